@@ -1,0 +1,147 @@
+"""appy_amd - annotated Python loops on AMD MI355X (gfx950).
+
+``@jit`` rewrites every loop annotated with ``#pragma parallel for ...`` into a
+call of :func:`_kernel_launch`, which generates a HIP C++ kernel for the loop,
+compiles it with hiprtc and launches it through ``libappy_hip.so``.  The user
+surface (decorator, pragma grammar, by-value scalars, ``shared()`` scalars,
+NumPy arrays copied in and out, GPU tensors used in place) is the one of the
+reference package (reference tree: appy/__init__.py:18-151).
+"""
+from __future__ import annotations
+
+import ast
+import builtins as _builtins
+import inspect
+import sys
+import textwrap
+
+from .__version__ import __version__
+from . import dispatcher
+from .frontend import source as _source
+from .frontend import static_rewrite as _static_rewrite
+
+_DEFAULT_OPTIONS = (
+    ("backend", None),
+    ("dry_run", False),
+    ("dump_code", False),
+    ("dump_code_to_file", None),
+    ("verbose_static_rewrite", False),
+    ("verbose_block_loop", False),
+)
+
+
+def _kernel_launch(loop_source, loop_name, scope, global_scope, options):
+    """Run-time stub that stands where an annotated loop stood.
+
+    ``loop_source`` is the pragma line followed by the loop, ``loop_name`` is
+    ``kernel_loop_N``, ``scope``/``global_scope`` are ``locals()``/``globals()``
+    of the calling function (reference: appy/__init__.py:18-35)."""
+    dispatcher.codegen(options.get("backend"), loop_source, loop_name, scope, global_scope, options)
+
+
+def set_default_options(options):
+    for key, val in _DEFAULT_OPTIONS:
+        options.setdefault(key, val)
+
+
+def rewrite_loops(fn, **options):
+    """Source of ``fn`` -> rewritten function object (reference:
+    appy/__init__.py:38-65)."""
+    source = textwrap.dedent(inspect.getsource(fn))
+    tree = _source.parse(source)
+    if options.get("shader", False):
+        raise NotImplementedError("shader loops are not part of the HIP execution path")
+    tree, _loops = _static_rewrite.transform(tree, options)
+    new_source = ast.unparse(tree)
+    if options["verbose_static_rewrite"]:
+        print("[Static Rewrite] new code:\n", new_source)
+    code = compile(new_source, filename=f"<appy:{fn.__name__}>", mode="exec")
+    import numpy
+
+    g = fn.__globals__
+    g["numpy"] = numpy
+    # The stub is spelled `appy._kernel_launch`; make that name resolve even if
+    # the caller imported this package under another name.
+    g.setdefault("appy", sys.modules[__name__])
+    namespace = {}
+    exec(code, g, namespace)
+    new_fn = namespace[fn.__name__]
+    new_fn.__appy_source__ = new_source
+    return new_fn
+
+
+def jit(fn=None, **options):
+    set_default_options(options)
+    if fn:
+        return rewrite_loops(fn, **options)
+
+    def jit_with_args(fn1):
+        return rewrite_loops(fn1, **options)
+
+    return jit_with_args
+
+
+# ---- names usable inside annotated functions -------------------------------
+def vidx(start, stepsize, bound=None):
+    """Slice of at most ``stepsize`` indices from ``start``, clipped at
+    ``bound`` (reference: appy/__init__.py:95-100)."""
+    stop = start + stepsize
+    if bound:
+        stop = min(bound, stop)
+    return slice(start, stop)
+
+
+class prange(object):
+    """Parallel range: identical to ``range`` when executed by the interpreter
+    (reference: appy/__init__.py:105-110)."""
+
+    def __new__(cls, *args, shared=None):
+        return _builtins.range(*args)
+
+
+built_in_range = _builtins.range
+
+
+def range(*args, parallel=False, simd=False):  # noqa: A001 - mirrors the reference's name
+    return _builtins.range(*args)
+
+
+# ---- explicit data placement -------------------------------------------------
+def _to_gpu(a):
+    import torch
+
+    kind = f"{type(a).__module__}.{type(a).__name__}"
+    if kind == "numpy.ndarray":
+        return torch.from_numpy(a).to("cuda")
+    if isinstance(a, torch.Tensor):
+        return a.to("cuda")
+    if isinstance(a, list):
+        return torch.tensor(a).to("cuda")
+    if type(a) in (int, float):
+        return a
+    raise AssertionError("Unsupported type to transfer to GPU")
+
+
+def to_gpu(*args):
+    """NumPy arrays / tensors / lists -> tensors resident in HBM (reference:
+    appy/__init__.py:118-135; 'cuda' is the device name of ROCm builds of
+    PyTorch as well)."""
+    if len(args) == 1:
+        return _to_gpu(args[0])
+    return [_to_gpu(a) for a in args]
+
+
+def _to_cpu(a):
+    import torch
+
+    if isinstance(a, torch.Tensor):
+        if a.ndim == 0:
+            return a.item()
+        return a.to("cpu").numpy()
+    return a
+
+
+def to_cpu(*args):
+    if len(args) == 1:
+        return _to_cpu(args[0])
+    return [_to_cpu(a) for a in args]

@@ -1,0 +1,519 @@
+"""HIP back end: loop text + run-time values -> launcher.
+
+Entry point :func:`codegen` has the calling convention of the reference's back
+ends (reference tree: appy/backends/triton/codegen.py:9-74 and the call in
+appy/dispatcher.py:19-60): ``codegen(loop_source, loop_name, val_map, options)
+-> (f, code_src)`` where ``f(*args)`` takes the non-module values of
+``val_map`` positionally, returns nothing and delivers results by mutating its
+array arguments; ``code_src`` is the generated source (here: HIP C++).
+
+The launcher moves data as the reference's generated host code does
+(appy/backends/triton/passes/host_passes/gen_data_movement.py:25-87): NumPy
+arrays and CPU tensors are copied to the device before the launch and the ones
+the loop stores to are copied back afterwards; tensors that already live on
+the GPU are used in place, on PyTorch's current stream, without a
+synchronisation.
+"""
+from __future__ import annotations
+
+import ast
+import ctypes as C
+import hashlib
+import math
+import os
+import threading
+import types as _types
+
+import numpy as np
+
+from ...frontend import loop_ir
+from . import array_expr
+from . import dtypes as T
+from . import runtime as rt
+from .exprs import ArrayParam, ScalarParam
+from .kernelgen import KernelBuilder, KernelSource, LoopAnalysis, Spec, Unsupported
+
+ARCH = "gfx950"
+_HEADER_PATH = os.path.join(os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__)))), "csrc", "appy_device.h")
+
+code_cache = {}
+_cache_lock = threading.Lock()
+_device_header = None
+
+# Hardware facts used by the launch heuristics (MI355X: 256 CUs in 8 XCDs).
+DEFAULT_CUS = 256
+
+
+def device_header() -> str:
+    global _device_header
+    if _device_header is None:
+        with open(_HEADER_PATH) as f:
+            _device_header = f.read()
+    return _device_header
+
+
+# ---------------------------------------------------------------------------
+# classification of run-time values
+# ---------------------------------------------------------------------------
+def _kind(v) -> str:
+    return f"{type(v).__module__}.{type(v).__name__}"
+
+
+def is_numpy_array(v) -> bool:
+    return _kind(v) == "numpy.ndarray"
+
+
+def is_torch_tensor(v) -> bool:
+    return _kind(v) == "torch.Tensor" or (type(v).__module__.startswith("torch") and hasattr(v, "data_ptr"))
+
+
+def _torch_np_dtype(t):
+    import torch
+
+    table = {
+        torch.float32: np.float32, torch.float64: np.float64, torch.float16: np.float16,
+        torch.int8: np.int8, torch.uint8: np.uint8, torch.int16: np.int16, torch.int32: np.int32,
+        torch.int64: np.int64, torch.bool: np.bool_,
+    }
+    if t.dtype not in table:
+        raise TypeError(f"tensor dtype {t.dtype} is not supported in generated kernels")
+    return np.dtype(table[t.dtype])
+
+
+def array_dtype(v) -> np.dtype:
+    return v.dtype if is_numpy_array(v) else _torch_np_dtype(v)
+
+
+def _signature(val_map):
+    sig = []
+    for k, v in val_map.items():
+        if isinstance(v, _types.ModuleType):
+            sig.append((k, "module"))
+        elif is_numpy_array(v) or is_torch_tensor(v):
+            sig.append((k, _kind(v), str(array_dtype(v)), v.ndim))
+        else:
+            ty = T.of_python_value(v)
+            sig.append((k, _kind(v), str(ty)))
+    return tuple(sig)
+
+
+# ---------------------------------------------------------------------------
+# compiled kernels
+# ---------------------------------------------------------------------------
+def _disk_cache_dir():
+    if os.environ.get("APPY_HIP_NO_DISK_CACHE") == "1":
+        return None
+    d = os.environ.get("APPY_HIP_CACHE_DIR") or os.path.join(os.path.expanduser("~"), ".cache", "appy_hip")
+    try:
+        os.makedirs(d, exist_ok=True)
+    except OSError:
+        return None
+    return d
+
+
+def compile_source(text: str, name: str) -> bytes:
+    """HIP C++ -> gfx950 code object, through hiprtc, with an on-disk cache
+    keyed on the source text and the compiler options."""
+    d = _disk_cache_dir()
+    path = None
+    if d:
+        h = hashlib.sha256()
+        h.update(text.encode())
+        h.update(repr(rt.BASE_COMPILE_OPTIONS).encode())
+        h.update(ARCH.encode())
+        path = os.path.join(d, h.hexdigest() + ".co")
+        if os.path.exists(path):
+            with open(path, "rb") as f:
+                return f.read()
+    code = rt.compile_to_code_object(text, name + ".hip", ARCH)
+    if path:
+        tmp = path + f".{os.getpid()}.tmp"
+        try:
+            with open(tmp, "wb") as f:
+                f.write(code)
+            os.replace(tmp, path)
+        except OSError:
+            pass
+    return code
+
+
+class Kernel:
+    """One compiled variant of a loop."""
+
+    def __init__(self, src: KernelSource):
+        self.src = src
+        self.code = compile_source(src.text, src.name)
+        self._funcs = {}   # device -> function handle
+        fields = [(f"f{i}", p.ctype) for i, p in enumerate(src.params)]
+        self.ArgStruct = type("Args" + src.name, (C.Structure,), {"_fields_": fields})
+        self._field_names = [f for f, _ in fields]
+
+    def function(self, device: int):
+        f = self._funcs.get(device)
+        if f is None:
+            mod = rt.Module(self.code)
+            f = (mod, mod.function(self.src.name))
+            self._funcs[device] = f
+        return f[1]
+
+
+# ---------------------------------------------------------------------------
+# the launcher
+# ---------------------------------------------------------------------------
+_current_device = [None]
+
+
+def _ensure_device(dev: int):
+    if _current_device[0] != dev:
+        rt.init(dev)
+        _current_device[0] = dev
+
+
+def _pow2ceil(x: float) -> int:
+    n = 1
+    while n < x:
+        n <<= 1
+    return n
+
+
+class CompiledLoop:
+    """Callable launcher of one annotated loop for one argument signature."""
+
+    def __init__(self, loop_source, loop_name, val_map, options):
+        self.loop_name = loop_name
+        self.options = dict(options)
+        self.arg_names = [k for k, v in val_map.items() if not isinstance(v, _types.ModuleType)]
+        self.module_names = [k for k, v in val_map.items() if isinstance(v, _types.ModuleType)]
+
+        tree = loop_ir.build(loop_source)
+        tree, shape_refs = array_expr.transform(tree, val_map)
+        self.tree = tree
+
+        arrays, scalars = {}, {}
+        for k, v in val_map.items():
+            if isinstance(v, _types.ModuleType):
+                continue
+            if is_numpy_array(v) or is_torch_tensor(v):
+                dt = array_dtype(v)
+                if not T.supported(dt):
+                    raise TypeError(f"array `{k}` has dtype {dt}, which is not supported in generated kernels")
+                arrays[k] = ArrayParam(k, T.from_dtype(dt), v.ndim)
+            else:
+                ty = T.of_python_value(v)
+                if ty is not None:
+                    scalars[k] = ScalarParam(k, ty)
+        # extents introduced by array statements: scalars filled in from the shapes at launch
+        self.derived_shapes = {}
+        for arr, dim in shape_refs:
+            nm = f"{arr}_shape_{dim}"
+            if nm not in scalars:
+                scalars[nm] = ScalarParam(nm, T.WEAK_INT)
+                self.derived_shapes[nm] = (arr, dim)
+        self.analysis = LoopAnalysis(tree, arrays, scalars)
+        a = self.analysis
+        self._lo_code = compile(ast.Expression(body=ast.fix_missing_locations(_copy(a.lo_node))), "<lo>", "eval")
+        self._hi_code = compile(ast.Expression(body=ast.fix_missing_locations(_copy(a.hi_node))), "<hi>", "eval")
+        self._simd_loops = self._collect_simd_loops()
+        self.kernels = {}   # Spec -> Kernel
+        self._lock = threading.Lock()
+        # default variant now: generation / compilation errors surface at first use of the loop
+        self.default_spec = self._default_spec()
+        self.code_src = self.kernel_for(self.default_spec).src.text
+        self.last_launch = None
+
+    # ---- variants ------------------------------------------------------------------
+    def _elem_sizes(self):
+        return [arr.ty.size for arr in self.analysis.arrays.values()] or [4]
+
+    def _default_spec(self) -> Spec:
+        a = self.analysis
+        v = max(1, min(4, 16 // max(self._elem_sizes())))
+        if a.kind == "flat":
+            if "simd" in a.pragma:
+                return Spec("flat", block=256, vec=v, unroll=4)
+            return Spec("flat", block=256, vec=1, unroll=1)
+        return Spec("team", block=256, vec=v, width=64)
+
+    def kernel_for(self, spec: Spec) -> Kernel:
+        k = self.kernels.get(spec)
+        if k is None:
+            with self._lock:
+                k = self.kernels.get(spec)
+                if k is None:
+                    builder = KernelBuilder(self.analysis, self.loop_name, self.module_names, spec)
+                    k = Kernel(builder.build(device_header()))
+                    self.kernels[spec] = k
+        return k
+
+    def _collect_simd_loops(self):
+        out = []
+        for n in ast.walk(self.analysis.outer):
+            if n is self.analysis.outer or not isinstance(n, ast.For):
+                continue
+            if "simd" not in (getattr(n, "pragma", None) or {}):
+                continue
+            lo, hi, _ = n.iter.args
+            extent = ast.Expression(body=ast.fix_missing_locations(ast.BinOp(left=_copy(hi), op=ast.Sub(), right=_copy(lo))))
+            streamed = []
+            for s in ast.walk(n):
+                if (isinstance(s, ast.Subscript) and isinstance(s.value, ast.Name)
+                        and s.value.id in self.analysis.arrays and isinstance(s.slice, ast.Name)
+                        and s.slice.id == n.target.id):
+                    streamed.append(s.value.id)
+            out.append((compile(extent, "<extent>", "eval"), streamed))
+        return out
+
+    def _estimate_trip(self, env, arrays, n_outer) -> float:
+        best = 0.0
+        for code, streamed in self._simd_loops:
+            try:
+                best = max(best, float(eval(code, {"__builtins__": {}}, env)))
+                continue
+            except Exception:
+                pass
+            for name in streamed:
+                v = arrays.get(name)
+                if v is not None and v.ndim == 1 and n_outer > 0:
+                    best = max(best, v.shape[0] / n_outer)
+        return best
+
+    def choose_spec(self, n_outer, env, arrays, restrict=True) -> Spec:
+        forced = self.options.get("hip_spec")
+        d = self.default_spec
+        if isinstance(forced, dict):
+            base = dict(kind=d.kind, block=d.block, vec=d.vec, unroll=d.unroll, width=d.width,
+                        restrict=restrict, stream_loads=d.stream_loads)
+            base.update(forced)
+            return Spec(**base)
+        if d.kind == "flat":
+            if d.vec > 1 and n_outer < d.block * d.vec * d.unroll:
+                return Spec("flat", block=d.block, vec=d.vec, unroll=1, restrict=restrict)
+            return Spec("flat", block=d.block, vec=d.vec, unroll=d.unroll, restrict=restrict)
+        trip = self._estimate_trip(env, arrays, n_outer)
+        v = d.vec
+        if trip < 2 * v:
+            v = 1
+        w = max(1, min(64, _pow2ceil(trip / (v * 1.0)) if trip > 0 else 1))
+        # keep at least two vector steps per lane before widening to the full wavefront
+        return Spec("team", block=d.block, vec=v, width=w, restrict=restrict)
+
+    def grid_for(self, spec: Spec, n_outer: int, cus: int = DEFAULT_CUS) -> int:
+        if spec.kind == "flat":
+            per_block = spec.block * spec.vec * spec.unroll
+            need = max(1, -(-n_outer // per_block))
+            cap = self.options.get("hip_max_blocks") or cus * 8
+            if self.analysis.outer_reductions:
+                cap = self.options.get("hip_max_blocks") or cus * 8
+            return int(min(need, cap))
+        tpb = spec.block // spec.width
+        need = max(1, -(-n_outer // tpb))
+        return int(min(need, 1 << 24))
+
+    # ---- call ------------------------------------------------------------------------
+    def __call__(self, *args):
+        if len(args) != len(self.arg_names):
+            raise TypeError(f"{self.loop_name} expects {len(self.arg_names)} arguments, got {len(args)}")
+        vals = dict(zip(self.arg_names, args))
+        plan = self.prepare(vals)
+        if plan is None:
+            return
+        plan.run()
+
+    def prepare(self, vals):
+        """Stage arguments on the device and pick the kernel variant.  Returns
+        a :class:`Launch` (None for an empty iteration space)."""
+        a = self.analysis
+        env = {k: v for k, v in vals.items() if k not in a.arrays}
+        env["np"] = np
+        env["math"] = math
+        lo = int(eval(self._lo_code, {"__builtins__": {}}, env))
+        hi = int(eval(self._hi_code, {"__builtins__": {}}, env))
+        if hi <= lo:
+            return None
+        arrays = {k: vals[k] for k in a.arrays}
+        return Launch(self, vals, arrays, env, lo, hi)
+
+
+class Launch:
+    """One staged launch: device pointers, argument block, grid."""
+
+    def __init__(self, loop: CompiledLoop, vals, arrays, env, lo, hi):
+        self.loop = loop
+        a = loop.analysis
+        self.lo, self.hi = lo, hi
+        self.temps = []          # (dptr, host ndarray (contiguous), original, stored)
+        self.keepalive = []
+        self.stream = 0
+        device = 0
+        # -- device and stream: PyTorch's when a GPU tensor takes part
+        gpu_tensors = [v for v in arrays.values() if is_torch_tensor(v) and v.device.type == "cuda"]
+        if gpu_tensors:
+            import torch
+
+            device = gpu_tensors[0].device.index or 0
+            self.stream = torch.cuda.current_stream(device).cuda_stream
+        _ensure_device(device)
+        self.device = device
+
+        # -- bounds of accesses indexed by the parallel loop variable
+        for name, dim, off in a.bound_checks:
+            ext = arrays[name].shape[dim]
+            if lo + off < 0 or hi - 1 + off >= ext:
+                raise IndexError(
+                    f"{loop.loop_name}: `{name}` has extent {ext} in dimension {dim} but the loop "
+                    f"range [{lo}, {hi}) indexes it at offset {off:+d}"
+                )
+
+        # -- device pointers and strides
+        self.ptr = {}
+        self.strides = {}
+        extents = []
+        for name, v in arrays.items():
+            arr = a.arrays[name]
+            if not (arr.loaded or arr.stored):
+                continue
+            if is_numpy_array(v):
+                host = v if v.flags["C_CONTIGUOUS"] else np.ascontiguousarray(v)
+                self._stage_host(name, host, v, arr.stored)
+            elif v.device.type == "cuda":
+                t = v
+                if t.ndim >= 1 and t.numel() > 1 and t.stride(-1) != 1:
+                    t = v.contiguous()
+                    if arr.stored:
+                        self.keepalive.append(("copy_back", v, t))
+                self.keepalive.append(t)
+                self.ptr[name] = t.data_ptr()
+                self.strides[name] = [t.stride(d) for d in range(t.ndim)]
+                extents.append((name, t.data_ptr(), t.numel() * t.element_size(), arr.stored))
+            else:
+                # CPU tensor: same path as NumPy through a shared-memory view
+                tc = v if v.is_contiguous() else v.contiguous()
+                host = tc.numpy()
+                self._stage_host(name, host, v if tc is v else ("tensor", v, tc), arr.stored)
+        for dptr, host, _orig, stored, name in self.temps:
+            extents.append((name, dptr, host.nbytes, stored))
+        restrict = not _overlaps(extents)
+
+        # -- kernel variant, argument block, grid
+        n_outer = hi - lo
+        spec = loop.choose_spec(n_outer, env, arrays, restrict=restrict)
+        self.kernel = loop.kernel_for(spec)
+        self.spec = spec
+        st = self.kernel.ArgStruct()
+        for fname, p in zip(self.kernel._field_names, self.kernel.src.params):
+            if p.role == "array":
+                val = self.ptr[p.source]
+            elif p.role == "stride":
+                val = int(self.strides[p.source][p.dim])
+            elif p.role == "scalar":
+                if p.source in loop.derived_shapes:
+                    an, dim = loop.derived_shapes[p.source]
+                    val = int(arrays[an].shape[dim])
+                else:
+                    val = vals[p.source]
+                    if isinstance(val, np.generic):
+                        val = val.item()
+            elif p.role == "shape":
+                val = int(arrays[p.source].shape[p.dim])
+            elif p.role == "lo":
+                val = lo
+            else:
+                val = hi
+            setattr(st, fname, val)
+        self.args = st
+        self.grid = (loop.grid_for(spec, n_outer), 1, 1)
+        self.block = (spec.block, 1, 1)
+        loop.last_launch = self
+
+    def _stage_host(self, name, host, original, stored):
+        nbytes = host.nbytes
+        dptr = rt.malloc(max(nbytes, 1))
+        if nbytes:
+            rt.memcpy_h2d(dptr, host.ctypes.data, nbytes, self.stream)
+        self.temps.append((dptr, host, original, stored, name))
+        self.ptr[name] = dptr
+        self.strides[name] = [s // host.itemsize for s in host.strides]
+
+    def function(self):
+        return self.kernel.function(self.device)
+
+    def launch_only(self):
+        rt.launch(self.function(), self.grid, self.block, self.args, self.stream)
+
+    def time_kernel(self, warmup=3, reps=20) -> float:
+        """Mean milliseconds per launch (HIP events on the launch stream)."""
+        return rt.launch_timed(self.function(), self.grid, self.block, self.args, self.stream, warmup=warmup, reps=reps)
+
+    def finish(self):
+        """Copy stored host arrays back and release staging buffers."""
+        try:
+            for dptr, host, original, stored, _name in self.temps:
+                if stored and host.nbytes:
+                    rt.memcpy_d2h(host.ctypes.data, dptr, host.nbytes, self.stream)
+                    if isinstance(original, tuple):          # non-contiguous CPU tensor
+                        _, dst, src = original
+                        dst.copy_(src)
+                    elif original is not host and is_numpy_array(original):
+                        original[...] = host
+            if self.temps:
+                rt.sync(self.stream)
+            for item in self.keepalive:
+                if isinstance(item, tuple) and item[0] == "copy_back":
+                    item[1].copy_(item[2])
+        finally:
+            for dptr, *_ in self.temps:
+                rt.free(dptr)
+            self.temps = []
+            self.keepalive = []
+
+    def run(self):
+        try:
+            self.launch_only()
+        except Exception:
+            for dptr, *_ in self.temps:
+                rt.free(dptr)
+            self.temps = []
+            raise
+        self.finish()
+
+
+def _overlaps(extents) -> bool:
+    """True if a stored array shares bytes with any other array argument."""
+    for i, (n1, p1, s1, st1) in enumerate(extents):
+        for j, (n2, p2, s2, st2) in enumerate(extents):
+            if i >= j or not (st1 or st2):
+                continue
+            if p1 < p2 + s2 and p2 < p1 + s1:
+                return True
+    return False
+
+
+def _copy(node):
+    import copy
+
+    return copy.deepcopy(node)
+
+
+# ---------------------------------------------------------------------------
+# entry point
+# ---------------------------------------------------------------------------
+def codegen(loop_source, loop_name, val_map, options):
+    key = (loop_source, loop_name, _signature(val_map), options.get("hip_spec") and repr(options.get("hip_spec")),
+           options.get("hip_max_blocks"))
+    hit = code_cache.get(key)
+    if hit is not None:
+        return hit
+    with _cache_lock:
+        hit = code_cache.get(key)
+        if hit is not None:
+            return hit
+        f = CompiledLoop(loop_source, loop_name, val_map, options)
+        code_cache[key] = (f, f.code_src)
+    if options.get("dump_code"):
+        print(f"--- Dumped code for loop {loop_name} ---")
+        print(f.code_src)
+        print(f"--- End of dumped code for loop {loop_name} ---")
+    if options.get("dump_code_to_file"):
+        with open(options["dump_code_to_file"], "w") as fh:
+            fh.write(f.code_src)
+    return f, f.code_src

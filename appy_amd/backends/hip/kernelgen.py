@@ -1,0 +1,724 @@
+"""Loop IR -> HIP C++ kernel text for gfx950.
+
+Two execution shapes cover every annotated loop:
+
+``flat``
+    ``#pragma parallel for simd`` (and parallel loops without inner ``simd``
+    loops): one lane per iteration.  Lanes take V consecutive iterations so
+    that ``X[i]`` accesses become one 128-bit load/store; a workgroup walks
+    tiles of ``BLOCK*U*V`` iterations with all loads of a tile issued before
+    its arithmetic.  Replaces the reference's 256-wide masked Triton program
+    per 256 iterations (reference tree: appy/backends/triton/passes/
+    block_loop.py:111-149, device_passes/remove_loop_head.py:20-48).
+
+``team``
+    ``#pragma parallel for`` whose body holds ``#pragma simd`` loops: one
+    team of W adjacent lanes (W = 1..64, a power of two) per outer iteration.
+    Statements outside ``simd`` loops run on every lane of the team with
+    identical values and their stores are issued by lane 0; ``simd`` loops are
+    spread over the lanes (V consecutive iterations per lane where the
+    accesses allow) and their reductions end with a DPP/shuffle butterfly over
+    the team.  Replaces the reference's one-program-per-outer-iteration
+    mapping with masked 256-wide chunks (SURVEY of the same passes).
+
+Reductions of the parallel loop itself (``shared`` scalars, detected as in
+appy/frontend/reduction_detection.py:76-104 of the reference) are kept in a
+register per lane, reduced over the wavefront with DPP moves, over the
+workgroup through LDS, and combined into memory with one atomic per
+workgroup - instead of the reference's one atomic per 256 iterations
+(device_passes/rewrite_par_reduce_to_atomics.py:18-55).
+"""
+from __future__ import annotations
+
+import ast
+import ctypes as C
+from dataclasses import dataclass, field
+
+from ...frontend import loop_ir
+from . import dtypes as T
+from .dtypes import Ty
+from .exprs import ArrayParam, ExprEmitter, ScalarParam, cast, cname, truth
+
+_OPS = {"+": "appy::OpAdd", "*": "appy::OpMul", "max": "appy::OpMax", "min": "appy::OpMin"}
+
+_CTYPES = {
+    "bool": C.c_bool, "int8": C.c_int8, "uint8": C.c_uint8, "int16": C.c_int16, "uint16": C.c_uint16,
+    "int32": C.c_int32, "uint32": C.c_uint32, "int64": C.c_int64, "uint64": C.c_uint64,
+    "float32": C.c_float, "float64": C.c_double,
+}
+
+
+@dataclass(frozen=True)
+class Spec:
+    """Launch-time selectable shape of a kernel."""
+
+    kind: str            # 'flat' | 'team'
+    block: int = 256     # threads per workgroup
+    vec: int = 1         # consecutive iterations per lane (V)
+    unroll: int = 1      # vectors per lane and tile (U), flat only
+    width: int = 1       # lanes per team (W), team only
+    restrict: bool = True
+    stream_loads: bool = False   # non-temporal loads for vectorised accesses
+
+    def tag(self) -> str:
+        return (f"{self.kind}_b{self.block}_v{self.vec}_u{self.unroll}_w{self.width}"
+                f"{'_r' if self.restrict else ''}{'_nt' if self.stream_loads else ''}")
+
+
+@dataclass
+class Param:
+    cname: str
+    ctype_decl: str      # C++ parameter declaration
+    ctype: object        # ctypes type
+    role: str            # 'array' | 'stride' | 'scalar' | 'shape' | 'lo' | 'hi'
+    source: str = ""     # python-side name (array / scalar name)
+    dim: int = 0
+
+
+@dataclass
+class OuterReduction:
+    key: str             # e.g. 's[0]'
+    op: str
+    array: str
+    index: int
+    ty: Ty
+    acc: str             # register name
+
+
+@dataclass
+class KernelSource:
+    name: str
+    text: str
+    params: list
+    spec: Spec
+    reductions: list
+    stored_arrays: list
+    bound_checks: list   # (array, dim, offset) accesses indexed by the parallel loop variable
+
+
+class Unsupported(NotImplementedError):
+    pass
+
+
+def _elts(sub: ast.Subscript):
+    return sub.slice.elts if isinstance(sub.slice, ast.Tuple) else [sub.slice]
+
+
+def _uses_name(node, name: str) -> bool:
+    return any(isinstance(n, ast.Name) and n.id == name for n in ast.walk(node))
+
+
+def _var_offset(node, var: str):
+    """``var`` -> 0, ``var + 3`` -> 3, ``var - 1`` -> -1, else None."""
+    if isinstance(node, ast.Name) and node.id == var:
+        return 0
+    if isinstance(node, ast.BinOp) and isinstance(node.op, (ast.Add, ast.Sub)):
+        l, r = node.left, node.right
+        if isinstance(l, ast.Name) and l.id == var and isinstance(r, ast.Constant) and type(r.value) is int:
+            return r.value if isinstance(node.op, ast.Add) else -r.value
+        if (isinstance(node.op, ast.Add) and isinstance(r, ast.Name) and r.id == var
+                and isinstance(l, ast.Constant) and type(l.value) is int):
+            return l.value
+    return None
+
+
+def _has_simd_loop(stmts) -> bool:
+    for st in stmts:
+        for n in ast.walk(st):
+            if isinstance(n, ast.For) and "simd" in (getattr(n, "pragma", None) or {}):
+                return True
+    return False
+
+
+class LoopAnalysis:
+    """Facts about a loop nest that do not depend on the launch shape."""
+
+    def __init__(self, tree: ast.Module, val_arrays: dict, val_scalars: dict):
+        self.tree = tree
+        self.outer = loop_ir.outer_loop(tree)
+        if not (isinstance(self.outer.iter, ast.Call) and isinstance(self.outer.iter.func, ast.Name)
+                and self.outer.iter.func.id in ("range", "prange") and len(self.outer.iter.args) == 3):
+            raise Unsupported(f"Parallel loops iterate over range(...): {ast.unparse(self.outer.iter)}")
+        if not isinstance(self.outer.target, ast.Name):
+            raise Unsupported("The loop variable must be a plain name")
+        self.var = self.outer.target.id
+        self.pragma = getattr(self.outer, "pragma", None) or {"parallel_for": True}
+        self.lo_node, self.hi_node, _ = self.outer.iter.args
+        self.arrays = val_arrays      # name -> ArrayParam
+        self.scalars = val_scalars    # name -> ScalarParam
+
+        self.assigned = []            # local names in order of first assignment
+        self.loop_vars = []
+        self.stored = set()
+        for n in ast.walk(self.outer):
+            if isinstance(n, ast.Assign):
+                t = n.targets[0]
+                if isinstance(t, ast.Name) and t.id not in self.assigned:
+                    self.assigned.append(t.id)
+                elif isinstance(t, ast.Subscript) and isinstance(t.value, ast.Name):
+                    self.stored.add(t.value.id)
+            elif isinstance(n, ast.For):
+                if isinstance(n.target, ast.Name):
+                    self.loop_vars.append(n.target.id)
+                else:
+                    raise Unsupported("Loop variables must be plain names")
+            elif isinstance(n, (ast.While, ast.Break, ast.Continue, ast.Return, ast.With, ast.Try, ast.FunctionDef,
+                                ast.Lambda, ast.ListComp, ast.Yield)):
+                raise Unsupported(f"Statement not supported in a kernel: {type(n).__name__}")
+        for name in self.stored:
+            if name in self.arrays:
+                self.arrays[name].stored = True
+            elif name not in self.assigned:
+                raise Unsupported(f"`{name}` is subscripted but is not an array argument")
+
+        is_simd = "simd" in self.pragma
+        self.kind = "flat" if (is_simd or not _has_simd_loop(self.outer.body)) else "team"
+
+        # reductions of the parallel loop: constant-subscript elements of arrays
+        self.outer_reductions = []
+        for key, op in loop_ir.reductions_of(self.outer).items():
+            try:
+                node = ast.parse(key, mode="eval").body
+            except SyntaxError:
+                continue
+            if (isinstance(node, ast.Subscript) and isinstance(node.value, ast.Name)
+                    and node.value.id in self.arrays and isinstance(node.slice, ast.Constant)
+                    and type(node.slice.value) is int and self.arrays[node.value.id].ndim == 1):
+                arr = self.arrays[node.value.id]
+                if arr.ty.size < 4:
+                    raise Unsupported(f"Reduction into a {arr.ty.name} element is not supported: {key}")
+                self.outer_reductions.append(
+                    OuterReduction(key, op, arr.name, node.slice.value, arr.ty, f"__acc{len(self.outer_reductions)}")
+                )
+
+        # accesses indexed directly by the parallel loop variable: checked on
+        # the host against the array extents before every launch
+        self.bound_checks = []
+        for n in ast.walk(self.outer):
+            if isinstance(n, ast.Subscript) and isinstance(n.value, ast.Name) and n.value.id in self.arrays:
+                for d, e in enumerate(_elts(n)):
+                    off = _var_offset(e, self.var)
+                    if off is not None and (n.value.id, d, off) not in self.bound_checks:
+                        self.bound_checks.append((n.value.id, d, off))
+
+
+class KernelBuilder:
+    def __init__(self, analysis: LoopAnalysis, kernel_name: str, module_names, spec: Spec):
+        self.a = analysis
+        self.name = kernel_name
+        self.spec = spec
+        self.ex = ExprEmitter(analysis.arrays, analysis.scalars, module_names)
+        self.lines = []
+        self.ind = 1
+        self.mode = "lane"
+        self.partials = {}        # reduction variable -> partial register, inside a spread simd loop
+        self.store_subst = {}     # unparsed subscript -> (lvalue code, Ty)
+        self.dirty = False
+        self.counter = 0
+        self.shadowed = [n for n in analysis.assigned if n in analysis.scalars]
+        self.red_by_key = {r.key: r for r in analysis.outer_reductions}
+
+    # ---- text helpers ------------------------------------------------------------
+    def w(self, line=""):
+        self.lines.append("    " * self.ind + line if line else "")
+
+    def fresh(self, stem):
+        self.counter += 1
+        return f"__{stem}{self.counter}"
+
+    # ---- types of locals ---------------------------------------------------------------
+    def set_local(self, name, ty: Ty):
+        old = self.ex.locals.get(name)
+        new = T.join(old, ty)
+        if new != old:
+            self.ex.locals[name] = new
+            self.dirty = True
+
+    # ---- statements ---------------------------------------------------------------
+    def block(self, stmts):
+        for st in stmts:
+            self.stmt(st)
+
+    def stmt(self, st):
+        if isinstance(st, ast.Assign):
+            return self.assign(st)
+        if isinstance(st, ast.For):
+            return self.for_(st)
+        if isinstance(st, ast.If):
+            return self.if_(st)
+        if isinstance(st, ast.Pass):
+            return
+        if isinstance(st, ast.Expr) and isinstance(st.value, ast.Constant):
+            return  # docstring-like
+        raise Unsupported(f"Statement not supported in a kernel: {ast.unparse(st)}")
+
+    def if_(self, st: ast.If):
+        c, t = self.ex.emit(st.test)
+        self.w(f"if ({truth(c, t)}) {{")
+        self.ind += 1
+        self.block(st.body)
+        self.ind -= 1
+        if st.orelse:
+            self.w("} else {")
+            self.ind += 1
+            self.block(st.orelse)
+            self.ind -= 1
+        self.w("}")
+
+    def assign(self, st: ast.Assign):
+        tgt = st.targets[0]
+        red_op = getattr(st, "reduce", None)
+        if isinstance(tgt, ast.Name):
+            name = tgt.id
+            if red_op and name in self.partials:
+                oc, ot = self.ex.emit(loop_ir.reduction_operand(st))
+                p, pty = self.partials[name]
+                self.w(f"{p} = {_OPS[red_op]}::f<{pty.c}>({p}, {cast(oc, ot, pty)});")
+                return
+            vc, vt = self.ex.emit(st.value)
+            self.set_local(name, vt)
+            lt = self.ex.locals[name]
+            self.w(f"{cname(name)} = {cast(vc, vt, lt)};")
+            return
+        if not (isinstance(tgt, ast.Subscript) and isinstance(tgt.value, ast.Name)):
+            raise Unsupported(f"Assignment target not supported in a kernel: {ast.unparse(tgt)}")
+        key = ast.unparse(tgt)
+        if red_op and key in self.red_by_key and self.red_by_key[key].op == red_op:
+            r = self.red_by_key[key]
+            oc, ot = self.ex.emit(loop_ir.reduction_operand(st))
+            upd = f"{r.acc} = {_OPS[r.op]}::f<{r.ty.c}>({r.acc}, {cast(oc, ot, r.ty)});"
+            if self.mode == "team":
+                self.w(f"if (__lane == 0) {{ {upd} }}")
+            else:
+                self.w(upd)
+            return
+        arr = self.a.arrays.get(tgt.value.id)
+        if arr is None:
+            raise Unsupported(f"`{tgt.value.id}` is subscripted but is not an array argument")
+        vc, vt = self.ex.emit(st.value)
+        if key in self.store_subst:
+            lv, lty = self.store_subst[key]
+            self.w(f"{lv} = {self._store_value(vc, vt, arr)};")
+            self.ex.load_subst[key] = ((f"({lv} != 0)" if arr.ty.is_bool else lv), arr.ty)
+            return
+        idx = self.ex.index_code(arr, tgt)
+        store = f"{cname(arr.name)}[{idx}] = {self._store_value(vc, vt, arr)};"
+        if self.mode == "team":
+            self.w(f"if (__lane == 0) {{ {store} }}")
+        else:
+            self.w(store)
+        # a later read of the same element in this iteration goes to memory again
+        self.ex.load_subst.pop(key, None)
+
+    def _store_value(self, vc, vt, arr: ArrayParam):
+        if arr.ty.is_bool:
+            return f"(unsigned char)({truth(vc, vt)})"
+        return cast(vc, vt, arr.ty)
+
+    # ---- loops ---------------------------------------------------------------------
+    def _range_args(self, st: ast.For):
+        it = st.iter
+        if not (isinstance(it, ast.Call) and isinstance(it.func, ast.Name) and it.func.id == "range"
+                and len(it.args) == 3):
+            raise Unsupported(f"Loops in a kernel iterate over range(...): {ast.unparse(it)}")
+        lc, lt = self.ex.emit(it.args[0])
+        hc, ht = self.ex.emit(it.args[1])
+        return cast(lc, lt, T.I64), cast(hc, ht, T.I64)
+
+    def for_(self, st: ast.For):
+        pragma = getattr(st, "pragma", None) or {}
+        if self.mode == "team" and "simd" in pragma:
+            return self.spread_loop(st)
+        var = st.target.id
+        lo, hi = self._range_args(st)
+        self.ex.locals[var] = T.WEAK_INT
+        hi_v = self.fresh("hi")
+        self.w(f"const appy::i64 {hi_v} = {hi};")
+        self.w(f"for (appy::i64 {cname(var)} = {lo}; {cname(var)} < {hi_v}; ++{cname(var)}) {{")
+        self.ind += 1
+        self.block(st.body)
+        self.ind -= 1
+        self.w("}")
+
+    def _vector_accesses(self, body, var: str):
+        """Loads ``X[.., var+c]`` (any depth) and unconditional top-level
+        stores ``X[.., var+c] = e`` of a loop body that can move V elements at
+        once.  Returns (loads, stores): lists of (key, array, subscript)."""
+        loads, stores = {}, {}
+        blocked = set()
+        inner_vars = {n.target.id for s in body for n in ast.walk(s) if isinstance(n, ast.For)}
+        for s in body:
+            for n in ast.walk(s):
+                if not (isinstance(n, ast.Subscript) and isinstance(n.value, ast.Name)
+                        and n.value.id in self.a.arrays):
+                    continue
+                arr = self.a.arrays[n.value.id]
+                el = _elts(n)
+                if len(el) != arr.ndim or any(isinstance(e, ast.Slice) for e in el):
+                    continue
+                off = _var_offset(el[-1], var)
+                ok = off is not None and not any(_uses_name(e, var) for e in el[:-1])
+                # indices that depend on variables of loops nested in the body change per inner iteration
+                ok = ok and not any(_uses_name(e, v) for e in el for v in inner_vars)
+                # indices may only use values that exist before the body starts
+                ok = ok and not any(_uses_name(e, v) for e in el[:-1] for v in self._assigned_in(body))
+                key = ast.unparse(n)
+                if isinstance(n.ctx, ast.Load):
+                    if ok:
+                        loads[key] = (arr, n)
+                else:
+                    top = any(isinstance(t, ast.Assign) and t.targets[0] is n for t in body)
+                    if ok and top:
+                        stores[key] = (arr, n)
+                    else:
+                        blocked.add(arr.name)
+        # an array written through a non-vector path must not be cached in registers
+        for key in [k for k, (arr, _) in loads.items() if arr.name in blocked]:
+            del loads[key]
+        for key in [k for k, (arr, _) in stores.items() if arr.name in blocked]:
+            del stores[key]
+        # a vector store to an array that is also read at another offset would reorder accesses
+        for key, (arr, _) in list(stores.items()):
+            if any(a2.name == arr.name and k2 != key for k2, (a2, _) in loads.items()):
+                del stores[key]
+                loads = {k: v for k, v in loads.items() if v[0].name != arr.name}
+        return loads, stores
+
+    def _assigned_in(self, body):
+        names = set()
+        for s in body:
+            for n in ast.walk(s):
+                if isinstance(n, ast.Assign) and isinstance(n.targets[0], ast.Name):
+                    names.add(n.targets[0].id)
+        return names
+
+    def _addr(self, arr: ArrayParam, sub: ast.Subscript, var: str, base_code: str) -> str:
+        """Address of ``sub`` with ``var`` replaced by ``base_code``."""
+        saved = self.ex.locals.get(var)
+        self.ex.locals[var] = T.WEAK_INT
+        try:
+            repl = _Rename(var, "__vbase").visit(_copy(sub))
+            self.ex.locals["__vbase"] = T.WEAK_INT
+            idx = self.ex.index_code(arr, repl)
+        finally:
+            self.ex.locals.pop("__vbase", None)
+            if saved is None:
+                self.ex.locals.pop(var, None)
+            else:
+                self.ex.locals[var] = saved
+        return f"{cname(arr.name)} + ({idx.replace('__vbase', base_code)})"
+
+    def vector_body(self, body, var: str, base_code: str, V: int, loads, stores, declare_locals=False):
+        """Emit V consecutive iterations starting at ``base_code``: vector
+        loads first, the V scalar bodies, vector stores last."""
+        regs = {}
+        comp = "xyzw"
+        ld = "vload_stream" if self.spec.stream_loads else "vload"
+        for key, (arr, sub) in loads.items():
+            r = self.fresh(f"ld_{arr.name}_")
+            regs[key] = r
+            self.w(f"const appy::vec<{arr.elem_c}, {V}>::type {r} = "
+                   f"appy::{ld}<{arr.elem_c}, {V}>({self._addr(arr, sub, var, base_code)});")
+        sregs = {}
+        for key, (arr, sub) in stores.items():
+            r = self.fresh(f"st_{arr.name}_")
+            sregs[key] = r
+            self.w(f"appy::vec<{arr.elem_c}, {V}>::type {r};")
+        for k in range(V):
+            self.w("{")
+            self.ind += 1
+            self.w(f"const appy::i64 {cname(var)} = {base_code} + {k};")
+            if declare_locals:
+                self._declare_locals()
+            saved_loads = dict(self.ex.load_subst)
+            for key, (arr, _) in loads.items():
+                code = f"{regs[key]}.{comp[k]}" if V > 1 else regs[key]
+                self.ex.load_subst[key] = ((f"({code} != 0)" if arr.ty.is_bool else code), arr.ty)
+            saved_stores = dict(self.store_subst)
+            for key, (arr, _) in stores.items():
+                self.store_subst[key] = ((f"{sregs[key]}.{comp[k]}" if V > 1 else sregs[key]), arr.ty)
+            self.block(body)
+            self.ex.load_subst = saved_loads
+            self.store_subst = saved_stores
+            self.ind -= 1
+            self.w("}")
+        for key, (arr, sub) in stores.items():
+            self.w(f"appy::vstore<{arr.elem_c}, {V}>({self._addr(arr, sub, var, base_code)}, {sregs[key]});")
+
+    def spread_loop(self, st: ast.For):
+        """A ``simd`` loop inside a team: iterations dealt to the W lanes."""
+        var = st.target.id
+        W, V = self.spec.width, self.spec.vec
+        lo, hi = self._range_args(st)
+        self.ex.locals[var] = T.WEAK_INT
+        reds = {}
+        for key, op in loop_ir.reductions_of(st).items():
+            if key in self.ex.locals or key in self.a.assigned:
+                reds[key] = op
+        self.w("{")
+        self.ind += 1
+        lo_v, hi_v = self.fresh("lo"), self.fresh("hi")
+        self.w(f"const appy::i64 {lo_v} = {lo};")
+        self.w(f"const appy::i64 {hi_v} = {hi};")
+        saved_partials = dict(self.partials)
+        for name, op in reds.items():
+            ty = self.ex.locals.get(name)
+            if ty is None:
+                raise NameError(f"reduction variable `{name}` has no value before the loop")
+            p = self.fresh(f"part_{name}_")
+            self.partials[name] = (p, ty)
+            self.w(f"{ty.c} {p} = {T.identity_literal(op, ty)};")
+        saved_mode = self.mode
+        self.mode = "lane"
+        loads, stores = self._vector_accesses(st.body, var) if V > 1 else ({}, {})
+        if V > 1 and (loads or stores):
+            nv = self.fresh("nv")
+            q = self.fresh("q")
+            self.w(f"const appy::i64 {nv} = ({hi_v} - {lo_v}) / {V};")
+            self.w("#pragma unroll 2")
+            self.w(f"for (appy::i64 {q} = __lane; {q} < {nv}; {q} += {W}) {{")
+            self.ind += 1
+            base = self.fresh("j")
+            self.w(f"const appy::i64 {base} = {lo_v} + {q} * {V};")
+            self.vector_body(st.body, var, base, V, loads, stores)
+            self.ind -= 1
+            self.w("}")
+            start = f"{lo_v} + {nv} * {V} + __lane"
+        else:
+            start = f"{lo_v} + __lane"
+        self.w(f"for (appy::i64 {cname(var)} = {start}; {cname(var)} < {hi_v}; {cname(var)} += {W}) {{")
+        self.ind += 1
+        self.block(st.body)
+        self.ind -= 1
+        self.w("}")
+        self.mode = saved_mode
+        for name, op in reds.items():
+            p, ty = self.partials[name]
+            if ty.size < 4:
+                raise Unsupported(f"Reduction variable `{name}` of type {ty.name} is not supported")
+            self.w(f"{cname(name)} = {_OPS[op]}::f<{ty.c}>({cname(name)}, appy::team_reduce<{_OPS[op]}, {W}, {ty.c}>({p}));")
+        self.partials = saved_partials
+        self.ind -= 1
+        self.w("}")
+
+    # ---- kernel skeletons ---------------------------------------------------------
+    def _declare_locals(self):
+        for name in self.a.assigned:
+            ty = self.ex.locals.get(name)
+            if ty is None:
+                continue
+            init = f" = {cname(name)}__arg" if name in self.shadowed else " = 0"
+            self.w(f"{ty.c} {cname(name)}{init};")
+
+    def _iteration(self, idx_code: str):
+        self.w("{")
+        self.ind += 1
+        self.w(f"const appy::i64 {cname(self.a.var)} = {idx_code};")
+        self._declare_locals()
+        self.block(self.a.outer.body)
+        self.ind -= 1
+        self.w("}")
+
+    def _body_flat(self):
+        s = self.spec
+        V, U, B = s.vec, s.unroll, s.block
+        var = self.a.var
+        self.ex.locals[var] = T.WEAK_INT
+        loads, stores = self._vector_accesses(self.a.outer.body, var) if V > 1 else ({}, {})
+        vectorised = V > 1 and (loads or stores)
+        self.w("const appy::i64 __tid = threadIdx.x;")
+        self.w("const appy::i64 __nblk = gridDim.x;")
+        if vectorised:
+            tile = B * U * V
+            self.w(f"const appy::i64 __ntiles = (__hi - __lo) / {tile};")
+            self.w("for (appy::i64 __t = blockIdx.x; __t < __ntiles; __t += __nblk) {")
+            self.ind += 1
+            self.w(f"const appy::i64 __tile0 = __lo + __t * {tile} + __tid * {V};")
+            if U == 1:
+                self.vector_body(self.a.outer.body, var, "__tile0", V, loads, stores, declare_locals=True)
+            else:
+                # all loads of the tile first, then the arithmetic, then the stores
+                self._flat_unrolled_tile(V, U, B, loads, stores)
+            self.ind -= 1
+            self.w("}")
+            self.w(f"const appy::i64 __rest0 = __lo + __ntiles * {tile};")
+            self.w(f"const appy::i64 __nrv = (__hi - __rest0) / {V};")
+            self.w(f"for (appy::i64 __q = blockIdx.x * {B}LL + __tid; __q < __nrv; __q += __nblk * {B}LL) {{")
+            self.ind += 1
+            self.w(f"const appy::i64 __vb = __rest0 + __q * {V};")
+            self.vector_body(self.a.outer.body, var, "__vb", V, loads, stores, declare_locals=True)
+            self.ind -= 1
+            self.w("}")
+            tail0 = f"__rest0 + __nrv * {V}"
+        else:
+            tail0 = "__lo"
+        self.w(f"for (appy::i64 __i = {tail0} + blockIdx.x * {B}LL + __tid; __i < __hi; __i += __nblk * {B}LL) {{")
+        self.ind += 1
+        self._iteration("__i")
+        self.ind -= 1
+        self.w("}")
+
+    def _flat_unrolled_tile(self, V, U, B, loads, stores):
+        comp = "xyzw"
+        ld = "vload_stream" if self.spec.stream_loads else "vload"
+        var = self.a.var
+        regs = {}
+        for u in range(U):
+            base = f"(__tile0 + {u * B * V})"
+            for key, (arr, sub) in loads.items():
+                r = self.fresh(f"ld_{arr.name}_")
+                regs[(u, key)] = r
+                self.w(f"const appy::vec<{arr.elem_c}, {V}>::type {r} = "
+                       f"appy::{ld}<{arr.elem_c}, {V}>({self._addr(arr, sub, var, base)});")
+        sregs = {}
+        for u in range(U):
+            for key, (arr, sub) in stores.items():
+                r = self.fresh(f"st_{arr.name}_")
+                sregs[(u, key)] = r
+                self.w(f"appy::vec<{arr.elem_c}, {V}>::type {r};")
+        for u in range(U):
+            base = f"(__tile0 + {u * B * V})"
+            for k in range(V):
+                self.w("{")
+                self.ind += 1
+                self.w(f"const appy::i64 {cname(var)} = {base} + {k};")
+                self._declare_locals()
+                saved_loads = dict(self.ex.load_subst)
+                saved_stores = dict(self.store_subst)
+                for key, (arr, _) in loads.items():
+                    code = f"{regs[(u, key)]}.{comp[k]}"
+                    self.ex.load_subst[key] = ((f"({code} != 0)" if arr.ty.is_bool else code), arr.ty)
+                for key, (arr, _) in stores.items():
+                    self.store_subst[key] = (f"{sregs[(u, key)]}.{comp[k]}", arr.ty)
+                self.block(self.a.outer.body)
+                self.ex.load_subst = saved_loads
+                self.store_subst = saved_stores
+                self.ind -= 1
+                self.w("}")
+        for u in range(U):
+            base = f"(__tile0 + {u * B * V})"
+            for key, (arr, sub) in stores.items():
+                self.w(f"appy::vstore<{arr.elem_c}, {V}>({self._addr(arr, sub, var, base)}, {sregs[(u, key)]});")
+
+    def _body_team(self):
+        s = self.spec
+        W, B = s.width, s.block
+        tpb = B // W
+        var = self.a.var
+        self.ex.locals[var] = T.WEAK_INT
+        self.w(f"const int __lane = threadIdx.x & {W - 1};")
+        self.w(f"const appy::i64 __team = threadIdx.x / {W};")
+        self.w(f"for (appy::i64 __i = __lo + blockIdx.x * {tpb}LL + __team; __i < __hi; __i += gridDim.x * {tpb}LL) {{")
+        self.ind += 1
+        self.mode = "team"
+        self._iteration("__i")
+        self.mode = "lane"
+        self.ind -= 1
+        self.w("}")
+
+    def _epilogue(self):
+        B = self.spec.block
+        for r in self.a.outer_reductions:
+            ident = T.identity_literal(r.op, r.ty)
+            self.w("{")
+            self.ind += 1
+            self.w(f"const {r.ty.c} __tot = appy::block_reduce<{_OPS[r.op]}, {B}, {r.ty.c}>({r.acc}, {ident});")
+            self.w(f"if (threadIdx.x == 0) appy::atomic_combine<{_OPS[r.op]}, {r.ty.c}>::run(&{cname(r.array)}[{r.index}], __tot);")
+            self.ind -= 1
+            self.w("}")
+
+    # ---- parameters -----------------------------------------------------------------
+    def _params(self):
+        params = []
+        used_arrays = [a for a in self.a.arrays.values() if a.loaded or a.stored]
+        rs = " __restrict__" if self.spec.restrict else ""
+        for arr in used_arrays:
+            const = "" if arr.stored else "const "
+            params.append(Param(cname(arr.name), f"{const}{arr.elem_c}*{rs} {cname(arr.name)}", C.c_void_p, "array", arr.name))
+        for arr in used_arrays:
+            for d in range(arr.ndim - 1):
+                nm = f"{cname(arr.name)}_stride_{d}"
+                params.append(Param(nm, f"const appy::i64 {nm}", C.c_int64, "stride", arr.name, d))
+        for sc in self.a.scalars.values():
+            if sc.name not in self.used_scalars:
+                continue
+            nm = cname(sc.name) + ("__arg" if sc.name in self.shadowed else "")
+            params.append(Param(nm, f"const {sc.ty.c} {nm}", _CTYPES[sc.ty.name], "scalar", sc.name))
+        for arr, dim in sorted(self.ex.shape_scalars):
+            nm = cname(f"{arr}_shape_{dim}")
+            if any(p.cname == nm for p in params):
+                continue
+            params.append(Param(nm, f"const appy::i64 {nm}", C.c_int64, "shape", arr, dim))
+        params.append(Param("__lo", "const appy::i64 __lo", C.c_int64, "lo"))
+        params.append(Param("__hi", "const appy::i64 __hi", C.c_int64, "hi"))
+        return params
+
+    # ---- driver ------------------------------------------------------------------------
+    def _emit_body(self):
+        self.lines = []
+        self.ind = 1
+        self.counter = 0
+        self.ex.load_subst = {}
+        self.store_subst = {}
+        self.partials = {}
+        for r in self.a.outer_reductions:
+            self.w(f"{r.ty.c} {r.acc} = {T.identity_literal(r.op, r.ty)};")
+        if self.spec.kind == "flat":
+            self._body_flat()
+        else:
+            self._body_team()
+        self._epilogue()
+
+    def build(self, header: str) -> KernelSource:
+        # names of shapes produced by array-statement lowering act as scalars
+        for it in range(8):
+            self.dirty = False
+            self._emit_body()
+            if not self.dirty:
+                break
+        else:
+            raise Unsupported("types of local variables do not settle")
+        body = "\n".join(self.lines)
+        self.used_scalars = set()
+        for sc in self.a.scalars.values():
+            if _word_in(cname(sc.name), body) or sc.name in self.shadowed:
+                self.used_scalars.add(sc.name)
+        params = self._params()
+        sig = ",\n    ".join(p.ctype_decl for p in params)
+        text = (
+            f"{header}\n"
+            f"// kernel for {self.name}: {self.spec.tag()}\n"
+            f'extern "C" __global__ void __launch_bounds__({self.spec.block})\n'
+            f"_{self.name}(\n    {sig})\n{{\n{body}\n}}\n"
+        )
+        return KernelSource(
+            name="_" + self.name,
+            text=text,
+            params=params,
+            spec=self.spec,
+            reductions=list(self.a.outer_reductions),
+            stored_arrays=sorted(n for n in self.a.stored if n in self.a.arrays),
+            bound_checks=list(self.a.bound_checks),
+        )
+
+
+def _word_in(word: str, text: str) -> bool:
+    import re
+
+    return re.search(r"(?<![A-Za-z0-9_])" + re.escape(word) + r"(?![A-Za-z0-9_])", text) is not None
+
+
+def _copy(node):
+    import copy
+
+    return copy.deepcopy(node)
+
+
+class _Rename(ast.NodeTransformer):
+    def __init__(self, old, new):
+        self.old, self.new = old, new
+
+    def visit_Name(self, node):
+        if node.id == self.old:
+            return ast.copy_location(ast.Name(id=self.new, ctx=node.ctx), node)
+        return node

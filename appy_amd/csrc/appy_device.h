@@ -1,0 +1,221 @@
+// appy_device.h - device-side support code for generated kernels (gfx950).
+//
+// This text is placed in front of every generated kernel before it is handed
+// to hiprtc, so it may only use compiler builtins and the HIP device headers.
+// Wavefronts are 64 lanes wide; a "team" is a power-of-two group of adjacent
+// lanes (2..64) that executes one iteration of a parallel loop together.
+#if !defined(__HIPCC_RTC__)
+#include <hip/hip_runtime.h>  // hiprtc has the device API built in; hipcc needs the header
+#endif
+
+namespace appy {
+
+typedef long long i64;
+
+// ---- unaligned-tolerant vector access ---------------------------------------
+// Element-aligned vectors: global memory accepts dwordx2/x4 accesses at any
+// element-aligned address, so rows that start at arbitrary offsets can still be
+// streamed with wide loads.
+template <typename T, int V>
+struct vec {
+    typedef T type __attribute__((ext_vector_type(V), aligned(alignof(T))));
+};
+
+template <typename T, int V>
+__device__ __forceinline__ typename vec<T, V>::type vload(const T* p) {
+    return *reinterpret_cast<const typename vec<T, V>::type*>(p);
+}
+
+template <typename T, int V>
+__device__ __forceinline__ void vstore(T* p, typename vec<T, V>::type v) {
+    *reinterpret_cast<typename vec<T, V>::type*>(p) = v;
+}
+
+// Streaming variants: data that is touched once should not displace reused
+// lines (x of SpMV/GEMV, B rows of SpMM) from the L2.
+template <typename T, int V>
+__device__ __forceinline__ typename vec<T, V>::type vload_stream(const T* p) {
+    return __builtin_nontemporal_load(reinterpret_cast<const typename vec<T, V>::type*>(p));
+}
+
+template <typename T, int V>
+__device__ __forceinline__ void vstore_stream(T* p, typename vec<T, V>::type v) {
+    __builtin_nontemporal_store(v, reinterpret_cast<typename vec<T, V>::type*>(p));
+}
+
+template <typename T>
+__device__ __forceinline__ T load_stream(const T* p) {
+    return __builtin_nontemporal_load(p);
+}
+
+// ---- Python arithmetic that differs from C ------------------------------------
+template <typename T>
+__device__ __forceinline__ T floordiv_int(T a, T b) {
+    T q = a / b;
+    T r = a % b;
+    return ((r != 0) && ((r < 0) != (b < 0))) ? q - 1 : q;
+}
+
+template <typename T>
+__device__ __forceinline__ T mod_int(T a, T b) {
+    T r = a % b;
+    return ((r != 0) && ((r < 0) != (b < 0))) ? r + b : r;
+}
+
+__device__ __forceinline__ float mod_float(float a, float b) {
+    float r = fmodf(a, b);
+    return ((r != 0.0f) && ((r < 0.0f) != (b < 0.0f))) ? r + b : r;
+}
+
+__device__ __forceinline__ double mod_float(double a, double b) {
+    double r = fmod(a, b);
+    return ((r != 0.0) && ((r < 0.0) != (b < 0.0))) ? r + b : r;
+}
+
+template <typename T>
+__device__ __forceinline__ T ipow(T base, i64 e) {
+    T r = (T)1;
+    if (e < 0) return (T)0;
+    while (e) {
+        if (e & 1) r *= base;
+        base *= base;
+        e >>= 1;
+    }
+    return r;
+}
+
+// ---- reduction operators --------------------------------------------------------
+struct OpAdd {
+    template <typename T>
+    __device__ static __forceinline__ T f(T a, T b) { return a + b; }
+};
+struct OpMul {
+    template <typename T>
+    __device__ static __forceinline__ T f(T a, T b) { return a * b; }
+};
+struct OpMax {  // Python's max(a, b): b only if it is greater
+    template <typename T>
+    __device__ static __forceinline__ T f(T a, T b) { return (b > a) ? b : a; }
+};
+struct OpMin {
+    template <typename T>
+    __device__ static __forceinline__ T f(T a, T b) { return (b < a) ? b : a; }
+};
+
+// ---- cross-lane movement ----------------------------------------------------------
+// DPP controls (GFX9): quad_perm[1,0,3,2]=0xB1, quad_perm[2,3,0,1]=0x4E,
+// row_half_mirror=0x141, row_mirror=0x140.  All four stay inside a row of 16
+// lanes, so teams of up to 16 lanes reduce without touching the LDS crossbar.
+template <int CTRL>
+__device__ __forceinline__ int dpp_i32(int x) {
+    return __builtin_amdgcn_update_dpp(x, x, CTRL, 0xf, 0xf, false);
+}
+
+template <int CTRL, typename T>
+__device__ __forceinline__ T dpp_move(T v) {
+    static_assert(sizeof(T) == 4 || sizeof(T) == 8, "cross-lane values are 4 or 8 bytes");
+    if constexpr (sizeof(T) == 4) {
+        return __builtin_bit_cast(T, dpp_i32<CTRL>(__builtin_bit_cast(int, v)));
+    } else {
+        unsigned long long u = __builtin_bit_cast(unsigned long long, v);
+        unsigned lo = (unsigned)dpp_i32<CTRL>((int)(unsigned)(u & 0xffffffffull));
+        unsigned hi = (unsigned)dpp_i32<CTRL>((int)(unsigned)(u >> 32));
+        return __builtin_bit_cast(T, ((unsigned long long)hi << 32) | (unsigned long long)lo);
+    }
+}
+
+template <typename T>
+__device__ __forceinline__ T lane_xor(T v, int mask) {
+    static_assert(sizeof(T) == 4 || sizeof(T) == 8, "cross-lane values are 4 or 8 bytes");
+    const int src = ((int)__lane_id() ^ mask) << 2;
+    if constexpr (sizeof(T) == 4) {
+        return __builtin_bit_cast(T, __builtin_amdgcn_ds_bpermute(src, __builtin_bit_cast(int, v)));
+    } else {
+        unsigned long long u = __builtin_bit_cast(unsigned long long, v);
+        unsigned lo = (unsigned)__builtin_amdgcn_ds_bpermute(src, (int)(unsigned)(u & 0xffffffffull));
+        unsigned hi = (unsigned)__builtin_amdgcn_ds_bpermute(src, (int)(unsigned)(u >> 32));
+        return __builtin_bit_cast(T, ((unsigned long long)hi << 32) | (unsigned long long)lo);
+    }
+}
+
+// Butterfly reduction over a team of W adjacent lanes (W = 1,2,4,...,64, teams
+// aligned to W).  Every lane of the team must be active; every lane returns the
+// same total.
+template <typename Op, int W, typename T>
+__device__ __forceinline__ T team_reduce(T v) {
+    static_assert(W >= 1 && W <= 64 && (W & (W - 1)) == 0, "team width is a power of two up to 64");
+    if constexpr (W >= 2) v = Op::f(v, dpp_move<0xB1>(v));
+    if constexpr (W >= 4) v = Op::f(v, dpp_move<0x4E>(v));
+    if constexpr (W >= 8) v = Op::f(v, dpp_move<0x141>(v));
+    if constexpr (W >= 16) v = Op::f(v, dpp_move<0x140>(v));
+    if constexpr (W >= 32) v = Op::f(v, lane_xor(v, 16));
+    if constexpr (W >= 64) v = Op::f(v, lane_xor(v, 32));
+    return v;
+}
+
+// Workgroup reduction: wavefront butterfly, one LDS slot per wavefront, then a
+// butterfly over the slots.  Must be reached by every thread of the workgroup.
+// The total is returned in every lane of wavefront 0 (only).
+template <typename Op, int BLOCK, typename T>
+__device__ __forceinline__ T block_reduce(T v, T identity) {
+    static_assert(BLOCK % 64 == 0 && BLOCK <= 1024, "workgroup is a whole number of wavefronts");
+    constexpr int NW = BLOCK / 64;
+    v = team_reduce<Op, 64>(v);
+    if constexpr (NW == 1) {
+        return v;
+    } else {
+        __shared__ T slots[NW];
+        const int wave = threadIdx.x >> 6;
+        const int lane = threadIdx.x & 63;
+        if (lane == 0) slots[wave] = v;
+        __syncthreads();
+        T r = identity;
+        if (wave == 0) {
+            r = (lane < NW) ? slots[lane] : identity;
+            constexpr int W2 = NW <= 2 ? 2 : NW <= 4 ? 4 : NW <= 8 ? 8 : 16;
+            r = team_reduce<Op, W2>(r);
+        }
+        __syncthreads();  // slots may be reused by the next reduction
+        return r;
+    }
+}
+
+// ---- atomics on device memory -------------------------------------------------------
+template <int N>
+struct uint_of;
+template <>
+struct uint_of<4> {
+    typedef unsigned int type;
+};
+template <>
+struct uint_of<8> {
+    typedef unsigned long long type;
+};
+
+template <typename Op, typename T>
+__device__ __forceinline__ void atomic_cas_combine(T* p, T v) {
+    typedef typename uint_of<sizeof(T)>::type U;
+    U* up = reinterpret_cast<U*>(p);
+    U seen = __hip_atomic_load(up, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    for (;;) {
+        const T next = Op::f(__builtin_bit_cast(T, seen), v);
+        const U want = __builtin_bit_cast(U, next);
+        if (want == seen) return;
+        if (__hip_atomic_compare_exchange_strong(up, &seen, want, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                                 __HIP_MEMORY_SCOPE_AGENT))
+            return;
+    }
+}
+
+template <typename Op, typename T>
+struct atomic_combine {
+    __device__ static __forceinline__ void run(T* p, T v) { atomic_cas_combine<Op, T>(p, v); }
+};
+template <typename T>
+struct atomic_combine<OpAdd, T> {  // hardware add for 32/64-bit integers, float and double
+    __device__ static __forceinline__ void run(T* p, T v) {
+        __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+};
+
+}  // namespace appy

@@ -1,0 +1,250 @@
+"""Per-loop front end: loop text -> loop IR.
+
+The loop IR is a standard ``ast.Module`` holding one ``For`` nest in which
+
+* every ``range`` call has the three arguments ``(start, stop, 1)``,
+* tuple assignments and augmented assignments are expanded to plain ones,
+* ``For`` and ``Assign`` nodes that follow a pragma carry a ``pragma`` dict,
+* assignments that are reductions carry ``reduce`` (one of ``+ * max min``)
+  and the annotated loop around them lists them as
+  ``pragma['reduction'] = 'op:target,...'``.
+
+This is the form the reference's back ends consume (reference tree:
+appy/backends/triton/codegen.py:18-32 runs sanity_check, rewrite_tuple_assign,
+rewrite_aug_assign, rewrite_range, attach_pragma and reduction_detection from
+appy/frontend/ in that order); the rules below restate those passes.
+"""
+from __future__ import annotations
+
+import ast
+import copy
+
+from . import source as src
+from .pragma import is_pragma_text, parse_pragma
+
+REDUCTION_OPS = ("+", "*", "max", "min")
+
+
+# --------------------------------------------------------------------------
+# structure checks (reference: appy/frontend/sanity_check.py:4-18)
+# --------------------------------------------------------------------------
+def check_structure(tree: ast.Module) -> None:
+    loops = sum(isinstance(n, ast.For) for n in tree.body)
+    if loops > 1:
+        raise Exception(f"Input AST should only contain a single for loop while {loops} found.")
+    assert tree.body and src.pragma_text(tree.body[0]) is not None, "Input AST should start with a pragma"
+
+
+# --------------------------------------------------------------------------
+# statement normalisation
+# --------------------------------------------------------------------------
+class _Normalise(ast.NodeTransformer):
+    """Tuple assignment, augmented assignment and ``range`` normal forms
+    (reference: appy/frontend/rewrite_tuple_assign.py:4-17,
+    rewrite_aug_assign.py:5-20, rewrite_range.py:4-27)."""
+
+    def visit_Assign(self, node):
+        self.generic_visit(node)
+        if isinstance(node.value, ast.Tuple):
+            tgt = node.targets[0]
+            assert isinstance(tgt, ast.Tuple) and len(tgt.elts) == len(node.value.elts), (
+                "a tuple on the right-hand side needs a tuple of the same length on the left"
+            )
+            return [
+                ast.copy_location(ast.Assign(targets=[t], value=v), node)
+                for t, v in zip(tgt.elts, node.value.elts)
+            ]
+        return node
+
+    def visit_AugAssign(self, node):
+        self.generic_visit(node)
+        read = copy.deepcopy(node.target)
+        read.ctx = ast.Load()
+        return ast.copy_location(
+            ast.Assign(targets=[node.target], value=ast.BinOp(left=read, op=node.op, right=node.value)), node
+        )
+
+    def visit_Call(self, node):
+        self.generic_visit(node)
+        if isinstance(node.func, ast.Name) and node.func.id == "range":
+            n = len(node.args)
+            if n == 1:
+                node.args = [ast.Constant(value=0), node.args[0], ast.Constant(value=1)]
+            elif n == 2:
+                node.args = [node.args[0], node.args[1], ast.Constant(value=1)]
+            elif n == 3:
+                step = node.args[2]
+                if not (isinstance(step, ast.Constant) and step.value == 1 and not isinstance(step.value, bool)):
+                    raise Exception(f"Only step 1 is supported in range, got: {ast.unparse(node)}")
+            else:
+                raise Exception(f"range expects 1 to 3 arguments, got: {ast.unparse(node)}")
+        return node
+
+
+# --------------------------------------------------------------------------
+# pragma attachment (reference: appy/frontend/attach_pragma.py:4-24)
+# --------------------------------------------------------------------------
+def _attach_pragmas(stmts, pending):
+    """A pragma belongs to the next ``For`` or ``Assign`` in program order; an
+    assignment consumes it (so ``#pragma simd`` written above ``s = 0.0``
+    leaves the following loop sequential).  Marker statements are removed."""
+    out = []
+    for st in stmts:
+        text = src.pragma_text(st)
+        if text is not None:
+            if is_pragma_text(text):
+                pending = text
+            continue
+        if isinstance(st, ast.For):
+            if pending is not None:
+                st.pragma = parse_pragma(pending)
+                pending = None
+            st.body, pending = _attach_pragmas(st.body, pending)
+            st.orelse, pending = _attach_pragmas(st.orelse, pending)
+        elif isinstance(st, ast.Assign):
+            if pending is not None:
+                st.pragma = parse_pragma(pending)
+                pending = None
+        else:
+            for f in ("body", "orelse"):
+                sub = getattr(st, f, None)
+                if isinstance(sub, list) and sub and isinstance(sub[0], ast.stmt):
+                    new, pending = _attach_pragmas(sub, pending)
+                    setattr(st, f, new)
+        out.append(st)
+    return out, pending
+
+
+# --------------------------------------------------------------------------
+# reduction detection (reference: appy/frontend/reduction_detection.py:19-104)
+# --------------------------------------------------------------------------
+def is_scalar_location(node) -> bool:
+    """A name, or an array element with a literal subscript (``s[0]``)."""
+    return isinstance(node, ast.Name) or (
+        isinstance(node, ast.Subscript) and isinstance(node.slice, ast.Constant)
+    )
+
+
+def reduction_operator(assign: ast.Assign):
+    """``+``/``*`` for ``t = t + e`` / ``t = e * t``; ``max``/``min`` for
+    ``t = max(t, e)``; None when the assignment is not of that shape."""
+    tgt = assign.targets[0]
+    if not is_scalar_location(tgt):
+        return None
+    key = ast.unparse(tgt)
+    val = assign.value
+
+    def same(e):
+        return is_scalar_location(e) and ast.unparse(e) == key
+
+    if isinstance(val, ast.BinOp) and isinstance(val.op, (ast.Add, ast.Mult)):
+        if same(val.left) or same(val.right):
+            return "+" if isinstance(val.op, ast.Add) else "*"
+    elif (
+        isinstance(val, ast.Call)
+        and isinstance(val.func, ast.Name)
+        and val.func.id in ("max", "min")
+        and len(val.args) >= 2
+    ):
+        if same(val.args[0]) or same(val.args[1]):
+            return val.func.id
+    return None
+
+
+def reduction_operand(assign: ast.Assign):
+    """The expression combined into the target by a reduction assignment."""
+    key = ast.unparse(assign.targets[0])
+    val = assign.value
+    if isinstance(val, ast.BinOp):
+        if is_scalar_location(val.left) and ast.unparse(val.left) == key:
+            return val.right
+        return val.left
+    a, b = val.args[0], val.args[1]
+    if is_scalar_location(a) and ast.unparse(a) == key:
+        return b
+    return a
+
+
+def _assignments_in(node):
+    for n in ast.walk(node):
+        if isinstance(n, ast.Assign):
+            yield n
+
+
+def _mark_all(tree: ast.Module) -> None:
+    seen = set()
+
+    def visit(node):
+        for child in ast.iter_child_nodes(node):
+            visit(child)
+        if isinstance(node, ast.For) and id(node) not in seen:
+            seen.add(id(node))
+            _mark_one(node)
+
+    def _mark_one(loop):
+        if not hasattr(loop, "pragma"):
+            return
+        ops_of = {}
+        for a in _assignments_in(loop):
+            tgt = a.targets[0]
+            if is_scalar_location(tgt):
+                ops_of.setdefault(ast.unparse(tgt), set()).add(reduction_operator(a))
+        found = {}
+        for a in _assignments_in(loop):
+            tgt = a.targets[0]
+            if not is_scalar_location(tgt):
+                continue
+            key = ast.unparse(tgt)
+            ops = ops_of.get(key, set())
+            if len(ops) == 1:
+                op = next(iter(ops))
+                if op is not None:
+                    a.reduce = op
+                    found[key] = op
+        pragma = loop.pragma
+        if found and ("parallel_for" in pragma or "simd" in pragma):
+            entries = []
+            if "reduction" in pragma:
+                spec = pragma["reduction"]
+                entries = list(spec) if isinstance(spec, (tuple, list)) else spec.split(",")
+            for key, op in found.items():
+                entry = f"{op}:{key}"
+                if entry not in entries:
+                    entries.append(entry)
+            pragma["reduction"] = ",".join(entries)
+
+    visit(tree)
+
+
+def reductions_of(loop: ast.For) -> dict:
+    """``{'s[0]': '+'}`` from ``loop.pragma['reduction']``."""
+    pragma = getattr(loop, "pragma", None) or {}
+    out = {}
+    if "reduction" in pragma:
+        spec = pragma["reduction"]
+        items = spec if isinstance(spec, (tuple, list)) else spec.split(",")
+        for item in items:
+            op, _, var = item.partition(":")
+            out[var.strip()] = op.strip()
+    return out
+
+
+# --------------------------------------------------------------------------
+# entry point
+# --------------------------------------------------------------------------
+def build(loop_source: str) -> ast.Module:
+    """Loop text (pragma line + ``for`` statement) -> loop IR."""
+    tree = src.parse(loop_source)
+    check_structure(tree)
+    tree = _Normalise().visit(tree)
+    tree.body, _ = _attach_pragmas(tree.body, None)
+    _mark_all(tree)
+    ast.fix_missing_locations(tree)
+    return tree
+
+
+def outer_loop(tree: ast.Module) -> ast.For:
+    for n in tree.body:
+        if isinstance(n, ast.For):
+            return n
+    raise Exception("The launch unit holds no for loop.")

@@ -1,0 +1,201 @@
+"""Decoration-time rewrite of an annotated function.
+
+Turns every loop annotated with ``#pragma parallel for ...`` (or iterating over
+``prange``) into a call of the run-time stub, keeping the rest of the function
+as ordinary Python.  The observable result follows the reference's four
+decoration-time passes (reference tree: appy/__init__.py:38-65,
+appy/frontend/hoist_shape_attr.py:4-48, appy/frontend/process_shared.py:4-75,
+appy/frontend/replace_pfor_with_stub.py:3-81):
+
+* ``X.shape[k]`` inside a ``for`` statement becomes the name ``X_shape_k`` and
+  the assignment ``X_shape_k = X.shape[k]`` is placed in front of the
+  (outermost) loop;
+* for ``shared(v, ...)`` the loop is bracketed by ``v = numpy.array([v])`` and
+  ``v = v.item()`` and every use of ``v`` in the loop reads ``v[0]``;
+* the loop is replaced by ``appy._kernel_launch(<loop text>, 'kernel_loop_N',
+  locals(), globals(), {options})`` where the loop text starts with the pragma
+  line and loops are numbered per function starting at 1;
+* decorators of the function are dropped so that executing the new source
+  does not decorate again.
+
+The implementation works on statement lists with pragma marker statements
+(see :mod:`appy_amd.frontend.source`) instead of comment nodes.
+"""
+from __future__ import annotations
+
+import ast
+import copy
+import re
+
+from . import source as src
+from .pragma import is_parallel_for_text
+
+_SHARED_CLAUSE = re.compile(r"shared\(([^)]*)\)")
+
+_BODY_FIELDS = ("body", "orelse", "finalbody")
+
+
+# --------------------------------------------------------------------------
+# X.shape[k] hoisting
+# --------------------------------------------------------------------------
+class _ShapeRefs(ast.NodeTransformer):
+    def __init__(self):
+        self.seen = []  # (array name, dim) in first-use order, no duplicates
+
+    def visit_Subscript(self, node):
+        self.generic_visit(node)
+        v = node.value
+        if (
+            isinstance(v, ast.Attribute)
+            and v.attr == "shape"
+            and isinstance(v.value, ast.Name)
+            and isinstance(node.slice, ast.Constant)
+            and isinstance(node.slice.value, int)
+            and isinstance(node.ctx, ast.Load)
+        ):
+            key = (v.value.id, node.slice.value)
+            if key not in self.seen:
+                self.seen.append(key)
+            return ast.copy_location(ast.Name(id=f"{key[0]}_shape_{key[1]}", ctx=ast.Load()), node)
+        return node
+
+
+def _hoist_shapes_in_block(stmts):
+    out = []
+    for st in stmts:
+        if isinstance(st, ast.For):
+            refs = _ShapeRefs()
+            st = refs.visit(st)
+            for name, dim in refs.seen:
+                out.append(ast.parse(f"{name}_shape_{dim} = {name}.shape[{dim}]").body[0])
+            out.append(st)
+            continue
+        for f in _BODY_FIELDS:
+            sub = getattr(st, f, None)
+            if isinstance(sub, list) and sub and isinstance(sub[0], ast.stmt):
+                setattr(st, f, _hoist_shapes_in_block(sub))
+        if isinstance(st, ast.Try):
+            for h in st.handlers:
+                h.body = _hoist_shapes_in_block(h.body)
+        out.append(st)
+    return out
+
+
+# --------------------------------------------------------------------------
+# shared(...) scalars and stub replacement
+# --------------------------------------------------------------------------
+class _NameToElement0(ast.NodeTransformer):
+    def __init__(self, names):
+        self.names = set(names)
+
+    def visit_Name(self, node):
+        if node.id in self.names:
+            return ast.copy_location(
+                ast.Subscript(value=ast.Name(id=node.id, ctx=ast.Load()), slice=ast.Constant(value=0), ctx=node.ctx),
+                node,
+            )
+        return node
+
+
+def shared_names(pragma_text: str):
+    names = []
+    for group in _SHARED_CLAUSE.findall(pragma_text):
+        names.extend(v.strip() for v in group.split(",") if v.strip())
+    return names
+
+
+def _is_prange_loop(node: ast.For) -> bool:
+    it = node.iter
+    if not isinstance(it, ast.Call):
+        return False
+    f = it.func
+    if isinstance(f, ast.Name) and f.id == "prange":
+        return True
+    return (
+        isinstance(f, ast.Attribute)
+        and f.attr == "prange"
+        and isinstance(f.value, ast.Name)
+        and f.value.id == "appy"
+    )
+
+
+class _LoopOutliner:
+    def __init__(self, options):
+        self.options = dict(options)
+        self.count = 0
+        self.pending = None  # text of the last unconsumed '#pragma parallel for' comment
+        self.loops = []      # (loop name, loop text) in order, for inspection
+
+    def _stub(self, loop_text: str, loop_name: str) -> ast.Expr:
+        call = ast.Call(
+            func=ast.Attribute(value=ast.Name(id="appy", ctx=ast.Load()), attr="_kernel_launch", ctx=ast.Load()),
+            args=[
+                ast.Constant(value=loop_text),
+                ast.Constant(value=loop_name),
+                ast.Call(func=ast.Name(id="locals", ctx=ast.Load()), args=[], keywords=[]),
+                ast.Call(func=ast.Name(id="globals", ctx=ast.Load()), args=[], keywords=[]),
+                ast.Dict(
+                    keys=[ast.Constant(value=k) for k in self.options],
+                    values=[ast.Constant(value=v) for v in self.options.values()],
+                ),
+            ],
+            keywords=[],
+        )
+        return ast.fix_missing_locations(ast.Expr(value=call))
+
+    def _outline(self, loop: ast.For):
+        pragma, self.pending = self.pending, None
+        self.count += 1
+        loop_name = f"kernel_loop_{self.count}"
+        pre, post = [], []
+        if pragma:
+            shared = shared_names(pragma)
+            if shared:
+                loop = _NameToElement0(shared).visit(copy.deepcopy(loop))
+                for v in shared:
+                    pre.append(ast.parse(f"{v} = numpy.array([{v}])").body[0])
+                    post.append(ast.parse(f"{v} = {v}.item()").body[0])
+            loop_text = pragma + "\n" + src.unparse(loop)
+        else:
+            loop_text = src.unparse(loop)
+        self.loops.append((loop_name, loop_text))
+        return pre + [self._stub(loop_text, loop_name)] + post
+
+    def block(self, stmts):
+        out = []
+        for st in stmts:
+            text = src.pragma_text(st)
+            if text is not None:
+                if is_parallel_for_text(text):
+                    self.pending = text
+                # any other pragma outside a parallel loop has no meaning here
+                continue
+            if isinstance(st, ast.For) and (self.pending or _is_prange_loop(st)):
+                out.extend(self._outline(st))
+                continue
+            for f in _BODY_FIELDS:
+                sub = getattr(st, f, None)
+                if isinstance(sub, list) and sub and isinstance(sub[0], ast.stmt):
+                    new = self.block(sub)
+                    setattr(st, f, new if new or f != "body" else [ast.Pass()])
+            if isinstance(st, ast.Try):
+                for h in st.handlers:
+                    h.body = self.block(h.body) or [ast.Pass()]
+            out.append(st)
+        return out
+
+
+def transform(tree: ast.Module, options) -> tuple[ast.Module, list]:
+    """Rewrite a module holding one function definition.
+
+    Returns the new module and the list of ``(loop name, loop text)`` pairs
+    that were outlined.
+    """
+    tree.body = _hoist_shapes_in_block(tree.body)
+    for node in tree.body:
+        if isinstance(node, (ast.FunctionDef, ast.AsyncFunctionDef)):
+            node.decorator_list = []
+    outliner = _LoopOutliner(options)
+    tree.body = outliner.block(tree.body) or [ast.Pass()]
+    ast.fix_missing_locations(tree)
+    return tree, outliner.loops

@@ -1,0 +1,138 @@
+/*
+ * appy_hip.h - C ABI of libappy_hip.so, the device runtime underneath the APPy
+ * HIP code generator (gfx950 / MI355X).
+ *
+ * The reference has no native layer: its generated host launchers reach the GPU
+ * through PyTorch + Triton calls emitted as Python text.  Each entry point below
+ * names the reference construct whose job it takes over (paths are relative to
+ * the reference tree).  All functions are plain C: pointers, sizes and ints,
+ * no C++ or torch types.  Every function returns 0 on success; a non-zero value
+ * is a hipError_t (1..9999) or 10000 + hiprtcResult, and appy_hip_last_error()
+ * returns the matching text for the calling thread.
+ *
+ * Threading: all entry points may be called from several host threads at once.
+ * Streams are caller supplied (NULL = the null stream); launches and *_async
+ * calls are asynchronous with respect to the host.
+ */
+#ifndef APPY_HIP_H
+#define APPY_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define APPY_HIP_ABI_VERSION 1
+
+typedef struct appy_hip_props {
+    char     name[128];        /* marketing name */
+    char     arch[64];         /* gcnArchName, e.g. "gfx950:sramecc+:xnack-" */
+    int32_t  compute_units;    /* CUs on the device */
+    int32_t  wavefront_size;   /* 64 on CDNA */
+    int32_t  max_threads_per_block;
+    int32_t  lds_bytes_per_block;
+    int32_t  l2_bytes;
+    int32_t  clock_khz;
+    int32_t  mem_clock_khz;
+    int32_t  mem_bus_bits;
+    uint64_t hbm_bytes;
+} appy_hip_props;
+
+typedef struct appy_hip_func_info {
+    int32_t num_vgprs;         /* hipFuncAttributes.numRegs */
+    int32_t static_lds_bytes;  /* sharedSizeBytes */
+    int32_t scratch_bytes;     /* localSizeBytes: >0 means register spills */
+    int32_t max_threads_per_block;
+} appy_hip_func_info;
+
+/* ---- library ---------------------------------------------------------- */
+
+/* ABI version of the loaded library (APPY_HIP_ABI_VERSION). */
+int appy_hip_abi_version(void);
+
+/* Text of the last error raised on the calling thread ("" if none). */
+const char* appy_hip_last_error(void);
+
+/* ---- device ------------------------------------------------------------
+ * Replaces the reference's device discovery: shutil.which("nvidia-smi") in
+ * appy/dispatcher.py:37 and the literal 'cuda' device string in
+ * appy/backends/triton/passes/host_passes/gen_data_movement.py:48-62. */
+int appy_hip_device_count(int* count_out);
+int appy_hip_init(int device);                 /* make `device` current for this thread */
+int appy_hip_device_props(int device, appy_hip_props* out);
+
+/* ---- run-time compilation ----------------------------------------------
+ * Replaces @triton.jit on the generated `_kernel_loop_N`
+ * (appy/backends/triton/passes/gen_device_code.py:36-41) and the
+ * load_module_from_str step (appy/backends/triton/codegen.py:51-55): HIP C++
+ * source text -> gfx950 code object, via hiprtc.  Needs no GPU.
+ * `arch` is e.g. "gfx950"; `opts` are extra hiprtc options.  On success
+ * *code_out / *size_out hold a malloc'ed code object (free with
+ * appy_hip_code_free).  The compiler log of the last compile on this thread
+ * (warnings or errors) is returned by appy_hip_compile_log(). */
+int appy_hip_compile(const char* src, const char* name, const char* arch,
+                     const char* const* opts, int nopts,
+                     void** code_out, size_t* size_out);
+const char* appy_hip_compile_log(void);
+void appy_hip_code_free(void* code);
+
+/* Load a code object on the current device / look up an extern "C" kernel. */
+int appy_hip_module_load(const void* code, size_t size, void** module_out);
+int appy_hip_module_get_function(void* module, const char* kernel_name, void** func_out);
+int appy_hip_module_unload(void* module);
+int appy_hip_func_get_info(void* func, appy_hip_func_info* out);
+/* Resident workgroups per CU for `func` at this block size / dynamic LDS. */
+int appy_hip_occupancy(void* func, int block_threads, size_t dynamic_lds_bytes,
+                       int* blocks_per_cu_out);
+
+/* ---- device memory ------------------------------------------------------
+ * Replaces `__tg_x = __tc_x.to('cuda')` and `__tc_x.copy_(__tg_x)`
+ * (appy/backends/triton/passes/host_passes/gen_data_movement.py:25-87) for
+ * NumPy / CPU-tensor arguments.  Buffers come from a size-bucketed pool so a
+ * repeated call does not pay hipMalloc/hipFree; appy_hip_pool_trim releases
+ * everything the pool holds. */
+int appy_hip_malloc(size_t nbytes, void** dptr_out);
+int appy_hip_free(void* dptr);
+int appy_hip_pool_trim(void);
+int appy_hip_pool_stats(uint64_t* bytes_in_use_out, uint64_t* bytes_cached_out);
+/* Stream-ordered copies; both return after the copy has completed. */
+int appy_hip_memcpy_h2d(void* dst_dev, const void* src_host, size_t nbytes, void* stream);
+int appy_hip_memcpy_d2h(void* dst_host, const void* src_dev, size_t nbytes, void* stream);
+int appy_hip_memcpy_d2d_async(void* dst_dev, const void* src_dev, size_t nbytes, void* stream);
+int appy_hip_memset_async(void* dst_dev, int byte_value, size_t nbytes, void* stream);
+
+/* ---- launch --------------------------------------------------------------
+ * Replaces `_kernel_loop_N[grid](args..., num_warps=4)`
+ * (appy/backends/triton/passes/host_passes/gen_kernel_launch.py:27-66).
+ * `args` is the kernel's argument block laid out as the C struct of its
+ * parameters (natural alignment); it is copied before the call returns. */
+int appy_hip_launch(void* func,
+                    uint32_t grid_x, uint32_t grid_y, uint32_t grid_z,
+                    uint32_t block_x, uint32_t block_y, uint32_t block_z,
+                    uint32_t dynamic_lds_bytes, void* stream,
+                    const void* args, size_t args_bytes);
+int appy_hip_sync(void* stream);               /* hipStreamSynchronize */
+
+/* ---- timing ---------------------------------------------------------------
+ * Replaces torch.utils.benchmark.Timer in examples/benchmark_utils.py:4-15:
+ * HIP events recorded on the stream the kernel is launched on. */
+int appy_hip_event_create(void** event_out);
+int appy_hip_event_record(void* event, void* stream);
+int appy_hip_event_sync(void* event);
+int appy_hip_event_elapsed_ms(void* start, void* stop, float* ms_out);
+int appy_hip_event_destroy(void* event);
+/* `reps` back-to-back launches of one kernel between two events, after
+ * `warmup` untimed launches; *mean_ms_out = elapsed / reps. */
+int appy_hip_launch_timed(void* func,
+                          uint32_t grid_x, uint32_t grid_y, uint32_t grid_z,
+                          uint32_t block_x, uint32_t block_y, uint32_t block_z,
+                          uint32_t dynamic_lds_bytes, void* stream,
+                          const void* args, size_t args_bytes,
+                          int warmup, int reps, float* mean_ms_out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* APPY_HIP_H */
