@@ -223,7 +223,14 @@ class CompiledLoop:
 
     # ---- variants ------------------------------------------------------------------
     def _elem_sizes(self):
-        return [arr.ty.size for arr in self.analysis.arrays.values()] or [4]
+        """Element sizes of the arrays that are indexed by a variable (the
+        candidates for wide loads); reduction targets like ``s[0]`` do not count."""
+        sizes = []
+        for n in ast.walk(self.analysis.outer):
+            if (isinstance(n, ast.Subscript) and isinstance(n.value, ast.Name)
+                    and n.value.id in self.analysis.arrays and not isinstance(n.slice, ast.Constant)):
+                sizes.append(self.analysis.arrays[n.value.id].ty.size)
+        return sizes or [4]
 
     def _default_spec(self) -> Spec:
         a = self.analysis
@@ -307,7 +314,7 @@ class CompiledLoop:
             return int(min(need, cap))
         tpb = spec.block // spec.width
         need = max(1, -(-n_outer // tpb))
-        return int(min(need, 1 << 24))
+        return int(min(need, 1 << 22))
 
     # ---- call ------------------------------------------------------------------------
     def __call__(self, *args):

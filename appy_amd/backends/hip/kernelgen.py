@@ -273,6 +273,8 @@ class KernelBuilder:
             if red_op and name in self.partials:
                 oc, ot = self.ex.emit(loop_ir.reduction_operand(st))
                 p, pty = self.partials[name]
+                # the variable takes the type NumPy gives `name (op) operand`
+                self.set_local(name, T.promote(pty, ot) if red_op in "+*" else T.join(pty, ot))
                 self.w(f"{p} = {_OPS[red_op]}::f<{pty.c}>({p}, {cast(oc, ot, pty)});")
                 return
             vc, vt = self.ex.emit(st.value)

@@ -49,10 +49,14 @@ def codegen(backend_name, loop_source, loop_name, local_scope, global_scope, opt
 
     if options.get("dry_run"):
         # Code generation has run (its errors surface); now interpret the loop
-        # text itself in the caller's scope (reference: appy/dispatcher.py:46-53).
+        # text itself with the caller's values (reference: appy/dispatcher.py:46-53).
+        # The caller's locals take precedence over its globals; results travel
+        # through in-place mutation of arrays, exactly as for a kernel launch.
         try:
             code_obj = compile(loop_source, filename=f"<{loop_name}>", mode="exec")
-            exec(code_obj, local_scope, global_scope)
+            scope = dict(global_scope)
+            scope.update(local_scope)
+            exec(code_obj, scope)
         except Exception as e:
             raise RuntimeError(f"Error executing loop {loop_name} in dry_run mode: {e}")
         return

@@ -1,0 +1,158 @@
+"""Parity of the HIP path with the CPU oracle on identical seeded inputs.
+
+Bars: bit-exact for elementwise and integer work; for float32 reductions,
+GEMV, SpMV and SpMM ``|out - oracle| <= 1e-5 * sum(|terms|)`` per output, the
+oracle being float64 (oracle/vectorised.py).  Every call goes through
+``@jit`` -> generated HIP kernel -> libappy_hip.so (C ABI).
+"""
+import numpy as np
+import pytest
+
+from appy_amd.backends.hip import selfcheck
+from oracle import loops as lo
+from oracle import vectorised as vo
+from oracle import workloads as wl
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-5  # the tolerance of the parity bar, relative to sum(|terms|)
+
+
+@pytest.fixture(scope="module")
+def k(gpu):
+    return selfcheck.kernels()
+
+
+@pytest.mark.parametrize("n", [1, 3, 255, 256, 4096, 4097, 100_003, 1 << 20, (1 << 22) + 5])
+def test_vec_add_bit_exact(k, n):
+    a, b = wl.vec_add(n)
+    c = k.vec_add(a, b)
+    assert c.dtype == np.float32
+    assert np.array_equal(c, vo.vec_add(a, b))
+
+
+def test_vec_add_float64_and_int(k):
+    rng = np.random.default_rng(7)
+    a = rng.standard_normal(10_001)
+    b = rng.standard_normal(10_001)
+    assert np.array_equal(k.vec_add(a, b), a + b)
+    ai = rng.integers(-1000, 1000, 5003, dtype=np.int32)
+    bi = rng.integers(-1000, 1000, 5003, dtype=np.int32)
+    assert np.array_equal(k.vec_add(ai, bi), ai + bi)
+
+
+def test_vec_add_empty(k):
+    a = np.empty(0, dtype=np.float32)
+    assert k.vec_add(a, a).shape == (0,)
+
+
+@pytest.mark.parametrize("n", [1, 7, 1000, 4096, 65_537, 1 << 20, (1 << 24) + 3])
+def test_vector_sum(k, n):
+    A, _ = wl.reduce_inputs(n)
+    ref, budget = vo.vector_sum(A)
+    got = k.vector_sum(A)
+    assert isinstance(got, float)
+    assert abs(got - ref) <= TOL * budget
+
+
+@pytest.mark.parametrize("n", [1, 7, 1000, 4099, 1 << 20, (1 << 24) + 3])
+def test_masked_sum(k, n):
+    A, M = wl.reduce_inputs(n)
+    ref, budget = vo.masked_sum(A, M)
+    got = k.masked_sum(A, M)
+    assert abs(got - ref) <= TOL * budget
+
+
+def test_masked_sum_special_masks(k):
+    A, _ = wl.reduce_inputs(50_001)
+    assert k.masked_sum(A, np.zeros(A.shape, dtype=bool)) == 0.0
+    ref, budget = vo.vector_sum(A)
+    assert abs(k.masked_sum(A, np.ones(A.shape, dtype=bool)) - ref) <= TOL * budget
+
+
+def test_small_cases_against_literal_loops(k):
+    A, M = wl.reduce_inputs(777)
+    assert abs(k.vector_sum(A) - lo.vector_sum(A)) <= TOL * float(np.abs(A).sum())
+    assert abs(k.masked_sum(A, M) - lo.masked_sum_ternary(A, M)) <= TOL * float(np.abs(A).sum())
+    a, b = wl.vec_add(333)
+    assert np.array_equal(k.vec_add(a, b), lo.vec_add(a, b))
+
+
+@pytest.mark.parametrize("shape", [(1, 1), (3, 5), (64, 64), (100, 1000), (513, 1027), (2048, 4096), (37, 16384)])
+def test_gemv(k, shape):
+    A, x = wl.gemv(*shape)
+    ref, budget = vo.gemv(A, x)
+    y = k.gemv(A, x)
+    assert y.dtype == np.float32
+    ok, worst = vo.within_budget(y, ref, budget, TOL)
+    assert ok, worst
+
+
+def test_gemv_unit_vectors_select_columns(k):
+    A, _ = wl.gemv(40, 70)
+    for col in (0, 33, 69):
+        e = np.zeros(70, dtype=np.float32)
+        e[col] = 1.0
+        assert np.array_equal(k.gemv(A, e), A[:, col])
+
+
+@pytest.mark.parametrize("m,per_row", [(1, 1), (10, 3), (1000, 16), (4096, 16), (50_000, 16), (3000, 100)])
+def test_spmv_uniform(k, m, per_row):
+    data, indptr, indices, x = wl.spmv_uniform(m, max(m, per_row * 2), per_row)
+    n = x.shape[0]
+    ref, budget = vo.spmv_csr(data, indptr, indices, x, (m, n))
+    y = k.spmv(data, indptr, indices, x, m, n)
+    ok, worst = vo.within_budget(y, ref, budget, TOL)
+    assert ok, worst
+
+
+@pytest.mark.parametrize("m,clip", [(2000, 64), (8192, 512), (20_000, 4096)])
+def test_spmv_powerlaw(k, m, clip):
+    data, indptr, indices, x = wl.spmv_powerlaw(m, m, clip=clip)
+    ref, budget = vo.spmv_csr(data, indptr, indices, x, (m, m))
+    y = k.spmv(data, indptr, indices, x, m, m)
+    ok, worst = vo.within_budget(y, ref, budget, TOL)
+    assert ok, worst
+
+
+def test_spmv_empty_rows_and_identity(k):
+    # rows 0 and 2 empty
+    indptr = np.array([0, 0, 2, 2, 3], dtype=np.int32)
+    indices = np.array([1, 3, 0], dtype=np.int32)
+    data = np.array([2.0, -1.0, 0.5], dtype=np.float32)
+    x = np.array([4.0, 3.0, 2.0, 1.0], dtype=np.float32)
+    y = k.spmv(data, indptr, indices, x, 4, 4)
+    assert np.array_equal(y, np.array([0.0, 5.0, 0.0, 2.0], dtype=np.float32))
+    n = 1000
+    eye_ptr = np.arange(n + 1, dtype=np.int32)
+    eye_idx = np.arange(n, dtype=np.int32)
+    xs = np.random.default_rng(3).standard_normal(n, dtype=np.float32)
+    assert np.array_equal(k.spmv(np.ones(n, dtype=np.float32), eye_ptr, eye_idx, xs, n, n), xs)
+
+
+def test_spmv_int64_indices(k):
+    data, indptr, indices, x = wl.spmv_uniform(3000, 3000, 9)
+    ref, budget = vo.spmv_csr(data, indptr, indices, x, (3000, 3000))
+    y = k.spmv(data, indptr.astype(np.int64), indices.astype(np.int64), x, 3000, 3000)
+    assert vo.within_budget(y, ref, budget, TOL)[0]
+
+
+@pytest.mark.parametrize("m,ncols", [(1, 128), (100, 128), (4096, 128), (1000, 200), (500, 7)])
+def test_spmm(k, m, ncols):
+    data, indptr, indices, B = wl.spmm(m, max(m, 64), ncols)
+    n = B.shape[0]
+    ref, budget = vo.spmm_csr(data, indptr, indices, B, (m, n))
+    Y = np.full((m, ncols), np.nan, dtype=np.float32)
+    k.spmm(data, indptr, indices, B, Y, m)
+    ok, worst = vo.within_budget(Y, ref, budget, TOL)
+    assert ok, worst
+
+
+def test_spmm_columns_equal_spmv(k):
+    data, indptr, indices, B = wl.spmm(700, 700, 128)
+    Y = np.empty((700, 128), dtype=np.float32)
+    k.spmm(data, indptr, indices, B, Y, 700)
+    for col in (0, 64, 127):
+        x = np.ascontiguousarray(B[:, col])
+        ref, budget = vo.spmv_csr(data, indptr, indices, x, (700, 700))
+        assert vo.within_budget(Y[:, col], ref, budget, TOL)[0]
