@@ -1,0 +1,355 @@
+#!/usr/bin/env python3
+"""Benchmark of the annotated-loop hot path on one MI355X.
+
+``python bench.py [--gpus 1] [--steps K] [--warmup W]`` prints ONE JSON line.
+
+Headline (``value``): achieved HBM GB/s of the ``shared()`` scalar reduction
+``vector_sum`` over float32 N = 2^28 (1 GiB), inputs resident in HBM, one step
+= clear the float64 accumulator + one launch of the generated kernel, timed
+over K steps between device synchronisations.  ``roofline`` gives the same
+kernel's algorithmic bytes per launch divided by its mean launch duration
+measured with HIP events on the launch stream, against the 8 TB/s HBM peak.
+``kernels`` lists the same figures for the other generated kernels
+(vec_add, masked_sum, GEMV, CSR SpMV uniform and power-law, CSR SpMM), each
+checked against the float64 oracle on the identical inputs in the same run.
+``cpu_baseline`` times the oracle (NumPy, one core) on the host.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_BPS = 8.0e12  # MI355X HBM3E, bytes per second
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def parse_args():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=50)
+    p.add_argument("--warmup", type=int, default=5)
+    p.add_argument("--workloads", default="vector_sum,masked_sum,vec_add,gemv,spmv_uniform,spmv_powerlaw,spmm",
+                   help="comma separated subset; vector_sum is always run (headline)")
+    p.add_argument("--scale", type=float, default=1.0, help="shrink every size by this factor (debugging)")
+    p.add_argument("--no-cpu-baseline", action="store_true")
+    return p.parse_args()
+
+
+class Runner:
+    """Times one compiled loop on resident inputs."""
+
+    def __init__(self, torch, rt, cg):
+        self.torch, self.rt, self.cg = torch, rt, cg
+
+    def loop_of(self, before):
+        new = [k for k in self.cg.code_cache if k not in before]
+        assert len(new) == 1, f"expected one new compiled loop, got {len(new)}"
+        return self.cg.code_cache[new[0]][0]
+
+    def measure(self, loop, vals, nbytes, steps, warmup, clear=None):
+        """Returns dict(ms_per_step, gbps_step, kernel_ms, gbps_kernel, frac, spec, grid)."""
+        torch, rt = self.torch, self.rt
+        launch = loop.prepare(vals)
+        stream = launch.stream
+
+        def step():
+            if clear is not None:
+                clear.zero_()           # fill kernel on the same (current) stream
+            launch.launch_only()
+
+        for _ in range(warmup):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / steps
+        kernel_ms = launch.time_kernel(warmup=2, reps=max(10, min(steps, 50)))
+        info = rt.func_info(launch.function())
+        return {
+            "ms_per_step": dt * 1e3,
+            "gbps_step": nbytes / dt / 1e9,
+            "kernel_ms": kernel_ms,
+            "gbps_kernel": nbytes / (kernel_ms * 1e-3) / 1e9,
+            "frac": nbytes / (kernel_ms * 1e-3) / HBM_PEAK_BPS,
+            "algorithmic_bytes": int(nbytes),
+            "spec": launch.spec.tag(),
+            "grid": launch.grid[0],
+            "vgprs": info["num_vgprs"],
+            "scratch_bytes": info["scratch_bytes"],
+        }
+
+
+def device_csr(torch, lengths_np, ncols, seed):
+    """CSR structure with sorted distinct uniform columns per row, built on the
+    device (the host generator of oracle/workloads.py needs minutes at 4e8
+    non-zeros).  Returns (data f32, indptr i32, indices i32) device tensors."""
+    dev = "cuda"
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed)
+    lengths = torch.from_numpy(lengths_np).to(dev)
+    m = lengths.numel()
+    indptr = torch.zeros(m + 1, dtype=torch.int64, device=dev)
+    torch.cumsum(lengths, 0, out=indptr[1:])
+    nnz = int(indptr[-1].item())
+    assert nnz < 2**31
+    row_of = torch.repeat_interleave(torch.arange(m, device=dev, dtype=torch.int64), lengths)
+    cols = torch.randint(0, ncols, (nnz,), generator=g, device=dev, dtype=torch.int64)
+    for _ in range(64):
+        key = row_of * ncols + cols
+        sk, order = torch.sort(key)
+        dup_sorted = torch.zeros(nnz, dtype=torch.bool, device=dev)
+        dup_sorted[1:] = sk[1:] == sk[:-1]
+        ndup = int(dup_sorted.sum().item())
+        if ndup == 0:
+            cols = sk % ncols
+            break
+        idx = order[dup_sorted]
+        cols[idx] = torch.randint(0, ncols, (ndup,), generator=g, device=dev, dtype=torch.int64)
+        del key, sk, order, dup_sorted, idx
+    else:
+        raise RuntimeError("could not draw distinct columns")
+    data = torch.randn(nnz, generator=g, device=dev, dtype=torch.float32)
+    return data, indptr.to(torch.int32), cols.to(torch.int32)
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported in this build "
+              "(every kernel here is a single-device kernel)", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    from appy_amd.backends.hip import codegen as cg
+    from appy_amd.backends.hip import runtime as rt
+    from appy_amd.backends.hip import selfcheck
+    from oracle import loops as olo
+    from oracle import vectorised as vo
+    from oracle import workloads as wl
+
+    if not torch.cuda.is_available() or rt.device_count() < 1:
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+    torch.cuda.set_device(0)
+    props = rt.device_props(0)
+    log(f"device: {props['name']} {props['arch']} CUs={props['compute_units']} HBM={props['hbm_bytes'] / 2**30:.0f} GiB")
+
+    k = selfcheck.kernels()
+    run = Runner(torch, rt, cg)
+    want = set(args.workloads.split(",")) | {"vector_sum"}
+    sc = args.scale
+    results = {}
+    parity = {}
+    K, W = args.steps, args.warmup
+
+    def shrink(n, lo=1024):
+        return max(lo, int(n * sc))
+
+    # ---------------- config 2a / 2b: shared() scalar reductions ----------------------
+    n = shrink(1 << 28)
+    t0 = time.time()
+    A, M = wl.reduce_inputs(n)
+    log(f"reduce inputs N={n} generated in {time.time() - t0:.1f}s")
+    A_d = torch.from_numpy(A).cuda()
+    s_d = torch.zeros(1, dtype=torch.float64, device="cuda")
+
+    before = set(cg.code_cache)
+    got = k.vector_sum(A_d)                                # product path end to end
+    loop = run.loop_of(before)
+    ref, budget = vo.vector_sum(A)
+    parity["vector_sum"] = {"abs_err": abs(got - ref), "bound": vo.TOL * budget, "ok": abs(got - ref) <= vo.TOL * budget}
+    results["vector_sum"] = run.measure(loop, {"s": s_d, "A": A_d, "A_shape_0": n}, 4 * n + 8, K, W, clear=s_d)
+    # end-to-end call of the decorated function (shared scalar travels host<->device)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(10):
+        k.vector_sum(A_d)
+    results["vector_sum"]["jit_call_ms"] = (time.perf_counter() - t0) / 10 * 1e3
+    log("vector_sum", results["vector_sum"], parity["vector_sum"])
+
+    cpu_baseline = None
+    if not args.no_cpu_baseline:
+        # oracle (NumPy float64 accumulation, one core) on the full array, best of 3,
+        # and the literal interpreter loop on a 2^20 sample
+        best = 1e30
+        for _ in range(3):
+            t0 = time.perf_counter()
+            A.sum(dtype=np.float64)
+            best = min(best, time.perf_counter() - t0)
+        m = min(n, 1 << 20)
+        t0 = time.perf_counter()
+        olo.vector_sum(A[:m])
+        lit = (time.perf_counter() - t0) / m * 1e9
+        cpu_baseline = {
+            "value": (4 * n + 8) / best / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"oracle A.sum(dtype=float64) over all N={n} float32, best of 3 ({best * 1e3:.1f} ms); "
+                      f"literal interpreter loop on the first {m} elements: {lit:.0f} ns/element",
+            "host_cpus": os.cpu_count(), "affinity": len(os.sched_getaffinity(0)),
+        }
+        log("cpu_baseline", cpu_baseline)
+
+    if "masked_sum" in want:
+        M_d = torch.from_numpy(M).cuda()
+        before = set(cg.code_cache)
+        got = k.masked_sum(A_d, M_d)
+        loop = run.loop_of(before)
+        ref, budget = vo.masked_sum(A, M)
+        parity["masked_sum"] = {"abs_err": abs(got - ref), "bound": vo.TOL * budget, "ok": abs(got - ref) <= vo.TOL * budget}
+        results["masked_sum"] = run.measure(loop, {"s": s_d, "A": A_d, "M": M_d, "A_shape_0": n}, 5 * n + 8, K, W, clear=s_d)
+        log("masked_sum", results["masked_sum"], parity["masked_sum"])
+        del M_d
+    del A_d, A, M
+    torch.cuda.empty_cache()
+
+    # ---------------- config 1: vec_add ---------------------------------------------------
+    if "vec_add" in want:
+        n1 = shrink(1 << 24)
+        a, b = wl.vec_add(n1)
+        a_d, b_d = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()
+        before = set(cg.code_cache)
+        c_d = k.vec_add(a_d, b_d)
+        loop = run.loop_of(before)
+        ok = bool(np.array_equal(c_d.cpu().numpy(), vo.vec_add(a, b)))
+        parity["vec_add"] = {"bit_exact": ok, "ok": ok}
+        results["vec_add"] = run.measure(loop, {"c": c_d, "a": a_d, "b": b_d, "a_shape_0": n1}, 12 * n1, K, W)
+        log("vec_add", results["vec_add"], parity["vec_add"])
+        del a_d, b_d, c_d
+
+    # ---------------- config 3: GEMV ---------------------------------------------------------
+    if "gemv" in want:
+        r = shrink(16384, 64)
+        t0 = time.time()
+        Am, x = wl.gemv(r, r)
+        log(f"gemv inputs {r}x{r} generated in {time.time() - t0:.1f}s")
+        A_d, x_d = torch.from_numpy(Am).cuda(), torch.from_numpy(x).cuda()
+        before = set(cg.code_cache)
+        y_d = k.gemv(A_d, x_d)
+        loop = run.loop_of(before)
+        ref, budget = vo.gemv(Am, x)
+        ok, worst = vo.within_budget(y_d.cpu().numpy(), ref, budget)
+        parity["gemv"] = {"worst_err_over_bound": worst, "ok": ok}
+        vals = {"A": A_d, "x": x_d, "y": y_d, "A_shape_0": r, "A_shape_1": r}
+        results["gemv"] = run.measure(loop, vals, 4 * (r * r + r + r), K, W)
+        log("gemv", results["gemv"], parity["gemv"])
+        del A_d, x_d, y_d, Am, ref, budget
+        torch.cuda.empty_cache()
+
+    # ---------------- config 4: CSR SpMV -----------------------------------------------------
+    def spmv_case(name, data_d, indptr_d, indices_d, x_d, m, ncol):
+        before = set(cg.code_cache)
+        y_d = k.spmv(data_d, indptr_d, indices_d, x_d, m, ncol)
+        new = [kk for kk in cg.code_cache if kk not in before]
+        loop = cg.code_cache[new[0]][0] if new else spmv_case.loop
+        spmv_case.loop = loop
+        nnz = data_d.numel()
+        t0 = time.time()
+        ref, budget = vo.spmv_csr(data_d.cpu().numpy(), indptr_d.cpu().numpy(), indices_d.cpu().numpy(),
+                                  x_d.cpu().numpy(), (m, ncol))
+        ok, worst = vo.within_budget(y_d.cpu().numpy(), ref, budget)
+        log(f"{name}: oracle in {time.time() - t0:.1f}s")
+        lens = (indptr_d[1:] - indptr_d[:-1])
+        parity[name] = {"worst_err_over_bound": worst, "ok": ok}
+        vals = {"A_data": data_d, "A_indptr": indptr_d, "A_indices": indices_d, "x": x_d, "y": y_d, "M": m}
+        nbytes = 8 * nnz + 4 * (m + 1) + 4 * ncol + 4 * m
+        results[name] = run.measure(loop, vals, nbytes, K, W)
+        results[name].update({"nnz": int(nnz), "rows": m, "mean_row": float(nnz) / m, "max_row": int(lens.max().item())})
+        log(name, results[name], parity[name])
+
+    spmv_case.loop = None
+    if "spmv_uniform" in want:
+        m4 = shrink(1 << 22)
+        lengths = np.full(m4, 16, dtype=np.int64)
+        data_d, indptr_d, indices_d = device_csr(torch, lengths, m4, seed=4)
+        gx = torch.Generator(device="cuda"); gx.manual_seed(40)
+        x_d = torch.randn(m4, generator=gx, device="cuda", dtype=torch.float32)
+        spmv_case("spmv_uniform", data_d, indptr_d, indices_d, x_d, m4, m4)
+        del data_d, indptr_d, indices_d, x_d
+        torch.cuda.empty_cache()
+    if "spmv_powerlaw" in want:
+        m4 = shrink(1 << 22)
+        rng = np.random.default_rng(104)
+        lengths = np.clip(rng.zipf(1.5, m4), 1, min(4096, m4)).astype(np.int64)
+        t0 = time.time()
+        data_d, indptr_d, indices_d = device_csr(torch, lengths, m4, seed=5)
+        log(f"power-law CSR nnz={data_d.numel()} built in {time.time() - t0:.1f}s")
+        gx = torch.Generator(device="cuda"); gx.manual_seed(41)
+        x_d = torch.randn(m4, generator=gx, device="cuda", dtype=torch.float32)
+        spmv_case("spmv_powerlaw", data_d, indptr_d, indices_d, x_d, m4, m4)
+        del data_d, indptr_d, indices_d, x_d
+        torch.cuda.empty_cache()
+
+    # ---------------- config 5: CSR SpMM -------------------------------------------------------
+    if "spmm" in want:
+        m5 = shrink(1 << 20)
+        rng = np.random.default_rng(5)
+        lengths = np.minimum(rng.poisson(32, m5), m5).astype(np.int64)
+        data_d, indptr_d, indices_d = device_csr(torch, lengths, m5, seed=6)
+        gx = torch.Generator(device="cuda"); gx.manual_seed(42)
+        B_d = torch.randn((m5, 128), generator=gx, device="cuda", dtype=torch.float32)
+        Y_d = torch.empty((m5, 128), device="cuda", dtype=torch.float32)
+        before = set(cg.code_cache)
+        k.spmm(data_d, indptr_d, indices_d, B_d, Y_d, m5)
+        loop = run.loop_of(before)
+        # oracle on a row sample (the full float64 product needs ~10 s of one core)
+        rows = np.unique(np.concatenate([np.arange(min(m5, 4096)), rng.integers(0, m5, 4096)]))
+        ip = indptr_d.cpu().numpy().astype(np.int64)
+        sel = np.concatenate([np.arange(ip[r0], ip[r0 + 1]) for r0 in rows]) if len(rows) else np.empty(0, np.int64)
+        sub_ptr = np.zeros(len(rows) + 1, dtype=np.int64)
+        np.cumsum(ip[rows + 1] - ip[rows], out=sub_ptr[1:])
+        ref, budget = vo.spmm_csr(data_d.cpu().numpy()[sel], sub_ptr, indices_d.cpu().numpy()[sel],
+                                  B_d.cpu().numpy(), (len(rows), m5))
+        ok, worst = vo.within_budget(Y_d.cpu().numpy()[rows], ref, budget)
+        parity["spmm"] = {"worst_err_over_bound": worst, "ok": ok, "rows_checked": int(len(rows))}
+        nnz = data_d.numel()
+        nbytes = 8 * nnz + 4 * (m5 + 1) + 4 * m5 * 128 + 4 * m5 * 128
+        vals = {"A_data": data_d, "A_indptr": indptr_d, "A_indices": indices_d, "B": B_d, "y": Y_d, "M": m5}
+        results["spmm"] = run.measure(loop, vals, nbytes, max(5, K // 5), min(W, 2))
+        results["spmm"].update({"nnz": int(nnz), "gather_model_bytes": int(nnz * (8 + 512) + 4 * (m5 + 1) + 512 * m5)})
+        log("spmm", results["spmm"], parity["spmm"])
+
+    head = results["vector_sum"]
+    all_ok = all(p["ok"] for p in parity.values())
+    line = {
+        "metric": "achieved HBM GB/s of the generated shared()-reduction kernel (vector_sum), 1 GPU",
+        "value": head["gbps_step"],
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": K,
+        "warmup": W,
+        "ms_per_step": head["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32 loads, f64 accumulate",
+        "data": "synthetic",
+        "config": {"workload": f"configs[1](a) shared() scalar reduction vector_sum, float32 N={n}, uniform[0,1), seed 2",
+                   "step": "clear float64 accumulator + one kernel launch, inputs resident in HBM"},
+        "roofline": {"bound": "hbm", "achieved": head["gbps_kernel"], "peak": HBM_PEAK_BPS / 1e9, "unit": "GB/s",
+                     "frac": head["frac"], "traffic": None},
+        "cpu_baseline": cpu_baseline,
+        "parity_ok": all_ok,
+        "parity": parity,
+        "kernels": results,
+        "device": {"name": props["name"], "arch": props["arch"], "compute_units": props["compute_units"]},
+    }
+    print(json.dumps(line), flush=True)
+    if not all_ok:
+        sys.exit(3)
+
+
+if __name__ == "__main__":
+    main()

@@ -41,6 +41,16 @@ def _sorted_unique_columns(rng, lengths, ncols):
     indptr = np.zeros(len(lengths) + 1, dtype=np.int64)
     np.cumsum(lengths, out=indptr[1:])
     nnz = int(indptr[-1])
+    if len(lengths) and np.all(lengths == lengths[0]) and lengths[0] > 0:
+        # equal rows: sort each row on its own, redraw the rows that hold a duplicate
+        L = int(lengths[0])
+        cols = np.sort(rng.integers(0, ncols, size=(len(lengths), L), dtype=np.int64), axis=1)
+        for _ in range(64):
+            bad = np.flatnonzero((cols[:, 1:] == cols[:, :-1]).any(axis=1)) if L > 1 else np.empty(0, dtype=np.int64)
+            if bad.size == 0:
+                return indptr, cols.reshape(-1)
+            cols[bad] = np.sort(rng.integers(0, ncols, size=(bad.size, L), dtype=np.int64), axis=1)
+        raise RuntimeError("could not draw distinct columns")
     row_of = np.repeat(np.arange(len(lengths), dtype=np.int64), lengths)
     cols = rng.integers(0, ncols, size=nnz, dtype=np.int64)
     for _ in range(64):
