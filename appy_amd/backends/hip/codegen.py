@@ -40,8 +40,10 @@ code_cache = {}
 _cache_lock = threading.Lock()
 _device_header = None
 
-# Hardware facts used by the launch heuristics (MI355X: 256 CUs in 8 XCDs).
+# Hardware facts used by the launch heuristics (MI355X: 256 CUs in 8 XCDs,
+# 256 MiB of memory-side cache in front of the HBM3E).
 DEFAULT_CUS = 256
+MALL_BYTES = 256 << 20
 
 
 def device_header() -> str:
@@ -214,6 +216,7 @@ class CompiledLoop:
         self._lo_code = compile(ast.Expression(body=ast.fix_missing_locations(_copy(a.lo_node))), "<lo>", "eval")
         self._hi_code = compile(ast.Expression(body=ast.fix_missing_locations(_copy(a.hi_node))), "<hi>", "eval")
         self._simd_loops = self._collect_simd_loops()
+        self._row_extent_code = self._find_row_extent()
         self.kernels = {}   # Spec -> Kernel
         self._lock = threading.Lock()
         # default variant now: generation / compilation errors surface at first use of the loop
@@ -237,7 +240,7 @@ class CompiledLoop:
         v = max(1, min(4, 16 // max(self._elem_sizes())))
         if a.kind == "flat":
             if "simd" in a.pragma:
-                return Spec("flat", block=256, vec=v, unroll=4)
+                return Spec("flat", block=256, vec=v, unroll=4 if a.outer_reductions else 2)
             return Spec("flat", block=256, vec=1, unroll=1)
         return Spec("team", block=256, vec=v, width=64)
 
@@ -270,6 +273,22 @@ class CompiledLoop:
             out.append((compile(extent, "<extent>", "eval"), streamed))
         return out
 
+    def _find_row_extent(self):
+        """Extent expression of a row that a sequential loop updates through a
+        ``simd`` loop (``y[i, :] += a * B[k, :]`` inside ``for k``): such rows
+        are kept in registers when the extent is known at compile time."""
+        for n in ast.walk(self.analysis.outer):
+            if (isinstance(n, ast.For) and n is not self.analysis.outer
+                    and "simd" not in (getattr(n, "pragma", None) or {}) and len(n.body) == 1):
+                inner = n.body[0]
+                if (isinstance(inner, ast.For) and "simd" in (getattr(inner, "pragma", None) or {})
+                        and len(inner.body) == 1 and isinstance(inner.body[0], ast.Assign)
+                        and isinstance(inner.body[0].targets[0], ast.Subscript)):
+                    lo, hi, _ = inner.iter.args
+                    if isinstance(lo, ast.Constant) and lo.value == 0:
+                        return compile(ast.Expression(body=ast.fix_missing_locations(_copy(hi))), "<extent>", "eval")
+        return None
+
     def _estimate_trip(self, env, arrays, n_outer) -> float:
         best = 0.0
         for code, streamed in self._simd_loops:
@@ -293,24 +312,45 @@ class CompiledLoop:
             base.update(forced)
             return Spec(**base)
         if d.kind == "flat":
+            stream = self._bytes_touched(arrays) > MALL_BYTES
             if d.vec > 1 and n_outer < d.block * d.vec * d.unroll:
                 return Spec("flat", block=d.block, vec=d.vec, unroll=1, restrict=restrict)
-            return Spec("flat", block=d.block, vec=d.vec, unroll=d.unroll, restrict=restrict)
-        trip = self._estimate_trip(env, arrays, n_outer)
+            return Spec("flat", block=d.block, vec=d.vec, unroll=d.unroll, restrict=restrict, stream_loads=stream)
+        stream = self._bytes_touched(arrays) > MALL_BYTES
         v = d.vec
+        if self._row_extent_code is not None:
+            try:
+                ext = int(eval(self._row_extent_code, {"__builtins__": {}}, env))
+            except Exception:
+                ext = 0
+            if ext > 0 and ext % v == 0:
+                w = max(1, min(64, _pow2ceil(ext / v)))
+                if -(-ext // (w * v)) <= 8:
+                    return Spec("team", block=d.block, vec=v, width=w, restrict=restrict,
+                                stream_loads=False, extent=ext)
+        trip = self._estimate_trip(env, arrays, n_outer)
         if trip < 2 * v:
             v = 1
-        w = max(1, min(64, _pow2ceil(trip / (v * 1.0)) if trip > 0 else 1))
-        # keep at least two vector steps per lane before widening to the full wavefront
-        return Spec("team", block=d.block, vec=v, width=w, restrict=restrict)
+        # one vector step per lane for short rows; two rows per wavefront at most
+        # (two independent rows in flight per wavefront stream better than one)
+        w = max(1, min(32, _pow2ceil(trip / float(v)) if trip > 0 else 1))
+        return Spec("team", block=d.block, vec=v, width=w, restrict=restrict, stream_loads=stream)
+
+    def _bytes_touched(self, arrays) -> int:
+        total = 0
+        for name, v in arrays.items():
+            arr = self.analysis.arrays[name]
+            if arr.loaded or arr.stored:
+                total += int(np.prod(v.shape)) * arr.ty.size
+        return total
 
     def grid_for(self, spec: Spec, n_outer: int, cus: int = DEFAULT_CUS) -> int:
         if spec.kind == "flat":
             per_block = spec.block * spec.vec * spec.unroll
             need = max(1, -(-n_outer // per_block))
-            cap = self.options.get("hip_max_blocks") or cus * 8
-            if self.analysis.outer_reductions:
-                cap = self.options.get("hip_max_blocks") or cus * 8
+            # reductions end with one atomic per workgroup: few, persistent
+            # workgroups (4 per CU); pure streaming loops take up to 32 per CU
+            cap = self.options.get("hip_max_blocks") or (cus * 4 if self.analysis.outer_reductions else cus * 32)
             return int(min(need, cap))
         tpb = spec.block // spec.width
         need = max(1, -(-n_outer // tpb))
@@ -338,6 +378,8 @@ class CompiledLoop:
         if hi <= lo:
             return None
         arrays = {k: vals[k] for k in a.arrays}
+        for nm, (an, dim) in self.derived_shapes.items():
+            env[nm] = int(arrays[an].shape[dim])
         return Launch(self, vals, arrays, env, lo, hi)
 
 

@@ -58,11 +58,13 @@ class Spec:
     unroll: int = 1      # vectors per lane and tile (U), flat only
     width: int = 1       # lanes per team (W), team only
     restrict: bool = True
-    stream_loads: bool = False   # non-temporal loads for vectorised accesses
+    stream_loads: bool = False   # non-temporal loads for data that is read once
+    extent: int = 0      # compile-time extent of row accumulators (team only; 0 = none)
 
     def tag(self) -> str:
         return (f"{self.kind}_b{self.block}_v{self.vec}_u{self.unroll}_w{self.width}"
-                f"{'_r' if self.restrict else ''}{'_nt' if self.stream_loads else ''}")
+                f"{'_r' if self.restrict else ''}{'_nt' if self.stream_loads else ''}"
+                f"{'_e' + str(self.extent) if self.extent else ''}")
 
 
 @dataclass
@@ -212,6 +214,7 @@ class KernelBuilder:
         self.ind = 1
         self.mode = "lane"
         self.partials = {}        # reduction variable -> partial register, inside a spread simd loop
+        self.bounds_vary = False  # inside a spread loop whose bounds differ between outer iterations
         self.store_subst = {}     # unparsed subscript -> (lvalue code, Ty)
         self.dirty = False
         self.counter = 0
@@ -236,8 +239,15 @@ class KernelBuilder:
 
     # ---- statements ---------------------------------------------------------------
     def block(self, stmts):
-        for st in stmts:
-            self.stmt(st)
+        i = 0
+        while i < len(stmts):
+            if self.mode == "team" and self.spec.extent:
+                used = self.row_accumulate(stmts, i)
+                if used:
+                    i += used
+                    continue
+            self.stmt(stmts[i])
+            i += 1
 
     def stmt(self, st):
         if isinstance(st, ast.Assign):
@@ -410,15 +420,27 @@ class KernelBuilder:
                 self.ex.locals[var] = saved
         return f"{cname(arr.name)} + ({idx.replace('__vbase', base_code)})"
 
+    def _streamed(self, sub: ast.Subscript) -> bool:
+        """True if the data behind a vectorised load is read once by the whole
+        launch (then it is loaded non-temporally so that it does not displace
+        reused lines from the caches): always in a flat loop; in a team loop
+        when the address depends on the outer iteration, directly or through
+        row-dependent loop bounds."""
+        if not self.spec.stream_loads:
+            return False
+        if self.spec.kind == "flat":
+            return True
+        return self.bounds_vary or any(_uses_name(e, self.a.var) for e in _elts(sub))
+
     def vector_body(self, body, var: str, base_code: str, V: int, loads, stores, declare_locals=False):
         """Emit V consecutive iterations starting at ``base_code``: vector
         loads first, the V scalar bodies, vector stores last."""
         regs = {}
         comp = "xyzw"
-        ld = "vload_stream" if self.spec.stream_loads else "vload"
         for key, (arr, sub) in loads.items():
             r = self.fresh(f"ld_{arr.name}_")
             regs[key] = r
+            ld = "vload_stream" if self._streamed(sub) else "vload"
             self.w(f"const appy::vec<{arr.elem_c}, {V}>::type {r} = "
                    f"appy::{ld}<{arr.elem_c}, {V}>({self._addr(arr, sub, var, base_code)});")
         sregs = {}
@@ -472,6 +494,9 @@ class KernelBuilder:
             self.w(f"{ty.c} {p} = {T.identity_literal(op, ty)};")
         saved_mode = self.mode
         self.mode = "lane"
+        saved_vary = self.bounds_vary
+        outer_locals = set(self.a.assigned) | {self.a.var}
+        self.bounds_vary = any(_uses_name(b, n) for b in st.iter.args[:2] for n in outer_locals)
         loads, stores = self._vector_accesses(st.body, var) if V > 1 else ({}, {})
         if V > 1 and (loads or stores):
             nv = self.fresh("nv")
@@ -494,6 +519,7 @@ class KernelBuilder:
         self.ind -= 1
         self.w("}")
         self.mode = saved_mode
+        self.bounds_vary = saved_vary
         for name, op in reds.items():
             p, ty = self.partials[name]
             if ty.size < 4:
@@ -502,6 +528,137 @@ class KernelBuilder:
         self.partials = saved_partials
         self.ind -= 1
         self.w("}")
+
+    # ---- row accumulators ----------------------------------------------------------
+    def _match_row_update(self, loop):
+        """``for c in range(0, E): T[.., c] = T[.., c] (op) rest`` with ``simd``
+        -> (T subscript, op, rest, c, E node) or None."""
+        if not (isinstance(loop, ast.For) and "simd" in (getattr(loop, "pragma", None) or {})
+                and len(loop.body) == 1 and isinstance(loop.body[0], ast.Assign)):
+            return None
+        lo, hi, _ = loop.iter.args
+        if not (isinstance(lo, ast.Constant) and lo.value == 0):
+            return None
+        c = loop.target.id
+        st = loop.body[0]
+        tgt = st.targets[0]
+        if not (isinstance(tgt, ast.Subscript) and isinstance(tgt.value, ast.Name) and tgt.value.id in self.a.arrays):
+            return None
+        el = _elts(tgt)
+        if not (isinstance(el[-1], ast.Name) and el[-1].id == c) or any(_uses_name(e, c) for e in el[:-1]):
+            return None
+        key = ast.unparse(tgt)
+        arr_name = tgt.value.id
+        val = st.value
+        op, rest = None, None
+        if isinstance(val, ast.BinOp) and isinstance(val.op, (ast.Add, ast.Sub, ast.Mult)):
+            if ast.unparse(val.left) == key:
+                op, rest = val.op, val.right
+            elif ast.unparse(val.right) == key and not isinstance(val.op, ast.Sub):
+                op, rest = val.op, val.left
+        if op is None:
+            # plain store T[.., c] = rest (the initialisation form)
+            op, rest = None, val
+        if any(isinstance(n, ast.Name) and n.id == arr_name for n in ast.walk(rest)):
+            return None
+        return tgt, op, rest, c, hi
+
+    def row_accumulate(self, stmts, i) -> int:
+        """Keep a row ``T[.., :]`` that a sequential loop updates once per
+        iteration in registers: one load (or the initial value) before the
+        loop, one store after it, instead of a read-modify-write of the row in
+        memory per iteration.  Legal because the row belongs to this team's
+        outer iteration alone.  Returns the number of statements consumed."""
+        W, V, E = self.spec.width, self.spec.vec, self.spec.extent
+        init = None
+        k = i
+        m0 = self._match_row_update(stmts[k])
+        if m0 is not None and m0[1] is None and k + 1 < len(stmts):
+            init = m0
+            k += 1
+        kloop = stmts[k]
+        if not (isinstance(kloop, ast.For) and "simd" not in (getattr(kloop, "pragma", None) or {})
+                and len(kloop.body) == 1):
+            return 0
+        m1 = self._match_row_update(kloop.body[0])
+        if m1 is None or m1[1] is None:
+            return 0
+        tgt, op, rest, c, hi = m1
+        kvar = kloop.target.id
+        if _uses_name(tgt, kvar) or E % V != 0:
+            return 0
+        if init is not None:
+            itgt, _, ival, ic, ihi = init
+            same_row = ast.unparse(_Rename(ic, c).visit(_copy(itgt))) == ast.unparse(tgt)
+            if not same_row or ast.unparse(ihi) != ast.unparse(hi) or _uses_name(ival, ic):
+                return 0
+        arr = self.a.arrays[tgt.value.id]
+        arr.loaded = arr.loaded or init is None
+        nv = -(-E // (W * V))
+        if nv > 8:
+            return 0
+        vt = f"appy::vec<{arr.elem_c}, {V}>::type"
+        comp = "xyzw"
+        self.ex.locals[c] = T.WEAK_INT
+        self.w("{")
+        self.ind += 1
+        ec, et = self.ex.emit(hi)
+        self.w(f"// row accumulators: extent {E} is fixed at compile time (asserted by the launcher)")
+        accs = [self.fresh("acc") for _ in range(nv)]
+        bases = [f"(({t * W}LL + __lane) * {V})" for t in range(nv)]
+        full = [(t + 1) * W * V <= E for t in range(nv)]
+        for t in range(nv):
+            self.w(f"{vt} {accs[t]};")
+            guard = "" if full[t] else f"if ({bases[t]} < {E}LL) "
+            if init is not None:
+                vc, vty = self.ex.emit(init[2])
+                val = self._store_value(vc, vty, arr)
+                self.w(f"{guard}{{ " + " ".join(f"{accs[t]}.{comp[v]} = {val};" for v in range(V)) + " }")
+            else:
+                self.w(f"{guard}{accs[t]} = appy::vload<{arr.elem_c}, {V}>({self._addr(arr, tgt, c, bases[t])});")
+        lo_c, hi_c = self._range_args(kloop)
+        self.ex.locals[kvar] = T.WEAK_INT
+        hi_v = self.fresh("hi")
+        self.w(f"const appy::i64 {hi_v} = {hi_c};")
+        self.w("#pragma unroll 4")
+        self.w(f"for (appy::i64 {cname(kvar)} = {lo_c}; {cname(kvar)} < {hi_v}; ++{cname(kvar)}) {{")
+        self.ind += 1
+        saved_mode = self.mode
+        self.mode = "lane"
+        loads, _ = self._vector_accesses([ast.Assign(targets=[ast.Name(id="__rest", ctx=ast.Store())], value=rest)], c)
+        sym = {ast.Add: "+", ast.Sub: "-", ast.Mult: "*"}[type(op)]
+        for t in range(nv):
+            self.w("{" if full[t] else f"if ({bases[t]} < {E}LL) {{")
+            self.ind += 1
+            regs = {}
+            for key, (larr, lsub) in loads.items():
+                r = self.fresh(f"ld_{larr.name}_")
+                regs[key] = r
+                ld = "vload_stream" if (self.spec.stream_loads and _uses_name(lsub, self.a.var)) else "vload"
+                self.w(f"const appy::vec<{larr.elem_c}, {V}>::type {r} = "
+                       f"appy::{ld}<{larr.elem_c}, {V}>({self._addr(larr, lsub, c, bases[t])});")
+            for v in range(V):
+                saved = dict(self.ex.load_subst)
+                for key, (larr, _) in loads.items():
+                    code = f"{regs[key]}.{comp[v]}"
+                    self.ex.load_subst[key] = ((f"({code} != 0)" if larr.ty.is_bool else code), larr.ty)
+                self.w(f"{{ const appy::i64 {cname(c)} = {bases[t]} + {v};")
+                rc, rty = self.ex.emit(rest)
+                a = f"{accs[t]}.{comp[v]}"
+                rt_ = T.promote(arr.ty, rty)
+                self.w(f"  {a} = {cast(f'({cast(a, arr.ty, rt_)} {sym} {cast(rc, rty, rt_)})', rt_, arr.ty)}; }}")
+                self.ex.load_subst = saved
+            self.ind -= 1
+            self.w("}")
+        self.mode = saved_mode
+        self.ind -= 1
+        self.w("}")
+        for t in range(nv):
+            guard = "" if full[t] else f"if ({bases[t]} < {E}LL) "
+            self.w(f"{guard}appy::vstore<{arr.elem_c}, {V}>({self._addr(arr, tgt, c, bases[t])}, {accs[t]});")
+        self.ind -= 1
+        self.w("}")
+        return k - i + 1
 
     # ---- kernel skeletons ---------------------------------------------------------
     def _declare_locals(self):
@@ -562,7 +719,6 @@ class KernelBuilder:
 
     def _flat_unrolled_tile(self, V, U, B, loads, stores):
         comp = "xyzw"
-        ld = "vload_stream" if self.spec.stream_loads else "vload"
         var = self.a.var
         regs = {}
         for u in range(U):
@@ -570,6 +726,7 @@ class KernelBuilder:
             for key, (arr, sub) in loads.items():
                 r = self.fresh(f"ld_{arr.name}_")
                 regs[(u, key)] = r
+                ld = "vload_stream" if self._streamed(sub) else "vload"
                 self.w(f"const appy::vec<{arr.elem_c}, {V}>::type {r} = "
                        f"appy::{ld}<{arr.elem_c}, {V}>({self._addr(arr, sub, var, base)});")
         sregs = {}

@@ -41,6 +41,10 @@ def _sorted_unique_columns(rng, lengths, ncols):
     indptr = np.zeros(len(lengths) + 1, dtype=np.int64)
     np.cumsum(lengths, out=indptr[1:])
     nnz = int(indptr[-1])
+    if len(lengths) and int(lengths.max()) * 4 > ncols:
+        # dense rows: rejection would not terminate, draw each row without replacement
+        cols = np.concatenate([np.sort(rng.permutation(ncols)[: int(n)]) for n in lengths] or [np.empty(0, np.int64)])
+        return indptr, cols.astype(np.int64)
     if len(lengths) and np.all(lengths == lengths[0]) and lengths[0] > 0:
         # equal rows: sort each row on its own, redraw the rows that hold a duplicate
         L = int(lengths[0])
