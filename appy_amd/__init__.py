@@ -51,6 +51,9 @@ def rewrite_loops(fn, **options):
     tree = _source.parse(source)
     if options.get("shader", False):
         raise NotImplementedError("shader loops are not part of the HIP execution path")
+    # carried to the code generator through the stub: names the device kernels
+    # after the function they come from, which keeps profiles readable
+    options.setdefault("fn_name", fn.__name__)
     tree, _loops = _static_rewrite.transform(tree, options)
     new_source = ast.unparse(tree)
     if options["verbose_static_rewrite"]:

@@ -250,7 +250,9 @@ class CompiledLoop:
             with self._lock:
                 k = self.kernels.get(spec)
                 if k is None:
-                    builder = KernelBuilder(self.analysis, self.loop_name, self.module_names, spec)
+                    fn = self.options.get("fn_name")
+                    sym = f"{fn}_{self.loop_name}" if fn and str(fn).isidentifier() else self.loop_name
+                    builder = KernelBuilder(self.analysis, sym, self.module_names, spec)
                     k = Kernel(builder.build(device_header()))
                     self.kernels[spec] = k
         return k
@@ -392,6 +394,15 @@ class Launch:
         self.lo, self.hi = lo, hi
         self.temps = []          # (dptr, host ndarray (contiguous), original, stored)
         self.keepalive = []
+        # -- bounds of accesses indexed by the parallel loop variable (host check, before any device work)
+        for name, dim, off in a.bound_checks:
+            ext = arrays[name].shape[dim]
+            if lo + off < 0 or hi - 1 + off >= ext:
+                raise IndexError(
+                    f"{loop.loop_name}: `{name}` has extent {ext} in dimension {dim} but the loop "
+                    f"range [{lo}, {hi}) indexes it at offset {off:+d}"
+                )
+
         self.stream = 0
         device = 0
         # -- device and stream: PyTorch's when a GPU tensor takes part
@@ -403,15 +414,6 @@ class Launch:
             self.stream = torch.cuda.current_stream(device).cuda_stream
         _ensure_device(device)
         self.device = device
-
-        # -- bounds of accesses indexed by the parallel loop variable
-        for name, dim, off in a.bound_checks:
-            ext = arrays[name].shape[dim]
-            if lo + off < 0 or hi - 1 + off >= ext:
-                raise IndexError(
-                    f"{loop.loop_name}: `{name}` has extent {ext} in dimension {dim} but the loop "
-                    f"range [{lo}, {hi}) indexes it at offset {off:+d}"
-                )
 
         # -- device pointers and strides
         self.ptr = {}
@@ -548,7 +550,7 @@ def _copy(node):
 # ---------------------------------------------------------------------------
 def codegen(loop_source, loop_name, val_map, options):
     key = (loop_source, loop_name, _signature(val_map), options.get("hip_spec") and repr(options.get("hip_spec")),
-           options.get("hip_max_blocks"))
+           options.get("hip_max_blocks"), options.get("fn_name"))
     hit = code_cache.get(key)
     if hit is not None:
         return hit

@@ -39,6 +39,12 @@ def vec_add(a, b):
     return c
 
 
+def copy(a, c):
+    #pragma parallel for simd
+    for i in range(a.shape[0]):
+        c[i] = a[i]
+
+
 def vector_sum(A):
     s = 0.0
     #pragma parallel for simd shared(s)
@@ -89,7 +95,7 @@ def spmm(A_data, A_indptr, A_indices, B, y, M):
             y[i, :] += A_data[k] * B[A_indices[k], :]
 
 
-_RAW = (vec_add, vector_sum, masked_sum, gemv, spmv, spmm)
+_RAW = (vec_add, copy, vector_sum, masked_sum, gemv, spmv, spmm)
 _cache = {}
 
 
@@ -124,6 +130,7 @@ def compile_all_patterns() -> int:
     Y = np.empty((8, 128), dtype=np.float32)
     before = set(cg.code_cache)
     k.vec_add(a, a)
+    k.copy(a, np.empty_like(a))
     k.vector_sum(a)
     k.masked_sum(a, m)
     k.gemv(A, x)

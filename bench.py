@@ -38,7 +38,7 @@ def parse_args():
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=50)
     p.add_argument("--warmup", type=int, default=5)
-    p.add_argument("--workloads", default="vector_sum,masked_sum,vec_add,gemv,spmv_uniform,spmv_powerlaw,spmm",
+    p.add_argument("--workloads", default="vector_sum,masked_sum,copy,vec_add,gemv,spmv_uniform,spmv_powerlaw,spmm",
                    help="comma separated subset; vector_sum is always run (headline)")
     p.add_argument("--scale", type=float, default=1.0, help="shrink every size by this factor (debugging)")
     p.add_argument("--no-cpu-baseline", action="store_true")
@@ -214,6 +214,23 @@ def main():
         del M_d
     del A_d, A, M
     torch.cuda.empty_cache()
+
+    # ---------------- calibration: plain copy of known size -------------------------------
+    # c[i] = a[i] over 2^28 float32: 1 GiB read + 1 GiB written.  Used to scale the
+    # FETCH_SIZE / WRITE_SIZE counters of profiling runs and as the streaming reference.
+    if "copy" in want:
+        nc = shrink(1 << 28)
+        a_d = torch.empty(nc, dtype=torch.float32, device="cuda").uniform_(-1, 1)
+        c_d = torch.empty_like(a_d)
+        before = set(cg.code_cache)
+        selfcheck.kernels().copy(a_d, c_d)
+        loop = run.loop_of(before)
+        ok = bool(torch.equal(a_d, c_d))
+        parity["copy"] = {"bit_exact": ok, "ok": ok}
+        results["copy"] = run.measure(loop, {"c": c_d, "a": a_d, "a_shape_0": nc}, 8 * nc, K, W)
+        log("copy", results["copy"], parity["copy"])
+        del a_d, c_d
+        torch.cuda.empty_cache()
 
     # ---------------- config 1: vec_add ---------------------------------------------------
     if "vec_add" in want:

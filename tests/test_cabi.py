@@ -1,0 +1,71 @@
+"""The C-ABI library: loads, exports exactly what include/appy_hip.h declares,
+and its GPU-independent entry points (run-time compilation, error reporting)
+behave as documented.  No kernel is launched here."""
+import ctypes
+import os
+import re
+import subprocess
+
+import pytest
+
+from appy_amd.backends.hip import runtime as rt
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "appy_hip.h")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(appy_hip_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_and_binding_agree():
+    decl = declared_symbols()
+    assert len(decl) >= 25
+    assert sorted(rt.SIGNATURES) == decl
+
+
+def test_library_exports_every_declared_symbol():
+    lib = ctypes.CDLL(rt.library_path())
+    for name in declared_symbols():
+        assert hasattr(lib, name), name
+    out = subprocess.run(["nm", "-D", "--defined-only", rt.library_path()], capture_output=True, text=True, check=True).stdout
+    exported = set(re.findall(r"\bT (appy_hip_[a-z0-9_]+)", out))
+    assert exported == set(declared_symbols())          # nothing undeclared leaks out either
+
+
+def test_abi_version():
+    assert rt.lib().appy_hip_abi_version() == rt.ABI_VERSION
+    text = open(HEADER).read()
+    assert f"#define APPY_HIP_ABI_VERSION {rt.ABI_VERSION}" in text
+
+
+def test_compile_produces_a_gfx950_code_object():
+    src = 'extern "C" __global__ void k(float* a, long long n) { long long i = blockIdx.x * 64ll + threadIdx.x; if (i < n) a[i] += 1.0f; }'
+    code = rt.compile_to_code_object(src, "k.hip")
+    assert code[:4] == b"\x7fELF" and len(code) > 1000
+    assert b"gfx950" in code
+
+
+def test_compile_error_carries_the_compiler_log():
+    with pytest.raises(rt.HipError) as e:
+        rt.compile_to_code_object('extern "C" __global__ void k() { this is not C++; }', "bad.hip")
+    assert e.value.code >= 10000                          # hiprtc result space
+    assert "error" in str(e.value) and "bad.hip" in str(e.value)
+
+
+def test_invalid_arguments_are_reported_not_crashed():
+    lib = rt.lib()
+    assert lib.appy_hip_device_count(None) != 0
+    assert "count_out" in rt.last_error()
+    assert lib.appy_hip_launch(None, 1, 1, 1, 64, 1, 1, 0, None, None, 0) != 0
+    assert "func" in rt.last_error()
+    ms = ctypes.c_float()
+    assert lib.appy_hip_launch_timed(None, 1, 1, 1, 64, 1, 1, 0, None, None, 0, 0, 1, ctypes.byref(ms)) != 0
+    assert lib.appy_hip_free(None) == 0                   # freeing NULL is a no-op
+    assert lib.appy_hip_module_unload(None) == 0
+
+
+def test_device_count_without_gpu_is_zero_not_an_error():
+    assert rt.device_count() >= 0

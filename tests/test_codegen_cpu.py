@@ -1,0 +1,153 @@
+"""Code generator checks that need no GPU: every kernel is generated and
+compiled to a gfx950 code object through the C ABI (hiprtc), and the generated
+text is inspected for the properties the design relies on."""
+import numpy as np
+import pytest
+
+import appy_amd as appy
+from appy_amd.backends.hip import codegen as cg
+from appy_amd.backends.hip import dtypes as T
+from appy_amd.backends.hip import selfcheck
+from appy_amd.backends.hip.kernelgen import Spec
+
+
+def compiled(loop_source, **vals):
+    vals.setdefault("np", np)
+    f, src = cg.codegen(loop_source, "kernel_loop_1", vals, {"dump_code": False})
+    return f, src
+
+
+def body_of(src):
+    return src[src.index("// kernel for"):]
+
+
+def test_all_workload_patterns_compile_for_gfx950():
+    assert selfcheck.compile_all_patterns() >= 6
+
+
+def test_vec_add_uses_128_bit_accesses_and_restrict():
+    a = np.zeros(8, np.float32)
+    f, src = compiled("#pragma parallel for simd\nfor i in range(a_shape_0):\n    c[i] = a[i] + b[i]", c=a, a=a, b=a, a_shape_0=8)
+    k = body_of(src)
+    assert "appy::vload<float, 4>" in k and "appy::vstore<float, 4>" in k
+    assert "float* __restrict__ c" in k and "const float* __restrict__ a" in k
+    assert f.analysis.kind == "flat" and not f.analysis.outer_reductions
+    assert f.kernels[f.default_spec].code[:4] == b"\x7fELF"
+
+
+def test_shared_reduction_ends_in_one_atomic_per_workgroup():
+    s = np.zeros(1)
+    a = np.zeros(8, np.float32)
+    f, src = compiled("#pragma parallel for simd shared(s)\nfor i in range(n):\n    s[0] += a[i]", s=s, a=a, n=8)
+    k = body_of(src)
+    assert k.count("atomic_combine") == 1 and "block_reduce<appy::OpAdd, 256, double>" in k
+    assert "double __acc0" in k                      # accumulates in the dtype of the shared buffer
+    assert "if (threadIdx.x == 0)" in k
+    red = f.analysis.outer_reductions[0]
+    assert (red.key, red.op, red.ty.name) == ("s[0]", "+", "float64")
+    assert f.grid_for(f.default_spec, 1 << 28) == 1024        # persistent: 4 workgroups per CU
+
+
+def test_masked_sum_loads_mask_bytes_as_vectors():
+    s = np.zeros(1)
+    a = np.zeros(8, np.float32)
+    m = np.zeros(8, bool)
+    _, src = compiled("#pragma parallel for simd shared(s)\nfor i in range(n):\n    s[0] += a[i] if m[i] else 0.0",
+                      s=s, a=a, m=m, n=8)
+    k = body_of(src)
+    assert "appy::vload<unsigned char, 4>" in k and "appy::vload<float, 4>" in k
+
+
+def test_weak_scalars_follow_numpy_promotion():
+    a32 = np.zeros(8, np.float32)
+    _, src = compiled("#pragma parallel for simd\nfor i in range(n):\n    c[i] = alpha * a[i] + 1.5", c=a32, a=a32, alpha=2.0, n=8)
+    k = body_of(src)
+    assert "(float)(alpha)" in k and "(float)(1.5)" in k       # Python floats adopt float32
+    a_i = np.zeros(8, np.int32)
+    c64 = np.zeros(8)
+    _, src = compiled("#pragma parallel for simd\nfor i in range(n):\n    c[i] = a[i] * 0.5", c=c64, a=a_i, n=8)
+    assert "(double)" in body_of(src)                          # int32 * Python float -> float64
+    assert T.promote(T.F32, T.WEAK_FLOAT) == T.F32
+    assert T.promote(T.I32, T.WEAK_FLOAT) == T.F64
+    assert T.promote(T.I32, T.WEAK_INT) == T.I32
+    assert T.true_divide(T.I32, T.I32) == T.F64
+    assert T.join(T.WEAK_FLOAT, T.F32) == T.F32
+
+
+def test_local_accumulator_takes_the_numpy_type():
+    A = np.zeros((4, 8), np.float32)
+    x = np.zeros(8, np.float32)
+    y = np.zeros(4, np.float32)
+    text = ("#pragma parallel for\nfor i in range(r):\n    yi = 0.0\n    #pragma simd\n"
+            "    for j in range(c):\n        yi += A[i, j] * x[j]\n    y[i] = yi")
+    f, src = compiled(text, A=A, x=x, y=y, r=4, c=8)
+    k = body_of(src)
+    assert "float yi" in k and "team_reduce<appy::OpAdd" in k
+    assert f.analysis.kind == "team"
+    assert "if (__lane == 0) { y[i]" in k                      # one store per row
+
+
+def test_team_width_follows_the_row_length():
+    f, _ = selfcheck_loop("spmv")
+    arrays = {"A_data": np.zeros(16 * 1000, np.float32)}
+    assert f.choose_spec(1000, {}, arrays).width == 4           # 16 non-zeros, 4 per lane
+    arrays = {"A_data": np.zeros(97 * 1000, np.float32)}
+    assert f.choose_spec(1000, {}, arrays).width == 32
+    g, _ = selfcheck_loop("gemv")
+    assert g.choose_spec(16384, {"A_shape_1": 16384}, {}).width == 32
+
+
+def selfcheck_loop(name):
+    selfcheck.compile_all_patterns()
+    for key, (loop, src) in cg.code_cache.items():
+        if name == "spmv" and "x[A_indices[j]]" in key[0]:
+            return loop, src
+        if name == "gemv" and "A[i, j] * x[j]" in key[0]:
+            return loop, src
+        if name == "spmm" and "B[A_indices[k], :]" in key[0]:
+            return loop, src
+    raise AssertionError(name)
+
+
+def test_spmm_row_lives_in_registers():
+    loop, _ = selfcheck_loop("spmm")
+    spec = Spec("team", block=256, vec=4, width=32, extent=128)
+    k = body_of(loop.kernel_for(spec).src.text)
+    assert "row accumulators" in k
+    inner = k[k.index("for (appy::i64 k ="):]
+    loop_body = inner[: inner.index("appy::vstore")]
+    assert "y[" not in loop_body and "appy::vload<float, 4>(y" not in loop_body     # no traffic to y inside the k loop
+    assert k.count("appy::vstore<float, 4>(y") == 1
+    # without a compile-time extent the generic (memory read-modify-write) form is used
+    k2 = body_of(loop.kernel_for(Spec("team", block=256, vec=4, width=32)).src.text)
+    assert "row accumulators" not in k2
+
+
+def test_array_statement_lowering():
+    A = np.zeros((4, 8))
+    x = np.zeros(8)
+    y = np.zeros(4)
+    f, src = compiled("#pragma parallel for\nfor i in range(r):\n    y[i] = np.sum(alpha * A[i, :] * x[:])", A=A, x=x, y=y, r=4, alpha=1.5)
+    k = body_of(src)
+    assert "A_shape_1" in k and "team_reduce<appy::OpAdd" in k
+    assert f.derived_shapes["A_shape_1"] == ("A", 1)
+    _, src = compiled("#pragma parallel for\nfor i in range(r):\n    y[i] = A[i, :] @ x[:]", A=A, x=x, y=y, r=4)
+    assert "team_reduce<appy::OpAdd" in body_of(src)
+    _, src = compiled("#pragma parallel for\nfor i in range(r):\n    A[i, 2:6] = x[0:4] + 1.0", A=A, x=x, r=4)
+    assert "(6LL - 2LL)" in body_of(src)
+
+
+def test_non_simd_parallel_loop_with_control_flow():
+    a = np.zeros(8)
+    m = np.zeros(8, bool)
+    b = np.zeros(1)
+    f, src = compiled("#pragma parallel for shared(b)\nfor i in range(n):\n    if m[i]:\n        b[0] += a[i]", a=a, m=m, b=b, n=8)
+    k = body_of(src)
+    assert f.default_spec.vec == 1 and "if ((m[i] != 0))" in k and "atomic_combine" in k
+
+
+def test_out_of_range_loop_is_caught_on_the_host():
+    a = np.zeros(8, np.float32)
+    f, _ = compiled("#pragma parallel for simd\nfor i in range(n):\n    c[i] = a[i + 1]", c=a, a=a, n=8)
+    with pytest.raises(IndexError):
+        f.prepare({"c": a, "a": a, "n": 8})

@@ -1,0 +1,174 @@
+"""Decoration-time rewrite and per-loop IR.
+
+Expected forms are the worked rewrites of the reference's passes
+(appy/frontend/process_shared.py:59-74, replace_pfor_with_stub.py:4-13,
+hoist_shape_attr.py:19-48, reduction_detection.py:1-9)."""
+import ast
+
+import numpy as np
+import pytest
+
+import appy_amd as appy
+from appy_amd.frontend import loop_ir, names, source, static_rewrite
+
+
+def rewrite(src, **options):
+    appy.set_default_options(options)
+    tree, loops = static_rewrite.transform(source.parse(src), options)
+    return ast.unparse(tree), loops
+
+
+VEC_SUM = '''
+@appy.jit
+def vector_sum(A):
+    s = 0.0
+    #pragma parallel for simd shared(s)
+    for i in range(A.shape[0]):
+        s += A[i]
+    return s
+'''
+
+
+def test_shared_rewrite_and_stub():
+    text, loops = rewrite(VEC_SUM)
+    lines = [l.strip() for l in text.splitlines()]
+    assert lines[0] == "def vector_sum(A):"            # decorator removed
+    assert "A_shape_0 = A.shape[0]" in lines
+    assert "s = numpy.array([s])" in lines
+    assert "s = s.item()" in lines
+    assert lines.index("s = numpy.array([s])") < lines.index("s = s.item()")
+    assert loops == [("kernel_loop_1",
+                      "#pragma parallel for simd shared(s)\nfor i in range(A_shape_0):\n    s[0] += A[i]")]
+    assert "appy._kernel_launch(" in text and "locals(), globals()" in text
+
+
+def test_inner_pragmas_stay_in_the_loop_text_and_numbering():
+    src = '''
+def f(A, x, y, z):
+    #pragma parallel for
+    for i in range(A.shape[0]):
+        yi = 0.0
+        #pragma simd
+        for j in range(A.shape[1]):
+            yi += A[i, j] * x[j]
+        y[i] = yi
+    #pragma parallel for simd
+
+    for i in range(z.shape[0]):
+        z[i] = 0
+'''
+    text, loops = rewrite(src)
+    assert [n for n, _ in loops] == ["kernel_loop_1", "kernel_loop_2"]
+    assert "#pragma simd" in loops[0][1]
+    assert loops[0][1].startswith("#pragma parallel for\nfor i in range(A_shape_0):")
+    assert "A_shape_1" in loops[0][1]
+    assert loops[1][1].startswith("#pragma parallel for simd\n")   # blank line after the pragma is fine
+    assert "__appy_pragma__" not in text
+
+
+def test_options_are_embedded_as_literals():
+    text, _ = rewrite(VEC_SUM, dump_code=True)
+    assert "'dump_code': True" in text and "'backend': None" in text
+
+
+def test_function_without_pragma_is_unchanged_in_behaviour():
+    @appy.jit
+    def passthrough(x):
+        return x
+
+    @appy.jit
+    def bump(x):
+        for i in range(x.shape[0]):
+            x[i] += 1
+        return x
+
+    @appy.jit
+    def total(x):
+        s = 0
+        for i in range(x.shape[0]):
+            s += x[i]
+        return s
+
+    assert passthrough([1, 2, 3]) == [1, 2, 3]
+    assert all(bump(np.zeros(10)) == np.ones(10))
+    assert total(np.arange(10)) == 45
+
+
+def test_prange_loop_is_outlined():
+    src = '''
+def f(a):
+    for i in appy.prange(a.shape[0]):
+        a[i] = 1
+'''
+    _, loops = rewrite(src)
+    assert loops and loops[0][1].startswith("for i in appy.prange(")
+
+
+# ---- per-loop IR ---------------------------------------------------------------
+def test_ir_vec_add():
+    tree = loop_ir.build("#pragma parallel for simd\nfor i in range(a_shape_0):\n    c[i] = a[i] + b[i]")
+    loop = loop_ir.outer_loop(tree)
+    assert dict(loop.pragma) == {"parallel_for": True, "simd": True}
+    assert ast.unparse(loop.iter) == "range(0, a_shape_0, 1)"
+    assert "reduction" not in loop.pragma
+
+
+def test_ir_shared_sum_is_a_reduction():
+    tree = loop_ir.build("#pragma parallel for simd shared(b)\nfor i in range(n):\n    b[0] += a[i]")
+    loop = loop_ir.outer_loop(tree)
+    assert loop.pragma["reduction"] == "+:b[0]"
+    assert loop.body[0].reduce == "+"
+    assert ast.unparse(loop.body[0]) == "b[0] = b[0] + a[i]"
+    assert loop_ir.reductions_of(loop) == {"b[0]": "+"}
+
+
+def test_ir_max_min_and_product():
+    for fn in ("max", "min"):
+        tree = loop_ir.build(f"#pragma parallel for simd shared(m)\nfor i in range(n):\n    m[0] = {fn}(m[0], a[i])")
+        assert loop_ir.outer_loop(tree).pragma["reduction"] == f"{fn}:m[0]"
+    tree = loop_ir.build("#pragma parallel for simd shared(p)\nfor i in range(n):\n    p[0] = a[i] * p[0]")
+    assert loop_ir.outer_loop(tree).pragma["reduction"] == "*:p[0]"
+
+
+def test_ir_gemv_inner_reduction_only():
+    tree = loop_ir.build(
+        "#pragma parallel for\nfor i in range(A_shape_0):\n    yi = 0.0\n    #pragma simd\n"
+        "    for j in range(A_shape_1):\n        yi += A[i, j] * x[j]\n    y[i] = yi")
+    outer = loop_ir.outer_loop(tree)
+    inner = outer.body[1]
+    assert "reduction" not in outer.pragma          # yi has both a plain and a '+' assignment out here
+    assert dict(inner.pragma) == {"simd": True, "reduction": "+:yi"}
+
+
+def test_ir_tuple_assignment_split():
+    tree = loop_ir.build("#pragma parallel for\nfor i in range(M):\n    start, end = p[i], p[i + 1]\n    y[i] = end - start")
+    body = loop_ir.outer_loop(tree).body
+    assert [ast.unparse(s) for s in body[:2]] == ["start = p[i]", "end = p[i + 1]"]
+
+
+def test_ir_pragma_is_consumed_by_an_assignment():
+    # '#pragma simd' above 's = 0.0' annotates the assignment; the loop after it stays sequential
+    tree = loop_ir.build(
+        "#pragma parallel for\nfor i in range(n):\n    #pragma simd\n    s = 0.0\n"
+        "    for j in range(m):\n        s += a[i, j]\n    b[i] = s")
+    outer = loop_ir.outer_loop(tree)
+    assert hasattr(outer.body[0], "pragma") and not hasattr(outer.body[1], "pragma")
+
+
+def test_ir_step_must_be_one():
+    with pytest.raises(Exception) as e:
+        loop_ir.build("#pragma parallel for simd\nfor i in range(0, n, 2):\n    c[i] = a[i]")
+    assert "range" in str(e.value) and "step" in str(e.value)
+
+
+def test_ir_structure_checks():
+    with pytest.raises(AssertionError):
+        loop_ir.build("for i in range(n):\n    c[i] = a[i]")
+    with pytest.raises(Exception) as e:
+        loop_ir.build("#pragma parallel for\nfor i in range(n):\n    c[i] = 0\nfor j in range(n):\n    c[j] = 1")
+    assert "single for loop" in str(e.value)
+
+
+def test_used_names_order_and_callees():
+    text = "#pragma parallel for\nfor i in range(M):\n    s = max(A[i], x[idx[i]])\n    y[i] = np.sqrt(s)"
+    assert names.used_names(text) == ("i", "M", "s", "A", "x", "idx", "y", "np")

@@ -1,0 +1,245 @@
+"""The reference's GPU integration tests for the loop patterns, run through
+``import appy`` exactly as written there (tests/integration/triton/tutorial/:
+test_vec_add.py:4-19, test_global_reduction.py:4-44, test_rowwise_reduction.py:4-53,
+test_mat_add.py:5-20, test_spmv.py:10-30, test_pi.py:8-26, test_var_write.py:12-23;
+npbench/test_gesummv.py:26-55 for array expressions), plus in-place use of GPU
+tensors.  ``backend="triton"`` in those files selects "the GPU back end"."""
+import warnings
+
+import numpy as np
+import pytest
+import scipy.sparse as sp
+
+import appy
+
+pytestmark = pytest.mark.gpu
+warnings.filterwarnings("ignore", message="backend='triton'")
+
+
+@appy.jit(backend="triton")
+def t_vec_add(a, b):
+    c = np.empty_like(a)
+    #pragma parallel for simd
+    for i in range(a.shape[0]):
+        c[i] = a[i] + b[i]
+    return c
+
+
+@appy.jit(backend="triton", dry_run=0)
+def t_vec_sum(a):
+    sum = 0.0
+    #pragma parallel for simd shared(sum)
+    for i in range(a.shape[0]):
+        sum += a[i]
+    return sum
+
+
+@appy.jit(backend="triton", dry_run=0)
+def t_vec_max(a):
+    m = -np.inf
+    #pragma parallel for simd shared(m)
+    for i in range(a.shape[0]):
+        m = max(m, a[i])
+    return m
+
+
+@appy.jit(backend="triton", dry_run=0)
+def t_vec_min(a):
+    m = np.inf
+    #pragma parallel for simd shared(m)
+    for i in range(a.shape[0]):
+        m = min(m, a[i])
+    return m
+
+
+@appy.jit(backend="triton")
+def t_rowwise_sum(a, b):
+    #pragma parallel for
+    for i in range(a.shape[0]):
+        #pragma simd
+        s = 0.0
+        for j in range(a.shape[1]):
+            s += a[i, j]
+        b[i] = s
+
+
+@appy.jit(backend="triton")
+def t_rowwise_max(a, b):
+    #pragma parallel for
+    for i in range(a.shape[0]):
+
+        s = -1e308
+        #pragma simd
+        for j in range(a.shape[1]):
+            s = max(s, a[i, j])
+        b[i] = s
+
+
+@appy.jit(backend="triton")
+def t_rowwise_min(a, b):
+    #pragma parallel for
+    for i in range(a.shape[0]):
+
+        s = 1e308
+        #pragma simd
+        for j in range(a.shape[1]):
+            s = min(s, a[i, j])
+        b[i] = s
+
+
+@appy.jit(backend="triton")
+def t_mat_add(a, b):
+    c = np.empty_like(a)
+    #pragma parallel for
+    for i in range(a.shape[0]):
+        #pragma simd
+        for j in range(a.shape[1]):
+            c[i, j] = a[i, j] + b[i, j]
+    return c
+
+
+@appy.jit(backend="triton")
+def t_spmv(A_data, A_indptr, A_indices, x, M, N):
+    y = np.empty(M, dtype=x.dtype)
+    #pragma parallel for
+    for i in range(M):
+        start, end = A_indptr[i], A_indptr[i+1]
+        s = 0.0
+        #pragma simd
+        for j in range(start, end):
+            s += A_data[j] * x[A_indices[j]]
+        y[i] = s
+    return y
+
+
+@appy.jit
+def t_pi(num_steps, step):
+    sum = 0.0
+    #pragma parallel for simd shared(sum,step)
+    for i in range(1, num_steps + 1):
+        x = (i - 0.5) * step
+        sum += 4.0 / (1.0 + x * x)
+    return step * sum
+
+
+@appy.jit
+def t_var_write():
+    a = 0
+    #pragma parallel for shared(a)
+    for i in range(10):
+        if i == 3:
+            a = 1
+    return a
+
+
+@appy.jit(backend="triton")
+def t_gesummv(alpha, beta, A, B, x):
+    y = np.empty((A.shape[0], ), dtype=x.dtype)
+    #pragma parallel for
+    for i in range(A.shape[0]):
+        s = 0.0
+        #pragma simd
+        for j in range(A.shape[1]):
+            s += alpha * A[i, j] * x[j] + beta * B[i, j] * x[j]
+        y[i] = s
+    return y
+
+
+@appy.jit(backend="triton")
+def t_gesummv1(alpha, beta, A, B, x):
+    y = np.empty((A.shape[0], ), dtype=x.dtype)
+    #pragma parallel for
+    for i in range(A.shape[0]):
+        y[i] = np.sum(alpha * A[i, :] * x[:] + beta * B[i, :] * x[:])
+    return y
+
+
+def test_vec_add(gpu):
+    a = np.ones(100)
+    b = np.ones(100)
+    assert np.allclose(t_vec_add(a, b), a + b)
+
+
+def test_global_reductions(gpu):
+    a = np.random.default_rng(0).random(1000)
+    assert np.allclose(t_vec_sum(a), a.sum())
+    assert np.allclose(t_vec_max(a), a.max())
+    assert np.allclose(t_vec_min(a), a.min())
+    big = np.random.default_rng(1).standard_normal(1_000_003)
+    assert t_vec_max(big) == big.max() and t_vec_min(big) == big.min()
+
+
+def test_rowwise_reductions(gpu):
+    a = np.random.default_rng(2).random((100, 100))
+    b = np.empty(100)
+    t_rowwise_sum(a, b)
+    assert np.allclose(b, a.sum(axis=1))
+    t_rowwise_max(a, b)
+    assert np.allclose(b, a.max(axis=1))
+    t_rowwise_min(a, b)
+    assert np.allclose(b, a.min(axis=1))
+
+
+def test_mat_add(gpu):
+    a = np.ones((100, 100))
+    b = np.ones((100, 100))
+    assert np.allclose(t_mat_add(a, b), a + b)
+    r = np.random.default_rng(3).standard_normal((37, 211)).astype(np.float32)
+    assert np.array_equal(t_mat_add(r, r), r + r)
+
+
+def test_spmv_csr(gpu):
+    N = 1000
+    A = sp.random(N, N, density=0.01, format="csr", random_state=4)
+    x = np.random.default_rng(5).random(N)
+    y = t_spmv(A.data, A.indptr, A.indices, x, N, N)
+    assert np.allclose(y, A @ x, atol=1e-6)
+
+
+def test_pi(gpu):
+    num_steps = 1_000_000
+    step = 1.0 / num_steps
+    assert np.isclose(t_pi(num_steps, step), np.pi, rtol=1e-06, atol=1e-08)
+
+
+def test_var_write(gpu):
+    assert t_var_write() == 1
+
+
+def test_gesummv_loops_and_array_expressions(gpu):
+    N = 100
+    alpha, beta = 1.5, 1.2
+    A = np.fromfunction(lambda i, j: ((i * j + 1) % N) / N, (N, N), dtype=np.float64)
+    B = np.fromfunction(lambda i, j: ((i * j + 2) % N) / N, (N, N), dtype=np.float64)
+    x = np.fromfunction(lambda i: (i % N) / N, (N,), dtype=np.float64)
+    ref = alpha * A @ x + beta * B @ x
+    assert np.allclose(ref, t_gesummv(alpha, beta, A, B, x))
+    assert np.allclose(ref, t_gesummv1(alpha, beta, A, B, x))
+
+
+def test_gpu_tensors_are_used_in_place(gpu):
+    import torch
+
+    a = torch.arange(10_000, dtype=torch.float32, device="cuda")
+    b = torch.ones(10_000, dtype=torch.float32, device="cuda")
+
+    @appy.jit
+    def add_into(a, b, c):
+        #pragma parallel for simd
+        for i in range(a.shape[0]):
+            c[i] = a[i] + b[i]
+
+    c = torch.empty_like(a)
+    ptr = c.data_ptr()
+    add_into(a, b, c)
+    assert c.data_ptr() == ptr and torch.equal(c, a + b)
+    # a CPU tensor is copied in and out like a NumPy array
+    ac, bc, cc = a.cpu(), b.cpu(), torch.zeros(10_000)
+    add_into(ac, bc, cc)
+    assert torch.equal(cc, ac + bc)
+    # a strided view (last dimension not contiguous) goes through a packed copy
+    base = torch.zeros((100, 8), device="cuda")
+    col = base[:, 3]
+    ones = torch.ones(100, device="cuda")
+    add_into(ones, ones, col)
+    assert torch.equal(base[:, 3], 2 * ones) and float(base.sum()) == 200.0
