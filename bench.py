@@ -28,6 +28,20 @@ if ROOT not in sys.path:
 
 HBM_PEAK_BPS = 8.0e12  # MI355X HBM3E, bytes per second
 
+# HBM traffic per launch (bytes) at the default sizes, from the rocprofv3 counter
+# runs summarised in profiles/all_kernels_bench_pmc_fetch_write_size.txt:
+# FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 (factors from the plain copy kernel), KiB -> bytes.
+MEASURED_TRAFFIC = {
+    "vector_sum": int((524302.8 * 2 + 32.0) * 1024),
+    "masked_sum": int((655384.2 * 2 + 32.0) * 1024),
+    "vec_add": int((65549.0 * 2 + 65536.0) * 1024),
+    "gemv": int((524558.6 * 2 + 64.5) * 1024),
+    "spmv_uniform": int((3442492.9 * 2 + 18586.1) * 1024),
+    "spmv_powerlaw": int((21321323.6 * 2 + 37057.4) * 1024),
+    "spmm": int((8641737.3 * 2 + 524288.0) * 1024),
+    "copy": int((524304.4 * 2 + 1048576.1) * 1024),
+}
+
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
@@ -338,6 +352,9 @@ def main():
         results["spmm"].update({"nnz": int(nnz), "gather_model_bytes": int(nnz * (8 + 512) + 4 * (m5 + 1) + 512 * m5)})
         log("spmm", results["spmm"], parity["spmm"])
 
+    if sc == 1.0:
+        for name, r in results.items():
+            r["traffic_bytes_rocprof"] = MEASURED_TRAFFIC.get(name)
     head = results["vector_sum"]
     all_ok = all(p["ok"] for p in parity.values())
     line = {
@@ -356,7 +373,7 @@ def main():
         "config": {"workload": f"configs[1](a) shared() scalar reduction vector_sum, float32 N={n}, uniform[0,1), seed 2",
                    "step": "clear float64 accumulator + one kernel launch, inputs resident in HBM"},
         "roofline": {"bound": "hbm", "achieved": head["gbps_kernel"], "peak": HBM_PEAK_BPS / 1e9, "unit": "GB/s",
-                     "frac": head["frac"], "traffic": None},
+                     "frac": head["frac"], "traffic": MEASURED_TRAFFIC["vector_sum"] if sc == 1.0 else None},
         "cpu_baseline": cpu_baseline,
         "parity_ok": all_ok,
         "parity": parity,
