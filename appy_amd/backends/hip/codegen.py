@@ -44,6 +44,8 @@ _device_header = None
 # 256 MiB of memory-side cache in front of the HBM3E).
 DEFAULT_CUS = 256
 MALL_BYTES = 256 << 20
+BYTES_IN_FLIGHT = 6.5e6
+TEAM_BYTES_IN_FLIGHT = 8.0e6
 
 
 def device_header() -> str:
@@ -217,6 +219,7 @@ class CompiledLoop:
         self._hi_code = compile(ast.Expression(body=ast.fix_missing_locations(_copy(a.hi_node))), "<hi>", "eval")
         self._simd_loops = self._collect_simd_loops()
         self._row_extent_code = self._find_row_extent()
+        self._row_hint = (0.0, False)
         self.kernels = {}   # Spec -> Kernel
         self._lock = threading.Lock()
         # default variant now: generation / compilation errors surface at first use of the loop
@@ -240,7 +243,7 @@ class CompiledLoop:
         v = max(1, min(4, 16 // max(self._elem_sizes())))
         if a.kind == "flat":
             if "simd" in a.pragma:
-                return Spec("flat", block=256, vec=v, unroll=4 if a.outer_reductions else 2)
+                return Spec("flat", block=256, vec=v, unroll=2)
             return Spec("flat", block=256, vec=1, unroll=1)
         return Spec("team", block=256, vec=v, width=64)
 
@@ -291,19 +294,21 @@ class CompiledLoop:
                         return compile(ast.Expression(body=ast.fix_missing_locations(_copy(hi))), "<extent>", "eval")
         return None
 
-    def _estimate_trip(self, env, arrays, n_outer) -> float:
-        best = 0.0
+    def _estimate_trip(self, env, arrays, n_outer):
+        """Expected trip count of the inner ``simd`` loops and whether it is the
+        same for every outer iteration (bounds computable on the host)."""
+        best, uniform = 0.0, True
         for code, streamed in self._simd_loops:
             try:
                 best = max(best, float(eval(code, {"__builtins__": {}}, env)))
                 continue
             except Exception:
-                pass
+                uniform = False
             for name in streamed:
                 v = arrays.get(name)
                 if v is not None and v.ndim == 1 and n_outer > 0:
                     best = max(best, v.shape[0] / n_outer)
-        return best
+        return best, uniform
 
     def choose_spec(self, n_outer, env, arrays, restrict=True) -> Spec:
         forced = self.options.get("hip_spec")
@@ -317,6 +322,11 @@ class CompiledLoop:
             stream = self._bytes_touched(arrays) > MALL_BYTES
             if d.vec > 1 and n_outer < d.block * d.vec * d.unroll:
                 return Spec("flat", block=d.block, vec=d.vec, unroll=1, restrict=restrict)
+            if stream and not self.analysis.outer_reductions:
+                # pure streaming beyond the memory-side cache: one tile per workgroup,
+                # loads and stores non-temporal (copy: 0.82 of peak against 0.67)
+                return Spec("flat", block=d.block, vec=d.vec, unroll=1, restrict=restrict,
+                            stream_loads=True, stream_stores=True)
             return Spec("flat", block=d.block, vec=d.vec, unroll=d.unroll, restrict=restrict, stream_loads=stream)
         stream = self._bytes_touched(arrays) > MALL_BYTES
         v = d.vec
@@ -330,7 +340,8 @@ class CompiledLoop:
                 if -(-ext // (w * v)) <= 8:
                     return Spec("team", block=d.block, vec=v, width=w, restrict=restrict,
                                 stream_loads=False, extent=ext)
-        trip = self._estimate_trip(env, arrays, n_outer)
+        trip, uniform = self._estimate_trip(env, arrays, n_outer)
+        self._row_hint = (trip, uniform)
         if trip < 2 * v:
             v = 1
         # one vector step per lane for short rows; two rows per wavefront at most
@@ -346,17 +357,41 @@ class CompiledLoop:
                 total += int(np.prod(v.shape)) * arr.ty.size
         return total
 
-    def grid_for(self, spec: Spec, n_outer: int, cus: int = DEFAULT_CUS) -> int:
+    def grid_for(self, spec: Spec, n_outer: int, cus: int = DEFAULT_CUS, kernel=None) -> int:
         if spec.kind == "flat":
             per_block = spec.block * spec.vec * spec.unroll
             need = max(1, -(-n_outer // per_block))
+            step_bytes = kernel.src.lane_step_bytes if kernel is not None else 0
+            if self.analysis.outer_reductions and step_bytes and not self.options.get("hip_max_blocks"):
+                # persistent workgroups sized by the bytes they keep in flight: HBM at
+                # 8 TB/s with ~0.8 us of latency wants ~6.5 MB outstanding; more
+                # workgroups only add serialised atomics (measured optimum 6-8 MB)
+                want = BYTES_IN_FLIGHT / float(spec.block * spec.unroll * step_bytes)
+                cap = max(cus, min(cus * 8, int(round(want / 128.0)) * 128))
+                return int(min(need, cap))
             # reductions end with one atomic per workgroup: few, persistent
-            # workgroups (4 per CU); pure streaming loops take up to 32 per CU
-            cap = self.options.get("hip_max_blocks") or (cus * 4 if self.analysis.outer_reductions else cus * 32)
+            # workgroups (2 per CU); streaming loops take one tile per workgroup
+            if self.options.get("hip_max_blocks"):
+                cap = self.options["hip_max_blocks"]
+            elif self.analysis.outer_reductions:
+                cap = cus * 2
+            elif spec.stream_stores:
+                cap = 1 << 22
+            else:
+                cap = cus * 32
             return int(min(need, cap))
         tpb = spec.block // spec.width
         need = max(1, -(-n_outer // tpb))
-        return int(min(need, 1 << 22))
+        trip, uniform = getattr(self, "_row_hint", (0.0, False))
+        if uniform and not spec.extent and trip * spec.vec >= 4096 and not self.options.get("hip_max_blocks"):
+            # long dense rows stream like a flat loop: persistent workgroups holding
+            # ~8 MB in flight, each taking a whole number of row batches (GEMV
+            # 16384^2: 1024 workgroups x 2 batches = 0.89 of peak, 2048 x 1 = 0.81)
+            step = 16 * 2
+            target = max(cus, TEAM_BYTES_IN_FLIGHT / float(spec.block * step))
+            passes = max(1, int(round(need / target)))
+            return int(max(1, -(-need // passes)))
+        return int(min(need, self.options.get("hip_max_blocks") or (1 << 22)))
 
     # ---- call ------------------------------------------------------------------------
     def __call__(self, *args):
@@ -472,7 +507,7 @@ class Launch:
                 val = hi
             setattr(st, fname, val)
         self.args = st
-        self.grid = (loop.grid_for(spec, n_outer), 1, 1)
+        self.grid = (loop.grid_for(spec, n_outer, kernel=self.kernel), 1, 1)
         self.block = (spec.block, 1, 1)
         loop.last_launch = self
 

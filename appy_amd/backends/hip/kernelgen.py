@@ -60,11 +60,12 @@ class Spec:
     restrict: bool = True
     stream_loads: bool = False   # non-temporal loads for data that is read once
     extent: int = 0      # compile-time extent of row accumulators (team only; 0 = none)
+    stream_stores: bool = False  # non-temporal vector stores
 
     def tag(self) -> str:
         return (f"{self.kind}_b{self.block}_v{self.vec}_u{self.unroll}_w{self.width}"
                 f"{'_r' if self.restrict else ''}{'_nt' if self.stream_loads else ''}"
-                f"{'_e' + str(self.extent) if self.extent else ''}")
+                f"{'_e' + str(self.extent) if self.extent else ''}{'_nts' if self.stream_stores else ''}")
 
 
 @dataclass
@@ -96,6 +97,7 @@ class KernelSource:
     reductions: list
     stored_arrays: list
     bound_checks: list   # (array, dim, offset) accesses indexed by the parallel loop variable
+    lane_step_bytes: int = 0   # bytes one lane moves per vector step of a flat loop
 
 
 class Unsupported(NotImplementedError):
@@ -420,6 +422,9 @@ class KernelBuilder:
                 self.ex.locals[var] = saved
         return f"{cname(arr.name)} + ({idx.replace('__vbase', base_code)})"
 
+    def _vst(self) -> str:
+        return "vstore_stream" if self.spec.stream_stores else "vstore"
+
     def _streamed(self, sub: ast.Subscript) -> bool:
         """True if the data behind a vectorised load is read once by the whole
         launch (then it is loaded non-temporally so that it does not displace
@@ -467,7 +472,7 @@ class KernelBuilder:
             self.ind -= 1
             self.w("}")
         for key, (arr, sub) in stores.items():
-            self.w(f"appy::vstore<{arr.elem_c}, {V}>({self._addr(arr, sub, var, base_code)}, {sregs[key]});")
+            self.w(f"appy::{self._vst()}<{arr.elem_c}, {V}>({self._addr(arr, sub, var, base_code)}, {sregs[key]});")
 
     def spread_loop(self, st: ast.For):
         """A ``simd`` loop inside a team: iterations dealt to the W lanes."""
@@ -685,6 +690,7 @@ class KernelBuilder:
         self.ex.locals[var] = T.WEAK_INT
         loads, stores = self._vector_accesses(self.a.outer.body, var) if V > 1 else ({}, {})
         vectorised = V > 1 and (loads or stores)
+        self.lane_step_bytes = sum(V * arr.ty.size for arr, _ in list(loads.values()) + list(stores.values()))
         self.w("const appy::i64 __tid = threadIdx.x;")
         self.w("const appy::i64 __nblk = gridDim.x;")
         if vectorised:
@@ -757,7 +763,7 @@ class KernelBuilder:
         for u in range(U):
             base = f"(__tile0 + {u * B * V})"
             for key, (arr, sub) in stores.items():
-                self.w(f"appy::vstore<{arr.elem_c}, {V}>({self._addr(arr, sub, var, base)}, {sregs[(u, key)]});")
+                self.w(f"appy::{self._vst()}<{arr.elem_c}, {V}>({self._addr(arr, sub, var, base)}, {sregs[(u, key)]});")
 
     def _body_team(self):
         s = self.spec
@@ -858,6 +864,7 @@ class KernelBuilder:
             reductions=list(self.a.outer_reductions),
             stored_arrays=sorted(n for n in self.a.stored if n in self.a.arrays),
             bound_checks=list(self.a.bound_checks),
+            lane_step_bytes=getattr(self, "lane_step_bytes", 0),
         )
 
 
