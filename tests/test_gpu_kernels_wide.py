@@ -1,0 +1,377 @@
+"""Wider loop shapes on the GPU, each against NumPy on seeded inputs: the kernel
+families of the reference's NPBench / DPBench integration tests
+(tests/integration/triton/npbench/*.py, dpbench/test_black_scholes.py) -
+triangular ``simd`` loops, stencils with neighbour offsets, in-place row
+updates, strided (column) accesses, several reductions in one ``simd`` loop,
+slices of the first dimension, ``@`` of slices, maths functions, loops nested
+in host-side Python loops.  Tolerances are those of the reference's tests."""
+import math
+from math import erf
+
+import numpy as np
+import pytest
+
+import appy
+
+pytestmark = pytest.mark.gpu
+
+
+@appy.jit
+def syrk_loops(alpha, beta, C, A):
+    #pragma parallel for
+    for i in range(A.shape[0]):
+        #pragma simd
+        for j in range(i + 1):
+            C[i, j] *= beta
+        for k in range(A.shape[1]):
+            #pragma simd
+            for j in range(i + 1):
+                C[i, j] += alpha * A[i, k] * A[j, k]
+    return C
+
+
+@appy.jit
+def syrk_slices(alpha, beta, C, A):
+    #pragma parallel for
+    for i in range(A.shape[0]):
+        C[i, :i + 1] *= beta
+        for k in range(A.shape[1]):
+            C[i, :i + 1] += alpha * A[i, k] * A[:i + 1, k]
+    return C
+
+
+def test_syrk(gpu):
+    rng = np.random.default_rng(0)
+    n, m = 70, 50
+    A = rng.standard_normal((n, m))
+    C = rng.standard_normal((n, n))
+    alpha, beta = 1.5, 1.2
+    ref = C.copy()
+    for i in range(n):
+        ref[i, :i + 1] = beta * ref[i, :i + 1] + alpha * (A[:i + 1] @ A[i])
+    assert np.allclose(syrk_loops(alpha, beta, C.copy(), A), ref)
+    assert np.allclose(syrk_slices(alpha, beta, C.copy(), A), ref)
+
+
+@appy.jit
+def jacobi_1d(TSTEPS, A, B):
+    for t in range(1, TSTEPS):
+        #pragma parallel for simd
+        for i in range(1, A.shape[0] - 1):
+            B[i] = 0.33333 * (A[i - 1] + A[i] + A[i + 1])
+
+        #pragma parallel for simd
+        for i in range(1, B.shape[0] - 1):
+            A[i] = 0.33333 * (B[i - 1] + B[i] + B[i + 1])
+    return A, B
+
+
+def test_jacobi_1d(gpu):
+    n = 10_007
+    A = np.fromfunction(lambda i: (i + 2) / n, (n,), dtype=np.float64)
+    B = np.fromfunction(lambda i: (i + 3) / n, (n,), dtype=np.float64)
+    A1, B1 = A.copy(), B.copy()
+    for _ in range(1, 10):
+        B1[1:-1] = 0.33333 * (A1[:-2] + A1[1:-1] + A1[2:])
+        A1[1:-1] = 0.33333 * (B1[:-2] + B1[1:-1] + B1[2:])
+    A2, B2 = jacobi_1d(10, A.copy(), B.copy())
+    assert np.array_equal(A2, A1) and np.array_equal(B2, B1)      # same operations in the same order
+
+
+@appy.jit
+def jacobi_2d(TSTEPS, A, B):
+    for t in range(1, TSTEPS):
+        #pragma parallel for
+        for i in range(1, A.shape[0] - 1):
+            #pragma simd
+            for j in range(1, A.shape[1] - 1):
+                B[i, j] = 0.2 * (A[i, j] + A[i, j - 1] + A[i, j + 1] + A[i - 1, j] + A[i + 1, j])
+
+        #pragma parallel for
+        for i in range(1, B.shape[0] - 1):
+            #pragma simd
+            for j in range(1, B.shape[1] - 1):
+                A[i, j] = 0.2 * (B[i, j] + B[i, j - 1] + B[i, j + 1] + B[i - 1, j] + B[i + 1, j])
+    return A, B
+
+
+def test_jacobi_2d(gpu):
+    n = 131
+    rng = np.random.default_rng(1)
+    A, B = rng.random((n, n)), rng.random((n, n))
+    A1, B1 = A.copy(), B.copy()
+    for _ in range(1, 6):
+        B1[1:-1, 1:-1] = 0.2 * (A1[1:-1, 1:-1] + A1[1:-1, :-2] + A1[1:-1, 2:] + A1[:-2, 1:-1] + A1[2:, 1:-1])
+        A1[1:-1, 1:-1] = 0.2 * (B1[1:-1, 1:-1] + B1[1:-1, :-2] + B1[1:-1, 2:] + B1[:-2, 1:-1] + B1[2:, 1:-1])
+    A2, B2 = jacobi_2d(6, A.copy(), B.copy())
+    assert np.allclose(A2, A1) and np.allclose(B2, B1)
+
+
+@appy.jit
+def floyd_warshall(path):
+    for k in range(path.shape[0]):
+        #pragma parallel for
+        for i in range(path.shape[0]):
+            #pragma simd
+            for j in range(path.shape[1]):
+                path[i, j] = min(path[i, j], path[i, k] + path[k, j])
+    return path
+
+
+def test_floyd_warshall(gpu):
+    n = 90
+    path = np.fromfunction(lambda i, j: i * j % 7 + 1, (n, n), dtype=np.int32)
+    for i in range(n):
+        for j in range(n):
+            if (i + j) % 13 == 0 or (i + j) % 7 == 0 or (i + j) % 11 == 0:
+                path[i, j] = 999
+    ref = path.copy()
+    for k in range(n):
+        ref[:] = np.minimum(ref, np.add.outer(ref[:, k], ref[k, :]))
+    out = floyd_warshall(path.copy())
+    assert out.dtype == np.int32 and np.array_equal(out, ref)
+
+
+@appy.jit
+def go_fast(a):
+    trace = 0.0
+    #pragma parallel for simd shared(trace)
+    for i in range(a.shape[0]):
+        trace += np.tanh(a[i, i])
+    return a + trace
+
+
+def test_go_fast_diagonal_and_tanh(gpu):
+    a = np.random.default_rng(2).random((300, 300))
+    assert np.allclose(go_fast(a), a + np.tanh(np.diagonal(a)).sum(), atol=1e-6)
+
+
+@appy.jit
+def azimint(data, radius, npt):
+    rmax = radius.max()
+    res = np.zeros(npt, dtype=np.float64)
+    #pragma parallel for
+    for i in range(npt):
+        r1 = rmax * i / npt
+        r2 = rmax * (i + 1) / npt
+        s, count = 0.0, 0
+        #pragma simd
+        for j in range(radius.shape[0]):
+            mask_r12 = (r1 <= radius[j]) & (radius[j] < r2)
+            s += data[j] if mask_r12 else 0.0
+            count += 1 if mask_r12 else 0
+        res[i] = s / count
+    return res
+
+
+def test_azimint_two_reductions_in_one_loop(gpu):
+    rng = np.random.default_rng(3)
+    n, npt = 4000, 50
+    data, radius = rng.random(n), rng.random(n)
+    rmax = radius.max()
+    ref = np.zeros(npt)
+    for i in range(npt):
+        m = (rmax * i / npt <= radius) & (radius < rmax * (i + 1) / npt)
+        ref[i] = data[m].mean()
+    assert np.allclose(azimint(data, radius, npt), ref)
+
+
+@appy.jit
+def gemver(alpha, beta, A, u1, v1, u2, v2, w, x, y, z):
+    M, N = A.shape
+    #pragma parallel for
+    for i in range(M):
+        #pragma simd
+        for j in range(N):
+            A[i, j] += u1[i] * v1[j] + u2[i] * v2[j]
+
+    #pragma parallel for
+    for j in range(N):
+        s = 0.0
+        #pragma simd
+        for i in range(M):
+            s += beta * y[i] * A[i, j]
+        x[j] += s + z[j]
+
+    #pragma parallel for
+    for i in range(M):
+        s = 0.0
+        #pragma simd
+        for j in range(N):
+            s += alpha * A[i, j] * x[j]
+        w[i] += s
+    return A, x, w
+
+
+def test_gemver_three_loops_column_access(gpu):
+    rng = np.random.default_rng(4)
+    n = 120
+    A = rng.random((n, n))
+    u1, v1, u2, v2, w, x, y, z = (rng.random(n) for _ in range(8))
+    alpha, beta = 1.5, 1.2
+    A1 = A + np.outer(u1, v1) + np.outer(u2, v2)
+    x1 = x + beta * y @ A1 + z
+    w1 = w + alpha * A1 @ x1
+    A2, x2, w2 = gemver(alpha, beta, A.copy(), u1, v1, u2, v2, w.copy(), x.copy(), y, z)
+    assert np.allclose(A2, A1) and np.allclose(x2, x1) and np.allclose(w2, w1)
+
+
+@appy.jit
+def symm_loops(alpha, beta, C, A, B):
+    temp2 = np.empty((C.shape[1], ), dtype=C.dtype)
+    C *= beta
+    for i in range(C.shape[0]):
+        #pragma parallel for
+        for j in range(C.shape[1]):
+            s = 0.0
+            #pragma simd
+            for k in range(i):
+                C[k, j] += alpha * B[i, j] * A[i, k]
+                s += B[k, j] * A[i, k]
+            temp2[j] = s
+        C[i, :] += alpha * B[i, :] * A[i, i] + alpha * temp2
+    return C
+
+
+@appy.jit
+def symm_slices(alpha, beta, C, A, B):
+    temp2 = np.empty((C.shape[1], ), dtype=C.dtype)
+    C *= beta
+    for i in range(C.shape[0]):
+        #pragma parallel for
+        for j in range(C.shape[1]):
+            C[:i, j] += alpha * B[i, j] * A[i, :i]
+            temp2[j] = B[:i, j] @ A[i, :i]
+        C[i, :] += alpha * B[i, :] * A[i, i] + alpha * temp2
+    return C
+
+
+def test_symm_store_and_reduction_in_one_simd_loop(gpu):
+    rng = np.random.default_rng(5)
+    m, n = 40, 45
+    A, B, C = rng.random((m, m)), rng.random((m, n)), rng.random((m, n))
+    alpha, beta = 1.5, 1.2
+    ref = beta * C
+    for i in range(m):
+        for j in range(n):
+            ref[:i, j] += alpha * B[i, j] * A[i, :i]
+        ref[i, :] += alpha * B[i, :] * A[i, i] + alpha * (B[:i, :].T @ A[i, :i])
+    assert np.allclose(symm_loops(alpha, beta, C.copy(), A, B), ref)
+    assert np.allclose(symm_slices(alpha, beta, C.copy(), A, B), ref)
+
+
+@appy.jit
+def gramschmidt(A):
+    Q = np.zeros_like(A)
+    R = np.zeros((A.shape[1], A.shape[1]), dtype=A.dtype)
+    for k in range(A.shape[1]):
+        nrm = np.dot(A[:, k], A[:, k])
+        R[k, k] = np.sqrt(nrm)
+        Q[:, k] = A[:, k] / R[k, k]
+        #pragma parallel for
+        for j in range(k + 1, A.shape[1]):
+            s = 0.0
+            #pragma simd
+            for i in range(A.shape[0]):
+                s += Q[i, k] * A[i, j]
+
+            #pragma simd
+            for i in range(A.shape[0]):
+                A[i, j] -= Q[i, k] * s
+            R[k, j] = s
+    return Q, R
+
+
+def test_gramschmidt_two_simd_loops_per_iteration(gpu):
+    rng = np.random.default_rng(6)
+    A = rng.random((60, 40))
+    Q, R = gramschmidt(A.copy())
+    assert np.allclose(Q @ R, A) and np.allclose(Q.T @ Q, np.eye(40), atol=1e-8)
+    assert np.allclose(R, np.triu(R))
+
+
+@appy.jit
+def fdtd_2d(TMAX, ex, ey, hz, _fict_):
+    for t in range(TMAX):
+        ey[0, :] = _fict_[t]
+        #pragma parallel for
+        for i in range(1, ey.shape[0]):
+            #pragma simd
+            for j in range(ey.shape[1]):
+                ey[i, j] -= 0.5 * (hz[i, j] - hz[i - 1, j])
+        #pragma parallel for
+        for i in range(ex.shape[0]):
+            #pragma simd
+            for j in range(1, ex.shape[1]):
+                ex[i, j] -= 0.5 * (hz[i, j] - hz[i, j - 1])
+        #pragma parallel for
+        for i in range(hz.shape[0] - 1):
+            #pragma simd
+            for j in range(hz.shape[1] - 1):
+                hz[i, j] -= 0.7 * (ex[i, j + 1] - ex[i, j] + ey[i + 1, j] - ey[i, j])
+    return ey, ex, hz
+
+
+def test_fdtd_2d(gpu):
+    rng = np.random.default_rng(7)
+    nx, ny, tmax = 50, 60, 8
+    ex, ey, hz = rng.random((nx, ny)), rng.random((nx, ny)), rng.random((nx, ny))
+    fict = np.arange(tmax, dtype=np.float64)
+    ex1, ey1, hz1 = ex.copy(), ey.copy(), hz.copy()
+    for t in range(tmax):
+        ey1[0, :] = fict[t]
+        ey1[1:, :] -= 0.5 * (hz1[1:, :] - hz1[:-1, :])
+        ex1[:, 1:] -= 0.5 * (hz1[:, 1:] - hz1[:, :-1])
+        hz1[:-1, :-1] -= 0.7 * (ex1[:-1, 1:] - ex1[:-1, :-1] + ey1[1:, :-1] - ey1[:-1, :-1])
+    ey2, ex2, hz2 = fdtd_2d(tmax, ex.copy(), ey.copy(), hz.copy(), fict)
+    assert np.allclose(ey2, ey1) and np.allclose(ex2, ex1) and np.allclose(hz2, hz1)
+
+
+@appy.jit
+def black_scholes(nopt, price, strike, t, rate, volatility, call, put):
+    mr = -rate
+    sig_sig_two = volatility * volatility * 2
+    #pragma parallel for simd
+    for i in range(nopt):
+        P = price[i]
+        S = strike[i]
+        T = t[i]
+        a = np.log(P / S)
+        b = T * mr
+        z = T * sig_sig_two
+        c = 0.25 * z
+        y = 1.0 / np.sqrt(z)
+        w1 = (a - b + c) * y
+        w2 = (a - b - c) * y
+        d1 = 0.5 + 0.5 * erf(w1)
+        d2 = 0.5 + 0.5 * erf(w2)
+        Se = np.exp(b) * S
+        r = P * d1 - Se * d2
+        call[i] = r
+        put[i] = r - P + Se
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_black_scholes_maths_functions(gpu, dtype):
+    rng = np.random.default_rng(8)
+    n = 100_003
+    price = rng.uniform(10, 50, n).astype(dtype)
+    strike = rng.uniform(10, 50, n).astype(dtype)
+    t = rng.uniform(1, 2, n).astype(dtype)
+    rate, vol = dtype(0.1), dtype(0.2)
+    call, put = np.zeros(n, dtype), -np.ones(n, dtype)
+    black_scholes(n, price, strike, t, rate, vol, call, put)
+    P, S, T = (v.astype(np.float64) for v in (price, strike, t))
+    a = np.log(P / S)
+    b = T * -0.1
+    z = T * (0.2 * 0.2 * 2)
+    c = 0.25 * z
+    y = 1.0 / np.sqrt(z)
+    verf = np.vectorize(math.erf)
+    d1 = 0.5 + 0.5 * verf((a - b + c) * y)
+    d2 = 0.5 + 0.5 * verf((a - b - c) * y)
+    Se = np.exp(b) * S
+    r = P * d1 - Se * d2
+    tol = 1e-10 if dtype is np.float64 else 2e-4
+    assert call.dtype == dtype
+    assert np.allclose(call, r, rtol=tol, atol=tol * 50) and np.allclose(put, r - P + Se, rtol=tol, atol=tol * 50)
