@@ -61,11 +61,13 @@ class Spec:
     stream_loads: bool = False   # non-temporal loads for data that is read once
     extent: int = 0      # compile-time extent of row accumulators (team only; 0 = none)
     stream_stores: bool = False  # non-temporal vector stores
+    lds_tile: int = 0    # elements of a row-invariant operand staged in LDS per step (team only; 0 = off)
 
     def tag(self) -> str:
         return (f"{self.kind}_b{self.block}_v{self.vec}_u{self.unroll}_w{self.width}"
                 f"{'_r' if self.restrict else ''}{'_nt' if self.stream_loads else ''}"
-                f"{'_e' + str(self.extent) if self.extent else ''}{'_nts' if self.stream_stores else ''}")
+                f"{'_e' + str(self.extent) if self.extent else ''}{'_nts' if self.stream_stores else ''}"
+                f"{'_lds' + str(self.lds_tile) if self.lds_tile else ''}")
 
 
 @dataclass
@@ -217,6 +219,7 @@ class KernelBuilder:
         self.mode = "lane"
         self.partials = {}        # reduction variable -> partial register, inside a spread simd loop
         self.bounds_vary = False  # inside a spread loop whose bounds differ between outer iterations
+        self.lds_plan = None      # (spread loop node, [ArrayParam]) staged through LDS, or None
         self.store_subst = {}     # unparsed subscript -> (lvalue code, Ty)
         self.dirty = False
         self.counter = 0
@@ -302,7 +305,7 @@ class KernelBuilder:
             oc, ot = self.ex.emit(loop_ir.reduction_operand(st))
             upd = f"{r.acc} = {_OPS[r.op]}::f<{r.ty.c}>({r.acc}, {cast(oc, ot, r.ty)});"
             if self.mode == "team":
-                self.w(f"if (__lane == 0) {{ {upd} }}")
+                self.w(f"if ({self._leader()}) {{ {upd} }}")
             else:
                 self.w(upd)
             return
@@ -318,7 +321,7 @@ class KernelBuilder:
         idx = self.ex.index_code(arr, tgt)
         store = f"{cname(arr.name)}[{idx}] = {self._store_value(vc, vt, arr)};"
         if self.mode == "team":
-            self.w(f"if (__lane == 0) {{ {store} }}")
+            self.w(f"if ({self._leader()}) {{ {store} }}")
         else:
             self.w(store)
         # a later read of the same element in this iteration goes to memory again
@@ -422,6 +425,10 @@ class KernelBuilder:
                 self.ex.locals[var] = saved
         return f"{cname(arr.name)} + ({idx.replace('__vbase', base_code)})"
 
+    def _leader(self) -> str:
+        """Condition under which a team-level statement has its side effect."""
+        return "__lane == 0 && __active" if self.lds_plan else "__lane == 0"
+
     def _vst(self) -> str:
         return "vstore_stream" if self.spec.stream_stores else "vstore"
 
@@ -437,7 +444,7 @@ class KernelBuilder:
             return True
         return self.bounds_vary or any(_uses_name(e, self.a.var) for e in _elts(sub))
 
-    def vector_body(self, body, var: str, base_code: str, V: int, loads, stores, declare_locals=False):
+    def vector_body(self, body, var: str, base_code: str, V: int, loads, stores, declare_locals=False, extra=None):
         """Emit V consecutive iterations starting at ``base_code``: vector
         loads first, the V scalar bodies, vector stores last."""
         regs = {}
@@ -463,6 +470,8 @@ class KernelBuilder:
             for key, (arr, _) in loads.items():
                 code = f"{regs[key]}.{comp[k]}" if V > 1 else regs[key]
                 self.ex.load_subst[key] = ((f"({code} != 0)" if arr.ty.is_bool else code), arr.ty)
+            for key, (r, arr) in (extra or {}).items():
+                self.ex.load_subst[key] = (f"{r}.{comp[k]}", arr.ty)
             saved_stores = dict(self.store_subst)
             for key, (arr, _) in stores.items():
                 self.store_subst[key] = ((f"{sregs[key]}.{comp[k]}" if V > 1 else sregs[key]), arr.ty)
@@ -476,6 +485,8 @@ class KernelBuilder:
 
     def spread_loop(self, st: ast.For):
         """A ``simd`` loop inside a team: iterations dealt to the W lanes."""
+        if self.lds_plan is not None and st is self.lds_plan[0]:
+            return self.tiled_spread_loop(st)
         var = st.target.id
         W, V = self.spec.width, self.spec.vec
         lo, hi = self._range_args(st)
@@ -765,19 +776,161 @@ class KernelBuilder:
             for key, (arr, sub) in stores.items():
                 self.w(f"appy::{self._vst()}<{arr.elem_c}, {V}>({self._addr(arr, sub, var, base)}, {sregs[(u, key)]});")
 
+    def _find_lds_plan(self):
+        """A ``simd`` loop directly in the body of the parallel loop whose bounds
+        are the same for every outer iteration and that reads 1-D arrays indexed
+        by its own variable only (``x[j]`` of GEMV): those operands are the same
+        for every row, so a workgroup stages them in LDS once per tile and all
+        its teams read them from there."""
+        if not self.spec.lds_tile or self.a.outer_reductions:
+            return None
+        # teams past the end of the range run on a clamped row with their team-level
+        # side effects switched off; stores issued from inside simd loops cannot be
+        # switched off that way, so such kernels keep the plain form
+        for n in ast.walk(self.a.outer):
+            if isinstance(n, ast.For) and n is not self.a.outer and "simd" in (getattr(n, "pragma", None) or {}):
+                if any(isinstance(a, ast.Assign) and isinstance(a.targets[0], ast.Subscript) for a in ast.walk(n)):
+                    return None
+        outer_locals = set(self.a.assigned) | {self.a.var}
+        for st in self.a.outer.body:
+            if not (isinstance(st, ast.For) and "simd" in (getattr(st, "pragma", None) or {})):
+                continue
+            if any(_uses_name(b, n) for b in st.iter.args[:2] for n in outer_locals):
+                continue
+            j = st.target.id
+            found = {}
+            for n in ast.walk(st):
+                if (isinstance(n, ast.Subscript) and isinstance(n.value, ast.Name) and n.value.id in self.a.arrays
+                        and isinstance(n.ctx, ast.Load) and isinstance(n.slice, ast.Name) and n.slice.id == j):
+                    arr = self.a.arrays[n.value.id]
+                    if arr.ndim == 1 and arr.name not in self.a.stored and not arr.ty.is_bool:
+                        found[arr.name] = arr
+            if found:
+                return st, list(found.values())
+        return None
+
     def _body_team(self):
         s = self.spec
         W, B = s.width, s.block
         tpb = B // W
         var = self.a.var
         self.ex.locals[var] = T.WEAK_INT
+        self.lds_plan = self._find_lds_plan()
         self.w(f"const int __lane = threadIdx.x & {W - 1};")
         self.w(f"const appy::i64 __team = threadIdx.x / {W};")
-        self.w(f"for (appy::i64 __i = __lo + blockIdx.x * {tpb}LL + __team; __i < __hi; __i += gridDim.x * {tpb}LL) {{")
+        if self.lds_plan is None:
+            self.w(f"for (appy::i64 __i = __lo + blockIdx.x * {tpb}LL + __team; __i < __hi; __i += gridDim.x * {tpb}LL) {{")
+            self.ind += 1
+            self.mode = "team"
+            self._iteration("__i")
+            self.mode = "lane"
+            self.ind -= 1
+            self.w("}")
+            return
+        # Every thread of the workgroup takes part in filling the LDS tiles, so
+        # teams past the end of the range stay in the loop on a clamped row and
+        # only their side effects are switched off.
+        for arr in self.lds_plan[1]:
+            self.w(f"__shared__ __attribute__((aligned(16))) {arr.elem_c} __tile_{cname(arr.name)}[{s.lds_tile}];")
+        self.w(f"for (appy::i64 __ib = __lo + blockIdx.x * {tpb}LL; __ib < __hi; __ib += gridDim.x * {tpb}LL) {{")
         self.ind += 1
+        self.w("const bool __active = (__ib + __team) < __hi;")
+        self.w("const appy::i64 __i = __active ? (__ib + __team) : (__hi - 1);")
         self.mode = "team"
         self._iteration("__i")
         self.mode = "lane"
+        self.ind -= 1
+        self.w("}")
+
+    def tiled_spread_loop(self, st: ast.For):
+        """The LDS-staged form of :meth:`spread_loop` for the loop of the plan."""
+        var = st.target.id
+        W, V, TILE, B = self.spec.width, self.spec.vec, self.spec.lds_tile, self.spec.block
+        staged = self.lds_plan[1]
+        lo, hi = self._range_args(st)
+        self.ex.locals[var] = T.WEAK_INT
+        reds = {k: op for k, op in loop_ir.reductions_of(st).items() if k in self.ex.locals or k in self.a.assigned}
+        self.w("{")
+        self.ind += 1
+        lo_v, hi_v = self.fresh("lo"), self.fresh("hi")
+        self.w(f"const appy::i64 {lo_v} = {lo};")
+        self.w(f"const appy::i64 {hi_v} = {hi};")
+        saved_partials = dict(self.partials)
+        for name, op in reds.items():
+            ty = self.ex.locals.get(name)
+            if ty is None:
+                raise NameError(f"reduction variable `{name}` has no value before the loop")
+            p = self.fresh(f"part_{name}_")
+            self.partials[name] = (p, ty)
+            self.w(f"{ty.c} {p} = {T.identity_literal(op, ty)};")
+        jt = self.fresh("jt")
+        self.w(f"for (appy::i64 {jt} = {lo_v}; {jt} < {hi_v}; {jt} += {TILE}) {{")
+        self.ind += 1
+        n_t = self.fresh("nt")
+        self.w(f"const appy::i64 {n_t} = ({hi_v} - {jt}) < {TILE} ? ({hi_v} - {jt}) : {TILE};")
+        self.w("__syncthreads();   // the previous tile has been consumed")
+        for arr in staged:
+            t = f"__tile_{cname(arr.name)}"
+            q = self.fresh("f")
+            self.w(f"for (appy::i64 {q} = (appy::i64)threadIdx.x * {V}; {q} < {n_t}; {q} += {B * V}) {{")
+            self.ind += 1
+            self.w(f"if ({q} + {V} <= {n_t}) {{")
+            self.w(f"    appy::lds_vstore<{arr.elem_c}, {V}>(&{t}[{q}], appy::vload<{arr.elem_c}, {V}>({cname(arr.name)} + {jt} + {q}));")
+            self.w("} else {")
+            self.w(f"    for (appy::i64 __e = {q}; __e < {n_t}; ++__e) {t}[__e] = {cname(arr.name)}[{jt} + __e];")
+            self.w("}")
+            self.ind -= 1
+            self.w("}")
+        self.w("__syncthreads();   // the tile is complete")
+        saved_mode, self.mode = self.mode, "lane"
+        loads, stores = self._vector_accesses(st.body, var) if V > 1 else ({}, {})
+        staged_names = {a.name for a in staged}
+        staged_keys = {f"{a.name}[{var}]" for a in staged}
+        if V > 1 and (loads or stores):
+            nv = self.fresh("nv")
+            q = self.fresh("q")
+            self.w(f"const appy::i64 {nv} = {n_t} / {V};")
+            self.w("#pragma unroll 2")
+            self.w(f"for (appy::i64 {q} = __lane; {q} < {nv}; {q} += {W}) {{")
+            self.ind += 1
+            base = self.fresh("j")
+            self.w(f"const appy::i64 {base} = {jt} + {q} * {V};")
+            global_loads = {k: v for k, v in loads.items() if k not in staged_keys}
+            saved_loads = dict(self.ex.load_subst)
+            comp = "xyzw"
+            regs = {}
+            for key in staged_keys & set(loads):
+                arr = loads[key][0]
+                r = self.fresh(f"lds_{arr.name}_")
+                regs[key] = (r, arr)
+                self.w(f"const appy::vec<{arr.elem_c}, {V}>::type {r} = "
+                       f"appy::lds_vload<{arr.elem_c}, {V}>(&__tile_{cname(arr.name)}[{q} * {V}]);")
+            self._staged_regs = regs
+            self.vector_body(st.body, var, base, V, global_loads, stores, extra=regs)
+            self.ex.load_subst = saved_loads
+            self.ind -= 1
+            self.w("}")
+            start = f"{jt} + {nv} * {V} + __lane"
+        else:
+            start = f"{jt} + __lane"
+        self.w(f"for (appy::i64 {cname(var)} = {start}; {cname(var)} < {jt} + {n_t}; {cname(var)} += {W}) {{")
+        self.ind += 1
+        saved_loads = dict(self.ex.load_subst)
+        for arr in staged:
+            self.ex.load_subst[f"{arr.name}[{var}]"] = (f"__tile_{cname(arr.name)}[{cname(var)} - {jt}]", arr.ty)
+        self.block(st.body)
+        self.ex.load_subst = saved_loads
+        self.ind -= 1
+        self.w("}")
+        self.mode = saved_mode
+        self.ind -= 1
+        self.w("}")
+        for name, op in reds.items():
+            p, ty = self.partials[name]
+            if ty.size < 4:
+                raise Unsupported(f"Reduction variable `{name}` of type {ty.name} is not supported")
+            self.w(f"{cname(name)} = {_OPS[op]}::f<{ty.c}>({cname(name)}, appy::team_reduce<{_OPS[op]}, {W}, {ty.c}>({p}));")
+        self.partials = saved_partials
         self.ind -= 1
         self.w("}")
 
@@ -826,6 +979,7 @@ class KernelBuilder:
         self.ex.load_subst = {}
         self.store_subst = {}
         self.partials = {}
+        self.lds_plan = None
         for r in self.a.outer_reductions:
             self.w(f"{r.ty.c} {r.acc} = {T.identity_literal(r.op, r.ty)};")
         if self.spec.kind == "flat":

@@ -31,6 +31,30 @@ __device__ __forceinline__ void vstore(T* p, typename vec<T, V>::type v) {
     *reinterpret_cast<typename vec<T, V>::type*>(p) = v;
 }
 
+// LDS tiles are 16-byte aligned and indexed in whole vectors: naturally aligned
+// vector types give single ds_read_b128 / ds_write_b128 accesses.
+template <typename T, int V>
+struct avec {
+    typedef T type __attribute__((ext_vector_type(V)));
+};
+
+template <typename T, int V>
+__device__ __forceinline__ typename vec<T, V>::type lds_vload(const T* p) {
+    typename avec<T, V>::type a = *reinterpret_cast<const typename avec<T, V>::type*>(p);
+    typename vec<T, V>::type r;
+#pragma unroll
+    for (int k = 0; k < V; ++k) r[k] = a[k];
+    return r;
+}
+
+template <typename T, int V>
+__device__ __forceinline__ void lds_vstore(T* p, typename vec<T, V>::type v) {
+    typename avec<T, V>::type a;
+#pragma unroll
+    for (int k = 0; k < V; ++k) a[k] = v[k];
+    *reinterpret_cast<typename avec<T, V>::type*>(p) = a;
+}
+
 // Streaming variants: data that is touched once should not displace reused
 // lines (x of SpMV/GEMV, B rows of SpMM) from the L2.
 template <typename T, int V>

@@ -151,3 +151,17 @@ def test_out_of_range_loop_is_caught_on_the_host():
     f, _ = compiled("#pragma parallel for simd\nfor i in range(n):\n    c[i] = a[i + 1]", c=a, a=a, n=8)
     with pytest.raises(IndexError):
         f.prepare({"c": a, "a": a, "n": 8})
+
+
+def test_lds_staging_is_an_option_and_refuses_unsafe_loops():
+    g, _ = selfcheck_loop("gemv")
+    k = body_of(g.kernel_for(Spec("team", block=256, vec=4, width=32, lds_tile=2048)).src.text)
+    assert "__shared__" in k and "__tile_x[2048]" in k and k.count("__syncthreads()") == 2
+    assert "appy::lds_vload<float, 4>" in k and "__lane == 0 && __active" in k
+    # a loop that stores from inside its simd loop keeps the plain form (no clamped duplicate rows)
+    a = np.zeros((4, 8), np.float32)
+    x = np.zeros(8, np.float32)
+    text = "#pragma parallel for\nfor i in range(r):\n    #pragma simd\n    for j in range(c):\n        a[i, j] = a[i, j] + x[j]"
+    f, _ = compiled(text, a=a, x=x, r=4, c=8)
+    k2 = body_of(f.kernel_for(Spec("team", block=256, vec=4, width=32, lds_tile=2048)).src.text)
+    assert "__shared__" not in k2

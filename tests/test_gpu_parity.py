@@ -156,3 +156,31 @@ def test_spmm_columns_equal_spmv(k):
         x = np.ascontiguousarray(B[:, col])
         ref, budget = vo.spmv_csr(data, indptr, indices, x, (700, 700))
         assert vo.within_budget(Y[:, col], ref, budget, TOL)[0]
+
+
+@pytest.mark.parametrize("shape", [(3, 5), (513, 1027), (300, 9000)])
+def test_gemv_with_x_staged_in_lds(gpu, shape):
+    """The LDS-tiled schedule (row-invariant operand staged per workgroup) is an
+    option of the generator; it must give the same results as the default."""
+    import appy_amd as appy
+
+    @appy.jit(hip_spec={"lds_tile": 2048, "width": 32})
+    def gemv_lds(A, x, y):
+        #pragma parallel for
+        for i in range(A.shape[0]):
+            yi = 0.0
+            #pragma simd
+            for j in range(A.shape[1]):
+                yi += A[i, j] * x[j]
+            y[i] = yi
+
+    A, x = wl.gemv(*shape)
+    y = np.full(shape[0], np.nan, dtype=np.float32)
+    gemv_lds(A, x, y)
+    ref, budget = vo.gemv(A, x)
+    ok, worst = vo.within_budget(y, ref, budget, TOL)
+    assert ok, worst
+    from appy_amd.backends.hip import codegen as cg
+
+    loop = [v[0] for kk, v in cg.code_cache.items() if kk[-1] == "gemv_lds"][-1]
+    assert "__tile_x" in loop.last_launch.kernel.src.text
