@@ -89,15 +89,17 @@ def array_dtype(v) -> np.dtype:
 
 
 def _signature(val_map):
+    """Cache key part: names with the kind, dtype and rank of their values
+    (shapes are not part of it: extents reach the kernels as arguments)."""
     sig = []
     for k, v in val_map.items():
-        if isinstance(v, _types.ModuleType):
-            sig.append((k, "module"))
-        elif is_numpy_array(v) or is_torch_tensor(v):
-            sig.append((k, _kind(v), str(array_dtype(v)), v.ndim))
+        t = type(v)
+        if t is _types.ModuleType:
+            sig.append((k, t))
+        elif hasattr(v, "dtype") and hasattr(v, "ndim"):
+            sig.append((k, t, v.dtype, v.ndim))
         else:
-            ty = T.of_python_value(v)
-            sig.append((k, _kind(v), str(ty)))
+            sig.append((k, t))
     return tuple(sig)
 
 
@@ -354,7 +356,10 @@ class CompiledLoop:
         for name, v in arrays.items():
             arr = self.analysis.arrays[name]
             if arr.loaded or arr.stored:
-                total += int(np.prod(v.shape)) * arr.ty.size
+                n = 1
+                for d in v.shape:
+                    n *= int(d)
+                total += n * arr.ty.size
         return total
 
     def grid_for(self, spec: Spec, n_outer: int, cus: int = DEFAULT_CUS, kernel=None) -> int:

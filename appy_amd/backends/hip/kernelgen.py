@@ -19,7 +19,7 @@ Two execution shapes cover every annotated loop:
     spread over the lanes (V consecutive iterations per lane where the
     accesses allow) and their reductions end with a DPP/shuffle butterfly over
     the team.  Replaces the reference's one-program-per-outer-iteration
-    mapping with masked 256-wide chunks (SURVEY of the same passes).
+    mapping with masked 256-wide chunks (same passes of the reference).
 
 Reductions of the parallel loop itself (``shared`` scalars, detected as in
 appy/frontend/reduction_detection.py:76-104 of the reference) are kept in a

@@ -32,8 +32,12 @@ def _resolve_backend(name):
 
 
 def build_val_map(loop_source, local_scope, global_scope):
-    merged = {**global_scope, **local_scope}
-    val_map = {k: merged[k] for k in used_names(loop_source) if k in merged}
+    val_map = {}
+    for k in used_names(loop_source):      # locals shadow globals; no copy of either scope
+        if k in local_scope:
+            val_map[k] = local_scope[k]
+        elif k in global_scope:
+            val_map[k] = global_scope[k]
     val_map.setdefault("np", np)
     val_map.setdefault("math", math)
     return val_map
