@@ -30,16 +30,16 @@ HBM_PEAK_BPS = 8.0e12  # MI355X HBM3E, bytes per second
 
 # HBM traffic per launch (bytes) at the default sizes, from the rocprofv3 counter
 # runs summarised in profiles/all_kernels_bench_pmc_fetch_write_size.txt:
-# FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 (factors from the plain copy kernel), KiB -> bytes.
+# FETCH_SIZE x 2.000 + WRITE_SIZE x 0.999 (factors from the plain copy kernel), KiB -> bytes.
 MEASURED_TRAFFIC = {
-    "vector_sum": int((524302.8 * 2 + 32.0) * 1024),
-    "masked_sum": int((655384.2 * 2 + 32.0) * 1024),
-    "vec_add": int((65549.0 * 2 + 65536.0) * 1024),
-    "gemv": int((524558.6 * 2 + 64.5) * 1024),
-    "spmv_uniform": int((3442492.9 * 2 + 18586.1) * 1024),
-    "spmv_powerlaw": int((21321323.6 * 2 + 37057.4) * 1024),
-    "spmm": int((8641737.3 * 2 + 524288.0) * 1024),
-    "copy": int((524304.4 * 2 + 1048576.1) * 1024),
+    "vector_sum": int((524302.8 * 2.000 + 24.0 * 0.999) * 1024),
+    "masked_sum": int((655384.1 * 2.000 + 20.0 * 0.999) * 1024),
+    "vec_add": int((65549.0 * 2.000 + 65536.0 * 0.999) * 1024),
+    "gemv": int((524558.0 * 2.000 + 64.5 * 0.999) * 1024),
+    "spmv_uniform": int((3442370.0 * 2.000 + 18580.9 * 0.999) * 1024),
+    "spmv_powerlaw": int((21324000.0 * 2.000 + 37038.3 * 0.999) * 1024),
+    "spmm": int((8641800.0 * 2.000 + 524288.0 * 0.999) * 1024),
+    "copy": int((524301.2 * 2.000 + 1049486.1 * 0.999) * 1024),
 }
 
 
