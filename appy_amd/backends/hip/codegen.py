@@ -166,13 +166,14 @@ class Kernel:
 # ---------------------------------------------------------------------------
 # the launcher
 # ---------------------------------------------------------------------------
-_current_device = [None]
+_tls = threading.local()
 
 
 def _ensure_device(dev: int):
-    if _current_device[0] != dev:
+    """HIP's current device is a per-thread setting."""
+    if getattr(_tls, "device", None) != dev:
         rt.init(dev)
-        _current_device[0] = dev
+        _tls.device = dev
 
 
 def _pow2ceil(x: float) -> int:
@@ -221,7 +222,6 @@ class CompiledLoop:
         self._hi_code = compile(ast.Expression(body=ast.fix_missing_locations(_copy(a.hi_node))), "<hi>", "eval")
         self._simd_loops = self._collect_simd_loops()
         self._row_extent_code = self._find_row_extent()
-        self._row_hint = (0.0, False)
         self.kernels = {}   # Spec -> Kernel
         self._lock = threading.Lock()
         # default variant now: generation / compilation errors surface at first use of the loop
@@ -343,13 +343,18 @@ class CompiledLoop:
                     return Spec("team", block=d.block, vec=v, width=w, restrict=restrict,
                                 stream_loads=False, extent=ext)
         trip, uniform = self._estimate_trip(env, arrays, n_outer)
-        self._row_hint = (trip, uniform)
         if trip < 2 * v:
             v = 1
         # one vector step per lane for short rows; two rows per wavefront at most
         # (two independent rows in flight per wavefront stream better than one)
         w = max(1, min(32, _pow2ceil(trip / float(v)) if trip > 0 else 1))
         return Spec("team", block=d.block, vec=v, width=w, restrict=restrict, stream_loads=stream)
+
+    def row_hint(self, n_outer, env, arrays):
+        """(expected inner trip count, same for every row?) for grid sizing."""
+        if self.analysis.kind != "team":
+            return 0.0, False
+        return self._estimate_trip(env, arrays, n_outer)
 
     def _bytes_touched(self, arrays) -> int:
         total = 0
@@ -362,7 +367,7 @@ class CompiledLoop:
                 total += n * arr.ty.size
         return total
 
-    def grid_for(self, spec: Spec, n_outer: int, cus: int = DEFAULT_CUS, kernel=None) -> int:
+    def grid_for(self, spec: Spec, n_outer: int, cus: int = DEFAULT_CUS, kernel=None, row_hint=(0.0, False)) -> int:
         if spec.kind == "flat":
             per_block = spec.block * spec.vec * spec.unroll
             need = max(1, -(-n_outer // per_block))
@@ -387,7 +392,7 @@ class CompiledLoop:
             return int(min(need, cap))
         tpb = spec.block // spec.width
         need = max(1, -(-n_outer // tpb))
-        trip, uniform = getattr(self, "_row_hint", (0.0, False))
+        trip, uniform = row_hint
         if uniform and not spec.extent and trip * spec.vec >= 4096 and not self.options.get("hip_max_blocks"):
             # long dense rows stream like a flat loop: persistent workgroups holding
             # ~8 MB in flight, each taking a whole number of row batches (GEMV
@@ -512,7 +517,8 @@ class Launch:
                 val = hi
             setattr(st, fname, val)
         self.args = st
-        self.grid = (loop.grid_for(spec, n_outer, kernel=self.kernel), 1, 1)
+        self.grid = (loop.grid_for(spec, n_outer, kernel=self.kernel,
+                                   row_hint=loop.row_hint(n_outer, env, arrays)), 1, 1)
         self.block = (spec.block, 1, 1)
         loop.last_launch = self
 

@@ -32,12 +32,12 @@ from __future__ import annotations
 
 import ast
 import ctypes as C
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 
 from ...frontend import loop_ir
 from . import dtypes as T
 from .dtypes import Ty
-from .exprs import ArrayParam, ExprEmitter, ScalarParam, cast, cname, truth
+from .exprs import ArrayParam, ExprEmitter, cast, cname, truth
 
 _OPS = {"+": "appy::OpAdd", "*": "appy::OpMul", "max": "appy::OpMax", "min": "appy::OpMin"}
 
@@ -62,6 +62,23 @@ class Spec:
     extent: int = 0      # compile-time extent of row accumulators (team only; 0 = none)
     stream_stores: bool = False  # non-temporal vector stores
     lds_tile: int = 0    # elements of a row-invariant operand staged in LDS per step (team only; 0 = off)
+
+    def __post_init__(self):
+        def pow2(n):
+            return n >= 1 and (n & (n - 1)) == 0
+
+        if self.kind not in ("flat", "team"):
+            raise ValueError(f"kernel shape must be 'flat' or 'team', got {self.kind!r}")
+        if self.block % 64 or not 64 <= self.block <= 1024:
+            raise ValueError(f"workgroup size must be a multiple of 64 up to 1024, got {self.block}")
+        if self.vec not in (1, 2, 4):
+            raise ValueError(f"vector width must be 1, 2 or 4, got {self.vec}")
+        if not 1 <= self.unroll <= 8:
+            raise ValueError(f"unroll factor must be 1..8, got {self.unroll}")
+        if not pow2(self.width) or self.width > 64:
+            raise ValueError(f"team width must be a power of two up to 64, got {self.width}")
+        if self.extent < 0 or self.lds_tile < 0 or self.lds_tile % 4 or self.lds_tile > 16384:
+            raise ValueError("row extent / LDS tile out of range (tile: multiple of 4, at most 16384 elements)")
 
     def tag(self) -> str:
         return (f"{self.kind}_b{self.block}_v{self.vec}_u{self.unroll}_w{self.width}"
@@ -905,7 +922,6 @@ class KernelBuilder:
                 regs[key] = (r, arr)
                 self.w(f"const appy::vec<{arr.elem_c}, {V}>::type {r} = "
                        f"appy::lds_vload<{arr.elem_c}, {V}>(&__tile_{cname(arr.name)}[{q} * {V}]);")
-            self._staged_regs = regs
             self.vector_body(st.body, var, base, V, global_loads, stores, extra=regs)
             self.ex.load_subst = saved_loads
             self.ind -= 1

@@ -165,3 +165,57 @@ def test_lds_staging_is_an_option_and_refuses_unsafe_loops():
     f, _ = compiled(text, a=a, x=x, r=4, c=8)
     k2 = body_of(f.kernel_for(Spec("team", block=256, vec=4, width=32, lds_tile=2048)).src.text)
     assert "__shared__" not in k2
+
+
+def test_spec_validation():
+    for bad in (dict(kind="warp"), dict(kind="flat", block=100), dict(kind="flat", vec=3), dict(kind="team", width=48),
+                dict(kind="team", width=128), dict(kind="flat", unroll=0), dict(kind="team", lds_tile=1000002)):
+        with pytest.raises(ValueError):
+            Spec(**bad)
+
+
+def test_dump_code_to_file_and_kernel_names(tmp_path):
+    out = tmp_path / "kernel.hip"
+
+    @appy.jit(dry_run=True, dump_code_to_file=str(out))
+    def scale(a, f):
+        #pragma parallel for simd
+        for i in range(a.shape[0]):
+            a[i] = a[i] * f
+
+    a = np.arange(8, dtype=np.float32)
+    scale(a, 2.0)
+    text = out.read_text()
+    assert 'extern "C" __global__' in text and "_scale_kernel_loop_1(" in text     # kernels carry the function's name
+    assert np.array_equal(a, np.arange(8, dtype=np.float32) * 2)                    # dry_run interpreted the loop
+
+
+def test_by_value_scalar_assigned_in_the_loop_is_private():
+    a = np.zeros(8)
+    f, src = compiled("#pragma parallel for simd\nfor i in range(n):\n    t = t + 1.0\n    a[i] = t", a=a, t=5.0, n=8)
+    k = body_of(src)
+    assert "const double t__arg" in k and "double t = t__arg;" in k       # every iteration starts from the caller's value
+
+
+def test_codegen_is_cached_per_signature_not_per_shape():
+    text = "#pragma parallel for simd\nfor i in range(n):\n    c[i] = a[i] + 1"
+    f1, _ = compiled(text, c=np.zeros(8, np.float32), a=np.zeros(8, np.float32), n=8)
+    f2, _ = compiled(text, c=np.zeros(800, np.float32), a=np.zeros(800, np.float32), n=800)
+    f3, _ = compiled(text, c=np.zeros(8), a=np.zeros(8), n=8)
+    assert f1 is f2 and f3 is not f1
+
+
+def test_concurrent_code_generation_is_safe():
+    import threading
+
+    text = "#pragma parallel for simd\nfor i in range(n):\n    c[i] = a[i] * 3 + b[i]"
+    got = []
+
+    def work():
+        a = np.zeros(8, np.float32)
+        got.append(cg.codegen(text, "kernel_loop_9", {"c": a, "a": a, "b": a, "n": 8}, {})[0])
+
+    ts = [threading.Thread(target=work) for _ in range(8)]
+    [t.start() for t in ts]
+    [t.join() for t in ts]
+    assert len(got) == 8 and all(g is got[0] for g in got)

@@ -184,3 +184,67 @@ def test_gemv_with_x_staged_in_lds(gpu, shape):
 
     loop = [v[0] for kk, v in cg.code_cache.items() if kk[-1] == "gemv_lds"][-1]
     assert "__tile_x" in loop.last_launch.kernel.src.text
+
+
+def test_aliased_arguments_and_strided_numpy_views(gpu):
+    import appy_amd as appy
+
+    @appy.jit
+    def add_into(a, b, c):
+        #pragma parallel for simd
+        for i in range(a.shape[0]):
+            c[i] = a[i] + b[i]
+
+    a = np.arange(10_001, dtype=np.float32)
+    add_into(a, a, a)                       # all three names are one buffer: the no-restrict variant
+    assert np.array_equal(a, 2 * np.arange(10_001, dtype=np.float32))
+    base = np.zeros((5000, 3), dtype=np.float32)
+    ones = np.ones(5000, dtype=np.float32)
+    add_into(ones, ones, base[:, 1])        # strided output view: packed copy in, copy back out
+    assert np.array_equal(base[:, 1], 2 * ones) and base.sum() == 10_000
+    add_into(base[:, 1], ones, base[:, 2])  # strided input view
+    assert np.array_equal(base[:, 2], 3 * ones)
+
+
+def test_integer_reductions_and_products(gpu):
+    import appy_amd as appy
+
+    @appy.jit
+    def count_and_max(a):
+        n = 0
+        m = -2**62
+        #pragma parallel for simd shared(n, m)
+        for i in range(a.shape[0]):
+            n += 1 if a[i] > 0 else 0
+            m = max(m, a[i])
+        return n, m
+
+    @appy.jit
+    def product(a):
+        p = 1.0
+        #pragma parallel for simd shared(p)
+        for i in range(a.shape[0]):
+            p *= a[i]
+        return p
+
+    a = np.random.default_rng(9).integers(-1000, 1000, 100_003, dtype=np.int64)
+    n, m = count_and_max(a)
+    assert (n, m) == (int((a > 0).sum()), int(a.max())) and isinstance(n, int)
+    b = np.random.default_rng(10).uniform(0.999, 1.001, 50_000)
+    assert product(b) == pytest.approx(float(np.prod(b)), rel=1e-9)
+
+
+def test_repeated_calls_reuse_pooled_buffers(gpu):
+    from appy_amd.backends.hip import runtime as rt
+    import ctypes
+
+    k0 = selfcheck.kernels()
+    a, b = wl.vec_add(300_000)
+    k0.vec_add(a, b)
+    used, cached = ctypes.c_uint64(), ctypes.c_uint64()
+    rt.check(rt.lib().appy_hip_pool_stats(ctypes.byref(used), ctypes.byref(cached)))
+    first = cached.value
+    for _ in range(5):
+        assert np.array_equal(k0.vec_add(a, b), a + b)
+    rt.check(rt.lib().appy_hip_pool_stats(ctypes.byref(used), ctypes.byref(cached)))
+    assert used.value == 0 and cached.value == first          # nothing leaked, nothing newly allocated
