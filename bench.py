@@ -105,6 +105,16 @@ class Runner:
         }
 
 
+def cpu_time(fn, reps=3):
+    """Best wall time of ``fn`` over ``reps`` runs, seconds."""
+    best = 1e30
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        fn()
+        best = min(best, time.perf_counter() - t0)
+    return best
+
+
 def device_csr(torch, lengths_np, ncols, seed):
     """CSR structure with sorted distinct uniform columns per row, built on the
     device (the host generator of oracle/workloads.py needs minutes at 4e8
@@ -196,6 +206,8 @@ def main():
     log("vector_sum", results["vector_sum"], parity["vector_sum"])
 
     cpu_baseline = None
+    cpu_kernels = {}
+    do_cpu = not args.no_cpu_baseline
     if not args.no_cpu_baseline:
         # oracle (NumPy float64 accumulation, one core) on the full array, best of 3,
         # and the literal interpreter loop on a 2^20 sample
@@ -225,6 +237,10 @@ def main():
         parity["masked_sum"] = {"abs_err": abs(got - ref), "bound": vo.TOL * budget, "ok": abs(got - ref) <= vo.TOL * budget}
         results["masked_sum"] = run.measure(loop, {"s": s_d, "A": A_d, "M": M_d, "A_shape_0": n}, 5 * n + 8, K, W, clear=s_d)
         log("masked_sum", results["masked_sum"], parity["masked_sum"])
+        if do_cpu:
+            t = cpu_time(lambda: np.where(M, A, np.float32(0)).sum(dtype=np.float64), 2)
+            cpu_kernels["masked_sum"] = {"ms": t * 1e3, "gbps": (5 * n + 8) / t / 1e9,
+                                         "what": "np.where(M, A, 0).sum(dtype=float64), full size, 1 core"}
         del M_d
     del A_d, A, M
     torch.cuda.empty_cache()
@@ -258,6 +274,14 @@ def main():
         parity["vec_add"] = {"bit_exact": ok, "ok": ok}
         results["vec_add"] = run.measure(loop, {"c": c_d, "a": a_d, "b": b_d, "a_shape_0": n1}, 12 * n1, K, W)
         log("vec_add", results["vec_add"], parity["vec_add"])
+        if do_cpu:
+            out = np.empty_like(a)
+            t = cpu_time(lambda: np.add(a, b, out=out), 5)
+            m1 = min(n1, 1 << 20)
+            t0 = time.perf_counter()
+            olo.vec_add(a[:m1], b[:m1])
+            cpu_kernels["vec_add"] = {"ms": t * 1e3, "gbps": 12 * n1 / t / 1e9, "what": "np.add(a, b, out=c), full size, 1 core",
+                                      "literal_loop_ns_per_element": (time.perf_counter() - t0) / m1 * 1e9}
         del a_d, b_d, c_d
 
     # ---------------- config 3: GEMV ---------------------------------------------------------
@@ -276,6 +300,14 @@ def main():
         vals = {"A": A_d, "x": x_d, "y": y_d, "A_shape_0": r, "A_shape_1": r}
         results["gemv"] = run.measure(loop, vals, 4 * (r * r + r + r), K, W)
         log("gemv", results["gemv"], parity["gemv"])
+        if do_cpu:
+            t = cpu_time(lambda: Am @ x, 3)
+            rr = min(r, 256)
+            t0 = time.perf_counter()
+            olo.gemv(1.0, Am[:rr, :rr], x[:rr])
+            cpu_kernels["gemv"] = {"ms": t * 1e3, "gbps": 4 * (r * r + 2 * r) / t / 1e9,
+                                   "what": f"A @ x (BLAS sgemv, up to {len(os.sched_getaffinity(0))} threads), full size",
+                                   "literal_loop_ns_per_element": (time.perf_counter() - t0) / (rr * rr) * 1e9}
         del A_d, x_d, y_d, Am, ref, budget
         torch.cuda.empty_cache()
 
@@ -288,10 +320,24 @@ def main():
         spmv_case.loop = loop
         nnz = data_d.numel()
         t0 = time.time()
-        ref, budget = vo.spmv_csr(data_d.cpu().numpy(), indptr_d.cpu().numpy(), indices_d.cpu().numpy(),
-                                  x_d.cpu().numpy(), (m, ncol))
+        h_data, h_ptr, h_idx, h_x = (data_d.cpu().numpy(), indptr_d.cpu().numpy(), indices_d.cpu().numpy(),
+                                      x_d.cpu().numpy())
+        ref, budget = vo.spmv_csr(h_data, h_ptr, h_idx, h_x, (m, ncol))
         ok, worst = vo.within_budget(y_d.cpu().numpy(), ref, budget)
         log(f"{name}: oracle in {time.time() - t0:.1f}s")
+        if do_cpu:
+            import scipy.sparse as sp
+
+            A32 = sp.csr_matrix((h_data, h_idx, h_ptr), shape=(m, ncol))
+            t = cpu_time(lambda: A32 @ h_x, 2)
+            mm = min(m, 1 << 12)
+            t0 = time.perf_counter()
+            olo.spmv_csr(h_data, h_ptr, h_idx, h_x, mm, ncol)
+            cpu_kernels[name] = {"ms": t * 1e3, "gbps": (8 * nnz + 4 * (m + 1) + 4 * ncol + 4 * m) / t / 1e9,
+                                 "what": "scipy.sparse.csr_matrix (float32) @ x, full size, 1 core",
+                                 "literal_loop_ns_per_nnz": (time.perf_counter() - t0) / max(1, int(h_ptr[mm])) * 1e9}
+            del A32
+        del h_data, h_ptr, h_idx, h_x
         lens = (indptr_d[1:] - indptr_d[:-1])
         parity[name] = {"worst_err_over_bound": worst, "ok": ok}
         vals = {"A_data": data_d, "A_indptr": indptr_d, "A_indices": indices_d, "x": x_d, "y": y_d, "M": m}
@@ -345,6 +391,19 @@ def main():
                                   B_d.cpu().numpy(), (len(rows), m5))
         ok, worst = vo.within_budget(Y_d.cpu().numpy()[rows], ref, budget)
         parity["spmm"] = {"worst_err_over_bound": worst, "ok": ok, "rows_checked": int(len(rows))}
+        if do_cpu:
+            import scipy.sparse as sp
+
+            # bounded sample: the first 2^16 rows of A against all of B (the full product needs ~10 s of one core)
+            ms_rows = min(m5, 1 << 16)
+            e = int(ip[ms_rows])
+            Asub = sp.csr_matrix((data_d[:e].cpu().numpy(), indices_d[:e].cpu().numpy(), ip[:ms_rows + 1]), shape=(ms_rows, m5))
+            Bh = B_d.cpu().numpy()
+            t = cpu_time(lambda: Asub @ Bh, 2)
+            sub_bytes = 8 * e + 4 * (ms_rows + 1) + 512 * m5 + 512 * ms_rows
+            cpu_kernels["spmm"] = {"ms": t * 1e3, "gbps": sub_bytes / t / 1e9,
+                                   "what": f"scipy csr (float32) @ B on the first {ms_rows} rows (nnz {e}), 1 core"}
+            del Asub, Bh
         nnz = data_d.numel()
         nbytes = 8 * nnz + 4 * (m5 + 1) + 4 * m5 * 128 + 4 * m5 * 128
         vals = {"A_data": data_d, "A_indptr": indptr_d, "A_indices": indices_d, "B": B_d, "y": Y_d, "M": m5}
@@ -375,6 +434,7 @@ def main():
         "roofline": {"bound": "hbm", "achieved": head["gbps_kernel"], "peak": HBM_PEAK_BPS / 1e9, "unit": "GB/s",
                      "frac": head["frac"], "traffic": MEASURED_TRAFFIC["vector_sum"] if sc == 1.0 else None},
         "cpu_baseline": cpu_baseline,
+        "cpu_kernels": cpu_kernels,
         "parity_ok": all_ok,
         "parity": parity,
         "kernels": results,
