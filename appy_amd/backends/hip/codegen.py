@@ -38,6 +38,11 @@ _HEADER_PATH = os.path.join(os.path.dirname(os.path.dirname(os.path.dirname(os.p
 
 code_cache = {}
 _cache_lock = threading.Lock()
+
+# Loop bounds are evaluated on the host with the scalar arguments in scope and
+# only these builtins (a bound like ``range(min(n, m))`` is ordinary Python).
+_HOST_EVAL_GLOBALS = {"__builtins__": {"min": min, "max": max, "abs": abs, "int": int, "len": len, "float": float,
+                                       "round": round, "bool": bool}}
 _device_header = None
 
 # Hardware facts used by the launch heuristics (MI355X: 256 CUs in 8 XCDs,
@@ -302,7 +307,7 @@ class CompiledLoop:
         best, uniform = 0.0, True
         for code, streamed in self._simd_loops:
             try:
-                best = max(best, float(eval(code, {"__builtins__": {}}, env)))
+                best = max(best, float(eval(code, _HOST_EVAL_GLOBALS, env)))
                 continue
             except Exception:
                 uniform = False
@@ -334,7 +339,7 @@ class CompiledLoop:
         v = d.vec
         if self._row_extent_code is not None:
             try:
-                ext = int(eval(self._row_extent_code, {"__builtins__": {}}, env))
+                ext = int(eval(self._row_extent_code, _HOST_EVAL_GLOBALS, env))
             except Exception:
                 ext = 0
             if ext > 0 and ext % v == 0:
@@ -420,8 +425,8 @@ class CompiledLoop:
         env = {k: v for k, v in vals.items() if k not in a.arrays}
         env["np"] = np
         env["math"] = math
-        lo = int(eval(self._lo_code, {"__builtins__": {}}, env))
-        hi = int(eval(self._hi_code, {"__builtins__": {}}, env))
+        lo = int(eval(self._lo_code, _HOST_EVAL_GLOBALS, env))
+        hi = int(eval(self._hi_code, _HOST_EVAL_GLOBALS, env))
         if hi <= lo:
             return None
         arrays = {k: vals[k] for k in a.arrays}

@@ -219,3 +219,10 @@ def test_concurrent_code_generation_is_safe():
     [t.start() for t in ts]
     [t.join() for t in ts]
     assert len(got) == 8 and all(g is got[0] for g in got)
+
+
+def test_loop_bounds_may_use_plain_builtins():
+    a = np.zeros(8, np.float32)
+    f, _ = compiled("#pragma parallel for simd\nfor i in range(min(n, m) - 1):\n    c[i] = a[i] + 1", c=a, a=a, n=8, m=5)
+    import appy_amd.backends.hip.codegen as mod
+    assert eval(f._hi_code, mod._HOST_EVAL_GLOBALS, {"n": 8, "m": 5}) == 4
