@@ -249,9 +249,9 @@ class CompiledLoop:
         a = self.analysis
         v = max(1, min(4, 16 // max(self._elem_sizes())))
         if a.kind == "flat":
-            if "simd" in a.pragma:
-                return Spec("flat", block=256, vec=v, unroll=2)
-            return Spec("flat", block=256, vec=1, unroll=1)
+            # with or without `simd`: iterations of a parallel loop are independent, and
+            # lanes handle control flow on their own, so both forms take the vector shape
+            return Spec("flat", block=256, vec=v, unroll=2)
         return Spec("team", block=256, vec=v, width=64)
 
     def kernel_for(self, spec: Spec) -> Kernel:
@@ -389,7 +389,7 @@ class CompiledLoop:
             if self.options.get("hip_max_blocks"):
                 cap = self.options["hip_max_blocks"]
             elif self.analysis.outer_reductions:
-                cap = cus * 2
+                cap = cus * 16   # scalar accesses only: more lanes to keep bytes in flight
             elif spec.stream_stores:
                 cap = 1 << 22
             else:

@@ -248,3 +248,22 @@ def test_repeated_calls_reuse_pooled_buffers(gpu):
         assert np.array_equal(k0.vec_add(a, b), a + b)
     rt.check(rt.lib().appy_hip_pool_stats(ctypes.byref(used), ctypes.byref(cached)))
     assert used.value == 0 and cached.value == first          # nothing leaked, nothing newly allocated
+
+
+@pytest.mark.parametrize("n", [1, 1000, 4099, (1 << 22) + 7])
+def test_masked_sum_with_control_flow(gpu, n):
+    """The `if mask[i]: b += a[i]` form of examples/04-masked_sum.py:7-14 (no simd clause)."""
+    import appy_amd as appy
+
+    @appy.jit
+    def masked_sum_if(a, mask):
+        b = 0.0
+        #pragma parallel for shared(b)
+        for i in range(a.shape[0]):
+            if mask[i]:
+                b += a[i]
+        return b
+
+    A, M = wl.reduce_inputs(n)
+    ref, budget = vo.masked_sum(A, M)
+    assert abs(masked_sum_if(A, M) - ref) <= TOL * budget
