@@ -15,7 +15,7 @@ import inspect
 import sys
 import textwrap
 
-from .__version__ import __version__
+__version__ = "0.1.0"  # of this package, not of the reference it is compatible with
 from . import dispatcher
 from .frontend import source as _source
 from .frontend import static_rewrite as _static_rewrite
