@@ -243,3 +243,34 @@ def test_gpu_tensors_are_used_in_place(gpu):
     ones = torch.ones(100, device="cuda")
     add_into(ones, ones, col)
     assert torch.equal(base[:, 3], 2 * ones) and float(base.sum()) == 200.0
+
+
+def test_launches_follow_the_current_torch_stream(gpu):
+    import torch
+
+    @appy.jit
+    def scale_add(a, b, f):
+        #pragma parallel for simd
+        for i in range(a.shape[0]):
+            b[i] = a[i] * f + b[i]
+
+    side = torch.cuda.Stream()                      # default priority
+    n = 1 << 22
+    with torch.cuda.stream(side):
+        a = torch.full((n,), 2.0, device="cuda")    # produced on the side stream
+        b = torch.ones(n, device="cuda")
+        for _ in range(5):
+            scale_add(a, b, 0.5)                    # each launch depends on the previous one through b
+        total = b.sum()                             # consumed on the same stream, no synchronisation in between
+    side.synchronize()
+    assert float(total) == n * 6.0
+
+
+def test_to_gpu_and_to_cpu_helpers(gpu):
+    import torch
+
+    a = np.arange(6, dtype=np.float32)
+    t, u = appy.to_gpu(a, [1, 2, 3])
+    assert t.device.type == "cuda" and u.device.type == "cuda" and appy.to_gpu(3.5) == 3.5
+    assert np.array_equal(appy.to_cpu(t), a)
+    assert appy.to_cpu(torch.tensor(7.0, device="cuda")) == 7.0
