@@ -148,6 +148,11 @@ class _LoopOutliner:
         self.count += 1
         loop_name = f"kernel_loop_{self.count}"
         pre, post = [], []
+        if _is_prange_loop(loop):
+            # `prange` is `range` with the promise of independent iterations
+            loop = copy.deepcopy(loop)
+            loop.iter.func = ast.Name(id="range", ctx=ast.Load())
+            loop.iter.keywords = []
         if pragma:
             shared = shared_names(pragma)
             if shared:
@@ -157,7 +162,8 @@ class _LoopOutliner:
                     post.append(ast.parse(f"{v} = {v}.item()").body[0])
             loop_text = pragma + "\n" + src.unparse(loop)
         else:
-            loop_text = src.unparse(loop)
+            # `for i in prange(...)` without a pragma: a parallel loop over the same range
+            loop_text = "#pragma parallel for\n" + src.unparse(loop)
         self.loops.append((loop_name, loop_text))
         return pre + [self._stub(loop_text, loop_name)] + post
 

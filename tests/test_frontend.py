@@ -101,7 +101,15 @@ def f(a):
         a[i] = 1
 '''
     _, loops = rewrite(src)
-    assert loops and loops[0][1].startswith("for i in appy.prange(")
+    assert loops == [("kernel_loop_1", "#pragma parallel for\nfor i in range(a_shape_0):\n    a[i] = 1")]
+
+    @appy.jit(dry_run=True)
+    def fill(a):
+        for i in appy.prange(a.shape[0]):
+            a[i] = 1
+        return a
+
+    assert all(fill(np.zeros(5)) == 1)
 
 
 # ---- per-loop IR ---------------------------------------------------------------
