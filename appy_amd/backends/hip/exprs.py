@@ -12,7 +12,7 @@ from __future__ import annotations
 
 import ast
 import math
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 
 import numpy as np
 
@@ -81,6 +81,16 @@ _CONSTANTS = {"pi": math.pi, "e": math.e, "inf": math.inf, "nan": math.nan, "tau
 _NP_CASTS = {"float32", "float64", "float16", "int8", "int16", "int32", "int64", "uint8", "uint16", "uint32",
              "uint64", "bool_"}
 _MATH_MODULE_NAMES = ("np", "numpy", "math")
+
+
+def _negative_literal(node):
+    """k for the literal index ``-k`` (k > 0), else None."""
+    if isinstance(node, ast.UnaryOp) and isinstance(node.op, ast.USub) and isinstance(node.operand, ast.Constant) \
+            and type(node.operand.value) is int and node.operand.value > 0:
+        return node.operand.value
+    if isinstance(node, ast.Constant) and type(node.value) is int and node.value < 0:
+        return -node.value
+    return None
 
 
 def cast(code: str, src: Ty, dst: Ty) -> str:
@@ -153,7 +163,13 @@ class ExprEmitter:
         for d, e in enumerate(elts):
             if isinstance(e, ast.Slice):
                 raise NotImplementedError(f"Slice outside an array statement: {ast.unparse(sub)}")
-            code, ty = self.emit(e)
+            neg = _negative_literal(e)
+            if neg is not None:
+                # X[-k] counts from the end, as in Python
+                self.shape_scalars.add((arr.name, d))
+                code, ty = f"({cname(f'{arr.name}_shape_{d}')} - {neg}LL)", T.I64
+            else:
+                code, ty = self.emit(e)
             if not (ty.is_int or ty.is_bool):
                 raise TypeError(f"Array index must be an integer: {ast.unparse(sub)}")
             code = cast(code, ty, T.I64)
@@ -244,13 +260,11 @@ class ExprEmitter:
             return f"appy::mod_int<{t.c}>({a}, {b})", t
         if isinstance(op, ast.Pow):
             t = T.promote(lt, rt)
-            if isinstance(node.right, ast.Constant) and isinstance(node.right.value, int) and 0 <= node.right.value <= 4 \
-                    and not isinstance(node.right.value, bool):
-                n = node.right.value
+            if isinstance(node.right, ast.Constant) and type(node.right.value) is int and node.right.value == 2:
+                # x ** 2 is x * x exactly (one rounding either way); higher powers go through
+                # pow like NumPy's, where repeated multiplication would round differently
                 a = cast(lc, lt, t)
-                if n == 0:
-                    return f"(({t.c})1)", t
-                return "(" + " * ".join([a] * n) + ")", t
+                return f"({a} * {a})", t
             if t.is_float:
                 fn = "powf" if t.name == "float32" else "pow"
                 return f"{fn}({cast(lc, lt, t)}, {cast(rc, rt, t)})", t

@@ -226,3 +226,12 @@ def test_loop_bounds_may_use_plain_builtins():
     f, _ = compiled("#pragma parallel for simd\nfor i in range(min(n, m) - 1):\n    c[i] = a[i] + 1", c=a, a=a, n=8, m=5)
     import appy_amd.backends.hip.codegen as mod
     assert eval(f._hi_code, mod._HOST_EVAL_GLOBALS, {"n": 8, "m": 5}) == 4
+
+
+def test_negative_literal_index_counts_from_the_end():
+    a = np.zeros(8, np.float32)
+    f, src = compiled("#pragma parallel for simd\nfor i in range(n):\n    c[i] = a[i] + a[-1] + b[-2, i]", c=a, a=a,
+                      b=np.zeros((4, 8), np.float32), n=8)
+    k = body_of(src)
+    assert "a[(a_shape_0 - 1LL)]" in k and "(b_shape_0 - 2LL) * b_stride_0" in k
+    assert "const appy::i64 a_shape_0" in k and "const appy::i64 b_shape_0" in k

@@ -1,0 +1,170 @@
+"""Expression semantics of generated kernels against NumPy, element by element:
+integer division and modulo with negative operands (Python/NumPy floor
+semantics, not C truncation), powers, comparisons, boolean operators, dtype
+promotion with Python scalars, small integer and half-precision arrays,
+boolean outputs, gathers with computed indices, maths functions."""
+import math
+
+import numpy as np
+import pytest
+
+import appy
+
+pytestmark = pytest.mark.gpu
+N = 10_007
+
+
+@pytest.fixture(scope="module")
+def rng(gpu):
+    return np.random.default_rng(123)
+
+
+@appy.jit
+def int_ops(a, b, q, r, p, s):
+    #pragma parallel for simd
+    for i in range(a.shape[0]):
+        q[i] = a[i] // b[i]
+        r[i] = a[i] % b[i]
+        p[i] = a[i] ** 2 + abs(b[i])
+        s[i] = (a[i] << 2) ^ (b[i] & 7) | (a[i] >> 1)
+
+
+def test_integer_floor_division_modulo_shifts(rng):
+    a = rng.integers(-1000, 1000, N, dtype=np.int32)
+    b = rng.integers(1, 50, N, dtype=np.int32) * rng.choice([-1, 1], N).astype(np.int32)
+    q, r, p, s = (np.empty_like(a) for _ in range(4))
+    int_ops(a, b, q, r, p, s)
+    assert np.array_equal(q, a // b) and np.array_equal(r, a % b)
+    assert np.array_equal(p, a ** 2 + np.abs(b))
+    assert np.array_equal(s, (a << 2) ^ (b & 7) | (a >> 1))
+
+
+@appy.jit
+def float_ops(a, b, out_mod, out_fdiv, out_pow, out_cmp, out_sel):
+    #pragma parallel for simd
+    for i in range(a.shape[0]):
+        out_mod[i] = a[i] % b[i]
+        out_fdiv[i] = a[i] // b[i]
+        out_pow[i] = a[i] ** 3 - b[i] ** 2
+        out_cmp[i] = (0.0 < a[i] < 0.5) or (not b[i] > 0.0 and a[i] <= -0.5)
+        out_sel[i] = max(a[i], b[i], 0.25) - min(a[i], b[i])
+
+
+def test_float_modulo_floor_division_power_comparisons(rng):
+    a = rng.uniform(-1, 1, N).astype(np.float32)
+    b = rng.uniform(0.1, 1, N).astype(np.float32) * rng.choice([-1, 1], N).astype(np.float32)
+    m, f, p, s = (np.empty_like(a) for _ in range(4))
+    c = np.empty(N, dtype=bool)
+    float_ops(a, b, m, f, p, c, s)
+    assert np.allclose(m, np.mod(a, b), rtol=0, atol=1e-6)
+    assert np.array_equal(f, np.floor_divide(a, b))
+    assert p.dtype == np.float32 and np.allclose(p, a ** 3 - b ** 2, rtol=1e-6, atol=1e-7)
+    assert np.array_equal(c, ((0.0 < a) & (a < 0.5)) | (~(b > 0.0) & (a <= -0.5)))
+    assert np.array_equal(s, np.maximum(np.maximum(a, b), np.float32(0.25)) - np.minimum(a, b))
+
+
+@appy.jit
+def promote(i32, f32, u8, alpha, out_f32, out_f64, out_u8, out_i64):
+    #pragma parallel for simd
+    for i in range(i32.shape[0]):
+        out_f32[i] = f32[i] * alpha + 1          # Python scalars adopt float32
+        out_f64[i] = i32[i] * alpha + i32[i] / 4 # int32 with a Python float / true division: float64
+        out_u8[i] = u8[i] + u8[i]                # wraps in uint8
+        out_i64[i] = i32[i] * 3 + i             # the loop index is a Python int
+
+
+def test_dtype_promotion_follows_numpy(rng):
+    i32 = rng.integers(-100, 100, N, dtype=np.int32)
+    f32 = rng.standard_normal(N).astype(np.float32)
+    u8 = rng.integers(0, 256, N, dtype=np.uint8)
+    alpha = 0.1
+    o32, o64 = np.empty(N, np.float32), np.empty(N, np.float64)
+    ou8, oi64 = np.empty(N, np.uint8), np.empty(N, np.int64)
+    promote(i32, f32, u8, alpha, o32, o64, ou8, oi64)
+    assert np.array_equal(o32, f32 * alpha + 1) and (f32 * alpha + 1).dtype == np.float32
+    assert np.array_equal(o64, i32 * alpha + i32 / 4)
+    assert np.array_equal(ou8, u8 + u8)
+    assert np.array_equal(oi64, i32.astype(np.int64) * 3 + np.arange(N))
+
+
+@appy.jit
+def half_add(a, b, c):
+    #pragma parallel for simd
+    for i in range(a.shape[0]):
+        c[i] = a[i] + b[i] * 2.0
+
+
+def test_float16_arrays(rng):
+    a = rng.standard_normal(N).astype(np.float16)
+    b = rng.standard_normal(N).astype(np.float16)
+    c = np.empty_like(a)
+    half_add(a, b, c)
+    assert c.dtype == np.float16 and np.array_equal(c, a + b * np.float16(2.0))
+
+
+@appy.jit
+def gather_shifted(x, idx, y, flag):
+    #pragma parallel for simd
+    for i in range(idx.shape[0]):
+        y[i] = x[idx[i] + 1] - x[idx[i]]
+        flag[i] = x[idx[i]] > 0.5
+
+
+def test_gather_with_computed_index_and_bool_output(rng):
+    x = rng.random(5000)
+    idx = rng.integers(0, 4999, N, dtype=np.int64)
+    y = np.empty(N)
+    flag = np.zeros(N, dtype=bool)
+    gather_shifted(x, idx, y, flag)
+    assert np.array_equal(y, x[idx + 1] - x[idx]) and np.array_equal(flag, x[idx] > 0.5)
+
+
+@appy.jit
+def maths(a, out):
+    #pragma parallel for simd
+    for i in range(a.shape[0]):
+        v = np.sqrt(np.abs(a[i])) + np.exp(-a[i] * a[i]) + math.sin(a[i]) * np.cos(a[i])
+        w = np.log1p(np.abs(a[i])) + np.arctan2(a[i], 2.0) + np.floor(a[i]) + np.pi
+        out[i] = v + w if a[i] > -10 else float("inf")
+
+
+@pytest.mark.parametrize("dtype,tol", [(np.float64, 1e-13), (np.float32, 2e-6)])
+def test_maths_functions(rng, dtype, tol):
+    a = rng.uniform(-3, 3, N).astype(dtype)
+    out = np.empty_like(a)
+    maths(a, out)
+    a64 = a.astype(np.float64)
+    ref = (np.sqrt(np.abs(a64)) + np.exp(-a64 * a64) + np.sin(a64) * np.cos(a64)
+           + np.log1p(np.abs(a64)) + np.arctan2(a64, 2.0) + np.floor(a64) + np.pi)
+    assert out.dtype == dtype and np.allclose(out, ref, rtol=tol, atol=tol * 10)
+
+
+@appy.jit
+def private_scalar(a, t):
+    #pragma parallel for simd
+    for i in range(a.shape[0]):
+        u = t + i
+        t = 0.0
+        a[i] = u
+    return t
+
+
+def test_scalars_are_passed_by_value(rng):
+    a = np.zeros(100)
+    assert private_scalar(a, 5.0) == 5.0                 # writes to a by-value scalar are invisible afterwards
+    assert a[0] == 5.0 and np.all(a >= 0)
+
+
+@appy.jit
+def from_the_end(a, b, out):
+    #pragma parallel for simd
+    for i in range(out.shape[0]):
+        out[i] = a[-1] + b[-2, i] - a[i]
+
+
+def test_negative_literal_indices(rng):
+    a = rng.random(50)
+    b = rng.random((4, 50))
+    out = np.empty(50)
+    from_the_end(a, b, out)
+    assert np.array_equal(out, a[-1] + b[-2, :] - a)
