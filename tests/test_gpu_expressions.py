@@ -168,3 +168,35 @@ def test_negative_literal_indices(rng):
     out = np.empty(50)
     from_the_end(a, b, out)
     assert np.array_equal(out, a[-1] + b[-2, :] - a)
+
+
+@appy.jit
+def sum_2d(a):
+    s = 0.0
+    #pragma parallel for shared(s)
+    for i in range(a.shape[0]):
+        #pragma simd
+        for j in range(a.shape[1]):
+            s += a[i, j]
+    return s
+
+
+@appy.jit
+def sum_of_row_maxima(a):
+    s = 0.0
+    #pragma parallel for shared(s)
+    for i in range(a.shape[0]):
+        m = -1e30
+        #pragma simd
+        for j in range(a.shape[1]):
+            m = max(m, a[i, j])
+        s += m
+    return s
+
+
+def test_shared_reductions_in_team_loops(rng):
+    a = rng.standard_normal((301, 777))
+    assert sum_2d(a) == pytest.approx(a.sum(), rel=1e-12)
+    assert sum_of_row_maxima(a) == pytest.approx(a.max(axis=1).sum(), rel=1e-12)
+    a32 = a.astype(np.float32)
+    assert sum_2d(a32) == pytest.approx(float(a32.astype(np.float64).sum()), abs=1e-5 * float(np.abs(a32).sum()))
