@@ -350,10 +350,13 @@ class CompiledLoop:
                 ext = int(eval(self._row_extent_code, _HOST_EVAL_GLOBALS, env))
             except Exception:
                 ext = 0
-            if ext > 0 and ext % v == 0:
-                w = max(1, min(64, _pow2ceil(ext / v)))
-                if -(-ext // (w * v)) <= 8:
-                    return Spec("team", block=d.block, vec=v, width=w, restrict=restrict,
+            ve = v
+            while ve > 1 and ext % ve:      # widest vector that divides the extent
+                ve //= 2
+            if ext > 0:
+                w = max(1, min(64, _pow2ceil(ext / ve)))
+                if -(-ext // (w * ve)) <= 8:
+                    return Spec("team", block=d.block, vec=ve, width=w, restrict=restrict,
                                 stream_loads=False, extent=ext)
         trip, uniform = self._estimate_trip(env, arrays, n_outer)
         if trip < 2 * v:

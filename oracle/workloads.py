@@ -45,7 +45,7 @@ def _sorted_unique_columns(rng, lengths, ncols):
         # dense rows: rejection would not terminate, draw each row without replacement
         cols = np.concatenate([np.sort(rng.permutation(ncols)[: int(n)]) for n in lengths] or [np.empty(0, np.int64)])
         return indptr, cols.astype(np.int64)
-    if len(lengths) and np.all(lengths == lengths[0]) and lengths[0] > 0:
+    if len(lengths) and np.all(lengths == lengths[0]) and 0 < lengths[0] and 4 * int(lengths[0]) ** 2 < ncols:
         # equal rows: sort each row on its own, redraw the rows that hold a duplicate
         L = int(lengths[0])
         cols = np.sort(rng.integers(0, ncols, size=(len(lengths), L), dtype=np.int64), axis=1)
