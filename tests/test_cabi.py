@@ -69,3 +69,29 @@ def test_invalid_arguments_are_reported_not_crashed():
 
 def test_device_count_without_gpu_is_zero_not_an_error():
     assert rt.device_count() >= 0
+
+
+CLIENT_SRC = os.path.join(ROOT, "tests", "cabi", "client.c")
+
+
+def _build_client(tmp_path):
+    exe = tmp_path / "cabi_client"
+    lib_dir = os.path.dirname(rt.library_path())
+    subprocess.run(
+        ["gcc", "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", "-I" + os.path.join(ROOT, "include"), CLIENT_SRC,
+         "-o", str(exe), "-L" + lib_dir, "-lappy_hip", "-Wl,-rpath," + lib_dir],
+        check=True, capture_output=True, text=True)
+    return str(exe)
+
+
+def test_header_is_plain_c_and_a_c_client_can_compile_kernels(tmp_path):
+    exe = _build_client(tmp_path)
+    out = subprocess.run([exe, "compile"], check=True, capture_output=True, text=True).stdout
+    assert out.startswith("compiled ") and int(out.split()[1]) > 1000
+
+
+@pytest.mark.gpu
+def test_c_client_runs_a_kernel_end_to_end(tmp_path, gpu):
+    exe = _build_client(tmp_path)
+    out = subprocess.run([exe, "run"], check=True, capture_output=True, text=True, timeout=120).stdout
+    assert "ran 100003 elements, 0 mismatches" in out
