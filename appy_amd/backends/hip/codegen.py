@@ -364,7 +364,13 @@ class CompiledLoop:
         # one vector step per lane for short rows; two rows per wavefront at most
         # (two independent rows in flight per wavefront stream better than one)
         w = max(1, min(32, _pow2ceil(trip / float(v)) if trip > 0 else 1))
-        return Spec("team", block=d.block, vec=v, width=w, restrict=restrict, stream_loads=stream)
+        block = d.block
+        if uniform and n_outer * 32 < DEFAULT_CUS * 256 and trip >= 64 * v * 32:
+            # few, very long rows: wavefront teams would leave most of the chip idle,
+            # so a whole workgroup takes each row (the more lanes the fewer rows there are)
+            block = 1024 if n_outer <= DEFAULT_CUS else 256
+            w = block
+        return Spec("team", block=block, vec=v, width=w, restrict=restrict, stream_loads=stream)
 
     def row_hint(self, n_outer, env, arrays):
         """(expected inner trip count, same for every row?) for grid sizing."""

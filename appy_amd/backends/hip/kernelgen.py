@@ -75,8 +75,8 @@ class Spec:
             raise ValueError(f"vector width must be 1, 2 or 4, got {self.vec}")
         if not 1 <= self.unroll <= 8:
             raise ValueError(f"unroll factor must be 1..8, got {self.unroll}")
-        if not pow2(self.width) or self.width > 64:
-            raise ValueError(f"team width must be a power of two up to 64, got {self.width}")
+        if not pow2(self.width) or (self.width > 64 and self.width != self.block):
+            raise ValueError(f"team width must be a power of two up to 64, or the whole workgroup, got {self.width}")
         if self.extent < 0 or self.lds_tile < 0 or self.lds_tile % 4 or self.lds_tile > 16384:
             raise ValueError("row extent / LDS tile out of range (tile: multiple of 4, at most 16384 elements)")
 
@@ -442,6 +442,16 @@ class KernelBuilder:
                 self.ex.locals[var] = saved
         return f"{cname(arr.name)} + ({idx.replace('__vbase', base_code)})"
 
+    def _team_total(self, op: str, ty: Ty, partial: str) -> str:
+        """Combine the lanes' partial results of a team; every lane gets the total.
+        Teams of up to 64 lanes use the DPP/bpermute butterfly, a team that is the
+        whole workgroup (rows too long and too few for wavefront teams) goes
+        through LDS."""
+        W = self.spec.width
+        if W <= 64:
+            return f"appy::team_reduce<{_OPS[op]}, {W}, {ty.c}>({partial})"
+        return f"appy::workgroup_reduce_all<{_OPS[op]}, {self.spec.block}, {ty.c}>({partial}, {T.identity_literal(op, ty)})"
+
     def _leader(self) -> str:
         """Condition under which a team-level statement has its side effect."""
         return "__lane == 0 && __active" if self.lds_plan else "__lane == 0"
@@ -557,7 +567,7 @@ class KernelBuilder:
             p, ty = self.partials[name]
             if ty.size < 4:
                 raise Unsupported(f"Reduction variable `{name}` of type {ty.name} is not supported")
-            self.w(f"{cname(name)} = {_OPS[op]}::f<{ty.c}>({cname(name)}, appy::team_reduce<{_OPS[op]}, {W}, {ty.c}>({p}));")
+            self.w(f"{cname(name)} = {_OPS[op]}::f<{ty.c}>({cname(name)}, {self._team_total(op, ty, p)});")
         self.partials = saved_partials
         self.ind -= 1
         self.w("}")
@@ -945,7 +955,7 @@ class KernelBuilder:
             p, ty = self.partials[name]
             if ty.size < 4:
                 raise Unsupported(f"Reduction variable `{name}` of type {ty.name} is not supported")
-            self.w(f"{cname(name)} = {_OPS[op]}::f<{ty.c}>({cname(name)}, appy::team_reduce<{_OPS[op]}, {W}, {ty.c}>({p}));")
+            self.w(f"{cname(name)} = {_OPS[op]}::f<{ty.c}>({cname(name)}, {self._team_total(op, ty, p)});")
         self.partials = saved_partials
         self.ind -= 1
         self.w("}")

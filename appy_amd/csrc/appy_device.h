@@ -204,6 +204,30 @@ __device__ __forceinline__ T block_reduce(T v, T identity) {
     }
 }
 
+// Workgroup reduction whose total is returned in every thread (a team that
+// spans the whole workgroup).  Must be reached by every thread.
+template <typename Op, int BLOCK, typename T>
+__device__ __forceinline__ T workgroup_reduce_all(T v, T identity) {
+    static_assert(BLOCK % 64 == 0 && BLOCK <= 1024, "workgroup is a whole number of wavefronts");
+    constexpr int NW = BLOCK / 64;
+    v = team_reduce<Op, 64>(v);
+    if constexpr (NW == 1) {
+        return v;
+    } else {
+        __shared__ T slots[NW];
+        const int wave = threadIdx.x >> 6;
+        const int lane = threadIdx.x & 63;
+        if (lane == 0) slots[wave] = v;
+        __syncthreads();
+        constexpr int W2 = NW <= 2 ? 2 : NW <= 4 ? 4 : NW <= 8 ? 8 : 16;
+        const int slot = lane & (W2 - 1);   // every aligned group of W2 lanes reduces the same NW slots
+        T r = (slot < NW) ? slots[slot] : identity;
+        r = team_reduce<Op, W2>(r);
+        __syncthreads();                    // slots may be reused by the next reduction
+        return r;
+    }
+}
+
 // ---- atomics on device memory -------------------------------------------------------
 template <int N>
 struct uint_of;

@@ -30,4 +30,8 @@ appy_device_check(const float* __restrict__ a, const double* __restrict__ b, con
         appy::atomic_combine<appy::OpAdd, long long>::run(ol, bl);
         appy::atomic_combine<appy::OpMul, double>::run(od + 1, appy::mod_float(bd, 3.0));
     }
+    {
+        const float wf = appy::workgroup_reduce_all<appy::OpAdd, 256>(f, 0.f);
+        if (threadIdx.x == 255) of[1] = wf;
+    }
 }

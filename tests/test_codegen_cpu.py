@@ -239,3 +239,16 @@ def test_negative_literal_index_counts_from_the_end():
     k = body_of(src)
     assert "a[(a_shape_0 - 1LL)]" in k and "(b_shape_0 - 2LL) * b_stride_0" in k
     assert "const appy::i64 a_shape_0" in k and "const appy::i64 b_shape_0" in k
+
+
+def test_few_very_long_rows_get_a_workgroup_each():
+    g, _ = selfcheck_loop("gemv")
+    sp = g.choose_spec(100, {"A_shape_1": 1 << 20}, {})
+    assert (sp.width, sp.block) == (1024, 1024)
+    sp = g.choose_spec(2000, {"A_shape_1": 1 << 16}, {})
+    assert (sp.width, sp.block) == (256, 256)
+    k = body_of(g.kernel_for(sp).src.text)
+    assert "appy::workgroup_reduce_all<appy::OpAdd, 256, float>" in k and "threadIdx.x & 255" in k
+    assert g.choose_spec(16384, {"A_shape_1": 16384}, {}).width == 32      # many rows: wavefront teams
+    with pytest.raises(ValueError):
+        Spec("team", block=256, width=128)

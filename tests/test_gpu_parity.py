@@ -267,3 +267,13 @@ def test_masked_sum_with_control_flow(gpu, n):
     A, M = wl.reduce_inputs(n)
     ref, budget = vo.masked_sum(A, M)
     assert abs(masked_sum_if(A, M) - ref) <= TOL * budget
+
+
+@pytest.mark.parametrize("shape", [(1, 300_000), (3, 1 << 20), (100, 70_001), (2000, 9000)])
+def test_gemv_few_long_rows(k, shape):
+    """Few, very long rows: one workgroup per row with the LDS team reduction."""
+    A, x = wl.gemv(*shape)
+    ref, budget = vo.gemv(A, x)
+    y = k.gemv(A, x)
+    ok, worst = vo.within_budget(y, ref, budget, TOL)
+    assert ok, worst
