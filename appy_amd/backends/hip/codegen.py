@@ -365,7 +365,7 @@ class CompiledLoop:
         # (two independent rows in flight per wavefront stream better than one)
         w = max(1, min(32, _pow2ceil(trip / float(v)) if trip > 0 else 1))
         block = d.block
-        if uniform and n_outer * 32 < DEFAULT_CUS * 256 and trip >= 64 * v * 32:
+        if n_outer * 32 < DEFAULT_CUS * 256 and trip >= 64 * v * 32:
             # few, very long rows: wavefront teams would leave most of the chip idle,
             # so a whole workgroup takes each row (the more lanes the fewer rows there are)
             block = 1024 if n_outer <= DEFAULT_CUS else 256

@@ -252,3 +252,11 @@ def test_few_very_long_rows_get_a_workgroup_each():
     assert g.choose_spec(16384, {"A_shape_1": 16384}, {}).width == 32      # many rows: wavefront teams
     with pytest.raises(ValueError):
         Spec("team", block=256, width=128)
+
+
+def test_few_very_long_csr_rows_get_a_workgroup_each():
+    g, _ = selfcheck_loop("spmv")
+    arrays = {"A_data": np.zeros(37 * 40_000, np.float32)}       # ~40000 non-zeros per row on average
+    sp = g.choose_spec(37, {}, arrays)
+    assert (sp.width, sp.block) == (1024, 1024)
+

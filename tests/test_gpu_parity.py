@@ -277,3 +277,17 @@ def test_gemv_few_long_rows(k, shape):
     y = k.gemv(A, x)
     ok, worst = vo.within_budget(y, ref, budget, TOL)
     assert ok, worst
+
+
+def test_spmv_few_very_long_rows(k):
+    """A handful of rows with tens of thousands of non-zeros: workgroup teams on CSR rows."""
+    rng = np.random.default_rng(11)
+    m, n = 37, 400_000
+    lengths = rng.integers(20_000, 60_000, m)
+    lengths[5] = 0
+    data, indptr, indices = wl.csr_matrix(lengths, n, rng)
+    x = rng.standard_normal(n, dtype=np.float32)
+    ref, budget = vo.spmv_csr(data, indptr, indices, x, (m, n))
+    y = k.spmv(data, indptr, indices, x, m, n)
+    ok, worst = vo.within_budget(y, ref, budget, TOL)
+    assert ok, worst
