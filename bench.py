@@ -32,14 +32,14 @@ HBM_PEAK_BPS = 8.0e12  # MI355X HBM3E, bytes per second
 # runs summarised in profiles/all_kernels_bench_pmc_fetch_write_size.txt:
 # FETCH_SIZE x 2.000 + WRITE_SIZE x 0.999 (factors from the plain copy kernel), KiB -> bytes.
 MEASURED_TRAFFIC = {
-    "vector_sum": int((524302.8 * 2.000 + 24.0 * 0.999) * 1024),
-    "masked_sum": int((655384.1 * 2.000 + 20.0 * 0.999) * 1024),
+    "vector_sum": int((524302.8 * 2.000 + 12.0 * 0.999) * 1024),
+    "masked_sum": int((655384.8 * 2.000 + 6.0 * 0.999) * 1024),
     "vec_add": int((65549.0 * 2.000 + 65536.0 * 0.999) * 1024),
-    "gemv": int((524558.0 * 2.000 + 64.5 * 0.999) * 1024),
-    "spmv_uniform": int((3442370.0 * 2.000 + 18580.9 * 0.999) * 1024),
-    "spmv_powerlaw": int((21324000.0 * 2.000 + 37038.3 * 0.999) * 1024),
-    "spmm": int((8641800.0 * 2.000 + 524288.0 * 0.999) * 1024),
-    "copy": int((524301.2 * 2.000 + 1049486.1 * 0.999) * 1024),
+    "gemv": int((524558.6 * 2.000 + 64.0 * 0.999) * 1024),
+    "spmv_uniform": int((3442392.1 * 2.000 + 18589.0 * 0.999) * 1024),
+    "spmv_powerlaw": int((21322939.7 * 2.000 + 37060.8 * 0.999) * 1024),
+    "spmm": int((8641723.2 * 2.000 + 524288.0 * 0.999) * 1024),
+    "copy": int((524301.6 * 2.000 + 1049511.1 * 0.999) * 1024),
 }
 
 
