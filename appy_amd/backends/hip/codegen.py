@@ -30,6 +30,7 @@ from ...frontend import loop_ir
 from . import array_expr
 from . import dtypes as T
 from . import runtime as rt
+from ... import residency
 from .exprs import ArrayParam, ScalarParam
 from .kernelgen import KernelBuilder, KernelSource, LoopAnalysis, Spec, Unsupported
 
@@ -462,6 +463,7 @@ class Launch:
         a = loop.analysis
         self.lo, self.hi = lo, hi
         self.temps = []          # (dptr, host ndarray (contiguous), original, stored)
+        self.mirrored = []       # (mirror, dptr, host ndarray, stored): arguments with a standing HBM mirror
         self.keepalive = []
         # -- bounds of accesses indexed by the parallel loop variable (host check, before any device work)
         for name, dim, off in a.bound_checks:
@@ -512,6 +514,8 @@ class Launch:
                 self._stage_host(name, host, v if tc is v else ("tensor", v, tc), arr.stored)
         for dptr, host, _orig, stored, name in self.temps:
             extents.append((name, dptr, host.nbytes, stored))
+        for _m, dptr, host, stored, name in self.mirrored:
+            extents.append((name, dptr, host.nbytes, stored))
         restrict = not _overlaps(extents)
 
         # -- kernel variant, argument block, grid
@@ -548,6 +552,20 @@ class Launch:
 
     def _stage_host(self, name, host, original, stored):
         nbytes = host.nbytes
+        hit = residency.lookup(host.ctypes.data, nbytes) if (residency.active() and original is host) else None
+        if hit is not None:
+            # the array (or the array this is a view of) has a standing mirror in HBM
+            m, off = hit
+            if m.resident:
+                if m.host_dirty:
+                    m.upload(self.stream)
+            elif nbytes:
+                rt.memcpy_h2d(m.device_ptr() + off, host.ctypes.data, nbytes, self.stream)
+            dptr = m.device_ptr() + off
+            self.mirrored.append((m, dptr, host, stored, name))
+            self.ptr[name] = dptr
+            self.strides[name] = [s // host.itemsize for s in host.strides]
+            return
         dptr = rt.malloc(max(nbytes, 1))
         if nbytes:
             rt.memcpy_h2d(dptr, host.ctypes.data, nbytes, self.stream)
@@ -576,7 +594,19 @@ class Launch:
                         dst.copy_(src)
                     elif original is not host and is_numpy_array(original):
                         original[...] = host
-            if self.temps:
+            waited = bool(self.temps)
+            for m, dptr, host, stored, _name in self.mirrored:
+                if not stored:
+                    continue
+                if m.resident:
+                    m.device_dirty = True       # downloaded on request, not per launch
+                    m.stream = self.stream
+                elif host.nbytes:
+                    rt.memcpy_d2h(host.ctypes.data, dptr, host.nbytes, self.stream)
+                    waited = True
+            if self.mirrored and not waited and any(not m.resident for m, *_ in self.mirrored):
+                waited = True    # uploads from pinned memory must have left the host buffer
+            if waited:
                 rt.sync(self.stream)
             for item in self.keepalive:
                 if isinstance(item, tuple) and item[0] == "copy_back":
@@ -585,6 +615,7 @@ class Launch:
             for dptr, *_ in self.temps:
                 rt.free(dptr)
             self.temps = []
+            self.mirrored = []
             self.keepalive = []
 
     def run(self):

@@ -185,8 +185,7 @@ class LoopAnalysis:
                     self.loop_vars.append(n.target.id)
                 else:
                     raise Unsupported("Loop variables must be plain names")
-            elif isinstance(n, (ast.While, ast.Break, ast.Continue, ast.Return, ast.With, ast.Try, ast.FunctionDef,
-                                ast.Lambda, ast.ListComp, ast.Yield)):
+            elif isinstance(n, (ast.Return, ast.With, ast.Try, ast.FunctionDef, ast.Lambda, ast.ListComp, ast.Yield)):
                 raise Unsupported(f"Statement not supported in a kernel: {type(n).__name__}")
         for name in self.stored:
             if name in self.arrays:
@@ -240,6 +239,7 @@ class KernelBuilder:
         self.store_subst = {}     # unparsed subscript -> (lvalue code, Ty)
         self.dirty = False
         self.counter = 0
+        self.seq_depth = 0        # sequential loops (for / while) around the current statement
         self.shadowed = [n for n in analysis.assigned if n in analysis.scalars]
         self.red_by_key = {r.key: r for r in analysis.outer_reductions}
 
@@ -278,6 +278,15 @@ class KernelBuilder:
             return self.for_(st)
         if isinstance(st, ast.If):
             return self.if_(st)
+        if isinstance(st, ast.While):
+            return self.while_(st)
+        if isinstance(st, (ast.Break, ast.Continue)):
+            # the iterations of parallel and simd loops are dealt to lanes, tiles and vector
+            # components: only a sequential loop has a C loop of its own to leave or to restart
+            if self.seq_depth == 0:
+                raise Unsupported("`break` / `continue` are only supported inside a sequential loop of the kernel")
+            self.w("break;" if isinstance(st, ast.Break) else "continue;")
+            return
         if isinstance(st, ast.Pass):
             return
         if isinstance(st, ast.Expr) and isinstance(st.value, ast.Constant):
@@ -295,6 +304,21 @@ class KernelBuilder:
             self.ind += 1
             self.block(st.orelse)
             self.ind -= 1
+        self.w("}")
+
+    def while_(self, st: ast.While):
+        if st.orelse:
+            raise Unsupported("`while ... else` is not supported in a kernel")
+        # the condition is evaluated again after every pass: as the last statement of an
+        # endless loop, so that it may hold loads and calls like any other expression
+        self.w("while (true) {")
+        self.ind += 1
+        c, t = self.ex.emit(st.test)
+        self.w(f"if (!({truth(c, t)})) break;")
+        self.seq_depth += 1
+        self.block(st.body)
+        self.seq_depth -= 1
+        self.ind -= 1
         self.w("}")
 
     def assign(self, st: ast.Assign):
@@ -370,7 +394,9 @@ class KernelBuilder:
         self.w(f"const appy::i64 {hi_v} = {hi};")
         self.w(f"for (appy::i64 {cname(var)} = {lo}; {cname(var)} < {hi_v}; ++{cname(var)}) {{")
         self.ind += 1
+        self.seq_depth += 1
         self.block(st.body)
+        self.seq_depth -= 1
         self.ind -= 1
         self.w("}")
 
@@ -537,6 +563,7 @@ class KernelBuilder:
             self.w(f"{ty.c} {p} = {T.identity_literal(op, ty)};")
         saved_mode = self.mode
         self.mode = "lane"
+        saved_depth, self.seq_depth = self.seq_depth, 0
         saved_vary = self.bounds_vary
         outer_locals = set(self.a.assigned) | {self.a.var}
         self.bounds_vary = any(_uses_name(b, n) for b in st.iter.args[:2] for n in outer_locals)
@@ -562,6 +589,7 @@ class KernelBuilder:
         self.ind -= 1
         self.w("}")
         self.mode = saved_mode
+        self.seq_depth = saved_depth
         self.bounds_vary = saved_vary
         for name, op in reds.items():
             p, ty = self.partials[name]
@@ -910,6 +938,7 @@ class KernelBuilder:
             self.w("}")
         self.w("__syncthreads();   // the tile is complete")
         saved_mode, self.mode = self.mode, "lane"
+        saved_depth, self.seq_depth = self.seq_depth, 0
         loads, stores = self._vector_accesses(st.body, var) if V > 1 else ({}, {})
         staged_names = {a.name for a in staged}
         staged_keys = {f"{a.name}[{var}]" for a in staged}
@@ -948,6 +977,7 @@ class KernelBuilder:
         self.ex.load_subst = saved_loads
         self.ind -= 1
         self.w("}")
+        self.seq_depth = saved_depth
         self.mode = saved_mode
         self.ind -= 1
         self.w("}")

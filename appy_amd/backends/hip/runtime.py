@@ -73,6 +73,9 @@ SIGNATURES = {
     "appy_hip_pool_stats": (C.c_int, [C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
     "appy_hip_memcpy_h2d": (C.c_int, [_vp, _vp, C.c_size_t, _vp]),
     "appy_hip_memcpy_d2h": (C.c_int, [_vp, _vp, C.c_size_t, _vp]),
+    "appy_hip_host_alloc": (C.c_int, [C.c_size_t, C.POINTER(_vp)]),
+    "appy_hip_host_free": (C.c_int, [_vp]),
+    "appy_hip_host_is_pinned": (C.c_int, [_vp, C.c_size_t]),
     "appy_hip_memcpy_d2d_async": (C.c_int, [_vp, _vp, C.c_size_t, _vp]),
     "appy_hip_memset_async": (C.c_int, [_vp, C.c_int, C.c_size_t, _vp]),
     "appy_hip_launch": (C.c_int, [_vp, _u32, _u32, _u32, _u32, _u32, _u32, _u32, _vp, _vp, C.c_size_t]),
@@ -228,6 +231,21 @@ def memcpy_h2d(dst: int, src_host_ptr: int, nbytes: int, stream: int = 0) -> Non
 
 def memcpy_d2h(dst_host_ptr: int, src: int, nbytes: int, stream: int = 0) -> None:
     check(lib().appy_hip_memcpy_d2h(_vp(dst_host_ptr), _vp(src), int(nbytes), _vp(stream)))
+
+
+def host_alloc(nbytes: int) -> int:
+    """Page-locked host memory (address as int)."""
+    out = _vp()
+    check(lib().appy_hip_host_alloc(int(nbytes), C.byref(out)))
+    return out.value
+
+
+def host_free(ptr: int) -> None:
+    check(lib().appy_hip_host_free(_vp(ptr)))
+
+
+def host_is_pinned(ptr: int, nbytes: int) -> bool:
+    return bool(lib().appy_hip_host_is_pinned(_vp(ptr), int(nbytes)))
 
 
 def memset_async(dst: int, value: int, nbytes: int, stream: int = 0) -> None:

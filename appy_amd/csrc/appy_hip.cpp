@@ -13,9 +13,12 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <algorithm>
+#include <atomic>
 #include <map>
 #include <mutex>
 #include <string>
+#include <thread>
 #include <unordered_map>
 #include <vector>
 
@@ -112,6 +115,170 @@ bool launch_shape_ok(uint32_t gx, uint32_t gy, uint32_t gz, uint32_t bx, uint32_
     if (uint64_t(gy) * by > 0xFFFFFFFFull) return false;
     if (uint64_t(gz) * bz > 0xFFFFFFFFull) return false;
     return true;
+}
+
+// ---------------------------------------------------------------------------
+// Host memory.  Pinned (page-locked) blocks handed out by appy_hip_host_alloc
+// are remembered by address range: a copy whose host side lies inside one is a
+// single DMA at link speed.  Any other host pointer is pageable memory: the
+// driver's own path for it moves 17-30 GB/s, so large pageable copies go
+// through the staging engine below instead.
+// ---------------------------------------------------------------------------
+struct HostBlocks {
+    std::mutex mu;
+    std::map<uintptr_t, size_t> ranges;   // base -> bytes
+    bool contains(const void* p, size_t n) {
+        std::lock_guard<std::mutex> g(mu);
+        const uintptr_t a = reinterpret_cast<uintptr_t>(p);
+        auto it = ranges.upper_bound(a);
+        if (it == ranges.begin()) return false;
+        --it;
+        return a >= it->first && a + n <= it->first + it->second;
+    }
+};
+
+HostBlocks& host_blocks() {
+    static HostBlocks* h = new HostBlocks();
+    return *h;
+}
+
+// Staging engine for pageable host memory: the buffer is cut into kLanes
+// contiguous slices; one host thread per slice copies its slice through a ring
+// of two pinned chunks of its own, on a stream of its own, so that the memcpy of
+// chunk k+1 overlaps the DMA of chunk k and the slices overlap each other.  Four
+// lanes of 8 MiB chunks reach the link rate measured for pinned memory
+// (53 of 57 GB/s in both directions on MI355X; one lane gives 28 GB/s).
+constexpr int kLanes = 4;
+constexpr int kRing = 2;
+constexpr size_t kChunk = size_t(8) << 20;
+constexpr size_t kStagedMin = size_t(16) << 20;   // below this the plain copy is as fast
+
+struct StageLane {
+    char* pinned[kRing] = {nullptr, nullptr};
+    hipEvent_t done[kRing] = {nullptr, nullptr};
+    hipStream_t stream = nullptr;
+};
+
+struct Stager {
+    std::mutex mu;            // one staged copy at a time per device
+    bool ready = false;
+    bool broken = false;      // pinned memory could not be had: use the plain path
+    StageLane lanes[kLanes];
+};
+
+Stager& stager(int device) {
+    static std::mutex mu;
+    static std::map<int, Stager*>* all = new std::map<int, Stager*>();
+    std::lock_guard<std::mutex> g(mu);
+    auto it = all->find(device);
+    if (it == all->end()) it = all->emplace(device, new Stager()).first;
+    return *it->second;
+}
+
+hipError_t stager_prepare(Stager& st) {
+    if (st.ready) return hipSuccess;
+    for (auto& lane : st.lanes) {
+        hipError_t e = hipStreamCreateWithFlags(&lane.stream, hipStreamNonBlocking);
+        if (e != hipSuccess) return e;
+        for (int r = 0; r < kRing; ++r) {
+            e = hipHostMalloc(reinterpret_cast<void**>(&lane.pinned[r]), kChunk, hipHostMallocDefault);
+            if (e != hipSuccess) return e;
+            e = hipEventCreateWithFlags(&lane.done[r], hipEventDisableTiming);
+            if (e != hipSuccess) return e;
+        }
+    }
+    st.ready = true;
+    return hipSuccess;
+}
+
+// One lane's share of a staged copy.  to_device: host -> pinned -> device;
+// otherwise device -> pinned -> host, the host memcpy trailing the DMA by one slot.
+hipError_t stage_slice(StageLane& lane, int device, char* dev, char* host, size_t n, bool to_device) {
+    hipError_t e = hipSetDevice(device);
+    if (e != hipSuccess) return e;
+    size_t pend_off[kRing] = {0, 0}, pend_len[kRing] = {0, 0};
+    size_t off = 0;
+    for (int i = 0; off < n; ++i) {
+        const int r = i % kRing;
+        const size_t m = std::min(kChunk, n - off);
+        if (i >= kRing) {
+            if ((e = hipEventSynchronize(lane.done[r])) != hipSuccess) return e;
+            if (!to_device) std::memcpy(host + pend_off[r], lane.pinned[r], pend_len[r]);
+        }
+        if (to_device) {
+            std::memcpy(lane.pinned[r], host + off, m);
+            e = hipMemcpyAsync(dev + off, lane.pinned[r], m, hipMemcpyHostToDevice, lane.stream);
+        } else {
+            e = hipMemcpyAsync(lane.pinned[r], dev + off, m, hipMemcpyDeviceToHost, lane.stream);
+        }
+        if (e != hipSuccess) return e;
+        if ((e = hipEventRecord(lane.done[r], lane.stream)) != hipSuccess) return e;
+        pend_off[r] = off;
+        pend_len[r] = m;
+        off += m;
+    }
+    if ((e = hipStreamSynchronize(lane.stream)) != hipSuccess) return e;
+    if (!to_device) {
+        // the last (up to kRing) chunks are still in the ring
+        const size_t chunks = (n + kChunk - 1) / kChunk;
+        const size_t first = chunks > size_t(kRing) ? chunks - kRing : 0;
+        for (size_t c = first; c < chunks; ++c) {
+            const int r = int(c % kRing);
+            std::memcpy(host + pend_off[r], lane.pinned[r], pend_len[r]);
+        }
+    }
+    return hipSuccess;
+}
+
+// Returns hipErrorNotSupported when the staged path is not available (the caller
+// then uses the plain copy).
+hipError_t staged_copy(void* dev, void* host, size_t n, bool to_device, hipStream_t order_after) {
+    int device = 0;
+    hipError_t e = hipGetDevice(&device);
+    if (e != hipSuccess) return e;
+    Stager& st = stager(device);
+    std::lock_guard<std::mutex> g(st.mu);
+    if (st.broken) return hipErrorNotSupported;
+    if ((e = stager_prepare(st)) != hipSuccess) {
+        st.broken = true;
+        (void)hipGetLastError();
+        return hipErrorNotSupported;
+    }
+    // work already queued on the caller's stream (the kernel whose results are
+    // fetched, or earlier users of the destination) comes first
+    if ((e = hipStreamSynchronize(order_after)) != hipSuccess) return e;
+    size_t per = (n + kLanes - 1) / kLanes;
+    per = (per + 4095) & ~size_t(4095);
+    hipError_t results[kLanes];
+    std::thread workers[kLanes];
+    int used = 0;
+    for (int t = 0; t < kLanes; ++t) {
+        results[t] = hipSuccess;
+        const size_t o = per * size_t(t);
+        if (o >= n) break;
+        const size_t m = std::min(per, n - o);
+        char* d = static_cast<char*>(dev) + o;
+        char* h = static_cast<char*>(host) + o;
+        StageLane* lane = &st.lanes[t];
+        hipError_t* out = &results[t];
+        if (t == 0) continue;   // the calling thread takes the first slice itself, below
+        workers[t] = std::thread([=] { *out = stage_slice(*lane, device, d, h, m, to_device); });
+        used = t;
+    }
+    results[0] = stage_slice(st.lanes[0], device, static_cast<char*>(dev), static_cast<char*>(host),
+                             std::min(per, n), to_device);
+    for (int t = 1; t <= used; ++t) workers[t].join();
+    for (int t = 0; t < kLanes; ++t)
+        if (results[t] != hipSuccess) return results[t];
+    return hipSuccess;
+}
+
+bool staging_enabled() {
+    static const bool on = [] {
+        const char* s = std::getenv("APPY_HIP_NO_STAGING");
+        return !(s && s[0] == '1');
+    }();
+    return on;
 }
 
 }  // namespace
@@ -365,6 +532,11 @@ int appy_hip_memcpy_h2d(void* dst_dev, const void* src_host, size_t nbytes, void
     if (nbytes == 0) return 0;
     if (!dst_dev || !src_host) return fail_arg("dst_dev/src_host is NULL");
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (nbytes >= kStagedMin && staging_enabled() && !host_blocks().contains(src_host, nbytes)) {
+        hipError_t e = staged_copy(dst_dev, const_cast<void*>(src_host), nbytes, true, s);
+        if (e == hipSuccess) return 0;
+        if (e != hipErrorNotSupported) return fail_hip(e, "staged host-to-device copy");
+    }
     HIP_TRY(hipMemcpyAsync(dst_dev, src_host, nbytes, hipMemcpyHostToDevice, s));
     HIP_TRY(hipStreamSynchronize(s));
     return 0;
@@ -374,9 +546,43 @@ int appy_hip_memcpy_d2h(void* dst_host, const void* src_dev, size_t nbytes, void
     if (nbytes == 0) return 0;
     if (!dst_host || !src_dev) return fail_arg("dst_host/src_dev is NULL");
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (nbytes >= kStagedMin && staging_enabled() && !host_blocks().contains(dst_host, nbytes)) {
+        hipError_t e = staged_copy(const_cast<void*>(src_dev), dst_host, nbytes, false, s);
+        if (e == hipSuccess) return 0;
+        if (e != hipErrorNotSupported) return fail_hip(e, "staged device-to-host copy");
+    }
     HIP_TRY(hipMemcpyAsync(dst_host, src_dev, nbytes, hipMemcpyDeviceToHost, s));
     HIP_TRY(hipStreamSynchronize(s));
     return 0;
+}
+
+int appy_hip_host_alloc(size_t nbytes, void** out) {
+    if (!out) return fail_arg("out is NULL");
+    *out = nullptr;
+    void* p = nullptr;
+    HIP_TRY(hipHostMalloc(&p, nbytes ? nbytes : 1, hipHostMallocDefault));
+    {
+        std::lock_guard<std::mutex> g(host_blocks().mu);
+        host_blocks().ranges[reinterpret_cast<uintptr_t>(p)] = nbytes ? nbytes : 1;
+    }
+    *out = p;
+    return 0;
+}
+
+int appy_hip_host_free(void* p) {
+    if (!p) return 0;
+    {
+        std::lock_guard<std::mutex> g(host_blocks().mu);
+        auto it = host_blocks().ranges.find(reinterpret_cast<uintptr_t>(p));
+        if (it == host_blocks().ranges.end()) return fail_arg("pointer was not returned by appy_hip_host_alloc");
+        host_blocks().ranges.erase(it);
+    }
+    HIP_TRY(hipHostFree(p));
+    return 0;
+}
+
+int appy_hip_host_is_pinned(const void* p, size_t nbytes) {
+    return host_blocks().contains(p, nbytes) ? 1 : 0;
 }
 
 int appy_hip_memcpy_d2d_async(void* dst_dev, const void* src_dev, size_t nbytes, void* stream) {

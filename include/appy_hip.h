@@ -97,9 +97,21 @@ int appy_hip_malloc(size_t nbytes, void** dptr_out);
 int appy_hip_free(void* dptr);
 int appy_hip_pool_trim(void);
 int appy_hip_pool_stats(uint64_t* bytes_in_use_out, uint64_t* bytes_cached_out);
-/* Stream-ordered copies; both return after the copy has completed. */
+/* Stream-ordered copies; both return after the copy has completed.  Host
+ * memory from appy_hip_host_alloc moves as one DMA; any other (pageable) host
+ * memory of 16 MiB or more is moved by four host threads through pinned staging
+ * chunks on streams of their own, after the work queued on `stream` has
+ * finished (set APPY_HIP_NO_STAGING=1 to use the driver's pageable path). */
 int appy_hip_memcpy_h2d(void* dst_dev, const void* src_host, size_t nbytes, void* stream);
 int appy_hip_memcpy_d2h(void* dst_host, const void* src_dev, size_t nbytes, void* stream);
+/* Page-locked host memory for arrays that travel often.  Replaces the device-
+ * visible buffers behind the reference's shared NumPy arrays
+ * (`device.buffer(n)` + `np.frombuffer`, appy/np_shared.py:11-17): on a
+ * discrete GPU the array lives in pinned host memory and is mirrored in HBM.
+ * appy_hip_host_is_pinned returns 1 if [p, p+nbytes) lies inside such a block. */
+int appy_hip_host_alloc(size_t nbytes, void** host_out);
+int appy_hip_host_free(void* host_ptr);
+int appy_hip_host_is_pinned(const void* p, size_t nbytes);
 int appy_hip_memcpy_d2d_async(void* dst_dev, const void* src_dev, size_t nbytes, void* stream);
 int appy_hip_memset_async(void* dst_dev, int byte_value, size_t nbytes, void* stream);
 

@@ -260,3 +260,28 @@ def test_few_very_long_csr_rows_get_a_workgroup_each():
     sp = g.choose_spec(37, {}, arrays)
     assert (sp.width, sp.block) == (1024, 1024)
 
+
+
+def test_while_break_continue_become_c_loops():
+    src = (
+        "#pragma parallel for\n"
+        "for i in range(0, n, 1):\n"
+        "    k = 0\n"
+        "    while k < 10 and a[i] > 0.0:\n"
+        "        k += 1\n"
+        "        if k == 3:\n"
+        "            continue\n"
+        "        if k > 7:\n"
+        "            break\n"
+        "    out[i] = k\n"
+    )
+    a = np.zeros(8, np.float32)
+    out = np.zeros(8, np.int64)
+    f, code = compiled(src, n=8, a=a, out=out)
+    k = body_of(f.kernel_for(f.choose_spec(8, {"n": 8}, {"a": a, "out": out})).src.text)
+    assert "while (true) {" in k and "if (!(" in k and "continue;" in k and "break;" in k
+
+    # the iterations of a parallel loop are dealt to lanes: it has no C loop to leave
+    bad = "#pragma parallel for\nfor i in range(0, n, 1):\n    if a[i] > 0.0:\n        continue\n    out[i] = 1\n"
+    with pytest.raises(NotImplementedError, match="break"):
+        compiled(bad, n=8, a=a, out=out)
