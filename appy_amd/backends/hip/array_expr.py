@@ -16,8 +16,9 @@ from NumPy's slice semantics:
     t = g(np.sum(E))
         ->  r = 0;  for c in range(0, n): r = r + E[c];  t = g(r)
 
-Slice bounds that are omitted come from the array's shape; the extent is the
-one of the assignment target (for reductions: of the first sliced operand).
+Slice bounds that are omitted come from the array's shape, literal negative
+bounds count from its end; the extent is the one of the assignment target (for
+reductions: of the first sliced operand).
 """
 from __future__ import annotations
 
@@ -83,7 +84,26 @@ def _bounds(sub: ast.Subscript, dim: int, sl: ast.Slice, ctx: _Ctx):
         raise RuntimeError(f"Only arrays defined outside of parallel region can be sliced: {ast.unparse(sub)}")
     lo = sl.lower if sl.lower is not None else ast.Constant(value=0)
     hi = sl.upper if sl.upper is not None else ctx.shape_name(sub.value.id, dim)
-    return lo, hi
+    return _from_end(lo, sub, dim, ctx), _from_end(hi, sub, dim, ctx)
+
+
+def _negative_literal(node):
+    """k for the literal ``-k`` (k > 0), else None."""
+    if isinstance(node, ast.UnaryOp) and isinstance(node.op, ast.USub) and isinstance(node.operand, ast.Constant) \
+            and type(node.operand.value) is int and node.operand.value > 0:
+        return node.operand.value
+    if isinstance(node, ast.Constant) and type(node.value) is int and node.value < 0:
+        return -node.value
+    return None
+
+
+def _from_end(bound, sub: ast.Subscript, dim: int, ctx: _Ctx):
+    """A literal negative slice bound counts from the end of the dimension
+    (``A[i, 1:-1]``); bounds computed at run time are taken as they are."""
+    k = _negative_literal(bound)
+    if k is None:
+        return bound
+    return ast.BinOp(left=ctx.shape_name(sub.value.id, dim), op=ast.Sub(), right=ast.Constant(value=k))
 
 
 def _extent(lo, hi):

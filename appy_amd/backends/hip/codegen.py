@@ -18,6 +18,7 @@ from __future__ import annotations
 
 import ast
 import ctypes as C
+import dataclasses
 import hashlib
 import math
 import os
@@ -521,6 +522,13 @@ class Launch:
         # -- kernel variant, argument block, grid
         n_outer = hi - lo
         spec = loop.choose_spec(n_outer, env, arrays, restrict=restrict)
+        if spec.kind == "flat" and spec.hoist_guarded and a.guarded_checks:
+            # loads the program guards with a condition may only be issued early when
+            # they cannot leave their array anywhere in the range
+            for name, dim, off in a.guarded_checks:
+                if lo + off < 0 or hi - 1 + off >= arrays[name].shape[dim]:
+                    spec = dataclasses.replace(spec, hoist_guarded=False)
+                    break
         self.kernel = loop.kernel_for(spec)
         self.spec = spec
         st = self.kernel.ArgStruct()

@@ -62,6 +62,8 @@ class Spec:
     extent: int = 0      # compile-time extent of row accumulators (team only; 0 = none)
     stream_stores: bool = False  # non-temporal vector stores
     lds_tile: int = 0    # elements of a row-invariant operand staged in LDS per step (team only; 0 = off)
+    hoist_guarded: bool = True   # flat only: loads the source guards with a condition may be issued
+                                 # unconditionally (the host has checked that they stay inside their arrays)
 
     def __post_init__(self):
         def pow2(n):
@@ -84,7 +86,7 @@ class Spec:
         return (f"{self.kind}_b{self.block}_v{self.vec}_u{self.unroll}_w{self.width}"
                 f"{'_r' if self.restrict else ''}{'_nt' if self.stream_loads else ''}"
                 f"{'_e' + str(self.extent) if self.extent else ''}{'_nts' if self.stream_stores else ''}"
-                f"{'_lds' + str(self.lds_tile) if self.lds_tile else ''}")
+                f"{'_lds' + str(self.lds_tile) if self.lds_tile else ''}{'' if self.hoist_guarded else '_g'}")
 
 
 @dataclass
@@ -143,6 +145,46 @@ def _var_offset(node, var: str):
                 and isinstance(l, ast.Constant) and type(l.value) is int):
             return l.value
     return None
+
+
+def guarded_nodes(stmts) -> set:
+    """ids of the subscripts that the program evaluates only under a condition:
+    in the arms of ``a if c else b``, after the first operand of ``and`` / ``or``
+    and of a comparison chain, in the bodies of ``if`` / ``while`` statements and
+    of nested loops (which may run zero times).  Such an access may lie outside
+    its array when the condition is false (``u[i - 1] if i > 0 else 0.0``), so it
+    must not be executed early."""
+    out = set()
+
+    def mark(node):
+        for n in ast.walk(node):
+            if isinstance(n, ast.Subscript):
+                out.add(id(n))
+
+    def visit(node):
+        if isinstance(node, ast.IfExp):
+            mark(node.body)
+            mark(node.orelse)
+        elif isinstance(node, ast.BoolOp):
+            for v in node.values[1:]:
+                mark(v)
+        elif isinstance(node, ast.Compare) and len(node.comparators) > 1:
+            for v in node.comparators[1:]:
+                mark(v)
+        elif isinstance(node, (ast.If, ast.While)):
+            for st in node.body + node.orelse:
+                mark(st)
+            if isinstance(node, ast.While):
+                mark(node.test)
+        elif isinstance(node, ast.For):
+            for st in node.body:
+                mark(st)
+        for child in ast.iter_child_nodes(node):
+            visit(child)
+
+    for st in stmts:
+        visit(st)
+    return out
 
 
 def _has_simd_loop(stmts) -> bool:
@@ -215,13 +257,20 @@ class LoopAnalysis:
 
         # accesses indexed directly by the parallel loop variable: checked on
         # the host against the array extents before every launch
+        # Accesses under a condition of the program are not checked (the condition is
+        # their guard); those a flat kernel may want to load early are listed apart, and
+        # the host picks the variant that leaves them in place when they could leave
+        # their array.
         self.bound_checks = []
+        self.guarded_checks = []
+        guarded = guarded_nodes(self.outer.body)
         for n in ast.walk(self.outer):
             if isinstance(n, ast.Subscript) and isinstance(n.value, ast.Name) and n.value.id in self.arrays:
+                into = self.guarded_checks if id(n) in guarded else self.bound_checks
                 for d, e in enumerate(_elts(n)):
                     off = _var_offset(e, self.var)
-                    if off is not None and (n.value.id, d, off) not in self.bound_checks:
-                        self.bound_checks.append((n.value.id, d, off))
+                    if off is not None and (n.value.id, d, off) not in into:
+                        into.append((n.value.id, d, off))
 
 
 class KernelBuilder:
@@ -400,12 +449,16 @@ class KernelBuilder:
         self.ind -= 1
         self.w("}")
 
-    def _vector_accesses(self, body, var: str):
+    def _vector_accesses(self, body, var: str, hoist_guarded: bool = False):
         """Loads ``X[.., var+c]`` (any depth) and unconditional top-level
         stores ``X[.., var+c] = e`` of a loop body that can move V elements at
-        once.  Returns (loads, stores): lists of (key, array, subscript)."""
+        once.  Returns (loads, stores): lists of (key, array, subscript).  Loads
+        the program guards with a condition are only taken when the caller
+        knows them to be in bounds (``hoist_guarded``)."""
         loads, stores = {}, {}
         blocked = set()
+        guarded = set() if hoist_guarded else guarded_nodes(body)
+        in_place = {}           # guarded loads that stay where the program has them: key -> array
         inner_vars = {n.target.id for s in body for n in ast.walk(s) if isinstance(n, ast.For)}
         for s in body:
             for n in ast.walk(s):
@@ -424,7 +477,9 @@ class KernelBuilder:
                 ok = ok and not any(_uses_name(e, v) for e in el[:-1] for v in self._assigned_in(body))
                 key = ast.unparse(n)
                 if isinstance(n.ctx, ast.Load):
-                    if ok:
+                    if id(n) in guarded:
+                        in_place[key] = arr
+                    elif ok:
                         loads[key] = (arr, n)
                 else:
                     top = any(isinstance(t, ast.Assign) and t.targets[0] is n for t in body)
@@ -439,7 +494,8 @@ class KernelBuilder:
             del stores[key]
         # a vector store to an array that is also read at another offset would reorder accesses
         for key, (arr, _) in list(stores.items()):
-            if any(a2.name == arr.name and k2 != key for k2, (a2, _) in loads.items()):
+            if (any(a2.name == arr.name and k2 != key for k2, (a2, _) in loads.items())
+                    or any(a2.name == arr.name and k2 != key for k2, a2 in in_place.items())):
                 del stores[key]
                 loads = {k: v for k, v in loads.items() if v[0].name != arr.name}
         return loads, stores
@@ -754,7 +810,7 @@ class KernelBuilder:
         V, U, B = s.vec, s.unroll, s.block
         var = self.a.var
         self.ex.locals[var] = T.WEAK_INT
-        loads, stores = self._vector_accesses(self.a.outer.body, var) if V > 1 else ({}, {})
+        loads, stores = self._vector_accesses(self.a.outer.body, var, s.hoist_guarded) if V > 1 else ({}, {})
         vectorised = V > 1 and (loads or stores)
         self.lane_step_bytes = sum(V * arr.ty.size for arr, _ in list(loads.values()) + list(stores.values()))
         self.w("const appy::i64 __tid = threadIdx.x;")
@@ -854,9 +910,11 @@ class KernelBuilder:
                 continue
             j = st.target.id
             found = {}
+            guarded = guarded_nodes(st.body)
             for n in ast.walk(st):
                 if (isinstance(n, ast.Subscript) and isinstance(n.value, ast.Name) and n.value.id in self.a.arrays
-                        and isinstance(n.ctx, ast.Load) and isinstance(n.slice, ast.Name) and n.slice.id == j):
+                        and isinstance(n.ctx, ast.Load) and isinstance(n.slice, ast.Name) and n.slice.id == j
+                        and id(n) not in guarded):
                     arr = self.a.arrays[n.value.id]
                     if arr.ndim == 1 and arr.name not in self.a.stored and not arr.ty.is_bool:
                         found[arr.name] = arr

@@ -285,3 +285,28 @@ def test_while_break_continue_become_c_loops():
     bad = "#pragma parallel for\nfor i in range(0, n, 1):\n    if a[i] > 0.0:\n        continue\n    out[i] = 1\n"
     with pytest.raises(NotImplementedError, match="break"):
         compiled(bad, n=8, a=a, out=out)
+
+
+def test_guarded_loads_are_hoisted_only_when_the_host_can_vouch_for_them():
+    from appy_amd.backends.hip.kernelgen import guarded_nodes
+    import ast
+    import dataclasses
+
+    src = ("#pragma parallel for simd\nfor i in range(0, n, 1):\n"
+           "    y[i] = (x[i - 1] if i > 0 else 0.0) + x[i] + (m[i] and x[i + 1] > 0.0)\n")
+    x = np.zeros(64)
+    m = np.zeros(64, bool)
+    f, _ = compiled(src, n=64, x=x, y=x.copy(), m=m)
+    assert ("x", 0, 0) in f.analysis.bound_checks and ("m", 0, 0) in f.analysis.bound_checks
+    assert ("x", 0, -1) in f.analysis.guarded_checks and ("x", 0, 1) in f.analysis.guarded_checks
+    assert ("x", 0, -1) not in f.analysis.bound_checks
+    sp = f.default_spec
+    fast = body_of(f.kernel_for(sp).src.text)
+    safe = body_of(f.kernel_for(dataclasses.replace(sp, hoist_guarded=False)).src.text)
+    assert fast.count("appy::vload<double") > safe.count("appy::vload<double") >= 1
+    assert "x[(i - 1LL)]" in safe and "x[(i - 1LL)]" not in fast.split("__rest0")[0]
+    assert dataclasses.replace(sp, hoist_guarded=False).tag().endswith("_g")
+
+    tree = ast.parse("a[0] if c[1] else b[2]\nfor k in r:\n    d[3]\nwhile e[4]:\n    pass\nif g[5]:\n    h[6]\nz = p[7] and q[8]")
+    names = {n.value.id for n in ast.walk(tree) if isinstance(n, ast.Subscript) and id(n) in guarded_nodes(tree.body)}
+    assert names == {"a", "b", "d", "e", "h", "q"}

@@ -1,0 +1,203 @@
+"""Array statements inside parallel loops on the GPU: the slice forms of the
+reference's Metal NPBench tests (tests/integration/metal/npbench/test_gemver.py,
+test_symm.py, test_gramschmidt.py, test_fdtd_2d.py, test_floyd_warshall.py,
+test_jacobi_2d.py, test_syr2k.py, test_jacobi_1d.py): whole-row and column
+slices, slices with negative and open bounds, ``@`` of two slices, ``np.minimum``
+of slices, in-place column updates.  The expected values are the same statements
+executed by NumPy (the un-jitted function) on the same inputs."""
+import numpy as np
+import pytest
+
+import appy
+
+pytestmark = pytest.mark.gpu
+
+
+def both(fn, *args):
+    """Run ``fn`` jitted and un-jitted on copies of the arguments."""
+    cp = lambda a: a.copy() if isinstance(a, np.ndarray) else a
+    got = appy.jit(fn)(*[cp(a) for a in args])
+    ref = fn(*[cp(a) for a in args])
+    return got, ref
+
+
+def close(got, ref, **kw):
+    if isinstance(ref, tuple):
+        return all(np.allclose(g, r, **kw) for g, r in zip(got, ref))
+    return np.allclose(got, ref, **kw)
+
+
+def gemver(alpha, beta, A, u1, u2, v1, v2, w, x, yv, z):
+    M, N = A.shape
+    #pragma parallel for
+    for i in range(M):
+        A[i, :] += u1[i] * v1[:] + u2[i] * v2[:]
+    #pragma parallel for
+    for j in range(N):
+        x[j] += beta * (yv[:] @ A[:, j]) + z[j]
+    #pragma parallel for
+    for i in range(M):
+        w[i] += alpha * (A[i, :] @ x[:])
+    return A, x, w
+
+
+def test_gemver_row_updates_and_dots_of_slices(gpu):
+    rng = np.random.default_rng(0)
+    n = 150
+    A = rng.random((n, n))
+    vecs = [rng.random(n) for _ in range(8)]
+    got, ref = both(gemver, 1.5, 1.2, A, *vecs)
+    assert close(got, ref, atol=1e-6)
+
+
+def symm(alpha, beta, C, A, B):
+    temp2 = np.empty((C.shape[1],), dtype=C.dtype)
+    C *= beta
+    for i in range(C.shape[0]):
+        #pragma parallel for
+        for j in range(C.shape[1]):
+            C[:i, j] += alpha * B[i, j] * A[i, :i]
+            temp2[j] = B[:i, j] @ A[i, :i]
+        C[i, :] += alpha * B[i, :] * A[i, i] + alpha * temp2
+    return C
+
+
+def test_symm_column_slices(gpu):
+    rng = np.random.default_rng(1)
+    m, n = 40, 50
+    got, ref = both(symm, 1.5, 1.2, rng.random((m, n)), rng.random((m, m)), rng.random((m, n)))
+    assert close(got, ref, atol=1e-6)
+
+
+def gramschmidt(A):
+    M, N = A.shape
+    Q = np.zeros((M, N), dtype=A.dtype)
+    R = np.zeros((N, N), dtype=A.dtype)
+    for k in range(N):
+        nrm = A[:, k] @ A[:, k]
+        R[k, k] = np.sqrt(nrm)
+        Q[:, k] = A[:, k] / R[k, k]
+        #pragma parallel for
+        for j in range(k + 1, N):
+            s = Q[:, k] @ A[:, j]
+            R[k, j] = s
+            A[:, j] -= Q[:, k] * s
+    return Q, R
+
+
+def test_gramschmidt_column_dot_and_update(gpu):
+    rng = np.random.default_rng(2)
+    A = rng.random((60, 40)) + np.eye(60, 40)
+    (Q, R), (Qr, Rr) = both(gramschmidt, A)
+    assert np.allclose(Q, Qr, atol=1e-6) and np.allclose(R, Rr, atol=1e-6)
+    assert np.allclose(Q @ R, A, atol=1e-8)
+
+
+def fdtd_2d(TMAX, ex, ey, hz, _fict_):
+    for t in range(TMAX):
+        ey[0, :] = _fict_[t]
+        #pragma parallel for
+        for i in range(1, ey.shape[0]):
+            ey[i, :] -= 0.5 * (hz[i, :] - hz[i - 1, :])
+        #pragma parallel for
+        for i in range(ex.shape[0]):
+            ex[i, 1:] -= 0.5 * (hz[i, 1:] - hz[i, :-1])
+        #pragma parallel for
+        for i in range(hz.shape[0] - 1):
+            hz[i, :-1] -= 0.7 * (ex[i, 1:] - ex[i, :-1] + ey[i + 1, :-1] -
+                                  ey[i, :-1])
+    return ey, ex, hz
+
+
+def test_fdtd_2d_shifted_slices(gpu):
+    rng = np.random.default_rng(3)
+    nx, ny, tmax = 70, 90, 8
+    got, ref = both(fdtd_2d, tmax, rng.random((nx, ny)), rng.random((nx, ny)), rng.random((nx, ny)),
+                    np.arange(tmax, dtype=np.float64))
+    assert close(got, ref, atol=1e-6)
+
+
+def floyd_warshall(path):
+    for k in range(path.shape[0]):
+        #pragma parallel for
+        for i in range(path.shape[0]):
+            path[i, :] = np.minimum(path[i, :], path[i, k] + path[k, :])
+    return path
+
+
+def test_floyd_warshall_np_minimum_of_slices(gpu):
+    rng = np.random.default_rng(4)
+    n = 64
+    path = rng.integers(1, 100, (n, n)).astype(np.int32)
+    got, ref = both(floyd_warshall, path)
+    assert np.array_equal(got, ref)
+
+
+def jacobi_2d(TSTEPS, A, B):
+    for t in range(1, TSTEPS):
+        #pragma parallel for
+        for i in range(1, A.shape[0] - 1):
+            B[i, 1:-1] = 0.2 * (A[i, 1:-1] + A[i, :-2] + A[i, 2:] +
+                                 A[i - 1, 1:-1] + A[i + 1, 1:-1])
+        #pragma parallel for
+        for i in range(1, B.shape[0] - 1):
+            A[i, 1:-1] = 0.2 * (B[i, 1:-1] + B[i, :-2] + B[i, 2:] +
+                                 B[i - 1, 1:-1] + B[i + 1, 1:-1])
+    return A, B
+
+
+def test_jacobi_2d_interior_slices(gpu):
+    rng = np.random.default_rng(5)
+    got, ref = both(jacobi_2d, 6, rng.random((80, 80)), rng.random((80, 80)))
+    assert close(got, ref, atol=1e-8)
+
+
+def syr2k(alpha, beta, C, A, B):
+    #pragma parallel for
+    for i in range(A.shape[0]):
+        C[i, :i + 1] *= beta
+        for k in range(A.shape[1]):
+            C[i, :i + 1] += (A[:i + 1, k] * alpha * B[i, k] +
+                             B[:i + 1, k] * alpha * A[i, k])
+    return C
+
+
+def syr2k_loops(alpha, beta, C, A, B):
+    #pragma parallel for
+    for i in range(A.shape[0]):
+        #pragma simd
+        for j in range(i + 1):
+            C[i, j] *= beta
+        for k in range(A.shape[1]):
+            #pragma simd
+            for j in range(i + 1):
+                C[i, j] += (A[j, k] * alpha * B[i, k] +
+                            B[j, k] * alpha * A[i, k])
+    return C
+
+
+def test_syr2k_triangular_slices_and_loops(gpu):
+    rng = np.random.default_rng(6)
+    n, m = 60, 45
+    C, A, B = rng.random((n, n)), rng.random((n, m)), rng.random((n, m))
+    got, ref = both(syr2k, 1.5, 1.2, C, A, B)
+    assert close(got, ref, atol=1e-6)
+    got2 = appy.jit(syr2k_loops)(1.5, 1.2, C.copy(), A, B)
+    assert close(got2, ref, atol=1e-6)
+
+
+def jacobi_1d(TSTEPS, A, B):
+    for t in range(1, TSTEPS):
+        #pragma parallel for simd
+        for i in range(1, A.shape[0] - 1):
+            B[i] = 0.33333 * (A[i - 1] + A[i] + A[i + 1])
+        #pragma parallel for simd
+        for i in range(1, A.shape[0] - 1):
+            A[i] = 0.33333 * (B[i - 1] + B[i] + B[i + 1])
+    return A, B
+
+
+def test_jacobi_1d(gpu):
+    rng = np.random.default_rng(7)
+    got, ref = both(jacobi_1d, 10, rng.random(4001), rng.random(4001))
+    assert close(got, ref, atol=0)

@@ -200,3 +200,53 @@ def test_shared_reductions_in_team_loops(rng):
     assert sum_of_row_maxima(a) == pytest.approx(a.max(axis=1).sum(), rel=1e-12)
     a32 = a.astype(np.float32)
     assert sum_2d(a32) == pytest.approx(float(a32.astype(np.float64).sum()), abs=1e-5 * float(np.abs(a32).sum()))
+
+
+def test_guarded_neighbour_accesses_stay_guarded(gpu):
+    """``x[i - 1] if i > 0 else 0.0``: the element before the array is never
+    touched, in flat and in team kernels (the reference's heat solver,
+    old-tests/codegen/triton/np_array/test_heat.py:60-76)."""
+    import appy_amd as appy
+
+    @appy.jit
+    def smooth(x, y):
+        #pragma parallel for simd
+        for i in range(x.shape[0]):
+            left = x[i - 1] if i > 0 else 0.0
+            right = x[i + 1] if i < x.shape[0] - 1 else 0.0
+            y[i] = 0.25 * left + 0.5 * x[i] + 0.25 * right
+
+    @appy.jit
+    def heat(n, alpha, dx, dt, u, u_tmp, nsteps):
+        r = alpha * dt / (dx * dx)
+        r2 = 1.0 - 4.0 * r
+        for _ in range(nsteps):
+            #pragma parallel for
+            for i in range(n):
+                #pragma simd
+                for j in range(n):
+                    center = u[i, j]
+                    left = u[i - 1, j] if i > 0 else 0.0
+                    right = u[i + 1, j] if i < n - 1 else 0.0
+                    down = u[i, j - 1] if j > 0 else 0.0
+                    up = u[i, j + 1] if j < n - 1 else 0.0
+                    u_tmp[i, j] = r2 * center + r * (left + right + down + up)
+            u, u_tmp = u_tmp, u
+        return u
+
+    rng = np.random.default_rng(21)
+    x = rng.standard_normal(100_003)
+    y = np.zeros_like(x)
+    smooth(x, y)
+    xp = np.concatenate([[0.0], x, [0.0]])
+    assert np.allclose(y, 0.25 * xp[:-2] + 0.5 * x + 0.25 * xp[2:], rtol=0, atol=1e-15)
+
+    n, nsteps = 37, 3
+    u0 = rng.random((n, n))
+    got = heat(n, 0.1, 0.5, 0.01, u0.copy(), np.zeros((n, n)), nsteps)
+    r = 0.1 * 0.01 / 0.25
+    ref = u0.copy()
+    for _ in range(nsteps):
+        p = np.pad(ref, 1)
+        ref = (1.0 - 4.0 * r) * ref + r * (p[:-2, 1:-1] + p[2:, 1:-1] + p[1:-1, :-2] + p[1:-1, 2:])
+    assert np.allclose(got, ref, rtol=1e-12, atol=1e-12)
