@@ -18,6 +18,7 @@ import textwrap
 __version__ = "0.1.0"  # of this package, not of the reference it is compatible with
 from . import dispatcher
 from .residency import invalidate, resident, sync_host  # noqa: F401 - part of the public interface
+from .graphs import graph  # noqa: F401
 from .frontend import source as _source
 from .frontend import static_rewrite as _static_rewrite
 

@@ -31,7 +31,7 @@ from ...frontend import loop_ir
 from . import array_expr
 from . import dtypes as T
 from . import runtime as rt
-from ... import residency
+from ... import graphs, residency
 from .exprs import ArrayParam, ScalarParam
 from .kernelgen import KernelBuilder, KernelSource, LoopAnalysis, Spec, Unsupported
 
@@ -484,6 +484,13 @@ class Launch:
 
             device = gpu_tensors[0].device.index or 0
             self.stream = torch.cuda.current_stream(device).cuda_stream
+        self.capture = graphs.current()
+        if self.capture is not None:
+            # the launch is recorded into the graph's stream, not executed
+            if device != self.capture.device:
+                raise RuntimeError(f"{loop.loop_name}: arguments live on device {device}, the graph being "
+                                   f"captured on device {self.capture.device}")
+            self.stream = self.capture.stream
         _ensure_device(device)
         self.device = device
 
@@ -501,6 +508,7 @@ class Launch:
             elif v.device.type == "cuda":
                 t = v
                 if t.ndim >= 1 and t.numel() > 1 and t.stride(-1) != 1:
+                    self._no_capture(name, "its last dimension is not contiguous (it would be repacked per launch)")
                     t = v.contiguous()
                     if arr.stored:
                         self.keepalive.append(("copy_back", v, t))
@@ -510,6 +518,7 @@ class Launch:
                 extents.append((name, t.data_ptr(), t.numel() * t.element_size(), arr.stored))
             else:
                 # CPU tensor: same path as NumPy through a shared-memory view
+                self._no_capture(name, "it is a CPU tensor (it would be copied per launch)")
                 tc = v if v.is_contiguous() else v.contiguous()
                 host = tc.numpy()
                 self._stage_host(name, host, v if tc is v else ("tensor", v, tc), arr.stored)
@@ -564,6 +573,10 @@ class Launch:
         if hit is not None:
             # the array (or the array this is a view of) has a standing mirror in HBM
             m, off = hit
+            if self.capture is not None and (not m.resident or m.host_dirty):
+                self._no_capture(name, "it is not resident on the device (use `with appy.resident(...)` around the "
+                                       "capture and the replays)" if not m.resident else
+                                       "its host copy has changed (appy.invalidate) and would be uploaded per launch")
             if m.resident:
                 if m.host_dirty:
                     m.upload(self.stream)
@@ -574,6 +587,8 @@ class Launch:
             self.ptr[name] = dptr
             self.strides[name] = [s // host.itemsize for s in host.strides]
             return
+        self._no_capture(name, "it is a host array that would be copied per launch (use GPU tensors, or NumPy "
+                               "arrays inside `with appy.resident(...)`; `shared()` scalars cannot be captured)")
         dptr = rt.malloc(max(nbytes, 1))
         if nbytes:
             rt.memcpy_h2d(dptr, host.ctypes.data, nbytes, self.stream)
@@ -581,11 +596,22 @@ class Launch:
         self.ptr[name] = dptr
         self.strides[name] = [s // host.itemsize for s in host.strides]
 
+    def _no_capture(self, name, why):
+        if self.capture is not None:
+            raise RuntimeError(f"{self.loop.loop_name} cannot be captured into a graph: argument `{name}`: {why}")
+
     def function(self):
         return self.kernel.function(self.device)
 
     def launch_only(self):
         rt.launch(self.function(), self.grid, self.block, self.args, self.stream)
+        g = self.capture
+        if g is not None:
+            g.launches += 1
+            g.keepalive.extend(self.keepalive)
+            for m, _dptr, _host, stored, _name in self.mirrored:
+                if stored and m not in g.stored_mirrors:
+                    g.stored_mirrors.append(m)
 
     def time_kernel(self, warmup=3, reps=20) -> float:
         """Mean milliseconds per launch (HIP events on the launch stream)."""

@@ -80,6 +80,12 @@ SIGNATURES = {
     "appy_hip_memset_async": (C.c_int, [_vp, C.c_int, C.c_size_t, _vp]),
     "appy_hip_launch": (C.c_int, [_vp, _u32, _u32, _u32, _u32, _u32, _u32, _u32, _vp, _vp, C.c_size_t]),
     "appy_hip_sync": (C.c_int, [_vp]),
+    "appy_hip_stream_create": (C.c_int, [C.POINTER(_vp)]),
+    "appy_hip_stream_destroy": (C.c_int, [_vp]),
+    "appy_hip_graph_begin": (C.c_int, [_vp]),
+    "appy_hip_graph_end": (C.c_int, [_vp, C.POINTER(_vp)]),
+    "appy_hip_graph_launch": (C.c_int, [_vp, _vp]),
+    "appy_hip_graph_destroy": (C.c_int, [_vp]),
     "appy_hip_event_create": (C.c_int, [C.POINTER(_vp)]),
     "appy_hip_event_record": (C.c_int, [_vp, _vp]),
     "appy_hip_event_sync": (C.c_int, [_vp]),
@@ -280,6 +286,34 @@ def launch_timed(func, grid, block, args_struct, stream: int = 0, dynamic_lds: i
 
 def sync(stream: int = 0) -> None:
     check(lib().appy_hip_sync(_vp(stream)))
+
+
+def stream_create() -> int:
+    out = _vp()
+    check(lib().appy_hip_stream_create(C.byref(out)))
+    return out.value
+
+
+def stream_destroy(stream: int) -> None:
+    check(lib().appy_hip_stream_destroy(_vp(stream)))
+
+
+def graph_begin(stream: int) -> None:
+    check(lib().appy_hip_graph_begin(_vp(stream)))
+
+
+def graph_end(stream: int) -> int:
+    out = _vp()
+    check(lib().appy_hip_graph_end(_vp(stream), C.byref(out)))
+    return out.value
+
+
+def graph_launch(graph_exec: int, stream: int) -> None:
+    check(lib().appy_hip_graph_launch(_vp(graph_exec), _vp(stream)))
+
+
+def graph_destroy(graph_exec: int) -> None:
+    check(lib().appy_hip_graph_destroy(_vp(graph_exec)))
 
 
 class Event:

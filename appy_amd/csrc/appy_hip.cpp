@@ -595,6 +595,13 @@ int appy_hip_memcpy_d2d_async(void* dst_dev, const void* src_dev, size_t nbytes,
 int appy_hip_memset_async(void* dst_dev, int byte_value, size_t nbytes, void* stream) {
     if (nbytes == 0) return 0;
     if (!dst_dev) return fail_arg("dst_dev is NULL");
+    if (stream) {
+        // memset nodes are kept out of graphs (replays of such nodes are not reliable
+        // on this platform): clear with a kernel inside a capture instead
+        hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+        HIP_TRY(hipStreamIsCapturing(static_cast<hipStream_t>(stream), &st));
+        if (st != hipStreamCaptureStatusNone) return fail_arg("memset on a stream that is being captured");
+    }
     HIP_TRY(hipMemsetAsync(dst_dev, byte_value, nbytes, static_cast<hipStream_t>(stream)));
     return 0;
 }
@@ -619,6 +626,56 @@ int appy_hip_launch(void* func,
 
 int appy_hip_sync(void* stream) {
     HIP_TRY(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+    return 0;
+}
+
+// ---- streams and graphs -------------------------------------------------------
+
+int appy_hip_stream_create(void** stream_out) {
+    if (!stream_out) return fail_arg("stream_out is NULL");
+    hipStream_t s = nullptr;
+    HIP_TRY(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));   // default priority
+    *stream_out = s;
+    return 0;
+}
+
+int appy_hip_stream_destroy(void* stream) {
+    if (!stream) return 0;
+    HIP_TRY(hipStreamDestroy(static_cast<hipStream_t>(stream)));
+    return 0;
+}
+
+int appy_hip_graph_begin(void* stream) {
+    if (!stream) return fail_arg("the null stream cannot be captured");
+    // Relaxed: code-object loads and pool growth triggered by the first launch of a
+    // kernel are legal while capturing; they are simply not part of the graph.
+    HIP_TRY(hipStreamBeginCapture(static_cast<hipStream_t>(stream), hipStreamCaptureModeRelaxed));
+    return 0;
+}
+
+int appy_hip_graph_end(void* stream, void** graph_exec_out) {
+    if (!stream || !graph_exec_out) return fail_arg("stream/graph_exec_out is NULL");
+    *graph_exec_out = nullptr;
+    hipGraph_t g = nullptr;
+    HIP_TRY(hipStreamEndCapture(static_cast<hipStream_t>(stream), &g));
+    if (!g) return fail_arg("the capture recorded nothing");
+    hipGraphExec_t ex = nullptr;
+    hipError_t e = hipGraphInstantiate(&ex, g, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(g);
+    if (e != hipSuccess) return fail_hip(e, "hipGraphInstantiate");
+    *graph_exec_out = ex;
+    return 0;
+}
+
+int appy_hip_graph_launch(void* graph_exec, void* stream) {
+    if (!graph_exec) return fail_arg("graph_exec is NULL");
+    HIP_TRY(hipGraphLaunch(static_cast<hipGraphExec_t>(graph_exec), static_cast<hipStream_t>(stream)));
+    return 0;
+}
+
+int appy_hip_graph_destroy(void* graph_exec) {
+    if (!graph_exec) return 0;
+    HIP_TRY(hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph_exec)));
     return 0;
 }
 

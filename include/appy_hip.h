@@ -127,6 +127,23 @@ int appy_hip_launch(void* func,
                     const void* args, size_t args_bytes);
 int appy_hip_sync(void* stream);               /* hipStreamSynchronize */
 
+/* ---- streams and graphs -----------------------------------------------------
+ * A loop nest that launches many short kernels (a time-stepping host loop
+ * around parallel loops, e.g. tests/integration/triton/npbench/test_jacobi_1d.py)
+ * is bound by the host's launch rate.  The launches can be recorded once into a
+ * HIP graph and replayed as one submission.  Nothing in the reference
+ * corresponds to this (its launches go through Triton one at a time,
+ * appy/backends/triton/passes/host_passes/gen_kernel_launch.py:27-66).
+ * Streams have the default priority.  Between graph_begin and graph_end only
+ * appy_hip_launch and appy_hip_memcpy_d2d_async may be issued on `stream`;
+ * appy_hip_memset_async is refused while a capture is active on the stream. */
+int appy_hip_stream_create(void** stream_out);
+int appy_hip_stream_destroy(void* stream);
+int appy_hip_graph_begin(void* stream);
+int appy_hip_graph_end(void* stream, void** graph_exec_out);
+int appy_hip_graph_launch(void* graph_exec, void* stream);
+int appy_hip_graph_destroy(void* graph_exec);
+
 /* ---- timing ---------------------------------------------------------------
  * Replaces torch.utils.benchmark.Timer in examples/benchmark_utils.py:4-15:
  * HIP events recorded on the stream the kernel is launched on. */
