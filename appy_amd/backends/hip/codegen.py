@@ -126,7 +126,7 @@ def _disk_cache_dir():
 
 def compile_source(text: str, name: str) -> bytes:
     """HIP C++ -> gfx950 code object, through hiprtc, with an on-disk cache
-    keyed on the source text and the compiler options."""
+    keyed on the source text, the compiler options and the compiler version."""
     d = _disk_cache_dir()
     path = None
     if d:
@@ -134,10 +134,13 @@ def compile_source(text: str, name: str) -> bytes:
         h.update(text.encode())
         h.update(repr(rt.BASE_COMPILE_OPTIONS).encode())
         h.update(ARCH.encode())
+        h.update(str(rt.rtc_version()).encode())
         path = os.path.join(d, h.hexdigest() + ".co")
         if os.path.exists(path):
             with open(path, "rb") as f:
-                return f.read()
+                code = f.read()
+            if code[:4] == b"\x7fELF":
+                return code
     code = rt.compile_to_code_object(text, name + ".hip", ARCH)
     if path:
         tmp = path + f".{os.getpid()}.tmp"

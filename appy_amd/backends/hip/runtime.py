@@ -80,6 +80,7 @@ SIGNATURES = {
     "appy_hip_memset_async": (C.c_int, [_vp, C.c_int, C.c_size_t, _vp]),
     "appy_hip_launch": (C.c_int, [_vp, _u32, _u32, _u32, _u32, _u32, _u32, _u32, _vp, _vp, C.c_size_t]),
     "appy_hip_sync": (C.c_int, [_vp]),
+    "appy_hip_rtc_version": (C.c_int, [C.POINTER(C.c_int)]),
     "appy_hip_stream_create": (C.c_int, [C.POINTER(_vp)]),
     "appy_hip_stream_destroy": (C.c_int, [_vp]),
     "appy_hip_graph_begin": (C.c_int, [_vp]),
@@ -188,6 +189,12 @@ def compile_to_code_object(source: str, name: str, arch: str = "gfx950", extra_o
         return C.string_at(code.value, size.value)
     finally:
         lib().appy_hip_code_free(code)
+
+
+def rtc_version() -> int:
+    out = C.c_int()
+    check(lib().appy_hip_rtc_version(C.byref(out)))
+    return out.value
 
 
 def compile_log() -> str:

@@ -388,6 +388,15 @@ int appy_hip_compile(const char* src, const char* name, const char* arch,
     return 0;
 }
 
+int appy_hip_rtc_version(int* version_out) {
+    if (!version_out) return fail_arg("version_out is NULL");
+    int major = 0, minor = 0;
+    hiprtcResult r = hiprtcVersion(&major, &minor);
+    if (r != HIPRTC_SUCCESS) return fail_rtc(r, "hiprtcVersion");
+    *version_out = major * 1000 + minor;
+    return 0;
+}
+
 const char* appy_hip_compile_log(void) { return g_compile_log.c_str(); }
 
 void appy_hip_code_free(void* code) { std::free(code); }

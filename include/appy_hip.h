@@ -76,6 +76,8 @@ int appy_hip_compile(const char* src, const char* name, const char* arch,
                      const char* const* opts, int nopts,
                      void** code_out, size_t* size_out);
 const char* appy_hip_compile_log(void);
+/* hiprtc's version as major * 1000 + minor (part of the key of code-object caches). */
+int appy_hip_rtc_version(int* version_out);
 void appy_hip_code_free(void* code);
 
 /* Load a code object on the current device / look up an extern "C" kernel. */
