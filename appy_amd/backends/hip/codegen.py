@@ -52,6 +52,7 @@ _device_header = None
 DEFAULT_CUS = 256
 MALL_BYTES = 256 << 20
 REDUCTION_WINDOW_BYTES = 6 << 20
+CACHED_REDUCTION_WINDOW_BYTES = 4 << 20
 TEAM_BYTES_IN_FLIGHT = 8.0e6
 
 
@@ -347,6 +348,11 @@ class CompiledLoop:
                 # input stream, four for several (vector_sum 0.90, masked_sum 0.92 of peak)
                 unroll = 2 if len(self._indexed_arrays()) <= 1 else 4
                 return Spec("flat", block=512, vec=d.vec, unroll=unroll, restrict=restrict, stream_loads=True)
+            if self.analysis.outer_reductions and d.vec > 1 and n_outer >= 16 * 1024 * d.vec * 2:
+                # input served by the caches: the atomics at the end (one per workgroup, all
+                # to one address, ~10 ns each) are what is left to save, so few workgroups of
+                # 1024 lanes (2^22 floats: 4.4 us against 12.0 us with 768 workgroups of 256)
+                return Spec("flat", block=1024, vec=d.vec, unroll=2, restrict=restrict)
             return Spec("flat", block=d.block, vec=d.vec, unroll=d.unroll, restrict=restrict, stream_loads=stream)
         stream = self._bytes_touched(arrays) > MALL_BYTES
         v = d.vec
@@ -405,7 +411,8 @@ class CompiledLoop:
                 # much outstanding; fewer workgroups starve it, more only add serialised
                 # atomics; measured optimum for every reduction tried)
                 widest = spec.vec * max(self._elem_sizes())
-                want = REDUCTION_WINDOW_BYTES / float(spec.block * spec.unroll * widest)
+                window = REDUCTION_WINDOW_BYTES if spec.stream_loads else CACHED_REDUCTION_WINDOW_BYTES
+                want = window / float(spec.block * spec.unroll * widest)
                 cap = max(64, min(cus * 8, int(round(want / 64.0)) * 64))
                 return int(min(need, cap))
             # reductions end with one atomic per workgroup: few, persistent

@@ -102,7 +102,7 @@ _cache = {}
 def kernels(**options):
     """Namespace with the six loops compiled by :func:`appy_amd.jit` under
     ``options`` (cached per option set)."""
-    key = tuple(sorted(options.items()))
+    key = repr(sorted(options.items()))
     ns = _cache.get(key)
     if ns is None:
         ns = types.SimpleNamespace(**{f.__name__: appy.jit(f, **options) if options else appy.jit(f) for f in _RAW})

@@ -45,7 +45,11 @@ def test_shared_reduction_ends_in_one_atomic_per_workgroup():
     assert "if (threadIdx.x == 0)" in k
     red = f.analysis.outer_reductions[0]
     assert (red.key, red.op, red.ty.name) == ("s[0]", "+", "float64")
-    assert f.grid_for(f.default_spec, 1 << 28, kernel=f.kernels[f.default_spec]) == 768   # 6 MiB window: 768 x 256 lanes x 2 x 16 B
+    assert f.grid_for(f.default_spec, 1 << 28, kernel=f.kernels[f.default_spec]) == 512   # 4 MiB window: 512 x 256 lanes x 2 x 16 B
+    mid = {"s": s, "a": np.broadcast_to(np.float32(0), (1 << 22,))}
+    sp = f.choose_spec(1 << 22, {}, mid)                 # served by the caches: few workgroups of 1024 lanes
+    assert (sp.block, sp.unroll, sp.stream_loads) == (1024, 2, False)
+    assert f.grid_for(sp, 1 << 22, kernel=f.kernel_for(sp)) == 128
     big = {"s": s, "a": np.broadcast_to(np.float32(0), (1 << 28,))}
     sp = f.choose_spec(1 << 28, {}, big)
     assert (sp.block, sp.unroll, sp.stream_loads) == (512, 2, True)
