@@ -291,3 +291,40 @@ def test_spmv_few_very_long_rows(k):
     y = k.spmv(data, indptr, indices, x, m, n)
     ok, worst = vo.within_budget(y, ref, budget, TOL)
     assert ok, worst
+
+
+def test_launches_from_several_threads(k):
+    """Four interpreter threads launch different loops on their own arrays at once:
+    the library's allocator, staging lanes and code caches are shared between them."""
+    import threading
+
+    rng = np.random.default_rng(13)
+    errors = []
+
+    def work(seed):
+        try:
+            r = np.random.default_rng(seed)
+            for rep in range(6):
+                n = int(r.integers(1000, 3_000_000))
+                a = r.standard_normal(n, dtype=np.float32)
+                b = r.standard_normal(n, dtype=np.float32)
+                if not np.array_equal(k.vec_add(a, b), a + b):
+                    errors.append((seed, rep, "vec_add"))
+                ref, budget = vo.vector_sum(a)
+                if abs(k.vector_sum(a) - ref) > TOL * budget:
+                    errors.append((seed, rep, "vector_sum"))
+                A = r.standard_normal((257, 300), dtype=np.float32)
+                x = r.standard_normal(300, dtype=np.float32)
+                gref, gb = vo.gemv(A, x)
+                ok, worst = vo.within_budget(k.gemv(A, x), gref, gb, TOL)
+                if not ok:
+                    errors.append((seed, rep, "gemv", worst))
+        except Exception as e:          # a failure in a thread must fail the test
+            errors.append((seed, repr(e)))
+
+    threads = [threading.Thread(target=work, args=(int(s),)) for s in rng.integers(0, 1 << 30, 4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
