@@ -182,9 +182,50 @@ def guarded_nodes(stmts) -> set:
         for child in ast.iter_child_nodes(node):
             visit(child)
 
+    def leaves_early(node) -> bool:
+        """The statement may end the iteration it belongs to (``continue`` / ``break``
+        not enclosed in a loop of its own)."""
+        if isinstance(node, (ast.Continue, ast.Break)):
+            return True
+        if isinstance(node, (ast.For, ast.While)):
+            return False
+        return any(leaves_early(c) for c in ast.iter_child_nodes(node))
+
+    def visit_block(block):
+        skipped = False
+        for st in block:
+            if skipped:
+                mark(st)
+            visit(st)
+            skipped = skipped or leaves_early(st)
+
+    def visit_blocks(node):
+        for f in ("body", "orelse"):
+            sub = getattr(node, f, None)
+            if isinstance(sub, list) and sub and isinstance(sub[0], ast.stmt):
+                visit_block(sub)
+                for st in sub:
+                    visit_blocks(st)
+
+    visit_block(stmts)
     for st in stmts:
-        visit(st)
+        visit_blocks(st)
     return out
+
+
+def skips_iterations(stmts) -> bool:
+    """True if the body holds a ``continue`` that ends an iteration of the loop
+    the body belongs to (not of a loop nested in it)."""
+    for st in stmts:
+        if isinstance(st, ast.Continue):
+            return True
+        if isinstance(st, (ast.For, ast.While)):
+            continue
+        for f in ("body", "orelse"):
+            sub = getattr(st, f, None)
+            if isinstance(sub, list) and sub and isinstance(sub[0], ast.stmt) and skips_iterations(sub):
+                return True
+    return False
 
 
 def _has_simd_loop(stmts) -> bool:
@@ -289,6 +330,7 @@ class KernelBuilder:
         self.dirty = False
         self.counter = 0
         self.seq_depth = 0        # sequential loops (for / while) around the current statement
+        self.skippable = False    # directly inside an iteration body that `continue` may leave
         self.shadowed = [n for n in analysis.assigned if n in analysis.scalars]
         self.red_by_key = {r.key: r for r in analysis.outer_reductions}
 
@@ -320,6 +362,19 @@ class KernelBuilder:
             self.stmt(stmts[i])
             i += 1
 
+    def iteration_body(self, stmts):
+        """One iteration of a parallel or simd loop."""
+        if not skips_iterations(stmts):
+            return self.block(stmts)
+        saved, self.skippable = self.skippable, True
+        saved_depth, self.seq_depth = self.seq_depth, 0
+        self.w("do {")
+        self.ind += 1
+        self.block(stmts)
+        self.ind -= 1
+        self.w("} while (0);")
+        self.skippable, self.seq_depth = saved, saved_depth
+
     def stmt(self, st):
         if isinstance(st, ast.Assign):
             return self.assign(st)
@@ -330,11 +385,15 @@ class KernelBuilder:
         if isinstance(st, ast.While):
             return self.while_(st)
         if isinstance(st, (ast.Break, ast.Continue)):
-            # the iterations of parallel and simd loops are dealt to lanes, tiles and vector
-            # components: only a sequential loop has a C loop of its own to leave or to restart
-            if self.seq_depth == 0:
-                raise Unsupported("`break` / `continue` are only supported inside a sequential loop of the kernel")
-            self.w("break;" if isinstance(st, ast.Break) else "continue;")
+            if self.seq_depth > 0:
+                self.w("break;" if isinstance(st, ast.Break) else "continue;")
+            elif isinstance(st, ast.Continue) and self.skippable:
+                # the iterations of parallel and simd loops are dealt to lanes, tiles and vector
+                # components, each in a `do { } while (0)` block of its own: leaving it ends the iteration
+                self.w("break;")
+            else:
+                raise Unsupported("`break` is only supported inside a sequential loop of the kernel "
+                                  "(the iterations of a parallel or simd loop do not run in order)")
             return
         if isinstance(st, ast.Pass):
             return
@@ -457,6 +516,7 @@ class KernelBuilder:
         knows them to be in bounds (``hoist_guarded``)."""
         loads, stores = {}, {}
         blocked = set()
+        skips = skips_iterations(body)      # then every store after the `continue` is conditional
         guarded = set() if hoist_guarded else guarded_nodes(body)
         in_place = {}           # guarded loads that stay where the program has them: key -> array
         inner_vars = {n.target.id for s in body for n in ast.walk(s) if isinstance(n, ast.For)}
@@ -483,7 +543,7 @@ class KernelBuilder:
                         loads[key] = (arr, n)
                 else:
                     top = any(isinstance(t, ast.Assign) and t.targets[0] is n for t in body)
-                    if ok and top:
+                    if ok and top and not skips:
                         stores[key] = (arr, n)
                     else:
                         blocked.add(arr.name)
@@ -584,7 +644,7 @@ class KernelBuilder:
             saved_stores = dict(self.store_subst)
             for key, (arr, _) in stores.items():
                 self.store_subst[key] = ((f"{sregs[key]}.{comp[k]}" if V > 1 else sregs[key]), arr.ty)
-            self.block(body)
+            self.iteration_body(body)
             self.ex.load_subst = saved_loads
             self.store_subst = saved_stores
             self.ind -= 1
@@ -641,7 +701,7 @@ class KernelBuilder:
             start = f"{lo_v} + __lane"
         self.w(f"for (appy::i64 {cname(var)} = {start}; {cname(var)} < {hi_v}; {cname(var)} += {W}) {{")
         self.ind += 1
-        self.block(st.body)
+        self.iteration_body(st.body)
         self.ind -= 1
         self.w("}")
         self.mode = saved_mode
@@ -801,7 +861,7 @@ class KernelBuilder:
         self.ind += 1
         self.w(f"const appy::i64 {cname(self.a.var)} = {idx_code};")
         self._declare_locals()
-        self.block(self.a.outer.body)
+        self.iteration_body(self.a.outer.body)
         self.ind -= 1
         self.w("}")
 
@@ -877,7 +937,7 @@ class KernelBuilder:
                     self.ex.load_subst[key] = ((f"({code} != 0)" if arr.ty.is_bool else code), arr.ty)
                 for key, (arr, _) in stores.items():
                     self.store_subst[key] = (f"{sregs[(u, key)]}.{comp[k]}", arr.ty)
-                self.block(self.a.outer.body)
+                self.iteration_body(self.a.outer.body)
                 self.ex.load_subst = saved_loads
                 self.store_subst = saved_stores
                 self.ind -= 1
@@ -895,6 +955,8 @@ class KernelBuilder:
         its teams read them from there."""
         if not self.spec.lds_tile or self.a.outer_reductions:
             return None
+        if skips_iterations(self.a.outer.body):
+            return None     # every thread has to reach the barriers of the tile loop
         # teams past the end of the range run on a clamped row with their team-level
         # side effects switched off; stores issued from inside simd loops cannot be
         # switched off that way, so such kernels keep the plain form
@@ -1031,7 +1093,7 @@ class KernelBuilder:
         saved_loads = dict(self.ex.load_subst)
         for arr in staged:
             self.ex.load_subst[f"{arr.name}[{var}]"] = (f"__tile_{cname(arr.name)}[{cname(var)} - {jt}]", arr.ty)
-        self.block(st.body)
+        self.iteration_body(st.body)
         self.ex.load_subst = saved_loads
         self.ind -= 1
         self.w("}")

@@ -285,8 +285,15 @@ def test_while_break_continue_become_c_loops():
     k = body_of(f.kernel_for(f.choose_spec(8, {"n": 8}, {"a": a, "out": out})).src.text)
     assert "while (true) {" in k and "if (!(" in k and "continue;" in k and "break;" in k
 
-    # the iterations of a parallel loop are dealt to lanes: it has no C loop to leave
-    bad = "#pragma parallel for\nfor i in range(0, n, 1):\n    if a[i] > 0.0:\n        continue\n    out[i] = 1\n"
+    # `continue` directly in a parallel loop ends the iteration: a do/while(0) block per iteration,
+    # and the store after it is not merged into a vector store
+    skip = "#pragma parallel for simd\nfor i in range(0, n, 1):\n    if a[i] > 0.0:\n        continue\n    out[i] = 1\n"
+    f2, _ = compiled(skip, n=8, a=a, out=out)
+    k2 = body_of(f2.kernel_for(f2.default_spec).src.text)
+    assert "do {" in k2 and "} while (0);" in k2 and "vstore" not in k2 and "continue;" not in k2
+    assert ("out", 0, 0) in f2.analysis.guarded_checks
+    # a parallel loop cannot be left
+    bad = "#pragma parallel for\nfor i in range(0, n, 1):\n    if a[i] > 0.0:\n        break\n    out[i] = 1\n"
     with pytest.raises(NotImplementedError, match="break"):
         compiled(bad, n=8, a=a, out=out)
 

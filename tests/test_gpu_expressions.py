@@ -250,3 +250,48 @@ def test_guarded_neighbour_accesses_stay_guarded(gpu):
         p = np.pad(ref, 1)
         ref = (1.0 - 4.0 * r) * ref + r * (p[:-2, 1:-1] + p[2:, 1:-1] + p[1:-1, :-2] + p[1:-1, 2:])
     assert np.allclose(got, ref, rtol=1e-12, atol=1e-12)
+
+
+def test_continue_in_parallel_and_simd_loops(gpu):
+    """``continue`` ends one iteration wherever that iteration runs: a lane of a
+    flat kernel, a team, a lane of a simd loop inside a team."""
+    import appy_amd as appy
+
+    @appy.jit
+    def clip_positive(a, out):
+        n = 0
+        #pragma parallel for simd shared(n)
+        for i in range(a.shape[0]):
+            if a[i] <= 0.0:
+                continue
+            out[i] = a[i] * 2.0
+            n += 1
+        return n
+
+    @appy.jit
+    def row_sums_of_marked_rows(A, mark, out):
+        #pragma parallel for
+        for i in range(A.shape[0]):
+            if mark[i] == 0:
+                continue
+            s = 0.0
+            #pragma simd
+            for j in range(A.shape[1]):
+                if A[i, j] < 0.0:
+                    continue
+                s += A[i, j]
+            out[i] = s
+
+    rng = np.random.default_rng(31)
+    a = rng.standard_normal(100_001)
+    out = np.full_like(a, -7.0)
+    n = clip_positive(a, out)
+    assert n == int((a > 0).sum())
+    assert np.array_equal(out, np.where(a > 0, a * 2.0, -7.0))
+
+    A = rng.standard_normal((513, 301))
+    mark = (rng.random(513) < 0.6).astype(np.int32)
+    res = np.full(513, -1.0)
+    row_sums_of_marked_rows(A, mark, res)
+    ref = np.where(mark == 1, np.where(A >= 0, A, 0.0).sum(axis=1), -1.0)
+    assert np.allclose(res, ref, rtol=1e-12, atol=1e-12)
