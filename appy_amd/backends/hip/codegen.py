@@ -375,6 +375,14 @@ class CompiledLoop:
         # one vector step per lane for short rows; two rows per wavefront at most
         # (two independent rows in flight per wavefront stream better than one)
         w = max(1, min(32, _pow2ceil(trip / float(v)) if trip > 0 else 1))
+        if uniform and trip > 0:
+            # dense rows of equal length.  Short ones stream best with two vector steps per
+            # lane (2^20 rows of 64 floats: 37 us with W = 8, 53 us with W = 16); when the
+            # rows are long but too few to keep 8 MB in flight with half a wavefront each,
+            # a whole wavefront takes a row (4096 x 16384: 42 us against 52 us)
+            w = max(1, min(32, _pow2ceil(trip / float(2 * v))))
+            if trip >= 128 * v and n_outer * 32 * 16 < TEAM_BYTES_IN_FLIGHT:
+                w = 64
         block = d.block
         if n_outer * 32 < DEFAULT_CUS * 256 and trip >= 64 * v * 32:
             # few, very long rows: wavefront teams would leave most of the chip idle,
