@@ -87,12 +87,20 @@ def _torch_np_dtype(t):
         torch.int8: np.int8, torch.uint8: np.uint8, torch.int16: np.int16, torch.int32: np.int32,
         torch.int64: np.int64, torch.bool: np.bool_,
     }
+    if t.dtype is torch.bfloat16:
+        return "bfloat16"       # no NumPy dtype: named, and typed by the generator's own rules
     if t.dtype not in table:
         raise TypeError(f"tensor dtype {t.dtype} is not supported in generated kernels")
     return np.dtype(table[t.dtype])
 
 
-def array_dtype(v) -> np.dtype:
+def _torch():
+    import torch
+
+    return torch
+
+
+def array_dtype(v):
     return v.dtype if is_numpy_array(v) else _torch_np_dtype(v)
 
 
@@ -538,7 +546,7 @@ class Launch:
                 # CPU tensor: same path as NumPy through a shared-memory view
                 self._no_capture(name, "it is a CPU tensor (it would be copied per launch)")
                 tc = v if v.is_contiguous() else v.contiguous()
-                host = tc.numpy()
+                host = tc.view(_torch().int16).numpy() if tc.dtype is _torch().bfloat16 else tc.numpy()
                 self._stage_host(name, host, v if tc is v else ("tensor", v, tc), arr.stored)
         for dptr, host, _orig, stored, name in self.temps:
             extents.append((name, dptr, host.nbytes, stored))

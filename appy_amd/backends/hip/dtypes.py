@@ -23,6 +23,7 @@ _C_NAMES = {
     "int64": "long long",
     "uint64": "unsigned long long",
     "float16": "_Float16",
+    "bfloat16": "__bf16",       # tensors only: NumPy has no such dtype
     "float32": "float",
     "float64": "double",
 }
@@ -41,6 +42,8 @@ class Ty:
 
     @property
     def kind(self) -> str:
+        if self.name == "bfloat16":
+            return "f"
         return self.dtype.kind  # 'b', 'i', 'u', 'f'
 
     @property
@@ -57,6 +60,8 @@ class Ty:
 
     @property
     def size(self) -> int:
+        if self.name == "bfloat16":
+            return 2
         return self.dtype.itemsize
 
     @property
@@ -80,12 +85,19 @@ WEAK_FLOAT = Ty("float64", True)
 WEAK_BOOL = Ty("bool", True)
 
 
+BF16 = Ty("bfloat16")
+
+
+def _dtype_name(dtype) -> str:
+    return "bfloat16" if isinstance(dtype, str) and dtype == "bfloat16" else np.dtype(dtype).name
+
+
 def supported(dtype) -> bool:
-    return np.dtype(dtype).name in _C_NAMES
+    return _dtype_name(dtype) in _C_NAMES
 
 
 def from_dtype(dtype) -> Ty:
-    name = np.dtype(dtype).name
+    name = _dtype_name(dtype)
     if name not in _C_NAMES:
         raise TypeError(f"dtype {name} is not supported in generated kernels")
     return Ty(name)
@@ -96,6 +108,13 @@ _WEAK_SAMPLE = {"b": True, "i": 1, "u": 1, "f": 1.0}
 
 def promote(a: Ty, b: Ty) -> Ty:
     """Type of ``a (op) b`` for an arithmetic operator."""
+    if "bfloat16" in (a.name, b.name):
+        # PyTorch's rules (the type only exists for tensors): Python scalars, integers and
+        # booleans adopt bfloat16, float16 meets it in float32, wider floats win
+        o = b if a.name == "bfloat16" else a
+        if o.weak or not o.is_float or o.name == "bfloat16":
+            return BF16
+        return F32 if o.name == "float16" else o.strong()
     if a.weak and b.weak:
         if a.is_float or b.is_float:
             return WEAK_FLOAT

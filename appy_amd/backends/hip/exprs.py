@@ -231,9 +231,13 @@ class ExprEmitter:
                     return f"({lc} && {rc})", t
                 raise TypeError("boolean subtract is not defined")
             sym = {ast.Add: "+", ast.Sub: "-", ast.Mult: "*"}[type(op)]
+            if t.name == "bfloat16":    # computed in float32 and rounded once, as PyTorch does
+                return f"((__bf16)({cast(lc, lt, T.F32)} {sym} {cast(rc, rt, T.F32)}))", t
             return f"({cast(lc, lt, t)} {sym} {cast(rc, rt, t)})", t
         if isinstance(op, ast.Div):
             t = T.true_divide(lt, rt)
+            if t.name == "bfloat16":
+                return f"((__bf16)({cast(lc, lt, T.F32)} / {cast(rc, rt, T.F32)}))", t
             return f"({cast(lc, lt, t)} / {cast(rc, rt, t)})", t
         if isinstance(op, ast.FloorDiv):
             t = T.promote(lt, rt)
@@ -252,8 +256,8 @@ class ExprEmitter:
                 t = T.WEAK_INT if t.weak else T.from_dtype(np.int8)
             a, b = cast(lc, lt, t), cast(rc, rt, t)
             if t.is_float:
-                if t.name == "float16":
-                    raise NotImplementedError("float16 modulo")
+                if t.size == 2:
+                    raise NotImplementedError(f"{t.name} modulo")
                 return f"appy::mod_float({a}, {b})", t
             if t.kind == "u":
                 return f"({a} % {b})", t
@@ -322,10 +326,14 @@ class ExprEmitter:
         t = None
         for _, at in args:
             t = T.join(t, T.to_float(at)) if t is not None else T.to_float(at)
-        if t.name == "float16":
+        half = t if t.size == 2 else None      # 16-bit floats: evaluated in float32, rounded back
+        if half is not None:
             t = T.F32
         fn = names[0] if t.name == "float32" else names[1]
-        return f"{fn}({', '.join(cast(c, at, t) for c, at in args)})", t
+        code = f"{fn}({', '.join(cast(c, at, t) for c, at in args)})"
+        if half is not None and half.name == "bfloat16":
+            return cast(code, t, half), half
+        return code, t
 
     def e_Call(self, node):
         f = node.func

@@ -438,7 +438,8 @@ class KernelBuilder:
                 oc, ot = self.ex.emit(loop_ir.reduction_operand(st))
                 p, pty = self.partials[name]
                 # the variable takes the type NumPy gives `name (op) operand`
-                self.set_local(name, T.promote(pty, ot) if red_op in "+*" else T.join(pty, ot))
+                vty = self.ex.locals.get(name, pty)
+                self.set_local(name, T.promote(vty, ot) if red_op in "+*" else T.join(vty, ot))
                 self.w(f"{p} = {_OPS[red_op]}::f<{pty.c}>({p}, {cast(oc, ot, pty)});")
                 return
             vc, vt = self.ex.emit(st.value)
@@ -675,6 +676,8 @@ class KernelBuilder:
             if ty is None:
                 raise NameError(f"reduction variable `{name}` has no value before the loop")
             p = self.fresh(f"part_{name}_")
+            if ty.is_float and ty.size < 4:
+                ty = T.F32      # lanes accumulate 16-bit floats in float32; rounded once when the team combines
             self.partials[name] = (p, ty)
             self.w(f"{ty.c} {p} = {T.identity_literal(op, ty)};")
         saved_mode = self.mode
@@ -711,7 +714,9 @@ class KernelBuilder:
             p, ty = self.partials[name]
             if ty.size < 4:
                 raise Unsupported(f"Reduction variable `{name}` of type {ty.name} is not supported")
-            self.w(f"{cname(name)} = {_OPS[op]}::f<{ty.c}>({cname(name)}, {self._team_total(op, ty, p)});")
+            vty = self.ex.locals.get(name, ty)
+            total = self._team_total(op, ty, p)
+            self.w(f"{cname(name)} = {cast(_OPS[op] + '::f<' + ty.c + '>(' + cast(cname(name), vty, ty) + ', ' + total + ')', ty, vty)};")
         self.partials = saved_partials
         self.ind -= 1
         self.w("}")
@@ -1036,6 +1041,8 @@ class KernelBuilder:
             if ty is None:
                 raise NameError(f"reduction variable `{name}` has no value before the loop")
             p = self.fresh(f"part_{name}_")
+            if ty.is_float and ty.size < 4:
+                ty = T.F32      # lanes accumulate 16-bit floats in float32; rounded once when the team combines
             self.partials[name] = (p, ty)
             self.w(f"{ty.c} {p} = {T.identity_literal(op, ty)};")
         jt = self.fresh("jt")
@@ -1105,7 +1112,9 @@ class KernelBuilder:
             p, ty = self.partials[name]
             if ty.size < 4:
                 raise Unsupported(f"Reduction variable `{name}` of type {ty.name} is not supported")
-            self.w(f"{cname(name)} = {_OPS[op]}::f<{ty.c}>({cname(name)}, {self._team_total(op, ty, p)});")
+            vty = self.ex.locals.get(name, ty)
+            total = self._team_total(op, ty, p)
+            self.w(f"{cname(name)} = {cast(_OPS[op] + '::f<' + ty.c + '>(' + cast(cname(name), vty, ty) + ', ' + total + ')', ty, vty)};")
         self.partials = saved_partials
         self.ind -= 1
         self.w("}")

@@ -321,3 +321,25 @@ def test_guarded_loads_are_hoisted_only_when_the_host_can_vouch_for_them():
     tree = ast.parse("a[0] if c[1] else b[2]\nfor k in r:\n    d[3]\nwhile e[4]:\n    pass\nif g[5]:\n    h[6]\nz = p[7] and q[8]")
     names = {n.value.id for n in ast.walk(tree) if isinstance(n, ast.Subscript) and id(n) in guarded_nodes(tree.body)}
     assert names == {"a", "b", "d", "e", "h", "q"}
+
+
+def test_bfloat16_tensors_follow_pytorch_promotion():
+    torch = pytest.importorskip("torch")
+    a = torch.zeros(8, dtype=torch.bfloat16)
+    h = torch.zeros(8, dtype=torch.float16)
+    w = torch.zeros(8, dtype=torch.float32)
+    o = torch.zeros(8, dtype=torch.bfloat16)
+    src = ("#pragma parallel for simd\nfor i in range(0, n, 1):\n"
+           "    t = a[i] * 2.5 + 1\n"
+           "    u = a[i] + h[i]\n"
+           "    v = a[i] * w[i]\n"
+           "    r = np.sqrt(a[i]) / a[i]\n"
+           "    o[i] = max(t, a[i]) + u + v + r\n")
+    f, code = compiled(src, n=8, a=a, h=h, w=w, o=o)
+    k = body_of(code)
+    assert "const __bf16* __restrict__ a" in k and "appy::vload<__bf16, 4>" in k
+    assert "__bf16 t" in k and "float u" in k and "float v" in k and "__bf16 r" in k
+    assert "(__bf16)(" in k and "sqrtf(" in k
+    assert T.promote(T.BF16, T.WEAK_FLOAT) == T.BF16 and T.promote(T.BF16, T.I64) == T.BF16
+    assert T.promote(T.BF16, T.from_dtype(np.float16)) == T.F32 and T.promote(T.F64, T.BF16) == T.F64
+    assert T.BF16.size == 2 and T.BF16.is_float

@@ -295,3 +295,48 @@ def test_continue_in_parallel_and_simd_loops(gpu):
     row_sums_of_marked_rows(A, mark, res)
     ref = np.where(mark == 1, np.where(A >= 0, A, 0.0).sum(axis=1), -1.0)
     assert np.allclose(res, ref, rtol=1e-12, atol=1e-12)
+
+
+def test_bfloat16_tensors(gpu):
+    """bfloat16 exists for tensors only; results must equal PyTorch's own
+    (every operation computed in float32 and rounded once)."""
+    import torch
+
+    import appy_amd as appy
+
+    @appy.jit
+    def fused(a, b, w, out, acc):
+        #pragma parallel for simd
+        for i in range(a.shape[0]):
+            out[i] = a[i] * b[i] + 2.5
+            acc[i] = a[i] * w[i]
+
+    @appy.jit
+    def row_dot(A, x, y):
+        #pragma parallel for
+        for i in range(A.shape[0]):
+            s = 0.0
+            #pragma simd
+            for j in range(A.shape[1]):
+                s += A[i, j] * x[j]
+            y[i] = s
+
+    g = torch.Generator(device="cuda").manual_seed(3)
+    n = 100_003
+    a = torch.randn(n, device="cuda", generator=g).to(torch.bfloat16)
+    b = torch.randn(n, device="cuda", generator=g).to(torch.bfloat16)
+    w = torch.randn(n, device="cuda", generator=g)
+    out = torch.empty(n, device="cuda", dtype=torch.bfloat16)
+    acc = torch.empty(n, device="cuda", dtype=torch.float32)
+    fused(a, b, w, out, acc)
+    assert torch.equal(out, a * b + 2.5)              # bf16 * bf16 -> bf16, + weak scalar -> bf16
+    assert torch.equal(acc, a * w)                    # bf16 * float32 -> float32
+
+    A = torch.randn(300, 1000, device="cuda", generator=g).to(torch.bfloat16)
+    x = torch.randn(1000, device="cuda", generator=g).to(torch.bfloat16)
+    y = torch.empty(300, device="cuda", dtype=torch.float32)
+    row_dot(A, x, y)
+    # `s = 0.0; s += bf16` makes s bfloat16 as the un-jitted tensor loop would: compare loosely with float64
+    ref = A.double() @ x.double()
+    budget = A.double().abs() @ x.double().abs()
+    assert ((y.double() - ref).abs() <= 2e-2 * budget + 1e-3).all()
