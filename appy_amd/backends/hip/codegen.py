@@ -335,6 +335,14 @@ class CompiledLoop:
         return best, uniform
 
     def choose_spec(self, n_outer, env, arrays, restrict=True) -> Spec:
+        spec = self._choose_spec(n_outer, env, arrays, restrict)
+        if self.options.get("check_bounds"):
+            # one element per access, every access through the checking path
+            spec = dataclasses.replace(spec, vec=1, unroll=1, extent=0, lds_tile=0, stream_loads=False,
+                                       stream_stores=False, checked=True)
+        return spec
+
+    def _choose_spec(self, n_outer, env, arrays, restrict=True) -> Spec:
         forced = self.options.get("hip_spec")
         d = self.default_spec
         if isinstance(forced, dict):
@@ -491,6 +499,7 @@ class Launch:
         self.lo, self.hi = lo, hi
         self.temps = []          # (dptr, host ndarray (contiguous), original, stored)
         self.mirrored = []       # (mirror, dptr, host ndarray, stored): arguments with a standing HBM mirror
+        self.oob = 0             # checked kernels: device word that receives the report
         self.keepalive = []
         # -- bounds of accesses indexed by the parallel loop variable (host check, before any device work)
         for name, dim, off in a.bound_checks:
@@ -582,6 +591,11 @@ class Launch:
                         val = val.item()
             elif p.role == "shape":
                 val = int(arrays[p.source].shape[p.dim])
+            elif p.role == "oob":
+                self._no_capture("__oob", "bounds-checked kernels report to the host after every launch")
+                self.oob = rt.malloc(4)
+                rt.memset_async(self.oob, 0, 4, self.stream)
+                val = self.oob
             elif p.role == "lo":
                 val = lo
             else:
@@ -643,9 +657,25 @@ class Launch:
         """Mean milliseconds per launch (HIP events on the launch stream)."""
         return rt.launch_timed(self.function(), self.grid, self.block, self.args, self.stream, warmup=warmup, reps=reps)
 
+    def _check_report(self):
+        if not self.oob:
+            return
+        word = C.c_int32(0)
+        try:
+            rt.memcpy_d2h(C.addressof(word), self.oob, 4, self.stream)
+        finally:
+            rt.free(self.oob)
+            self.oob = 0
+        if word.value:
+            sites = self.kernel.src.sites
+            text = sites[word.value - 1] if 0 < word.value <= len(sites) else "?"
+            raise IndexError(f"{self.loop.loop_name}: `{text}` was indexed outside the array "
+                             f"(negative indices other than literals count as outside)")
+
     def finish(self):
         """Copy stored host arrays back and release staging buffers."""
         try:
+            self._check_report()
             for dptr, host, original, stored, _name in self.temps:
                 if stored and host.nbytes:
                     rt.memcpy_d2h(host.ctypes.data, dptr, host.nbytes, self.stream)
@@ -685,6 +715,9 @@ class Launch:
             for dptr, *_ in self.temps:
                 rt.free(dptr)
             self.temps = []
+            if self.oob:
+                rt.free(self.oob)
+                self.oob = 0
             raise
         self.finish()
 
@@ -711,7 +744,7 @@ def _copy(node):
 # ---------------------------------------------------------------------------
 def codegen(loop_source, loop_name, val_map, options):
     key = (loop_source, loop_name, _signature(val_map), options.get("hip_spec") and repr(options.get("hip_spec")),
-           options.get("hip_max_blocks"), options.get("fn_name"))
+           options.get("hip_max_blocks"), bool(options.get("check_bounds")), options.get("fn_name"))
     hit = code_cache.get(key)
     if hit is not None:
         return hit

@@ -114,6 +114,8 @@ class ExprEmitter:
         self.locals = {}                # name -> Ty (loop variables included)
         self.load_subst = {}            # unparsed subscript -> (code, Ty)
         self.shape_scalars = set()      # 'X_shape_k' names referenced
+        self.checked = False            # compare every index with the extent of its dimension
+        self.sites = []                 # checked kernels: source text of the subscripts, by site number
 
     # ---- leaves ---------------------------------------------------------------
     def name_type(self, name: str):
@@ -153,7 +155,30 @@ class ExprEmitter:
         raise NotImplementedError(f"Attribute not supported in a kernel: {ast.unparse(node)}")
 
     # ---- memory -----------------------------------------------------------------
-    def index_code(self, arr: ArrayParam, sub: ast.Subscript) -> str:
+    def site(self, sub: ast.Subscript) -> int:
+        text = ast.unparse(sub)
+        if text not in self.sites:
+            self.sites.append(text)
+        return self.sites.index(text)
+
+    def inside_code(self, arr: ArrayParam, sub: ast.Subscript) -> str:
+        """Condition under which every index of ``sub`` lies inside ``arr``."""
+        elts = sub.slice.elts if isinstance(sub.slice, ast.Tuple) else [sub.slice]
+        conds = []
+        for d, e in enumerate(elts):
+            if _negative_literal(e) is not None:
+                k = _negative_literal(e)
+                self.shape_scalars.add((arr.name, d))
+                conds.append(f"({cname(f'{arr.name}_shape_{d}')} >= {k}LL)")
+                continue
+            code, ty = self.emit(e)
+            self.shape_scalars.add((arr.name, d))
+            conds.append(f"appy::inside({cast(code, ty, T.I64)}, {cname(f'{arr.name}_shape_{d}')})")
+        return " && ".join(conds)
+
+    def index_code(self, arr: ArrayParam, sub: ast.Subscript, check=None) -> str:
+        check = self.checked if check is None else check
+        site = self.site(sub) if check else -1
         elts = sub.slice.elts if isinstance(sub.slice, ast.Tuple) else [sub.slice]
         if len(elts) != arr.ndim:
             raise NotImplementedError(
@@ -173,6 +198,10 @@ class ExprEmitter:
             if not (ty.is_int or ty.is_bool):
                 raise TypeError(f"Array index must be an integer: {ast.unparse(sub)}")
             code = cast(code, ty, T.I64)
+            if check:
+                # an index outside its dimension is reported and replaced by 0, so the access itself stays legal
+                self.shape_scalars.add((arr.name, d))
+                code = f"appy::at({code}, {cname(f'{arr.name}_shape_{d}')}, {site}, __oob)"
             if d < arr.ndim - 1:
                 terms.append(f"{code} * {cname(arr.name)}_stride_{d}")
             else:

@@ -32,7 +32,7 @@ from __future__ import annotations
 
 import ast
 import ctypes as C
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 
 from ...frontend import loop_ir
 from . import dtypes as T
@@ -62,6 +62,7 @@ class Spec:
     extent: int = 0      # compile-time extent of row accumulators (team only; 0 = none)
     stream_stores: bool = False  # non-temporal vector stores
     lds_tile: int = 0    # elements of a row-invariant operand staged in LDS per step (team only; 0 = off)
+    checked: bool = False        # every subscript is compared with the extents; violations are reported
     hoist_guarded: bool = True   # flat only: loads the source guards with a condition may be issued
                                  # unconditionally (the host has checked that they stay inside their arrays)
 
@@ -79,6 +80,8 @@ class Spec:
             raise ValueError(f"unroll factor must be 1..8, got {self.unroll}")
         if not pow2(self.width) or (self.width > 64 and self.width != self.block):
             raise ValueError(f"team width must be a power of two up to 64, or the whole workgroup, got {self.width}")
+        if self.checked and (self.vec != 1 or self.unroll != 1 or self.extent or self.lds_tile):
+            raise ValueError("a bounds-checked kernel takes one element per access (vec = unroll = 1, no row extent, no LDS tile)")
         if self.extent < 0 or self.lds_tile < 0 or self.lds_tile % 4 or self.lds_tile > 16384:
             raise ValueError("row extent / LDS tile out of range (tile: multiple of 4, at most 16384 elements)")
 
@@ -86,7 +89,7 @@ class Spec:
         return (f"{self.kind}_b{self.block}_v{self.vec}_u{self.unroll}_w{self.width}"
                 f"{'_r' if self.restrict else ''}{'_nt' if self.stream_loads else ''}"
                 f"{'_e' + str(self.extent) if self.extent else ''}{'_nts' if self.stream_stores else ''}"
-                f"{'_lds' + str(self.lds_tile) if self.lds_tile else ''}{'' if self.hoist_guarded else '_g'}")
+                f"{'_lds' + str(self.lds_tile) if self.lds_tile else ''}{'' if self.hoist_guarded else '_g'}{'_chk' if self.checked else ''}")
 
 
 @dataclass
@@ -119,6 +122,7 @@ class KernelSource:
     stored_arrays: list
     bound_checks: list   # (array, dim, offset) accesses indexed by the parallel loop variable
     lane_step_bytes: int = 0   # bytes one lane moves per vector step of a flat loop
+    sites: list = field(default_factory=list)   # checked kernels: source text of every subscript, by site number
 
 
 class Unsupported(NotImplementedError):
@@ -320,6 +324,7 @@ class KernelBuilder:
         self.name = kernel_name
         self.spec = spec
         self.ex = ExprEmitter(analysis.arrays, analysis.scalars, module_names)
+        self.ex.checked = spec.checked
         self.lines = []
         self.ind = 1
         self.mode = "lane"
@@ -468,8 +473,14 @@ class KernelBuilder:
             self.w(f"{lv} = {self._store_value(vc, vt, arr)};")
             self.ex.load_subst[key] = ((f"({lv} != 0)" if arr.ty.is_bool else lv), arr.ty)
             return
-        idx = self.ex.index_code(arr, tgt)
-        store = f"{cname(arr.name)}[{idx}] = {self._store_value(vc, vt, arr)};"
+        if self.spec.checked:
+            idx = self.ex.index_code(arr, tgt, check=False)
+            site = self.ex.site(tgt)
+            store = (f"if ({self.ex.inside_code(arr, tgt)}) {cname(arr.name)}[{idx}] = {self._store_value(vc, vt, arr)}; "
+                     f"else appy::report(__oob, {site});")
+        else:
+            idx = self.ex.index_code(arr, tgt)
+            store = f"{cname(arr.name)}[{idx}] = {self._store_value(vc, vt, arr)};"
         if self.mode == "team":
             self.w(f"if ({self._leader()}) {{ {store} }}")
         else:
@@ -1152,6 +1163,8 @@ class KernelBuilder:
             if any(p.cname == nm for p in params):
                 continue
             params.append(Param(nm, f"const appy::i64 {nm}", C.c_int64, "shape", arr, dim))
+        if self.spec.checked:
+            params.append(Param("__oob", "int* __oob", C.c_void_p, "oob"))
         params.append(Param("__lo", "const appy::i64 __lo", C.c_int64, "lo"))
         params.append(Param("__hi", "const appy::i64 __hi", C.c_int64, "hi"))
         return params
@@ -1162,6 +1175,7 @@ class KernelBuilder:
         self.ind = 1
         self.counter = 0
         self.ex.load_subst = {}
+        self.ex.sites = []
         self.store_subst = {}
         self.partials = {}
         self.lds_plan = None
@@ -1203,6 +1217,7 @@ class KernelBuilder:
             reductions=list(self.a.outer_reductions),
             stored_arrays=sorted(n for n in self.a.stored if n in self.a.arrays),
             bound_checks=list(self.a.bound_checks),
+            sites=list(self.ex.sites),
             lane_step_bytes=getattr(self, "lane_step_bytes", 0),
         )
 

@@ -72,6 +72,21 @@ __device__ __forceinline__ T load_stream(const T* p) {
     return __builtin_nontemporal_load(p);
 }
 
+// ---- bounds-checked kernels --------------------------------------------------------
+// A checked kernel never leaves its arrays: an index outside its dimension is
+// reported (site number + 1 in *oob; any offending site may win) and the load
+// goes to element 0 instead, the store is dropped.  The host turns the report
+// into an IndexError after the launch.
+__device__ __forceinline__ bool inside(i64 idx, i64 extent) { return idx >= 0 && idx < extent; }
+
+__device__ __forceinline__ void report(int* oob, int site) { *oob = site + 1; }
+
+__device__ __forceinline__ i64 at(i64 idx, i64 extent, int site, int* oob) {
+    if (inside(idx, extent)) return idx;
+    report(oob, site);
+    return 0;
+}
+
 // ---- Python arithmetic that differs from C ------------------------------------
 template <typename T>
 __device__ __forceinline__ T floordiv_int(T a, T b) {

@@ -343,3 +343,22 @@ def test_bfloat16_tensors_follow_pytorch_promotion():
     assert T.promote(T.BF16, T.WEAK_FLOAT) == T.BF16 and T.promote(T.BF16, T.I64) == T.BF16
     assert T.promote(T.BF16, T.from_dtype(np.float16)) == T.F32 and T.promote(T.F64, T.BF16) == T.F64
     assert T.BF16.size == 2 and T.BF16.is_float
+
+
+def test_check_bounds_option_generates_a_kernel_that_cannot_leave_its_arrays():
+    src = ("#pragma parallel for\nfor i in range(0, n, 1):\n    s = 0.0\n    #pragma simd\n"
+           "    for j in range(lo[i], hi[i]):\n        s += v[j] * x[c[j]]\n    y[i + 1] = s\n")
+    v = np.zeros(8, np.float32)
+    c = np.zeros(8, np.int32)
+    f, _ = cg.codegen(src, "kernel_loop_1", {"n": 4, "lo": c, "hi": c, "v": v, "x": v, "c": c, "y": v, "np": np},
+                      {"check_bounds": True})
+    sp = f.choose_spec(4, {"n": 4}, {"lo": c, "hi": c, "v": v, "x": v, "c": c, "y": v})
+    assert sp.checked and sp.vec == 1 and sp.tag().endswith("_chk")
+    ksrc = f.kernel_for(sp).src
+    k = body_of(ksrc.text)
+    assert "int* __oob" in k and "vload" not in k
+    assert k.count("appy::at(") >= 5 and "appy::inside(" in k and "appy::report(__oob" in k
+    assert set(ksrc.sites) == {"lo[i]", "hi[i]", "v[j]", "c[j]", "x[c[j]]", "y[i + 1]"}
+    assert [p.role for p in ksrc.params].count("oob") == 1
+    with pytest.raises(ValueError):
+        Spec("flat", vec=4, checked=True)

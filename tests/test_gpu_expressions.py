@@ -340,3 +340,57 @@ def test_bfloat16_tensors(gpu):
     ref = A.double() @ x.double()
     budget = A.double().abs() @ x.double().abs()
     assert ((y.double() - ref).abs() <= 2e-2 * budget + 1e-3).all()
+
+
+def test_check_bounds_reports_instead_of_faulting(gpu):
+    """``check_bounds=True``: an index outside its array inside the kernel (where the
+    host cannot see it) becomes an IndexError after the launch; the access itself
+    never leaves the array.  A correct program computes the same as without the option."""
+    import appy_amd as appy
+
+    def spmv(data, indptr, indices, x, y):
+        #pragma parallel for
+        for i in range(y.shape[0]):
+            s = 0.0
+            #pragma simd
+            for j in range(indptr[i], indptr[i + 1]):
+                s += data[j] * x[indices[j]]
+            y[i] = s
+
+    checked = appy.jit(spmv, check_bounds=True)
+    plain = appy.jit(spmv)
+    rng = np.random.default_rng(8)
+    m, n = 500, 300
+    lengths = rng.integers(0, 20, m)
+    indptr = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    indices = rng.integers(0, n, indptr[-1]).astype(np.int32)
+    data = rng.standard_normal(indptr[-1]).astype(np.float32)
+    x = rng.standard_normal(n).astype(np.float32)
+    y1, y2 = np.zeros(m, np.float32), np.zeros(m, np.float32)
+    plain(data, indptr, indices, x, y1)
+    checked(data, indptr, indices, x, y2)
+    assert np.allclose(y1, y2, rtol=1e-5, atol=1e-5)     # same sums, elements dealt to the lanes differently
+
+    bad = indices.copy()
+    bad[indptr[250]] = n + 1000                      # one column index far outside x
+    y3 = np.full(m, 7.0, np.float32)
+    with pytest.raises(IndexError, match=r"x\[indices\[j\]\]"):
+        checked(data, indptr, bad, x, y3)
+    assert (y3 == 7.0).all()                         # nothing is copied back from a failed launch
+    bad[indptr[250]] = -1                            # negative run-time indices count as outside
+    with pytest.raises(IndexError, match=r"x\[indices\[j\]\]"):
+        checked(data, indptr, bad, x, y3)
+
+    @appy.jit(check_bounds=True)
+    def shifted_store(a, out):
+        #pragma parallel for simd
+        for i in range(a.shape[0]):
+            k = i * 2
+            out[k] = a[i]
+
+    a = np.arange(100.0)
+    out = np.zeros(150)
+    with pytest.raises(IndexError, match=r"out\[k\]"):
+        shifted_store(a, out)
+    checked(data, indptr, indices, x, y2)            # the runtime is fine afterwards
+    assert np.allclose(y1, y2, rtol=1e-5, atol=1e-5)
