@@ -41,6 +41,16 @@ def _kernel_launch(loop_source, loop_name, scope, global_scope, options):
     dispatcher.codegen(options.get("backend"), loop_source, loop_name, scope, global_scope, options)
 
 
+def _reduction_result(buffer, start):
+    """Value of a scalar that a ``prange`` loop reduced in a float64 buffer: the
+    type the un-jitted loop would most plausibly have produced - an ``int`` when
+    the start value was an ``int`` and the result is integral, else a ``float``."""
+    value = buffer.item()
+    if type(start) in (int, bool) and value == int(value) and abs(value) < 2.0 ** 53:
+        return int(value)
+    return value
+
+
 def set_default_options(options):
     for key, val in _DEFAULT_OPTIONS:
         options.setdefault(key, val)

@@ -119,6 +119,42 @@ def _is_prange_loop(node: ast.For) -> bool:
     )
 
 
+def prange_reductions(loop: ast.For):
+    """Scalars that a ``prange`` loop without a pragma reduces across its
+    iterations (reference behaviour as documented for ``appy.prange``,
+    docs/source/getting_started.rst:51-66: "APPy automatically detects
+    reductions"): names updated only by ``s += e`` / ``s *= e`` /
+    ``s = max(s, e)`` / ``s = min(s, e)`` with one and the same operator, never
+    assigned in any other way inside the loop (a name that is also plainly
+    assigned is a per-iteration temporary) and not a loop variable."""
+    ops = {}
+    loop_vars = {n.target.id for n in ast.walk(loop) if isinstance(n, ast.For) and isinstance(n.target, ast.Name)}
+
+    def note(name, op):
+        ops.setdefault(name, set()).add(op)
+
+    for n in ast.walk(loop):
+        if isinstance(n, ast.AugAssign) and isinstance(n.target, ast.Name):
+            note(n.target.id, {ast.Add: "+", ast.Mult: "*"}.get(type(n.op)))
+        elif isinstance(n, ast.Assign):
+            for t in n.targets:
+                for nm in (t.elts if isinstance(t, ast.Tuple) else [t]):
+                    if not isinstance(nm, ast.Name):
+                        continue
+                    v, op = n.value, None
+                    if len(n.targets) == 1 and not isinstance(t, ast.Tuple):
+                        if isinstance(v, ast.BinOp) and isinstance(v.op, (ast.Add, ast.Mult)) and any(
+                                isinstance(x, ast.Name) and x.id == nm.id for x in (v.left, v.right)):
+                            op = "+" if isinstance(v.op, ast.Add) else "*"
+                        elif (isinstance(v, ast.Call) and isinstance(v.func, ast.Name) and v.func.id in ("max", "min")
+                              and len(v.args) == 2 and any(isinstance(x, ast.Name) and x.id == nm.id for x in v.args)):
+                            op = v.func.id
+                    note(nm.id, op)
+        elif isinstance(n, (ast.NamedExpr,)) and isinstance(n.target, ast.Name):
+            note(n.target.id, None)
+    return [name for name, kinds in ops.items() if len(kinds) == 1 and None not in kinds and name not in loop_vars]
+
+
 class _LoopOutliner:
     def __init__(self, options):
         self.options = dict(options)
@@ -162,8 +198,20 @@ class _LoopOutliner:
                     post.append(ast.parse(f"{v} = {v}.item()").body[0])
             loop_text = pragma + "\n" + src.unparse(loop)
         else:
-            # `for i in prange(...)` without a pragma: a parallel loop over the same range
-            loop_text = "#pragma parallel for\n" + src.unparse(loop)
+            # `for i in prange(...)` without a pragma: a parallel loop over the same range;
+            # scalars it reduces are shared between the iterations.  Their buffer is float64
+            # whatever the start value (a Python `total = 0` may well receive floats); a
+            # start value that was an int gets an int back when the result is integral.
+            reduced = prange_reductions(loop)
+            pragma = "#pragma parallel for"
+            if reduced:
+                pragma += f" shared({', '.join(reduced)})"
+                loop = _NameToElement0(reduced).visit(copy.deepcopy(loop))
+                for v in reduced:
+                    pre.append(ast.parse(f"__appy_start_{v} = {v}").body[0])
+                    pre.append(ast.parse(f"{v} = numpy.array([{v}], dtype=numpy.float64)").body[0])
+                    post.append(ast.parse(f"{v} = appy._reduction_result({v}, __appy_start_{v})").body[0])
+            loop_text = pragma + "\n" + src.unparse(loop)
         self.loops.append((loop_name, loop_text))
         return pre + [self._stub(loop_text, loop_name)] + post
 

@@ -180,3 +180,37 @@ def test_ir_structure_checks():
 def test_used_names_order_and_callees():
     text = "#pragma parallel for\nfor i in range(M):\n    s = max(A[i], x[idx[i]])\n    y[i] = np.sqrt(s)"
     assert names.used_names(text) == ("i", "M", "s", "A", "x", "idx", "y", "np")
+
+
+def test_prange_loops_share_the_scalars_they_reduce():
+    from appy_amd.frontend.static_rewrite import prange_reductions
+
+    src = '''
+def f(a, N):
+    total = 0
+    big = -1.0
+    for i in prange(N):
+        t = a[i] * 2
+        total += t
+        big = max(big, a[i])
+    return total, big
+'''
+    new, loops = rewrite(src)
+    assert loops[0][1].startswith("#pragma parallel for shared(total, big)\nfor i in range(N):")
+    assert "total[0] += t" in loops[0][1] and "big[0] = max(big[0], a[i])" in loops[0][1]
+    assert "total = numpy.array([total], dtype=numpy.float64)" in new
+    assert "total = appy._reduction_result(total, __appy_start_total)" in new
+    loop = ast.parse("for i in prange(n):\n    s += 1\n    t = 0\n    t += 2\n    u = u * a[i]\n    v += 1\n    v -= 1").body[0]
+    assert prange_reductions(loop) == ["s", "u"]
+
+    @appy.jit(dry_run=True)
+    def sum_vector(a, N):
+        sum = 0
+        for i in appy.prange(N):
+            sum += a[i]
+        return sum
+
+    r = sum_vector(np.ones(10), 10)
+    assert r == 10 and type(r) is int                  # the documented example: "sum is now 10"
+    r = sum_vector(np.full(4, 0.25), 3)
+    assert r == 0.75 and type(r) is float

@@ -4,6 +4,7 @@ test_vec_add.py:4-19, test_global_reduction.py:4-44, test_rowwise_reduction.py:4
 test_mat_add.py:5-20, test_spmv.py:10-30, test_pi.py:8-26, test_var_write.py:12-23;
 npbench/test_gesummv.py:26-55 for array expressions), plus in-place use of GPU
 tensors.  ``backend="triton"`` in those files selects "the GPU back end"."""
+import math
 import warnings
 
 import numpy as np
@@ -274,3 +275,40 @@ def test_to_gpu_and_to_cpu_helpers(gpu):
     assert t.device.type == "cuda" and u.device.type == "cuda" and appy.to_gpu(3.5) == 3.5
     assert np.array_equal(appy.to_cpu(t), a)
     assert appy.to_cpu(torch.tensor(7.0, device="cuda")) == 7.0
+
+
+def test_prange_examples_of_the_getting_started_guide(gpu):
+    """docs/source/getting_started.rst:38-66: ``prange`` instead of ``range``,
+    reductions of scalars detected without a pragma."""
+    from appy import jit, prange
+
+    @jit
+    def add_one(a):
+        for i in prange(a.shape[0]):
+            a[i] += 1
+
+    @jit
+    def sum_vector(a, N):
+        sum = 0
+        for i in prange(N):
+            sum += a[i]
+        return sum
+
+    @jit
+    def stats(a):
+        lo = float("inf")
+        n_pos = 0
+        for i in prange(a.shape[0]):
+            lo = min(lo, a[i])
+            n_pos += 1 if a[i] > 0 else 0
+        return lo, n_pos
+
+    a = np.zeros(10)
+    add_one(a)
+    assert np.array_equal(a, np.ones(10))
+    assert sum_vector(np.ones(10), 10) == 10
+    x = np.random.default_rng(4).standard_normal(300_001)
+    s = sum_vector(x, x.shape[0])
+    assert abs(s - math.fsum(x)) <= 1e-9 * np.abs(x).sum()
+    lo, n_pos = stats(x)
+    assert lo == x.min() and n_pos == int((x > 0).sum()) and type(n_pos) is int
