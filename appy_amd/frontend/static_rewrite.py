@@ -104,19 +104,53 @@ def shared_names(pragma_text: str):
     return names
 
 
+def _range_flag(node: ast.For, flag: str) -> bool:
+    """``range(..., flag=True)`` / ``appy.range(..., flag=True)`` as the loop's iterator."""
+    it = node.iter
+    if not isinstance(it, ast.Call):
+        return False
+    f = it.func
+    is_range = (isinstance(f, ast.Name) and f.id == "range") or (
+        isinstance(f, ast.Attribute) and f.attr == "range" and isinstance(f.value, ast.Name) and f.value.id == "appy")
+    return is_range and any(k.arg == flag and isinstance(k.value, ast.Constant) and k.value.value is True
+                            for k in it.keywords)
+
+
 def _is_prange_loop(node: ast.For) -> bool:
+    """``prange(...)``, ``appy.prange(...)`` or its documented spelling
+    ``appy.range(..., parallel=True)`` (reference: docs/source/legacy.rst)."""
     it = node.iter
     if not isinstance(it, ast.Call):
         return False
     f = it.func
     if isinstance(f, ast.Name) and f.id == "prange":
         return True
-    return (
-        isinstance(f, ast.Attribute)
-        and f.attr == "prange"
-        and isinstance(f.value, ast.Name)
-        and f.value.id == "appy"
-    )
+    if isinstance(f, ast.Attribute) and f.attr == "prange" and isinstance(f.value, ast.Name) and f.value.id == "appy":
+        return True
+    return _range_flag(node, "parallel")
+
+
+class _SimdRanges(ast.NodeTransformer):
+    """``for j in appy.range(n, simd=True)`` inside a parallel loop is the
+    keyword spelling of ``#pragma simd`` above ``for j in range(n)``."""
+
+    def _fix(self, stmts):
+        out = []
+        for st in stmts:
+            st = self.visit(st)
+            if isinstance(st, ast.For) and _range_flag(st, "simd"):
+                st.iter.func = ast.Name(id="range", ctx=ast.Load())
+                st.iter.keywords = []
+                out.append(src.make_pragma_stmt("#pragma simd"))
+            out.append(st)
+        return out
+
+    def generic_visit(self, node):
+        for f in _BODY_FIELDS:
+            sub = getattr(node, f, None)
+            if isinstance(sub, list) and sub and isinstance(sub[0], ast.stmt):
+                setattr(node, f, self._fix(sub))
+        return node
 
 
 def prange_reductions(loop: ast.For):
@@ -184,11 +218,14 @@ class _LoopOutliner:
         self.count += 1
         loop_name = f"kernel_loop_{self.count}"
         pre, post = [], []
+        simd_outer = False
         if _is_prange_loop(loop):
             # `prange` is `range` with the promise of independent iterations
             loop = copy.deepcopy(loop)
+            simd_outer = _range_flag(loop, "simd")
             loop.iter.func = ast.Name(id="range", ctx=ast.Load())
             loop.iter.keywords = []
+        loop = _SimdRanges().visit(copy.deepcopy(loop))
         if pragma:
             shared = shared_names(pragma)
             if shared:
@@ -203,7 +240,7 @@ class _LoopOutliner:
             # whatever the start value (a Python `total = 0` may well receive floats); a
             # start value that was an int gets an int back when the result is integral.
             reduced = prange_reductions(loop)
-            pragma = "#pragma parallel for"
+            pragma = "#pragma parallel for simd" if simd_outer else "#pragma parallel for"
             if reduced:
                 pragma += f" shared({', '.join(reduced)})"
                 loop = _NameToElement0(reduced).visit(copy.deepcopy(loop))

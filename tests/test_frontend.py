@@ -214,3 +214,34 @@ def f(a, N):
     assert r == 10 and type(r) is int                  # the documented example: "sum is now 10"
     r = sum_vector(np.full(4, 0.25), 3)
     assert r == 0.75 and type(r) is float
+
+
+def test_keyword_spellings_of_parallel_and_simd_loops():
+    src = '''
+def f(A, x, y):
+    for i in appy.range(A.shape[0], parallel=True):
+        s = 0.0
+        for j in appy.range(A.shape[1], simd=True):
+            s += A[i, j] * x[j]
+        y[i] = s
+'''
+    _, loops = rewrite(src)
+    assert loops[0][1] == ("#pragma parallel for\nfor i in range(A_shape_0):\n    s = 0.0\n    #pragma simd\n"
+                           "    for j in range(A_shape_1):\n        s += A[i, j] * x[j]\n    y[i] = s")
+    tree = loop_ir.build(loops[0][1])
+    inner = [n for n in ast.walk(tree) if isinstance(n, ast.For)][1]
+    assert "simd" in inner.pragma and inner.pragma["reduction"] == "+:s"
+
+    @appy.jit(dry_run=True)
+    def gemv(A, x, y):
+        for i in appy.range(A.shape[0], parallel=True):
+            s = 0.0
+            for j in appy.range(A.shape[1], simd=True):
+                s += A[i, j] * x[j]
+            y[i] = s
+        return y
+
+    A = np.arange(12.0).reshape(3, 4)
+    assert np.allclose(gemv(A, np.ones(4), np.zeros(3)), A.sum(axis=1))
+    _, loops = rewrite("def g(a):\n    for i in range(a.shape[0], parallel=True, simd=True):\n        a[i] = 0\n")
+    assert loops[0][1].startswith("#pragma parallel for simd\nfor i in range(a_shape_0):")
