@@ -233,7 +233,7 @@ def f(A, x, y):
     assert "simd" in inner.pragma and inner.pragma["reduction"] == "+:s"
 
     @appy.jit(dry_run=True)
-    def gemv(A, x, y):
+    def rowdot_kw(A, x, y):
         for i in appy.range(A.shape[0], parallel=True):
             s = 0.0
             for j in appy.range(A.shape[1], simd=True):
@@ -242,6 +242,6 @@ def f(A, x, y):
         return y
 
     A = np.arange(12.0).reshape(3, 4)
-    assert np.allclose(gemv(A, np.ones(4), np.zeros(3)), A.sum(axis=1))
+    assert np.allclose(rowdot_kw(A, np.ones(4), np.zeros(3)), A.sum(axis=1))
     _, loops = rewrite("def g(a):\n    for i in range(a.shape[0], parallel=True, simd=True):\n        a[i] = 0\n")
     assert loops[0][1].startswith("#pragma parallel for simd\nfor i in range(a_shape_0):")
