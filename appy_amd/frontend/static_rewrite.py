@@ -27,6 +27,7 @@ import ast
 import copy
 import re
 
+from . import auto_simd
 from . import source as src
 from .pragma import is_parallel_for_text
 
@@ -241,6 +242,8 @@ class _LoopOutliner:
             # start value that was an int gets an int back when the result is integral.
             reduced = prange_reductions(loop)
             pragma = "#pragma parallel for simd" if simd_outer else "#pragma parallel for"
+            if not simd_outer:
+                auto_simd.vectorise_inner_loops(loop)
             if reduced:
                 pragma += f" shared({', '.join(reduced)})"
                 loop = _NameToElement0(reduced).visit(copy.deepcopy(loop))

@@ -245,3 +245,53 @@ def f(A, x, y):
     assert np.allclose(rowdot_kw(A, np.ones(4), np.zeros(3)), A.sum(axis=1))
     _, loops = rewrite("def g(a):\n    for i in range(a.shape[0], parallel=True, simd=True):\n        a[i] = 0\n")
     assert loops[0][1].startswith("#pragma parallel for simd\nfor i in range(a_shape_0):")
+
+
+def test_prange_loops_get_their_vectorisable_inner_loops_marked():
+    def loop_text(body_src):
+        return rewrite(body_src)[1][0][1]
+
+    gemv = loop_text('''
+def f(A, x, y, alpha):
+    for i in prange(A.shape[0]):
+        for j in range(A.shape[1]):
+            y[i] += alpha * A[i, j] * x[j]
+''')
+    assert gemv == ("#pragma parallel for\nfor i in range(A_shape_0):\n    __appy_acc1 = 0\n    #pragma simd\n"
+                    "    for j in range(A_shape_1):\n        __appy_acc1 += alpha * A[i, j] * x[j]\n    y[i] += __appy_acc1")
+    spmv = loop_text('''
+def f(data, indptr, indices, x, y):
+    for i in prange(y.shape[0]):
+        s = 0.0
+        for j in range(indptr[i], indptr[i + 1]):
+            s += data[j] * x[indices[j]]
+        y[i] = s
+''')
+    assert "#pragma simd\n    for j in range(indptr[i], indptr[i + 1]):" in spmv
+    spmm = loop_text('''
+def f(data, indptr, indices, B, C):
+    for i in prange(C.shape[0]):
+        for k in range(indptr[i], indptr[i + 1]):
+            for c in range(C.shape[1]):
+                C[i, c] += data[k] * B[indices[k], c]
+''')
+    assert "    for k in range(indptr[i], indptr[i + 1]):\n        #pragma simd\n        for c in range(C_shape_1):" in spmm
+    not_marked = [
+        # lanes walking j would stride through A
+        "def f(A, y):\n    for i in prange(A.shape[1]):\n        s = 0.0\n        for j in range(A.shape[0]):\n            s += A[j, i]\n        y[i] = s\n",
+        # iteration j reads what iteration j - 1 wrote
+        "def f(A):\n    for i in prange(A.shape[0]):\n        for j in range(1, A.shape[1]):\n            A[i, j] = A[i, j - 1] + 1\n",
+        # a scalar carried from one iteration to the next that is not a reduction
+        "def f(A, y):\n    for i in prange(A.shape[0]):\n        t = 0.0\n        for j in range(A.shape[1]):\n            t = t * 0.5 + A[i, j]\n        y[i] = t\n",
+        # the last value of a temporary is used after the loop
+        "def f(A, y):\n    for i in prange(A.shape[0]):\n        for j in range(A.shape[1]):\n            t = A[i, j]\n            A[i, j] = t * 2\n        y[i] = t\n",
+        # the accumulated element is read inside the loop
+        "def f(A, y, z):\n    for i in prange(A.shape[0]):\n        for j in range(A.shape[1]):\n            y[i] += A[i, j]\n            z[i, j] = y[i]\n",
+        # scatter through an index array
+        "def f(A, p, out):\n    for i in prange(A.shape[0]):\n        for j in range(A.shape[1]):\n            out[i, p[j]] = A[i, j]\n",
+    ]
+    for text in not_marked:
+        assert "#pragma simd" not in loop_text(text), text
+    # loops under a pragma are left as the programmer wrote them
+    kept = loop_text("def f(A, y):\n    #pragma parallel for\n    for i in range(A.shape[0]):\n        for j in range(A.shape[1]):\n            A[i, j] = 0\n")
+    assert "#pragma simd" not in kept

@@ -312,3 +312,76 @@ def test_prange_examples_of_the_getting_started_guide(gpu):
     assert abs(s - math.fsum(x)) <= 1e-9 * np.abs(x).sum()
     lo, n_pos = stats(x)
     assert lo == x.min() and n_pos == int((x > 0).sum()) and type(n_pos) is int
+
+
+def test_prange_only_programs_vectorise_their_inner_loops(gpu):
+    """High-level interface: no pragmas at all; the inner loops are spread over
+    lanes by the compiler (docs/source/developer.rst, "Inner Loop
+    Vectorization").  Results against NumPy / SciPy on the same inputs."""
+    from appy import jit, prange
+    from appy_amd.backends.hip import codegen as cg
+
+    @jit
+    def hl_gemv(A, x, y, alpha):
+        for i in prange(A.shape[0]):
+            for j in range(A.shape[1]):
+                y[i] += alpha * A[i, j] * x[j]
+
+    @jit
+    def hl_spmv(data, indptr, indices, x, y):
+        for i in prange(y.shape[0]):
+            s = 0.0
+            for j in range(indptr[i], indptr[i + 1]):
+                s += data[j] * x[indices[j]]
+            y[i] = s
+
+    @jit
+    def hl_spmm(data, indptr, indices, B, C):
+        for i in prange(C.shape[0]):
+            for k in range(indptr[i], indptr[i + 1]):
+                for c in range(C.shape[1]):
+                    C[i, c] += data[k] * B[indices[k], c]
+
+    @jit
+    def hl_mat_add(X, Z, Y):
+        for i in prange(X.shape[0]):
+            for j in range(X.shape[1]):
+                t = X[i, j] + Z[i, j]
+                Y[i, j] = t
+
+    @jit
+    def hl_colsum(A, y):
+        for i in prange(A.shape[1]):
+            s = 0.0
+            for j in range(A.shape[0]):
+                s += A[j, i]
+            y[i] = s
+
+    rng = np.random.default_rng(12)
+    A = rng.standard_normal((300, 517))
+    x = rng.standard_normal(517)
+    y0 = rng.standard_normal(300)
+    y = y0.copy()
+    hl_gemv(A, x, y, 1.5)
+    assert np.allclose(y, y0 + 1.5 * (A @ x), rtol=1e-12, atol=1e-12)
+
+    M = sp.random(400, 350, density=0.05, format="csr", random_state=3)
+    xv = rng.standard_normal(350)
+    ys = np.zeros(400)
+    hl_spmv(M.data, M.indptr, M.indices, xv, ys)
+    assert np.allclose(ys, M @ xv, rtol=1e-12, atol=1e-12)
+    B = rng.standard_normal((350, 64))
+    C = np.zeros((400, 64))
+    hl_spmm(M.data, M.indptr, M.indices, B, C)
+    assert np.allclose(C, M @ B, rtol=1e-12, atol=1e-12)
+
+    X, Z = rng.standard_normal((130, 257)), rng.standard_normal((130, 257))
+    Y = np.zeros_like(X)
+    hl_mat_add(X, Z, Y)
+    assert np.array_equal(Y, X + Z)
+    cs = np.zeros(517)
+    hl_colsum(A, cs)
+    assert np.allclose(cs, A.sum(axis=0), rtol=1e-12, atol=1e-12)
+
+    kinds = {key[-1]: loop.analysis.kind for key, (loop, _) in cg.code_cache.items() if str(key[-1]).startswith("hl_")}
+    assert kinds == {"hl_gemv": "team", "hl_spmv": "team", "hl_spmm": "team", "hl_mat_add": "team", "hl_colsum": "flat"}
