@@ -283,6 +283,14 @@ class LoopAnalysis:
         is_simd = "simd" in self.pragma
         self.kind = "flat" if (is_simd or not _has_simd_loop(self.outer.body)) else "team"
 
+        # sequential loops that every lane of a flat kernel runs by itself; if they index the
+        # contiguous dimension with the parallel variable, adjacent lanes must take adjacent iterations
+        nested = [n for st in self.outer.body for n in ast.walk(st) if isinstance(n, (ast.For, ast.While))]
+        self.lane_loops = self.kind == "flat" and bool(nested)
+        self.lane_loops_strided = self.lane_loops and any(
+            isinstance(n, ast.Subscript) and _uses_name(_elts(n)[-1], self.var)
+            for lp in nested for st in lp.body for n in ast.walk(st))
+
         # reductions of the parallel loop: constant-subscript elements of arrays
         self.outer_reductions = []
         for key, op in loop_ir.reductions_of(self.outer).items():
