@@ -241,6 +241,11 @@ class CompiledLoop:
         self._hi_code = compile(ast.Expression(body=ast.fix_missing_locations(_copy(a.hi_node))), "<hi>", "eval")
         self._simd_loops = self._collect_simd_loops()
         self._row_extent_code = self._find_row_extent()
+        self._strip_trip_code = None
+        if a.strip is not None:
+            lo, hi, _ = a.strip[1].iter.args
+            self._strip_trip_code = compile(ast.Expression(body=ast.fix_missing_locations(
+                ast.BinOp(left=_copy(hi), op=ast.Sub(), right=_copy(lo)))), "<trip>", "eval")
         self.kernels = {}   # Spec -> Kernel
         self._lock = threading.Lock()
         # default variant now: generation / compilation errors surface at first use of the loop
@@ -352,6 +357,20 @@ class CompiledLoop:
             return Spec(**base)
         if d.kind == "flat":
             stream = self._bytes_touched(arrays) > MALL_BYTES
+            if self.analysis.strip is not None and not self.analysis.outer_reductions:
+                # a column reduction: lanes side by side on the contiguous dimension, the
+                # wavefronts of a workgroup share out the inner loop (worth it when that
+                # loop is long; a trip count the host cannot evaluate is taken to be long)
+                try:
+                    trip = int(eval(self._strip_trip_code, _HOST_EVAL_GLOBALS, env))
+                except Exception:
+                    trip = 1 << 20
+                if trip >= 64:
+                    strips = -(-n_outer // 64)
+                    block = 1024 if strips < 4 * DEFAULT_CUS else (512 if strips < 16 * DEFAULT_CUS else 256)
+                    while block > 64 and trip < 4 * (block // 64):
+                        block //= 2
+                    return Spec("strip", block=block, vec=1, unroll=1, restrict=restrict)
             if self.analysis.lane_loops and not self.analysis.outer_reductions:
                 # every lane runs loops of its own: what it reads there per step is what adjacent
                 # lanes must find adjacent (one iteration per lane if the parallel variable indexes
@@ -433,6 +452,8 @@ class CompiledLoop:
         return total
 
     def grid_for(self, spec: Spec, n_outer: int, cus: int = DEFAULT_CUS, kernel=None, row_hint=(0.0, False)) -> int:
+        if spec.kind == "strip":
+            return int(min(max(1, -(-n_outer // 64)), self.options.get("hip_max_blocks") or (1 << 22)))
         if spec.kind == "flat":
             per_block = spec.block * spec.vec * spec.unroll
             need = max(1, -(-n_outer // per_block))

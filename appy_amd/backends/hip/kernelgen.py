@@ -52,7 +52,7 @@ _CTYPES = {
 class Spec:
     """Launch-time selectable shape of a kernel."""
 
-    kind: str            # 'flat' | 'team'
+    kind: str            # 'flat' | 'team' | 'strip'
     block: int = 256     # threads per workgroup
     vec: int = 1         # consecutive iterations per lane (V)
     unroll: int = 1      # vectors per lane and tile (U), flat only
@@ -70,8 +70,8 @@ class Spec:
         def pow2(n):
             return n >= 1 and (n & (n - 1)) == 0
 
-        if self.kind not in ("flat", "team"):
-            raise ValueError(f"kernel shape must be 'flat' or 'team', got {self.kind!r}")
+        if self.kind not in ("flat", "team", "strip"):
+            raise ValueError(f"kernel shape must be 'flat', 'team' or 'strip', got {self.kind!r}")
         if self.block % 64 or not 64 <= self.block <= 1024:
             raise ValueError(f"workgroup size must be a multiple of 64 up to 1024, got {self.block}")
         if self.vec not in (1, 2, 4):
@@ -243,6 +243,11 @@ def _has_simd_loop(stmts) -> bool:
 class LoopAnalysis:
     """Facts about a loop nest that do not depend on the launch shape."""
 
+    def _find_strip(self):
+        if self.kind != "flat":
+            return None
+        return _find_strip_parts(self.outer.body, self.var)
+
     def __init__(self, tree: ast.Module, val_arrays: dict, val_scalars: dict):
         self.tree = tree
         self.outer = loop_ir.outer_loop(tree)
@@ -291,6 +296,8 @@ class LoopAnalysis:
             isinstance(n, ast.Subscript) and _uses_name(_elts(n)[-1], self.var)
             for lp in nested for st in lp.body for n in ast.walk(st))
 
+        self.strip = self._find_strip() if self.lane_loops_strided else None
+
         # reductions of the parallel loop: constant-subscript elements of arrays
         self.outer_reductions = []
         for key, op in loop_ir.reductions_of(self.outer).items():
@@ -324,6 +331,43 @@ class LoopAnalysis:
                     off = _var_offset(e, self.var)
                     if off is not None and (n.value.id, d, off) not in into:
                         into.append((n.value.id, d, off))
+
+
+def _find_strip_parts(body, var):
+    """``(pre, loop, post, {scalar: op})`` if the body of a parallel loop is
+    scalar set-up, then ONE sequential loop that only folds values into scalars
+    with a reduction operator (``s += A[j, i] * y[j]``), then anything: the shape
+    of a column reduction.  None otherwise."""
+    loops = [k for k, st in enumerate(body) if isinstance(st, (ast.For, ast.While))]
+    if len(loops) != 1 or not isinstance(body[loops[0]], ast.For):
+        return None
+    k = loops[0]
+    pre, loop, post = body[:k], body[k], body[k + 1:]
+    if loop.orelse or not isinstance(loop.target, ast.Name) or getattr(loop, "pragma", None):
+        return None
+    for st in pre + post:
+        if any(isinstance(n, (ast.For, ast.While, ast.Break, ast.Continue)) for n in ast.walk(st)):
+            return None
+    for st in pre:      # run by every wavefront of the strip: values only, no effects
+        if not (isinstance(st, ast.Assign) and isinstance(st.targets[0], ast.Name)):
+            return None
+    ops = {}
+    for st in loop.body:
+        if not (isinstance(st, ast.Assign) and isinstance(st.targets[0], ast.Name)):
+            return None
+        op = loop_ir.reduction_operator(st)
+        name = st.targets[0].id
+        if op is None or ops.setdefault(name, op) != op:
+            return None
+        if _uses_name(loop_ir.reduction_operand(st), name):
+            return None
+    for name in ops:    # the running value is not looked at inside the loop
+        for st in loop.body:
+            if any(_uses_name(loop_ir.reduction_operand(s2), name) for s2 in loop.body):
+                return None
+    if not ops or any(_uses_name(a, n) for a in loop.iter.args for n in ops):
+        return None
+    return pre, loop, post, ops
 
 
 class KernelBuilder:
@@ -971,6 +1015,83 @@ class KernelBuilder:
             for key, (arr, sub) in stores.items():
                 self.w(f"appy::{self._vst()}<{arr.elem_c}, {V}>({self._addr(arr, sub, var, base)}, {sregs[(u, key)]});")
 
+    def _body_strip(self):
+        """Column reductions: the 64 lanes of a wavefront take 64 consecutive outer
+        iterations (so that ``A[j, i]`` is one contiguous row segment per step),
+        the wavefronts of the workgroup share out the iterations of the inner
+        loop, their partial results meet in LDS and the first wavefront finishes
+        the iteration."""
+        if self.a.strip is None or self.a.outer_reductions:
+            raise Unsupported("the loop does not have the shape of a column reduction")
+        pre, loop, post, ops = self.a.strip
+        B = self.spec.block
+        NW = B // 64
+        var = self.a.var
+        self.ex.locals[var] = T.WEAK_INT
+        self.w("const int __lane = threadIdx.x & 63;")
+        self.w("const int __wave = threadIdx.x >> 6;")
+        slots = {}
+        for name in ops:
+            ty = self.ex.locals.get(name)
+            if ty is None:
+                continue        # typed by the first pass over `pre`
+            pty = T.F32 if (ty.is_float and ty.size < 4) else ty
+            slots[name] = pty
+            self.w(f"__shared__ {pty.c} __strip_{cname(name)}[{NW}][64];")
+        self.w("for (appy::i64 __s = blockIdx.x; __lo + __s * 64 < __hi; __s += gridDim.x) {")
+        self.ind += 1
+        self.w(f"const appy::i64 {cname(var)} = __lo + __s * 64 + __lane;")
+        self.w(f"const bool __active = {cname(var)} < __hi;")
+        self._declare_locals()
+        for name, pty in slots.items():
+            self.w(f"{pty.c} __part_{cname(name)} = {T.identity_literal(ops[name], pty)};")
+        self.w("if (__active) {")
+        self.ind += 1
+        self.block(pre)
+        jv = loop.target.id
+        lo, hi = self._range_args(loop)
+        self.ex.locals[jv] = T.WEAK_INT
+        hi_v = self.fresh("hi")
+        self.w(f"const appy::i64 {hi_v} = {hi};")
+        self.w("#pragma unroll 4")
+        self.w(f"for (appy::i64 {cname(jv)} = {lo} + __wave; {cname(jv)} < {hi_v}; {cname(jv)} += {NW}) {{")
+        self.ind += 1
+        saved = dict(self.partials)
+        for name, pty in slots.items():
+            self.partials[name] = (f"__part_{cname(name)}", pty)
+        for st in loop.body:
+            st.reduce = ops[st.targets[0].id]
+            if st.targets[0].id not in slots:
+                # first typing pass: let the ordinary assignment give the variable its type
+                self.assign(ast.Assign(targets=st.targets, value=st.value))
+            else:
+                self.assign(st)
+        self.partials = saved
+        self.ind -= 1
+        self.w("}")
+        self.ind -= 1
+        self.w("}")
+        for name in slots:
+            self.w(f"__strip_{cname(name)}[__wave][__lane] = __part_{cname(name)};")
+        self.w("__syncthreads();")
+        self.w("if (__wave == 0 && __active) {")
+        self.ind += 1
+        for name, pty in slots.items():
+            vty = self.ex.locals[name]
+            op = _OPS[ops[name]]
+            self.w(f"for (int __w = 1; __w < {NW}; ++__w) __part_{cname(name)} = "
+                   f"{op}::f<{pty.c}>(__part_{cname(name)}, __strip_{cname(name)}[__w][__lane]);")
+            total = f"{op}::f<{pty.c}>({cast(cname(name), vty, pty)}, __part_{cname(name)})"
+            self.w(f"{cname(name)} = {cast(total, pty, vty)};")
+        self.block(post)
+        self.ind -= 1
+        self.w("}")
+        self.w("__syncthreads();   // the slots are free for the next strip")
+        self.ind -= 1
+        self.w("}")
+        if len(slots) != len(ops):
+            self.dirty = True
+
     def _find_lds_plan(self):
         """A ``simd`` loop directly in the body of the parallel loop whose bounds
         are the same for every outer iteration and that reads 1-D arrays indexed
@@ -1191,6 +1312,8 @@ class KernelBuilder:
             self.w(f"{r.ty.c} {r.acc} = {T.identity_literal(r.op, r.ty)};")
         if self.spec.kind == "flat":
             self._body_flat()
+        elif self.spec.kind == "strip":
+            self._body_strip()
         else:
             self._body_team()
         self._epilogue()

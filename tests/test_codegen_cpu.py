@@ -362,3 +362,27 @@ def test_check_bounds_option_generates_a_kernel_that_cannot_leave_its_arrays():
     assert [p.role for p in ksrc.params].count("oob") == 1
     with pytest.raises(ValueError):
         Spec("flat", vec=4, checked=True)
+
+
+def test_column_reductions_take_the_strip_shape():
+    src = ("#pragma parallel for\nfor i in range(0, n, 1):\n    s = 0.0\n    m = -1e30\n"
+           "    for j in range(0, r, 1):\n        s += A[j, i] * y[j]\n        m = max(m, A[j, i])\n"
+           "    x[i] += beta * s + m\n")
+    A = np.zeros((512, 300), np.float32)
+    y = np.zeros(512, np.float32)
+    x = np.zeros(300, np.float32)
+    f, _ = compiled(src, n=300, r=512, A=A, y=y, x=x, beta=1.5)
+    assert f.analysis.kind == "flat" and f.analysis.strip is not None
+    sp = f.choose_spec(300, {"n": 300, "r": 512, "beta": 1.5}, {"A": A, "y": y, "x": x})
+    assert (sp.kind, sp.block) == ("strip", 1024)
+    assert f.grid_for(sp, 300) == 5
+    k = body_of(f.kernel_for(sp).src.text)
+    assert "__shared__ float __strip_s[16][64];" in k and "__shared__ float __strip_m[16][64];" in k
+    assert "j += 16" in k and k.count("__syncthreads();") == 2 and "if (__wave == 0 && __active)" in k
+    assert "appy::OpMax::f<float>(__part_m" in k
+    # short inner loops stay with one lane per iteration
+    assert f.choose_spec(300, {"n": 300, "r": 8, "beta": 1.5}, {"A": A, "y": y, "x": x}).kind == "flat"
+    # a running value that the loop looks at is not a column reduction
+    g, _ = compiled("#pragma parallel for\nfor i in range(0, n, 1):\n    s = 0.0\n    for j in range(0, r, 1):\n"
+                    "        s = s * 0.5 + A[j, i]\n    x[i] = s\n", n=300, r=512, A=A, x=x)
+    assert g.analysis.strip is None

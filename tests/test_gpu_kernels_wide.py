@@ -375,3 +375,51 @@ def test_black_scholes_maths_functions(gpu, dtype):
     tol = 1e-10 if dtype is np.float64 else 2e-4
     assert call.dtype == dtype
     assert np.allclose(call, r, rtol=tol, atol=tol * 50) and np.allclose(put, r - P + Se, rtol=tol, atol=tol * 50)
+
+
+@appy.jit
+def column_stats(A, y, x, lo, beta):
+    #pragma parallel for
+    for i in range(A.shape[1]):
+        s = 0.0
+        m = -1e300
+        for j in range(A.shape[0]):
+            s += A[j, i] * y[j]
+            m = max(m, A[j, i])
+        x[i] += beta * s
+        lo[i] = m
+
+
+@appy.jit
+def upper_column_sums(A, out):
+    #pragma parallel for
+    for i in range(A.shape[1]):
+        s = 0.0
+        for j in range(i + 1):
+            s += A[j, i]
+        out[i] = s
+
+
+@pytest.mark.parametrize("shape", [(700, 1000), (64, 64), (5000, 37), (100, 129), (3, 500)])
+def test_column_reductions_run_as_strips(gpu, shape):
+    """``A[j, i]`` under a parallel ``i`` and a sequential ``j``: lanes side by
+    side along ``i``, the inner loop shared out between wavefronts (second loop of
+    tests/integration/triton/npbench/test_gemver.py:50-56 written as a column loop)."""
+    from appy_amd.backends.hip import codegen as cg
+
+    rng = np.random.default_rng(shape[0])
+    r, c = shape
+    A = rng.standard_normal((r, c))
+    y = rng.standard_normal(r)
+    x0 = rng.standard_normal(c)
+    x, lo = x0.copy(), np.zeros(c)
+    column_stats(A, y, x, lo, 1.2)
+    assert np.allclose(x, x0 + 1.2 * (y @ A), rtol=1e-11, atol=1e-11)
+    assert np.array_equal(lo, A.max(axis=0))
+    loop = [v[0] for kk, v in cg.code_cache.items() if kk[-1] == "column_stats"][-1]
+    assert loop.last_launch.spec.kind == ("strip" if r >= 64 else "flat")
+    if r == c or r > c:
+        S = rng.standard_normal((c, c))
+        out = np.zeros(c)
+        upper_column_sums(S, out)
+        assert np.allclose(out, np.triu(S).sum(axis=0), rtol=1e-11, atol=1e-11)
