@@ -355,22 +355,22 @@ class CompiledLoop:
                         restrict=restrict, stream_loads=d.stream_loads)
             base.update(forced)
             return Spec(**base)
+        if self.analysis.strip is not None and not self.analysis.outer_reductions:
+            # a column reduction: lanes side by side on the contiguous dimension, the
+            # wavefronts of a workgroup share out the inner loop (worth it when that
+            # loop is long; a trip count the host cannot evaluate is taken to be long)
+            try:
+                trip = int(eval(self._strip_trip_code, _HOST_EVAL_GLOBALS, env))
+            except Exception:
+                trip = 1 << 20
+            if trip >= 64:
+                strips = -(-n_outer // 64)
+                block = 1024 if strips < 4 * DEFAULT_CUS else (512 if strips < 16 * DEFAULT_CUS else 256)
+                while block > 64 and trip < 4 * (block // 64):
+                    block //= 2
+                return Spec("strip", block=block, vec=1, unroll=1, restrict=restrict)
         if d.kind == "flat":
             stream = self._bytes_touched(arrays) > MALL_BYTES
-            if self.analysis.strip is not None and not self.analysis.outer_reductions:
-                # a column reduction: lanes side by side on the contiguous dimension, the
-                # wavefronts of a workgroup share out the inner loop (worth it when that
-                # loop is long; a trip count the host cannot evaluate is taken to be long)
-                try:
-                    trip = int(eval(self._strip_trip_code, _HOST_EVAL_GLOBALS, env))
-                except Exception:
-                    trip = 1 << 20
-                if trip >= 64:
-                    strips = -(-n_outer // 64)
-                    block = 1024 if strips < 4 * DEFAULT_CUS else (512 if strips < 16 * DEFAULT_CUS else 256)
-                    while block > 64 and trip < 4 * (block // 64):
-                        block //= 2
-                    return Spec("strip", block=block, vec=1, unroll=1, restrict=restrict)
             if self.analysis.lane_loops and not self.analysis.outer_reductions:
                 # every lane runs loops of its own: what it reads there per step is what adjacent
                 # lanes must find adjacent (one iteration per lane if the parallel variable indexes

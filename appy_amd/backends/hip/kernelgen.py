@@ -244,9 +244,26 @@ class LoopAnalysis:
     """Facts about a loop nest that do not depend on the launch shape."""
 
     def _find_strip(self):
-        if self.kind != "flat":
+        """The parts of a column reduction (see ``_find_strip_parts``) when that
+        mapping is the coalesced one: inside the inner loop the parallel variable
+        indexes the contiguous dimension somewhere, the inner variable nowhere on
+        an array of two or more dimensions.  The inner loop may be sequential or
+        ``simd`` (a team walking ``A[j, i]`` along ``j`` would stride as well)."""
+        parts = _find_strip_parts(self.outer.body, self.var)
+        if parts is None:
             return None
-        return _find_strip_parts(self.outer.body, self.var)
+        loop = parts[1]
+        jv = loop.target.id
+        good = bad = False
+        for st in loop.body:
+            for n in ast.walk(st):
+                if isinstance(n, ast.Subscript) and isinstance(n.value, ast.Name) and n.value.id in self.arrays:
+                    last = _elts(n)[-1]
+                    if _uses_name(last, self.var):
+                        good = True
+                    if _uses_name(last, jv) and self.arrays[n.value.id].ndim >= 2:
+                        bad = True
+        return parts if good and not bad else None
 
     def __init__(self, tree: ast.Module, val_arrays: dict, val_scalars: dict):
         self.tree = tree
@@ -296,7 +313,7 @@ class LoopAnalysis:
             isinstance(n, ast.Subscript) and _uses_name(_elts(n)[-1], self.var)
             for lp in nested for st in lp.body for n in ast.walk(st))
 
-        self.strip = self._find_strip() if self.lane_loops_strided else None
+        self.strip = self._find_strip()
 
         # reductions of the parallel loop: constant-subscript elements of arrays
         self.outer_reductions = []
@@ -343,7 +360,9 @@ def _find_strip_parts(body, var):
         return None
     k = loops[0]
     pre, loop, post = body[:k], body[k], body[k + 1:]
-    if loop.orelse or not isinstance(loop.target, ast.Name) or getattr(loop, "pragma", None):
+    if loop.orelse or not isinstance(loop.target, ast.Name):
+        return None
+    if set(getattr(loop, "pragma", None) or {}) - {"simd", "reduction"}:
         return None
     for st in pre + post:
         if any(isinstance(n, (ast.For, ast.While, ast.Break, ast.Continue)) for n in ast.walk(st)):

@@ -423,3 +423,36 @@ def test_column_reductions_run_as_strips(gpu, shape):
         out = np.zeros(c)
         upper_column_sums(S, out)
         assert np.allclose(out, np.triu(S).sum(axis=0), rtol=1e-11, atol=1e-11)
+
+
+@appy.jit
+def column_dots_simd(A, y, x, beta):
+    #pragma parallel for
+    for j in range(A.shape[1]):
+        s = 0.0
+        #pragma simd
+        for i in range(A.shape[0]):
+            s += beta * y[i] * A[i, j]
+        x[j] += s
+
+
+@appy.jit
+def column_dots_slices(A, y, x, beta):
+    #pragma parallel for
+    for j in range(A.shape[1]):
+        x[j] += beta * (y[:] @ A[:, j])
+
+
+def test_simd_loops_down_a_column_run_as_strips_too(gpu):
+    from appy_amd.backends.hip import codegen as cg
+
+    rng = np.random.default_rng(77)
+    A = rng.standard_normal((900, 333))
+    y = rng.standard_normal(900)
+    x0 = rng.standard_normal(333)
+    for fn in (column_dots_simd, column_dots_slices):
+        x = x0.copy()
+        fn(A, y, x, 0.7)
+        assert np.allclose(x, x0 + 0.7 * (y @ A), rtol=1e-11, atol=1e-11), fn.__name__
+        loop = [v[0] for kk, v in cg.code_cache.items() if kk[-1] == fn.__name__][-1]
+        assert loop.last_launch.spec.kind == "strip", fn.__name__
