@@ -352,9 +352,14 @@ class LoopAnalysis:
 
 def _find_strip_parts(body, var):
     """``(pre, loop, post, {scalar: op})`` if the body of a parallel loop is
-    scalar set-up, then ONE sequential loop that only folds values into scalars
-    with a reduction operator (``s += A[j, i] * y[j]``), then anything: the shape
-    of a column reduction.  None otherwise."""
+    scalar set-up, then ONE inner loop, then anything, where the inner loop is
+
+    * a ``simd`` loop (its iterations are independent by declaration): any
+      statements without further loops, reductions into scalars included, or
+    * a sequential loop that only folds values into scalars with a reduction
+      operator (``s += A[j, i] * y[j]``) and never looks at the running value.
+
+    That is the shape of a column reduction or column update.  None otherwise."""
     loops = [k for k, st in enumerate(body) if isinstance(st, (ast.For, ast.While))]
     if len(loops) != 1 or not isinstance(body[loops[0]], ast.For):
         return None
@@ -362,29 +367,38 @@ def _find_strip_parts(body, var):
     pre, loop, post = body[:k], body[k], body[k + 1:]
     if loop.orelse or not isinstance(loop.target, ast.Name):
         return None
-    if set(getattr(loop, "pragma", None) or {}) - {"simd", "reduction"}:
+    pragma = getattr(loop, "pragma", None) or {}
+    if set(pragma) - {"simd", "reduction"}:
         return None
     for st in pre + post:
         if any(isinstance(n, (ast.For, ast.While, ast.Break, ast.Continue)) for n in ast.walk(st)):
+            return None
+    for st in loop.body:    # `continue` ends one iteration of the inner loop, wherever that runs
+        if any(isinstance(n, (ast.For, ast.While, ast.Break)) for n in ast.walk(st)):
             return None
     for st in pre:      # run by every wavefront of the strip: values only, no effects
         if not (isinstance(st, ast.Assign) and isinstance(st.targets[0], ast.Name)):
             return None
     ops = {}
-    for st in loop.body:
-        if not (isinstance(st, ast.Assign) and isinstance(st.targets[0], ast.Name)):
-            return None
-        op = loop_ir.reduction_operator(st)
-        name = st.targets[0].id
-        if op is None or ops.setdefault(name, op) != op:
-            return None
-        if _uses_name(loop_ir.reduction_operand(st), name):
-            return None
-    for name in ops:    # the running value is not looked at inside the loop
+    if "simd" in pragma:
+        for key, op in loop_ir.reductions_of(loop).items():
+            if not key.isidentifier():
+                return None
+            ops[key] = op
+    else:
         for st in loop.body:
+            if not (isinstance(st, ast.Assign) and isinstance(st.targets[0], ast.Name)):
+                return None
+            op = loop_ir.reduction_operator(st)
+            name = st.targets[0].id
+            if op is None or ops.setdefault(name, op) != op:
+                return None
+        for name in ops:    # the running value is not looked at inside the loop
             if any(_uses_name(loop_ir.reduction_operand(s2), name) for s2 in loop.body):
                 return None
-    if not ops or any(_uses_name(a, n) for a in loop.iter.args for n in ops):
+        if not ops:
+            return None
+    if any(_uses_name(a, n) for a in loop.iter.args for n in ops):
         return None
     return pre, loop, post, ops
 
@@ -1076,15 +1090,16 @@ class KernelBuilder:
         self.w(f"for (appy::i64 {cname(jv)} = {lo} + __wave; {cname(jv)} < {hi_v}; {cname(jv)} += {NW}) {{")
         self.ind += 1
         saved = dict(self.partials)
-        for name, pty in slots.items():
-            self.partials[name] = (f"__part_{cname(name)}", pty)
+        if len(slots) == len(ops):
+            for name, pty in slots.items():
+                self.partials[name] = (f"__part_{cname(name)}", pty)
+        # (while a reduced scalar still has no type, the pass only serves to type the
+        # locals: its updates are emitted as ordinary assignments and the pass is repeated)
         for st in loop.body:
-            st.reduce = ops[st.targets[0].id]
-            if st.targets[0].id not in slots:
-                # first typing pass: let the ordinary assignment give the variable its type
-                self.assign(ast.Assign(targets=st.targets, value=st.value))
-            else:
-                self.assign(st)
+            if (isinstance(st, ast.Assign) and isinstance(st.targets[0], ast.Name)
+                    and st.targets[0].id in ops and not hasattr(st, "reduce")):
+                st.reduce = ops[st.targets[0].id]
+        self.iteration_body(loop.body)
         self.partials = saved
         self.ind -= 1
         self.w("}")

@@ -456,3 +456,44 @@ def test_simd_loops_down_a_column_run_as_strips_too(gpu):
         assert np.allclose(x, x0 + 0.7 * (y @ A), rtol=1e-11, atol=1e-11), fn.__name__
         loop = [v[0] for kk, v in cg.code_cache.items() if kk[-1] == fn.__name__][-1]
         assert loop.last_launch.spec.kind == "strip", fn.__name__
+
+
+@appy.jit
+def scale_columns(A, f, colmax):
+    #pragma parallel for
+    for j in range(A.shape[1]):
+        m = 0.0
+        #pragma simd
+        for c in range(A.shape[0]):
+            if A[c, j] < 0.0:
+                continue
+            A[c, j] = A[c, j] * f[j]
+            m = max(m, A[c, j])
+        colmax[j] = m
+
+
+@appy.jit
+def subtract_from_columns(A, q, s):
+    #pragma parallel for
+    for j in range(A.shape[1]):
+        A[:, j] -= q[:] * s[j]
+
+
+def test_column_updates_run_as_strips(gpu):
+    from appy_amd.backends.hip import codegen as cg
+
+    rng = np.random.default_rng(5)
+    A = rng.standard_normal((777, 203))
+    f = rng.uniform(1.0, 2.0, 203)
+    ref = np.where(A < 0, A, A * f)
+    colmax = np.zeros(203)
+    scale_columns(A, f, colmax)
+    assert np.array_equal(A, ref)
+    assert np.array_equal(colmax, np.where(ref < 0, 0.0, ref).max(axis=0))
+    q, s = rng.standard_normal(777), rng.standard_normal(203)
+    B = ref.copy()
+    subtract_from_columns(B, q, s)
+    assert np.allclose(B, ref - np.outer(q, s), rtol=1e-13, atol=1e-13)
+    for name in ("scale_columns", "subtract_from_columns"):
+        loop = [v[0] for kk, v in cg.code_cache.items() if kk[-1] == name][-1]
+        assert loop.last_launch.spec.kind == "strip", name
