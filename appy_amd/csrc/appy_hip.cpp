@@ -198,9 +198,12 @@ hipError_t stage_slice(StageLane& lane, int device, char* dev, char* host, size_
     if (e != hipSuccess) return e;
     size_t pend_off[kRing] = {0, 0}, pend_len[kRing] = {0, 0};
     size_t off = 0;
+    // a slice is cut into at least eight pieces so that the host memcpy of one piece
+    // hides behind the DMA of the one before it, also for slices of a few MiB
+    size_t piece = std::min(kChunk, std::max(size_t(1) << 20, (n / 8 + 4095) & ~size_t(4095)));
     for (int i = 0; off < n; ++i) {
         const int r = i % kRing;
-        const size_t m = std::min(kChunk, n - off);
+        const size_t m = std::min(piece, n - off);
         if (i >= kRing) {
             if ((e = hipEventSynchronize(lane.done[r])) != hipSuccess) return e;
             if (!to_device) std::memcpy(host + pend_off[r], lane.pinned[r], pend_len[r]);
@@ -220,7 +223,7 @@ hipError_t stage_slice(StageLane& lane, int device, char* dev, char* host, size_
     if ((e = hipStreamSynchronize(lane.stream)) != hipSuccess) return e;
     if (!to_device) {
         // the last (up to kRing) chunks are still in the ring
-        const size_t chunks = (n + kChunk - 1) / kChunk;
+        const size_t chunks = (n + piece - 1) / piece;
         const size_t first = chunks > size_t(kRing) ? chunks - kRing : 0;
         for (size_t c = first; c < chunks; ++c) {
             const int r = int(c % kRing);
