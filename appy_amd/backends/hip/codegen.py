@@ -327,12 +327,21 @@ class CompiledLoop:
         """Expected trip count of the inner ``simd`` loops and whether it is the
         same for every outer iteration (bounds computable on the host)."""
         best, uniform = 0.0, True
+        mid = env.get("__appy_mid")
         for code, streamed in self._simd_loops:
             try:
                 best = max(best, float(eval(code, _HOST_EVAL_GLOBALS, env)))
                 continue
             except Exception:
                 uniform = False
+            # bounds that follow the parallel variable (triangular loops): the trip count in
+            # the middle of the range is the mean one
+            if mid is not None:
+                try:
+                    best = max(best, float(eval(code, _HOST_EVAL_GLOBALS, {**env, self.analysis.var: mid})))
+                    continue
+                except Exception:
+                    pass
             for name in streamed:
                 v = arrays.get(name)
                 if v is not None and v.ndim == 1 and n_outer > 0:
@@ -514,6 +523,7 @@ class CompiledLoop:
         if hi <= lo:
             return None
         arrays = {k: vals[k] for k in a.arrays}
+        env["__appy_mid"] = (lo + hi) // 2      # where triangular inner loops have their mean length
         for nm, (an, dim) in self.derived_shapes.items():
             env[nm] = int(arrays[an].shape[dim])
         return Launch(self, vals, arrays, env, lo, hi)

@@ -386,3 +386,13 @@ def test_column_reductions_take_the_strip_shape():
     g, _ = compiled("#pragma parallel for\nfor i in range(0, n, 1):\n    s = 0.0\n    for j in range(0, r, 1):\n"
                     "        s = s * 0.5 + A[j, i]\n    x[i] = s\n", n=300, r=512, A=A, x=x)
     assert g.analysis.strip is None
+
+
+def test_triangular_simd_loops_get_teams_sized_by_their_mean_length():
+    src = ("#pragma parallel for\nfor i in range(0, n, 1):\n    #pragma simd\n    for j in range(0, i + 1, 1):\n"
+           "        C[i, j] = C[i, j] * beta\n")
+    C = np.zeros((1200, 1200))
+    f, _ = compiled(src, n=1200, C=C, beta=1.2)
+    assert f.choose_spec(1200, {"n": 1200, "beta": 1.2, "__appy_mid": 600}, {"C": C}).width == 32
+    assert f.choose_spec(1200, {"n": 1200, "beta": 1.2}, {"C": C}).width == 1      # nothing known: one lane
+    assert f.choose_spec(16, {"n": 16, "beta": 1.2, "__appy_mid": 8}, {"C": C}).width == 8
