@@ -449,6 +449,9 @@ class KernelBuilder:
                 if used:
                     i += used
                     continue
+            if self.mode == "team" and self.interchange_row_update(stmts[i]):
+                i += 1
+                continue
             self.stmt(stmts[i])
             i += 1
 
@@ -806,6 +809,10 @@ class KernelBuilder:
         self.mode = saved_mode
         self.seq_depth = saved_depth
         self.bounds_vary = saved_vary
+        if W > 64 and any(isinstance(n, ast.Assign) and isinstance(n.targets[0], ast.Subscript)
+                          for b in st.body for n in ast.walk(b)):
+            # a team of several wavefronts: what one of them stored is read by the others only after this
+            self.w("__syncthreads();")
         for name, op in reds.items():
             p, ty = self.partials[name]
             if ty.size < 4:
@@ -947,6 +954,104 @@ class KernelBuilder:
         self.ind -= 1
         self.w("}")
         return k - i + 1
+
+    def interchange_row_update(self, kloop) -> bool:
+        """``for k in ...:  (simd) for c in range(0, n): T[.., c] = T[.., c] op rest(k, c)``
+        is emitted with the loops interchanged: every lane keeps its elements of the
+        row in registers while it runs the ``k`` loop, instead of reading and
+        writing the row in memory once per ``k`` (and waiting for that round trip
+        each time).  Legal because the elements are independent of each other
+        (``simd``), ``rest`` does not read ``T``, and the row belongs to this team's
+        outer iteration.  Same idea as the row accumulators, for extents that are
+        only known at run time."""
+        if not (isinstance(kloop, ast.For) and "simd" not in (getattr(kloop, "pragma", None) or {})
+                and len(kloop.body) == 1 and not kloop.orelse):
+            return False
+        m = self._match_row_update(kloop.body[0])
+        if m is None or m[1] is None:
+            return False
+        tgt, op, rest, c, hi = m
+        kvar = kloop.target.id
+        if _uses_name(tgt, kvar) or _uses_name(hi, kvar) or any(_uses_name(b, c) for b in kloop.iter.args):
+            return False
+        if loop_ir.reductions_of(kloop.body[0]):
+            return False
+        arr = self.a.arrays[tgt.value.id]
+        arr.loaded = True
+        W, V = self.spec.width, self.spec.vec
+        sym = {ast.Add: "+", ast.Sub: "-", ast.Mult: "*"}[type(op)]
+        comp = "xyzw"
+        self.w("{")
+        self.ind += 1
+        self.w("// loops interchanged: the row elements stay in registers across the sequential loop")
+        self.ex.locals[c] = T.WEAK_INT
+        self.ex.locals[kvar] = T.WEAK_INT
+        hc, ht = self.ex.emit(hi)
+        n_v = self.fresh("n")
+        self.w(f"const appy::i64 {n_v} = {cast(hc, ht, T.I64)};")
+        klo, khi = self._range_args(kloop)
+        klo_v, khi_v = self.fresh("klo"), self.fresh("khi")
+        self.w(f"const appy::i64 {klo_v} = {klo};")
+        self.w(f"const appy::i64 {khi_v} = {khi};")
+        saved_mode, self.mode = self.mode, "lane"
+        saved_depth, self.seq_depth = self.seq_depth, 0
+        probe = [ast.Assign(targets=[ast.Name(id="__rest", ctx=ast.Store())], value=rest)]
+        loads, _ = self._vector_accesses(probe, c) if V > 1 else ({}, {})
+        # loads of `rest` must not see elements of arrays that the k loop itself changes: there are none
+        # (its only statement is this update, and `rest` does not read T)
+        start = "__lane"
+        if V > 1:
+            nv, q, base, acc = self.fresh("nv"), self.fresh("q"), self.fresh("c0"), self.fresh("acc")
+            self.w(f"const appy::i64 {nv} = {n_v} / {V};")
+            self.w(f"for (appy::i64 {q} = __lane; {q} < {nv}; {q} += {W}) {{")
+            self.ind += 1
+            self.w(f"const appy::i64 {base} = {q} * {V};")
+            self.w(f"appy::vec<{arr.elem_c}, {V}>::type {acc} = appy::vload<{arr.elem_c}, {V}>({self._addr(arr, tgt, c, base)});")
+            self.w("#pragma unroll 2")
+            self.w(f"for (appy::i64 {cname(kvar)} = {klo_v}; {cname(kvar)} < {khi_v}; ++{cname(kvar)}) {{")
+            self.ind += 1
+            regs = {}
+            for key, (larr, lsub) in loads.items():
+                r = self.fresh(f"ld_{larr.name}_")
+                regs[key] = r
+                self.w(f"const appy::vec<{larr.elem_c}, {V}>::type {r} = "
+                       f"appy::vload<{larr.elem_c}, {V}>({self._addr(larr, lsub, c, base)});")
+            for v in range(V):
+                saved = dict(self.ex.load_subst)
+                for key, (larr, _) in loads.items():
+                    code = f"{regs[key]}.{comp[v]}"
+                    self.ex.load_subst[key] = ((f"({code} != 0)" if larr.ty.is_bool else code), larr.ty)
+                self.w(f"{{ const appy::i64 {cname(c)} = {base} + {v};")
+                rc, rty = self.ex.emit(rest)
+                a = f"{acc}.{comp[v]}"
+                rt_ = T.promote(arr.ty, rty)
+                self.w(f"  {a} = {cast(f'({cast(a, arr.ty, rt_)} {sym} {cast(rc, rty, rt_)})', rt_, arr.ty)}; }}")
+                self.ex.load_subst = saved
+            self.ind -= 1
+            self.w("}")
+            self.w(f"appy::vstore<{arr.elem_c}, {V}>({self._addr(arr, tgt, c, base)}, {acc});")
+            self.ind -= 1
+            self.w("}")
+            start = f"{nv} * {V} + __lane"
+        acc = self.fresh("acc")
+        self.w(f"for (appy::i64 {cname(c)} = {start}; {cname(c)} < {n_v}; {cname(c)} += {W}) {{")
+        self.ind += 1
+        idx = self.ex.index_code(arr, tgt)
+        self.w(f"{arr.ty.c} {acc} = {cname(arr.name)}[{idx}];")
+        self.w(f"for (appy::i64 {cname(kvar)} = {klo_v}; {cname(kvar)} < {khi_v}; ++{cname(kvar)}) {{")
+        self.ind += 1
+        rc, rty = self.ex.emit(rest)
+        rt_ = T.promote(arr.ty, rty)
+        self.w(f"{acc} = {cast(f'({cast(acc, arr.ty, rt_)} {sym} {cast(rc, rty, rt_)})', rt_, arr.ty)};")
+        self.ind -= 1
+        self.w("}")
+        self.w(f"{cname(arr.name)}[{idx}] = {acc};")
+        self.ind -= 1
+        self.w("}")
+        self.mode, self.seq_depth = saved_mode, saved_depth
+        self.ind -= 1
+        self.w("}")
+        return True
 
     # ---- kernel skeletons ---------------------------------------------------------
     def _declare_locals(self):
