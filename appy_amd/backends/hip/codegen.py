@@ -342,10 +342,16 @@ class CompiledLoop:
                     continue
                 except Exception:
                     pass
+            known = False
             for name in streamed:
                 v = arrays.get(name)
                 if v is not None and v.ndim == 1 and n_outer > 0:
                     best = max(best, v.shape[0] / n_outer)
+                    known = True
+            if not known:
+                # nothing to go by: a middling team (16 lanes x V) loses less on either side than
+                # one lane per row does on long rows
+                best = max(best, 64.0)
         return best, uniform
 
     def choose_spec(self, n_outer, env, arrays, restrict=True) -> Spec:

@@ -394,5 +394,5 @@ def test_triangular_simd_loops_get_teams_sized_by_their_mean_length():
     C = np.zeros((1200, 1200))
     f, _ = compiled(src, n=1200, C=C, beta=1.2)
     assert f.choose_spec(1200, {"n": 1200, "beta": 1.2, "__appy_mid": 600}, {"C": C}).width == 32
-    assert f.choose_spec(1200, {"n": 1200, "beta": 1.2}, {"C": C}).width == 1      # nothing known: one lane
+    assert f.choose_spec(1200, {"n": 1200, "beta": 1.2}, {"C": C}).width == 32     # nothing known: a middling team (64 / V)
     assert f.choose_spec(16, {"n": 16, "beta": 1.2, "__appy_mid": 8}, {"C": C}).width == 8
