@@ -195,6 +195,20 @@ def _ensure_device(dev: int):
         _tls.device = dev
 
 
+_raw_stream_getter = None
+
+
+def _current_raw_stream(device: int) -> int:
+    """PyTorch's current stream on ``device`` as a raw handle."""
+    global _raw_stream_getter
+    if _raw_stream_getter is None:
+        import torch
+
+        _raw_stream_getter = getattr(torch._C, "_cuda_getCurrentRawStream", None) or (
+            lambda dev: torch.cuda.current_stream(dev).cuda_stream)
+    return _raw_stream_getter(device)
+
+
 def _pow2ceil(x: float) -> int:
     n = 1
     while n < x:
@@ -247,6 +261,8 @@ class CompiledLoop:
             self._strip_trip_code = compile(ast.Expression(body=ast.fix_missing_locations(
                 ast.BinOp(left=_copy(hi), op=ast.Sub(), right=_copy(lo)))), "<trip>", "eval")
         self.kernels = {}   # Spec -> Kernel
+        self._replays = {}  # call identity -> Launch that can simply be launched again
+        self._replayable = not self.options.get("check_bounds")
         self._lock = threading.Lock()
         # default variant now: generation / compilation errors surface at first use of the loop
         self.default_spec = self._default_spec()
@@ -511,11 +527,50 @@ class CompiledLoop:
     def __call__(self, *args):
         if len(args) != len(self.arg_names):
             raise TypeError(f"{self.loop_name} expects {len(self.arg_names)} arguments, got {len(args)}")
+        key = self._replay_key(args) if self._replayable else None
+        if key is not None:
+            plan = self._replays.get(key)
+            if plan is not None:
+                # same tensors (address, shape, strides), same scalars, same stream: the staged
+                # launch of last time is still exact, so only the launch itself is repeated
+                _ensure_device(plan.device)
+                rt.launch(plan.function(), plan.grid, plan.block, plan.args, plan.stream)
+                self.last_launch = plan
+                return
         vals = dict(zip(self.arg_names, args))
         plan = self.prepare(vals)
         if plan is None:
             return
         plan.run()
+        if key is not None and plan.replayable():
+            if len(self._replays) >= 64:
+                self._replays.clear()
+            self._replays[key] = plan
+
+    def _replay_key(self, args):
+        """Identity of a call whose arrays all live on the GPU already; None for
+        any other call (host arrays are copied per call, captures record)."""
+        if graphs.current() is not None:
+            return None
+        key = []
+        device = -1
+        for v in args:
+            t = type(v)
+            if t is int or t is float or t is bool:
+                key.append((t, v))
+            elif isinstance(v, np.generic):
+                key.append((v.dtype.num, v.item()))
+            elif hasattr(v, "data_ptr"):        # a tensor
+                if not v.is_cuda:
+                    return None
+                device = v.device.index or 0
+                key.append((v.data_ptr(), v.shape, v.stride()))
+            else:
+                return None
+        if device < 0:
+            return None
+        key.append(_current_raw_stream(device))
+        return tuple(key)
 
     def prepare(self, vals):
         """Stage arguments on the device and pick the kernel variant.  Returns
@@ -545,6 +600,7 @@ class Launch:
         self.temps = []          # (dptr, host ndarray (contiguous), original, stored)
         self.mirrored = []       # (mirror, dptr, host ndarray, stored): arguments with a standing HBM mirror
         self.oob = 0             # checked kernels: device word that receives the report
+        self.keepalive_copies = False   # a non-contiguous tensor was repacked for this launch
         self.keepalive = []
         # -- bounds of accesses indexed by the parallel loop variable (host check, before any device work)
         for name, dim, off in a.bound_checks:
@@ -563,7 +619,7 @@ class Launch:
             import torch
 
             device = gpu_tensors[0].device.index or 0
-            self.stream = torch.cuda.current_stream(device).cuda_stream
+            self.stream = _current_raw_stream(device)
         self.capture = graphs.current()
         if self.capture is not None:
             # the launch is recorded into the graph's stream, not executed
@@ -590,6 +646,7 @@ class Launch:
                 if t.ndim >= 1 and t.numel() > 1 and t.stride(-1) != 1:
                     self._no_capture(name, "its last dimension is not contiguous (it would be repacked per launch)")
                     t = v.contiguous()
+                    self.keepalive_copies = True
                     if arr.stored:
                         self.keepalive.append(("copy_back", v, t))
                 self.keepalive.append(t)
@@ -680,6 +737,10 @@ class Launch:
         self.temps.append((dptr, host, original, stored, name))
         self.ptr[name] = dptr
         self.strides[name] = [s // host.itemsize for s in host.strides]
+
+    def replayable(self) -> bool:
+        """True if nothing but the kernel launch happens when this call is repeated."""
+        return not (self.temps or self.mirrored or self.keepalive_copies or self.oob or self.capture is not None)
 
     def _no_capture(self, name, why):
         if self.capture is not None:

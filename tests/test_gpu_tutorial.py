@@ -385,3 +385,41 @@ def test_prange_only_programs_vectorise_their_inner_loops(gpu):
 
     kinds = {key[-1]: loop.analysis.kind for key, (loop, _) in cg.code_cache.items() if str(key[-1]).startswith("hl_")}
     assert kinds == {"hl_gemv": "team", "hl_spmv": "team", "hl_spmm": "team", "hl_mat_add": "team", "hl_colsum": "flat"}
+
+
+def test_repeated_calls_on_gpu_tensors_replay_the_staged_launch(gpu):
+    """A call with the same tensors, scalars and stream as before repeats only the
+    launch; anything that differs goes through staging again."""
+    import torch
+
+    from appy_amd.backends.hip import codegen as cg
+
+    @appy.jit
+    def scaled_add(a, b, c, f):
+        #pragma parallel for simd
+        for i in range(a.shape[0]):
+            c[i] = a[i] * f + b[i]
+
+    a = torch.arange(1000, dtype=torch.float64, device="cuda")
+    b = torch.ones(1000, dtype=torch.float64, device="cuda")
+    c = torch.zeros(1000, dtype=torch.float64, device="cuda")
+    scaled_add(a, b, c, 2.0)
+    loop = [v[0] for kk, v in cg.code_cache.items() if kk[-1] == "scaled_add"][-1]
+    first = loop.last_launch
+    a.mul_(3.0)
+    scaled_add(a, b, c, 2.0)
+    assert loop.last_launch is first                          # replayed ...
+    assert torch.equal(c, a * 2.0 + b)                        # ... on the tensors' current contents
+    scaled_add(a, b, c, 5.0)                                  # another scalar
+    assert loop.last_launch is not first and torch.equal(c, a * 5.0 + b)
+    c2 = torch.zeros(500, dtype=torch.float64, device="cuda")
+    scaled_add(a[:500], b[:500], c2, 2.0)                     # other shapes
+    assert torch.equal(c2, a[:500] * 2.0 + b[:500])
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        scaled_add(a, b, c, 2.0)                              # another stream
+        assert loop.last_launch.stream == side.cuda_stream
+    side.synchronize()
+    assert torch.equal(c, a * 2.0 + b)
+    with pytest.raises(IndexError):
+        scaled_add(a, b[:10], c, 2.0)                         # host checks still run for new shapes
