@@ -52,7 +52,7 @@ def parse_args():
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=50)
     p.add_argument("--warmup", type=int, default=5)
-    p.add_argument("--workloads", default="vector_sum,masked_sum,copy,vec_add,gemv,spmv_uniform,spmv_powerlaw,spmm",
+    p.add_argument("--workloads", default="vector_sum,masked_sum,copy,vec_add,gemv,spmv_uniform,spmv_powerlaw,spmv_powerlaw16,spmm",
                    help="comma separated subset; vector_sum is always run (headline)")
     p.add_argument("--scale", type=float, default=1.0, help="shrink every size by this factor (debugging)")
     p.add_argument("--no-cpu-baseline", action="store_true")
@@ -334,6 +334,20 @@ def main():
         gx = torch.Generator(device="cuda"); gx.manual_seed(41)
         x_d = torch.randn(m4, generator=gx, device="cuda", dtype=torch.float32)
         spmv_case("spmv_powerlaw", data_d, indptr_d, indices_d, x_d, m4, m4)
+        del data_d, indptr_d, indices_d, x_d
+        torch.cuda.empty_cache()
+
+    if "spmv_powerlaw16" in want:
+        # same recipe with exponent 1.79: the power-law matrix whose mean row length is the
+        # 16 non-zeros the config text quotes (exponent 1.5 with clip 4096 gives a mean of 97)
+        m4 = shrink(1 << 22)
+        rng = np.random.default_rng(105)
+        lengths = np.clip(rng.zipf(1.79, m4), 1, min(4096, m4)).astype(np.int64)
+        data_d, indptr_d, indices_d = device_csr(torch, lengths, m4, seed=7)
+        log(f"power-law(1.79) CSR nnz={data_d.numel()}")
+        gx = torch.Generator(device="cuda"); gx.manual_seed(42)
+        x_d = torch.randn(m4, generator=gx, device="cuda", dtype=torch.float32)
+        spmv_case("spmv_powerlaw16", data_d, indptr_d, indices_d, x_d, m4, m4)
         del data_d, indptr_d, indices_d, x_d
         torch.cuda.empty_cache()
 
