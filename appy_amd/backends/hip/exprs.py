@@ -114,6 +114,7 @@ class ExprEmitter:
         self.locals = {}                # name -> Ty (loop variables included)
         self.load_subst = {}            # unparsed subscript -> (code, Ty)
         self.shape_scalars = set()      # 'X_shape_k' names referenced
+        self.stream_arrays = set()      # arrays whose scalar loads bypass the caches (read once by the launch)
         self.checked = False            # compare every index with the extent of its dimension
         self.sites = []                 # checked kernels: source text of the subscripts, by site number
 
@@ -224,6 +225,8 @@ class ExprEmitter:
         arr = self.arrays[base.id]
         arr.loaded = True
         code = f"{cname(arr.name)}[{self.index_code(arr, node)}]"
+        if arr.name in self.stream_arrays and not arr.stored:
+            code = f"__builtin_nontemporal_load(&{code})"
         if arr.ty.is_bool:
             code = f"({code} != 0)"
         return code, arr.ty

@@ -1191,7 +1191,15 @@ class KernelBuilder:
         self.ex.locals[jv] = T.WEAK_INT
         hi_v = self.fresh("hi")
         self.w(f"const appy::i64 {hi_v} = {hi};")
-        self.w("#pragma unroll 4")
+        saved_stream = set(self.ex.stream_arrays)
+        if self.spec.stream_loads:
+            # matrices walked once by the launch (indexed by both loop variables) bypass the caches
+            for st in loop.body:
+                for n in ast.walk(st):
+                    if (isinstance(n, ast.Subscript) and isinstance(n.value, ast.Name) and n.value.id in self.a.arrays
+                            and _uses_name(n, jv) and _uses_name(n, var)):
+                        self.ex.stream_arrays.add(n.value.id)
+        self.w(f"#pragma unroll {max(4, self.spec.unroll)}")
         self.w(f"for (appy::i64 {cname(jv)} = {lo} + __wave; {cname(jv)} < {hi_v}; {cname(jv)} += {NW}) {{")
         self.ind += 1
         saved = dict(self.partials)
@@ -1206,6 +1214,7 @@ class KernelBuilder:
                 st.reduce = ops[st.targets[0].id]
         self.iteration_body(loop.body)
         self.partials = saved
+        self.ex.stream_arrays = saved_stream
         self.ind -= 1
         self.w("}")
         self.ind -= 1

@@ -73,6 +73,18 @@ def gemv(A, x):
     return y
 
 
+def gemv_columns(A, y):
+    x = _empty(A.shape[1], y)
+    #pragma parallel for
+    for j in range(A.shape[1]):
+        s = 0.0
+        #pragma simd
+        for i in range(A.shape[0]):
+            s += A[i, j] * y[i]
+        x[j] = s
+    return x
+
+
 def spmv(A_data, A_indptr, A_indices, x, M, N):
     y = _empty(M, x)
     #pragma parallel for
@@ -95,7 +107,7 @@ def spmm(A_data, A_indptr, A_indices, B, y, M):
             y[i, :] += A_data[k] * B[A_indices[k], :]
 
 
-_RAW = (vec_add, copy, vector_sum, masked_sum, gemv, spmv, spmm)
+_RAW = (vec_add, copy, vector_sum, masked_sum, gemv, gemv_columns, spmv, spmm)
 _cache = {}
 
 
@@ -134,12 +146,16 @@ def compile_all_patterns() -> int:
     k.vector_sum(a)
     k.masked_sum(a, m)
     k.gemv(A, x)
+    k.gemv_columns(A, x[:8].copy())
     k.spmv(data, indptr, indices, x[:8].copy(), 8, 8)
     k.spmm(data, indptr, indices, B, Y, 8)
     count = 0
     for key in set(cg.code_cache) - before:
         loop, _src = cg.code_cache[key]
         count += len(loop.kernels)
+        if loop.analysis.strip is not None:
+            loop.kernel_for(Spec("strip", block=1024, vec=1, unroll=8, stream_loads=True))
+            count += 1
         if loop.analysis.kind == "team":
             for w in (1, 4, 16, 64):
                 loop.kernel_for(Spec("team", block=256, vec=loop.default_spec.vec, width=w))

@@ -52,7 +52,7 @@ def parse_args():
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=50)
     p.add_argument("--warmup", type=int, default=5)
-    p.add_argument("--workloads", default="vector_sum,masked_sum,copy,vec_add,gemv,spmv_uniform,spmv_powerlaw,spmv_powerlaw16,spmm",
+    p.add_argument("--workloads", default="vector_sum,masked_sum,copy,vec_add,gemv,gemv_columns,spmv_uniform,spmv_powerlaw,spmv_powerlaw16,spmm",
                    help="comma separated subset; vector_sum is always run (headline)")
     p.add_argument("--scale", type=float, default=1.0, help="shrink every size by this factor (debugging)")
     p.add_argument("--no-cpu-baseline", action="store_true")
@@ -277,6 +277,23 @@ def main():
                                    "what": f"A @ x (BLAS sgemv, up to {len(os.sched_getaffinity(0))} threads), full size",
                                    "literal_loop_ns_per_element": (time.perf_counter() - t0) / (rr * rr) * 1e9}
         del A_d, x_d, y_d, Am, ref, budget
+        torch.cuda.empty_cache()
+
+    # ---------------- column form of GEMV (second loop of gemver): the strip kernel shape -------
+    if "gemv_columns" in want:
+        r = shrink(16384, 64)
+        Am, yv = wl.gemv(r, r)
+        A_d, y_d = torch.from_numpy(Am).cuda(), torch.from_numpy(yv).cuda()
+        before = set(cg.code_cache)
+        x_d = k.gemv_columns(A_d, y_d)
+        loop = run.loop_of(before)
+        ref, budget = vo.gemv(Am.T, yv)
+        ok, worst = vo.within_budget(x_d.cpu().numpy(), ref, budget)
+        parity["gemv_columns"] = {"worst_err_over_bound": worst, "ok": ok}
+        vals = {"A": A_d, "y": y_d, "x": x_d, "A_shape_0": r, "A_shape_1": r}
+        results["gemv_columns"] = run.measure(loop, vals, 4 * (r * r + r + r), K, W)
+        log("gemv_columns", results["gemv_columns"], parity["gemv_columns"])
+        del A_d, y_d, x_d, Am, ref, budget
         torch.cuda.empty_cache()
 
     # ---------------- config 4: CSR SpMV -----------------------------------------------------

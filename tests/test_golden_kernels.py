@@ -21,6 +21,7 @@ CASES = {
     "vector_sum": Spec("flat", block=256, vec=4, unroll=2, stream_loads=True),
     "masked_sum": Spec("flat", block=256, vec=4, unroll=2, stream_loads=True),
     "gemv": Spec("team", block=256, vec=4, width=32, stream_loads=True),
+    "gemv_columns": Spec("strip", block=1024, vec=1, unroll=8, stream_loads=True),
     "spmv": Spec("team", block=256, vec=4, width=4, stream_loads=True),
     "spmm": Spec("team", block=256, vec=4, width=32, extent=128),
 }
