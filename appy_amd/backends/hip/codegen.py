@@ -257,7 +257,9 @@ class CompiledLoop:
         self._row_extent_code = self._find_row_extent()
         self._strip_trip_code = None
         if a.strip is not None:
-            lo, hi, _ = a.strip[1].iter.args
+            # trip count of the first shared-out loop, for the choice between strip and other shapes
+            first = next(n for n in ast.walk(a.outer) if isinstance(n, ast.For) and id(n) in a.strip)
+            lo, hi, _ = first.iter.args
             self._strip_trip_code = compile(ast.Expression(body=ast.fix_missing_locations(
                 ast.BinOp(left=_copy(hi), op=ast.Sub(), right=_copy(lo)))), "<trip>", "eval")
         self.kernels = {}   # Spec -> Kernel

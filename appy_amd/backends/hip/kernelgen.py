@@ -244,26 +244,84 @@ class LoopAnalysis:
     """Facts about a loop nest that do not depend on the launch shape."""
 
     def _find_strip(self):
-        """The parts of a column reduction (see ``_find_strip_parts``) when that
-        mapping is the coalesced one: inside the inner loop the parallel variable
-        indexes the contiguous dimension somewhere, the inner variable nowhere on
-        an array of two or more dimensions.  The inner loop may be sequential or
-        ``simd`` (a team walking ``A[j, i]`` along ``j`` would stride as well)."""
-        parts = _find_strip_parts(self.outer.body, self.var)
-        if parts is None:
+        """``{id(loop): {scalar: op}}`` for the inner loops that a *strip* kernel
+        shares out between wavefronts, or None if the loop nest does not suit that
+        shape.  In a strip the 64 lanes of a wavefront take 64 consecutive outer
+        iterations and the wavefronts of the workgroup form the team of each of
+        them; it is the coalesced mapping when the inner loops walk down columns
+        (``A[j, i]``: the parallel variable indexes the contiguous dimension).
+
+        Shared-out loops are the ``simd`` loops and, when the body has no ``simd``
+        loop, a single sequential loop that only folds values into scalars.  They
+        end in workgroup barriers, so they may only stand where every lane of the
+        workgroup arrives together: directly in the body or inside sequential
+        loops whose bounds are the same for every outer iteration - never under
+        ``if`` / ``while`` - and nothing outside them may ``break`` / ``continue``."""
+        body = self.outer.body
+        assigned = set(self.assigned) | {self.var}
+        spread = {}
+
+        def loop_free(stmts, allow_continue):
+            stop = (ast.For, ast.While, ast.Break) if allow_continue else (ast.For, ast.While, ast.Break, ast.Continue)
+            return not any(isinstance(n, stop) for st in stmts for n in ast.walk(st))
+
+        def has_simd(node):
+            return any(isinstance(n, ast.For) and "simd" in (getattr(n, "pragma", None) or {}) for n in ast.walk(node))
+
+        def walk(stmts) -> bool:
+            if skips_iterations(stmts):
+                return False                    # some lanes would miss the barriers that follow
+            for st in stmts:
+                if isinstance(st, ast.For) and "simd" in (getattr(st, "pragma", None) or {}):
+                    if st.orelse or not isinstance(st.target, ast.Name) or not loop_free(st.body, True):
+                        return False
+                    if set(st.pragma) - {"simd", "reduction"}:
+                        return False
+                    ops = {}
+                    for key, op in loop_ir.reductions_of(st).items():
+                        if not key.isidentifier():
+                            return False
+                        ops[key] = op
+                    if any(_uses_name(a, n) for a in st.iter.args for n in ops):
+                        return False
+                    spread[id(st)] = ops
+                elif isinstance(st, ast.For):
+                    if has_simd(st):
+                        if st.orelse or any(_uses_name(a, n) for a in st.iter.args for n in assigned):
+                            return False        # lanes would reach the barriers inside a different number of times
+                        if any(isinstance(n, ast.Break) for n in ast.walk(st)) or not walk(st.body):
+                            return False
+                elif isinstance(st, (ast.If, ast.While)) and has_simd(st):
+                    return False
+            return True
+
+        if has_simd(self.outer):
+            if not walk(body):
+                return None
+        else:
+            parts = _find_strip_parts(body, self.var)
+            if parts is None:
+                return None
+            _pre, loop, _post, ops = parts
+            for st in loop.body:
+                st.reduce = ops[st.targets[0].id]
+            spread[id(loop)] = ops
+        if not spread:
             return None
-        loop = parts[1]
-        jv = loop.target.id
+        # profitability: down the columns, never along a row of a matrix
         good = bad = False
-        for st in loop.body:
-            for n in ast.walk(st):
-                if isinstance(n, ast.Subscript) and isinstance(n.value, ast.Name) and n.value.id in self.arrays:
-                    last = _elts(n)[-1]
-                    if _uses_name(last, self.var):
-                        good = True
-                    if _uses_name(last, jv) and self.arrays[n.value.id].ndim >= 2:
-                        bad = True
-        return parts if good and not bad else None
+        for n in ast.walk(self.outer):
+            if isinstance(n, ast.For) and id(n) in spread:
+                jv = n.target.id
+                for st in n.body:
+                    for sub in ast.walk(st):
+                        if isinstance(sub, ast.Subscript) and isinstance(sub.value, ast.Name) and sub.value.id in self.arrays:
+                            last = _elts(sub)[-1]
+                            if _uses_name(last, self.var):
+                                good = True
+                            if _uses_name(last, jv) and self.arrays[sub.value.id].ndim >= 2:
+                                bad = True
+        return spread if good and not bad else None
 
     def __init__(self, tree: ast.Module, val_arrays: dict, val_scalars: dict):
         self.tree = tree
@@ -352,14 +410,10 @@ class LoopAnalysis:
 
 def _find_strip_parts(body, var):
     """``(pre, loop, post, {scalar: op})`` if the body of a parallel loop is
-    scalar set-up, then ONE inner loop, then anything, where the inner loop is
-
-    * a ``simd`` loop (its iterations are independent by declaration): any
-      statements without further loops, reductions into scalars included, or
-    * a sequential loop that only folds values into scalars with a reduction
-      operator (``s += A[j, i] * y[j]``) and never looks at the running value.
-
-    That is the shape of a column reduction or column update.  None otherwise."""
+    scalar set-up, then ONE sequential loop that only folds values into scalars
+    with a reduction operator (``s += A[j, i] * y[j]``) and never looks at the
+    running value, then anything without loops: a column reduction written
+    without ``simd``.  None otherwise."""
     loops = [k for k, st in enumerate(body) if isinstance(st, (ast.For, ast.While))]
     if len(loops) != 1 or not isinstance(body[loops[0]], ast.For):
         return None
@@ -368,7 +422,7 @@ def _find_strip_parts(body, var):
     if loop.orelse or not isinstance(loop.target, ast.Name):
         return None
     pragma = getattr(loop, "pragma", None) or {}
-    if set(pragma) - {"simd", "reduction"}:
+    if pragma:
         return None
     for st in pre + post:
         if any(isinstance(n, (ast.For, ast.While, ast.Break, ast.Continue)) for n in ast.walk(st)):
@@ -380,24 +434,18 @@ def _find_strip_parts(body, var):
         if not (isinstance(st, ast.Assign) and isinstance(st.targets[0], ast.Name)):
             return None
     ops = {}
-    if "simd" in pragma:
-        for key, op in loop_ir.reductions_of(loop).items():
-            if not key.isidentifier():
-                return None
-            ops[key] = op
-    else:
-        for st in loop.body:
-            if not (isinstance(st, ast.Assign) and isinstance(st.targets[0], ast.Name)):
-                return None
-            op = loop_ir.reduction_operator(st)
-            name = st.targets[0].id
-            if op is None or ops.setdefault(name, op) != op:
-                return None
-        for name in ops:    # the running value is not looked at inside the loop
-            if any(_uses_name(loop_ir.reduction_operand(s2), name) for s2 in loop.body):
-                return None
-        if not ops:
+    for st in loop.body:
+        if not (isinstance(st, ast.Assign) and isinstance(st.targets[0], ast.Name)):
             return None
+        op = loop_ir.reduction_operator(st)
+        name = st.targets[0].id
+        if op is None or ops.setdefault(name, op) != op:
+            return None
+    for name in ops:    # the running value is not looked at inside the loop
+        if any(_uses_name(loop_ir.reduction_operand(s2), name) for s2 in loop.body):
+            return None
+    if not ops:
+        return None
     if any(_uses_name(a, n) for a in loop.iter.args for n in ops):
         return None
     return pre, loop, post, ops
@@ -444,14 +492,14 @@ class KernelBuilder:
     def block(self, stmts):
         i = 0
         while i < len(stmts):
-            if self.mode == "team" and self.spec.extent:
-                used = self.row_accumulate(stmts, i)
+            if self.mode == "team" and self.spec.kind == "team":
+                used = self.row_accumulate(stmts, i) if self.spec.extent else 0
                 if used:
                     i += used
                     continue
-            if self.mode == "team" and self.interchange_row_update(stmts[i]):
-                i += 1
-                continue
+                if self.interchange_row_update(stmts[i]):
+                    i += 1
+                    continue
             self.stmt(stmts[i])
             i += 1
 
@@ -593,7 +641,10 @@ class KernelBuilder:
 
     def for_(self, st: ast.For):
         pragma = getattr(st, "pragma", None) or {}
-        if self.mode == "team" and "simd" in pragma:
+        if self.spec.kind == "strip":
+            if self.mode == "team" and id(st) in self.a.strip:
+                return self.strip_spread_loop(st)
+        elif self.mode == "team" and "simd" in pragma:
             return self.spread_loop(st)
         var = st.target.id
         lo, hi = self._range_args(st)
@@ -696,6 +747,8 @@ class KernelBuilder:
 
     def _leader(self) -> str:
         """Condition under which a team-level statement has its side effect."""
+        if self.spec.kind == "strip":
+            return "__wave == 0 && __active"
         return "__lane == 0 && __active" if self.lds_plan else "__lane == 0"
 
     def _vst(self) -> str:
@@ -1154,91 +1207,100 @@ class KernelBuilder:
                 self.w(f"appy::{self._vst()}<{arr.elem_c}, {V}>({self._addr(arr, sub, var, base)}, {sregs[(u, key)]});")
 
     def _body_strip(self):
-        """Column reductions: the 64 lanes of a wavefront take 64 consecutive outer
-        iterations (so that ``A[j, i]`` is one contiguous row segment per step),
-        the wavefronts of the workgroup share out the iterations of the inner
-        loop, their partial results meet in LDS and the first wavefront finishes
-        the iteration."""
+        """Column loops: the 64 lanes of a wavefront take 64 consecutive outer
+        iterations (so that ``A[j, i]`` is one contiguous row segment per step) and
+        the wavefronts of the workgroup are the team of each of them: statements
+        outside the shared-out loops run on every wavefront with equal values and
+        store from wavefront 0, the shared-out loops deal their iterations to the
+        wavefronts, partial results meet in LDS.  Lanes past the end of the range
+        run on the last iteration with their effects switched off, so that every
+        thread reaches every barrier."""
         if self.a.strip is None or self.a.outer_reductions:
-            raise Unsupported("the loop does not have the shape of a column reduction")
-        pre, loop, post, ops = self.a.strip
-        B = self.spec.block
-        NW = B // 64
+            raise Unsupported("the loop nest does not suit the strip shape")
+        NW = self.spec.block // 64
         var = self.a.var
         self.ex.locals[var] = T.WEAK_INT
         self.w("const int __lane = threadIdx.x & 63;")
         self.w("const int __wave = threadIdx.x >> 6;")
-        slots = {}
-        for name in ops:
-            ty = self.ex.locals.get(name)
-            if ty is None:
-                continue        # typed by the first pass over `pre`
-            pty = T.F32 if (ty.is_float and ty.size < 4) else ty
-            slots[name] = pty
-            self.w(f"__shared__ {pty.c} __strip_{cname(name)}[{NW}][64];")
+        self.w(f"__shared__ double __strip_slots[{NW}][64];   // one slot per wavefront and lane, any 4- or 8-byte type")
         self.w("for (appy::i64 __s = blockIdx.x; __lo + __s * 64 < __hi; __s += gridDim.x) {")
         self.ind += 1
-        self.w(f"const appy::i64 {cname(var)} = __lo + __s * 64 + __lane;")
-        self.w(f"const bool __active = {cname(var)} < __hi;")
+        self.w("const bool __active = __lo + __s * 64 + __lane < __hi;")
+        self.w(f"const appy::i64 {cname(var)} = __active ? __lo + __s * 64 + __lane : __hi - 1;")
         self._declare_locals()
-        for name, pty in slots.items():
-            self.w(f"{pty.c} __part_{cname(name)} = {T.identity_literal(ops[name], pty)};")
-        self.w("if (__active) {")
+        self.mode = "team"
+        self.block(self.a.outer.body)
+        self.mode = "lane"
+        self.ind -= 1
+        self.w("}")
+
+    def strip_spread_loop(self, st: ast.For):
+        """A loop of a strip kernel whose iterations are dealt to the wavefronts."""
+        ops = self.a.strip[id(st)]
+        NW = self.spec.block // 64
+        var = st.target.id
+        lo, hi = self._range_args(st)
+        self.ex.locals[var] = T.WEAK_INT
+        self.w("{")
         self.ind += 1
-        self.block(pre)
-        jv = loop.target.id
-        lo, hi = self._range_args(loop)
-        self.ex.locals[jv] = T.WEAK_INT
-        hi_v = self.fresh("hi")
+        lo_v, hi_v = self.fresh("lo"), self.fresh("hi")
+        self.w(f"const appy::i64 {lo_v} = {lo};")
         self.w(f"const appy::i64 {hi_v} = {hi};")
+        saved_partials = dict(self.partials)
+        typed = {}
+        for name, op in ops.items():
+            ty = self.ex.locals.get(name)
+            if ty is None:
+                raise NameError(f"reduction variable `{name}` has no value before the loop")
+            pty = T.F32 if (ty.is_float and ty.size < 4) else ty
+            if pty.size < 4:
+                raise Unsupported(f"Reduction variable `{name}` of type {ty.name} is not supported")
+            p = self.fresh(f"part_{name}_")
+            typed[name] = (p, pty)
+            self.partials[name] = (p, pty)
+            self.w(f"{pty.c} {p} = {T.identity_literal(op, pty)};")
+        saved_mode, self.mode = self.mode, "lane"
+        saved_depth, self.seq_depth = self.seq_depth, 0
         saved_stream = set(self.ex.stream_arrays)
         if self.spec.stream_loads:
             # matrices walked once by the launch (indexed by both loop variables) bypass the caches
-            for st in loop.body:
-                for n in ast.walk(st):
+            for b in st.body:
+                for n in ast.walk(b):
                     if (isinstance(n, ast.Subscript) and isinstance(n.value, ast.Name) and n.value.id in self.a.arrays
-                            and _uses_name(n, jv) and _uses_name(n, var)):
+                            and _uses_name(n, var) and _uses_name(n, self.a.var)):
                         self.ex.stream_arrays.add(n.value.id)
+        # lanes past the end of the range skip the loop as a whole (its bounds stay wavefront-uniform,
+        # which keeps the unrolled loads of a step in flight together); the barriers are outside
+        self.w("if (__active) {")
+        self.ind += 1
         self.w(f"#pragma unroll {max(4, self.spec.unroll)}")
-        self.w(f"for (appy::i64 {cname(jv)} = {lo} + __wave; {cname(jv)} < {hi_v}; {cname(jv)} += {NW}) {{")
+        self.w(f"for (appy::i64 {cname(var)} = {lo_v} + __wave; {cname(var)} < {hi_v}; {cname(var)} += {NW}) {{")
         self.ind += 1
-        saved = dict(self.partials)
-        if len(slots) == len(ops):
-            for name, pty in slots.items():
-                self.partials[name] = (f"__part_{cname(name)}", pty)
-        # (while a reduced scalar still has no type, the pass only serves to type the
-        # locals: its updates are emitted as ordinary assignments and the pass is repeated)
-        for st in loop.body:
-            if (isinstance(st, ast.Assign) and isinstance(st.targets[0], ast.Name)
-                    and st.targets[0].id in ops and not hasattr(st, "reduce")):
-                st.reduce = ops[st.targets[0].id]
-        self.iteration_body(loop.body)
-        self.partials = saved
+        self.iteration_body(st.body)
+        self.ind -= 1
+        self.w("}")
+        self.ind -= 1
+        self.w("}")
         self.ex.stream_arrays = saved_stream
-        self.ind -= 1
-        self.w("}")
-        self.ind -= 1
-        self.w("}")
-        for name in slots:
-            self.w(f"__strip_{cname(name)}[__wave][__lane] = __part_{cname(name)};")
-        self.w("__syncthreads();")
-        self.w("if (__wave == 0 && __active) {")
-        self.ind += 1
-        for name, pty in slots.items():
-            vty = self.ex.locals[name]
+        self.mode, self.seq_depth = saved_mode, saved_depth
+        self.partials = saved_partials
+        stores = any(isinstance(n, ast.Assign) and isinstance(n.targets[0], ast.Subscript)
+                     for b in st.body for n in ast.walk(b))
+        if stores and not typed:
+            self.w("__syncthreads();   // what one wavefront stored, the others may read from here on")
+        for name, (p, pty) in typed.items():
             op = _OPS[ops[name]]
-            self.w(f"for (int __w = 1; __w < {NW}; ++__w) __part_{cname(name)} = "
-                   f"{op}::f<{pty.c}>(__part_{cname(name)}, __strip_{cname(name)}[__w][__lane]);")
-            total = f"{op}::f<{pty.c}>({cast(cname(name), vty, pty)}, __part_{cname(name)})"
-            self.w(f"{cname(name)} = {cast(total, pty, vty)};")
-        self.block(post)
+            vty = self.ex.locals[name]
+            slot = f"reinterpret_cast<{pty.c}*>(&__strip_slots[0][0])"
+            self.w(f"{slot}[__wave * 64 + __lane] = {p};")
+            self.w("__syncthreads();")
+            t = self.fresh("tot")
+            self.w(f"{pty.c} {t} = {slot}[__lane];")
+            self.w(f"for (int __w = 1; __w < {NW}; ++__w) {t} = {op}::f<{pty.c}>({t}, {slot}[__w * 64 + __lane]);")
+            self.w(f"{cname(name)} = {cast(op + '::f<' + pty.c + '>(' + cast(cname(name), vty, pty) + ', ' + t + ')', pty, vty)};")
+            self.w("__syncthreads();   // the slots are free again")
         self.ind -= 1
         self.w("}")
-        self.w("__syncthreads();   // the slots are free for the next strip")
-        self.ind -= 1
-        self.w("}")
-        if len(slots) != len(ops):
-            self.dirty = True
 
     def _find_lds_plan(self):
         """A ``simd`` loop directly in the body of the parallel loop whose bounds

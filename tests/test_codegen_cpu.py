@@ -377,11 +377,28 @@ def test_column_reductions_take_the_strip_shape():
     assert (sp.kind, sp.block) == ("strip", 1024)
     assert f.grid_for(sp, 300) == 5
     k = body_of(f.kernel_for(sp).src.text)
-    assert "__shared__ float __strip_s[16][64];" in k and "__shared__ float __strip_m[16][64];" in k
-    assert "j += 16" in k and k.count("__syncthreads();") == 2 and "if (__wave == 0 && __active)" in k
-    assert "appy::OpMax::f<float>(__part_m" in k
+    assert "__shared__ double __strip_slots[16][64];" in k
+    assert "j += 16" in k and k.count("__syncthreads();") == 4 and "if (__wave == 0 && __active)" in k
+    assert "appy::OpMax::f<float>(__part_m" in k and "if (__active) {" in k
     # short inner loops stay with one lane per iteration
     assert f.choose_spec(300, {"n": 300, "r": 8, "beta": 1.5}, {"A": A, "y": y, "x": x}).kind == "flat"
+    # several shared-out loops, one of them under a sequential loop with the same bounds for every column
+    multi = ("#pragma parallel for\nfor j in range(0, n, 1):\n    s = 0.0\n    #pragma simd\n    for c in range(0, r, 1):\n"
+             "        s += Q[c, k] * A[c, j]\n    R[k, j] = s\n    for t in range(0, 3, 1):\n        #pragma simd\n"
+             "        for c in range(0, r, 1):\n            A[c, j] = A[c, j] - Q[c, k] * s\n")
+    Q = np.zeros((512, 300), np.float32)
+    R = np.zeros((300, 300), np.float32)
+    h, _ = compiled(multi, n=300, r=512, k=2, A=A, Q=Q, R=R)
+    assert h.analysis.kind == "team" and len(h.analysis.strip) == 2
+    hs = h.choose_spec(300, {"n": 300, "r": 512, "k": 2}, {"A": A, "Q": Q, "R": R})
+    assert hs.kind == "strip"
+    hk = body_of(h.kernel_for(hs).src.text)
+    assert hk.count("c += 16") == 2 and "if (__wave == 0 && __active) { R[" in hk and hk.count("__syncthreads();") == 3
+    # barriers under bounds or conditions that differ between columns: not a strip
+    for bad in ("    for t in range(0, j, 1):\n        #pragma simd\n        for c in range(0, r, 1):\n            A[c, j] = A[c, j] * 2.0\n",
+                "    if Q[0, j] > 0.0:\n        #pragma simd\n        for c in range(0, r, 1):\n            A[c, j] = A[c, j] * 2.0\n"):
+        b, _ = compiled("#pragma parallel for\nfor j in range(0, n, 1):\n" + bad, n=300, r=512, A=A, Q=Q)
+        assert b.analysis.strip is None
     # a running value that the loop looks at is not a column reduction
     g, _ = compiled("#pragma parallel for\nfor i in range(0, n, 1):\n    s = 0.0\n    for j in range(0, r, 1):\n"
                     "        s = s * 0.5 + A[j, i]\n    x[i] = s\n", n=300, r=512, A=A, x=x)

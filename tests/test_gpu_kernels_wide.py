@@ -497,3 +497,46 @@ def test_column_updates_run_as_strips(gpu):
     for name in ("scale_columns", "subtract_from_columns"):
         loop = [v[0] for kk, v in cg.code_cache.items() if kk[-1] == name][-1]
         assert loop.last_launch.spec.kind == "strip", name
+
+
+def test_gramschmidt_columns_run_as_strips_with_two_shared_out_loops(gpu):
+    """Tall matrix: both column loops of the Gram-Schmidt step are dealt to the
+    wavefronts of a strip (a reduction, then an update that uses its result)."""
+    from appy_amd.backends.hip import codegen as cg
+
+    rng = np.random.default_rng(9)
+    A = rng.random((700, 130)) + np.eye(700, 130)
+    Q, R = gramschmidt(A.copy())
+    assert np.allclose(Q @ R, A, atol=1e-10)
+    assert np.allclose(Q.T @ Q, np.eye(130), atol=1e-9)
+    loop = [v[0] for kk, v in cg.code_cache.items() if kk[-1] == "gramschmidt"][-1]
+    assert loop.last_launch.spec.kind == "strip" and len(loop.analysis.strip) == 2
+
+
+@appy.jit
+def repeated_column_smoothing(A, rounds):
+    #pragma parallel for
+    for j in range(A.shape[1]):
+        for t in range(rounds):
+            m = 0.0
+            #pragma simd
+            for i in range(A.shape[0]):
+                m += A[i, j]
+            m = m / A.shape[0]
+            #pragma simd
+            for i in range(A.shape[0]):
+                A[i, j] = 0.5 * (A[i, j] + m)
+
+
+def test_strip_loops_inside_a_sequential_loop_with_uniform_bounds(gpu):
+    from appy_amd.backends.hip import codegen as cg
+
+    rng = np.random.default_rng(10)
+    A = rng.standard_normal((333, 201))
+    ref = A.copy()
+    for _ in range(3):
+        ref = 0.5 * (ref + ref.mean(axis=0))
+    repeated_column_smoothing(A, 3)
+    assert np.allclose(A, ref, rtol=1e-12, atol=1e-12)
+    loop = [v[0] for kk, v in cg.code_cache.items() if kk[-1] == "repeated_column_smoothing"][-1]
+    assert loop.last_launch.spec.kind == "strip"
