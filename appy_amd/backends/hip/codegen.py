@@ -264,6 +264,16 @@ class CompiledLoop:
                 ast.BinOp(left=_copy(hi), op=ast.Sub(), right=_copy(lo)))), "<trip>", "eval")
         self.kernels = {}   # Spec -> Kernel
         self._replays = {}  # call identity -> Launch that can simply be launched again
+        # scalars that no host-side decision looks at (range of the loop, inner trip counts,
+        # row extents): a replayed launch may carry new values of these
+        steering = set()
+        for n in ast.walk(a.outer):
+            if isinstance(n, ast.For):
+                for arg in n.iter.args:
+                    steering.update(x.id for x in ast.walk(arg) if isinstance(x, ast.Name))
+        self._value_only = [i for i, k in enumerate(self.arg_names)
+                            if k in a.scalars and k not in steering and k not in a.assigned]
+        self._value_only_set = set(self._value_only)
         self._replayable = not self.options.get("check_bounds")
         self._lock = threading.Lock()
         # default variant now: generation / compilation errors surface at first use of the loop
@@ -539,7 +549,16 @@ class CompiledLoop:
                 # same tensors (address, shape, strides), same scalars, same stream: the staged
                 # launch of last time is still exact, so only the launch itself is repeated
                 _ensure_device(plan.device)
-                rt.launch(plan.function(), plan.grid, plan.block, plan.args, plan.stream)
+                if self._value_only:
+                    with self._lock:        # the argument block is shared by all replays of this plan
+                        for i in self._value_only:
+                            fname = plan.scalar_fields.get(self.arg_names[i])
+                            if fname is not None:
+                                v = args[i]
+                                setattr(plan.args, fname, v.item() if isinstance(v, np.generic) else v)
+                        rt.launch(plan.function(), plan.grid, plan.block, plan.args, plan.stream)
+                else:
+                    rt.launch(plan.function(), plan.grid, plan.block, plan.args, plan.stream)
                 self.last_launch = plan
                 return
         vals = dict(zip(self.arg_names, args))
@@ -559,12 +578,13 @@ class CompiledLoop:
             return None
         key = []
         device = -1
-        for v in args:
+        free = self._value_only_set
+        for i, v in enumerate(args):
             t = type(v)
             if t is int or t is float or t is bool:
-                key.append((t, v))
+                key.append(t if i in free else (t, v))
             elif isinstance(v, np.generic):
-                key.append((v.dtype.num, v.item()))
+                key.append(v.dtype.num if i in free else (v.dtype.num, v.item()))
             elif hasattr(v, "data_ptr"):        # a tensor
                 if not v.is_cuda:
                     return None
@@ -683,6 +703,7 @@ class Launch:
         self.kernel = loop.kernel_for(spec)
         self.spec = spec
         st = self.kernel.ArgStruct()
+        self.scalar_fields = {}      # by-value scalar -> field of the argument block
         for fname, p in zip(self.kernel._field_names, self.kernel.src.params):
             if p.role == "array":
                 val = self.ptr[p.source]
@@ -694,6 +715,7 @@ class Launch:
                     val = int(arrays[an].shape[dim])
                 else:
                     val = vals[p.source]
+                    self.scalar_fields[p.source] = fname
                     if isinstance(val, np.generic):
                         val = val.item()
             elif p.role == "shape":

@@ -410,8 +410,24 @@ def test_repeated_calls_on_gpu_tensors_replay_the_staged_launch(gpu):
     scaled_add(a, b, c, 2.0)
     assert loop.last_launch is first                          # replayed ...
     assert torch.equal(c, a * 2.0 + b)                        # ... on the tensors' current contents
-    scaled_add(a, b, c, 5.0)                                  # another scalar
-    assert loop.last_launch is not first and torch.equal(c, a * 5.0 + b)
+    scaled_add(a, b, c, 5.0)                                  # a scalar that only the kernel looks at: patched in
+    assert loop.last_launch is first and torch.equal(c, a * 5.0 + b)
+    scaled_add(a, b, c, 2)                                    # another type of scalar: another kernel altogether
+    assert torch.equal(c, a * 2 + b)
+
+    @appy.jit
+    def fill_from(c, start, v):
+        #pragma parallel for simd
+        for i in range(start, c.shape[0]):
+            c[i] = v
+
+    fill_from(c, 10, 1.0)
+    fl = [v[0] for kk, v in cg.code_cache.items() if kk[-1] == "fill_from"][-1]
+    plan = fl.last_launch
+    fill_from(c, 10, 3.0)                                     # `v` travels with the replay ...
+    assert fl.last_launch is plan and bool((c[10:] == 3.0).all())
+    fill_from(c, 500, 4.0)                                    # ... `start` steers the range: staged again
+    assert fl.last_launch is not plan and bool((c[10:500] == 3.0).all()) and bool((c[500:] == 4.0).all())
     c2 = torch.zeros(500, dtype=torch.float64, device="cuda")
     scaled_add(a[:500], b[:500], c2, 2.0)                     # other shapes
     assert torch.equal(c2, a[:500] * 2.0 + b[:500])
