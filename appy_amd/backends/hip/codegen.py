@@ -857,8 +857,8 @@ class Launch:
 
 def _overlaps(extents) -> bool:
     """True if a stored array shares bytes with any other array argument."""
-    for i, (n1, p1, s1, st1) in enumerate(extents):
-        for j, (n2, p2, s2, st2) in enumerate(extents):
+    for i, (_n1, p1, s1, st1) in enumerate(extents):
+        for j, (_n2, p2, s2, st2) in enumerate(extents):
             if i >= j or not (st1 or st2):
                 continue
             if p1 < p2 + s2 and p2 < p1 + s1:

@@ -605,7 +605,7 @@ class KernelBuilder:
             raise Unsupported(f"`{tgt.value.id}` is subscripted but is not an array argument")
         vc, vt = self.ex.emit(st.value)
         if key in self.store_subst:
-            lv, lty = self.store_subst[key]
+            lv, _lty = self.store_subst[key]
             self.w(f"{lv} = {self._store_value(vc, vt, arr)};")
             self.ex.load_subst[key] = ((f"({lv} != 0)" if arr.ty.is_bool else lv), arr.ty)
             return
@@ -950,7 +950,7 @@ class KernelBuilder:
         self.ex.locals[c] = T.WEAK_INT
         self.w("{")
         self.ind += 1
-        ec, et = self.ex.emit(hi)
+        self.ex.emit(hi)     # registers the extent as a kernel argument
         self.w(f"// row accumulators: extent {E} is fixed at compile time (asserted by the launcher)")
         accs = [self.fresh("acc") for _ in range(nv)]
         bases = [f"(({t * W}LL + __lane) * {V})" for t in range(nv)]
@@ -1417,7 +1417,6 @@ class KernelBuilder:
         saved_mode, self.mode = self.mode, "lane"
         saved_depth, self.seq_depth = self.seq_depth, 0
         loads, stores = self._vector_accesses(st.body, var) if V > 1 else ({}, {})
-        staged_names = {a.name for a in staged}
         staged_keys = {f"{a.name}[{var}]" for a in staged}
         if V > 1 and (loads or stores):
             nv = self.fresh("nv")
@@ -1430,7 +1429,6 @@ class KernelBuilder:
             self.w(f"const appy::i64 {base} = {jt} + {q} * {V};")
             global_loads = {k: v for k, v in loads.items() if k not in staged_keys}
             saved_loads = dict(self.ex.load_subst)
-            comp = "xyzw"
             regs = {}
             for key in staged_keys & set(loads):
                 arr = loads[key][0]

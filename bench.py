@@ -74,7 +74,6 @@ class Runner:
         """Returns dict(ms_per_step, gbps_step, kernel_ms, gbps_kernel, frac, spec, grid)."""
         torch, rt = self.torch, self.rt
         launch = loop.prepare(vals)
-        stream = launch.stream
 
         def step():
             if clear is not None:
