@@ -39,6 +39,9 @@ from . import dtypes as T
 from .dtypes import Ty
 from .exprs import ArrayParam, ExprEmitter, cast, cname, truth
 
+# accessors of the components of a vector register (the first four also have the usual names)
+_COMPONENTS = ["x", "y", "z", "w"] + [f"s{d:x}" for d in range(4, 16)]
+
 _OPS = {"+": "appy::OpAdd", "*": "appy::OpMul", "max": "appy::OpMax", "min": "appy::OpMin"}
 
 _CTYPES = {
@@ -74,8 +77,8 @@ class Spec:
             raise ValueError(f"kernel shape must be 'flat', 'team' or 'strip', got {self.kind!r}")
         if self.block % 64 or not 64 <= self.block <= 1024:
             raise ValueError(f"workgroup size must be a multiple of 64 up to 1024, got {self.block}")
-        if self.vec not in (1, 2, 4):
-            raise ValueError(f"vector width must be 1, 2 or 4, got {self.vec}")
+        if self.vec not in (1, 2, 4, 8, 16):
+            raise ValueError(f"vector width must be 1, 2, 4, 8 or 16, got {self.vec}")
         if not 1 <= self.unroll <= 8:
             raise ValueError(f"unroll factor must be 1..8, got {self.unroll}")
         if not pow2(self.width) or (self.width > 64 and self.width != self.block):
@@ -770,7 +773,7 @@ class KernelBuilder:
         """Emit V consecutive iterations starting at ``base_code``: vector
         loads first, the V scalar bodies, vector stores last."""
         regs = {}
-        comp = "xyzw"
+        comp = _COMPONENTS
         for key, (arr, sub) in loads.items():
             r = self.fresh(f"ld_{arr.name}_")
             regs[key] = r
@@ -946,7 +949,7 @@ class KernelBuilder:
         if nv > 8:
             return 0
         vt = f"appy::vec<{arr.elem_c}, {V}>::type"
-        comp = "xyzw"
+        comp = _COMPONENTS
         self.ex.locals[c] = T.WEAK_INT
         self.w("{")
         self.ind += 1
@@ -1033,7 +1036,7 @@ class KernelBuilder:
         arr.loaded = True
         W, V = self.spec.width, self.spec.vec
         sym = {ast.Add: "+", ast.Sub: "-", ast.Mult: "*"}[type(op)]
-        comp = "xyzw"
+        comp = _COMPONENTS
         self.w("{")
         self.ind += 1
         self.w("// loops interchanged: the row elements stay in registers across the sequential loop")
@@ -1165,7 +1168,7 @@ class KernelBuilder:
         self.w("}")
 
     def _flat_unrolled_tile(self, V, U, B, loads, stores):
-        comp = "xyzw"
+        comp = _COMPONENTS
         var = self.a.var
         regs = {}
         for u in range(U):

@@ -413,3 +413,17 @@ def test_triangular_simd_loops_get_teams_sized_by_their_mean_length():
     assert f.choose_spec(1200, {"n": 1200, "beta": 1.2, "__appy_mid": 600}, {"C": C}).width == 32
     assert f.choose_spec(1200, {"n": 1200, "beta": 1.2}, {"C": C}).width == 32     # nothing known: a middling team (64 / V)
     assert f.choose_spec(16, {"n": 16, "beta": 1.2, "__appy_mid": 8}, {"C": C}).width == 8
+
+
+def test_small_element_types_move_16_bytes_per_lane_too():
+    a8 = np.zeros(64, np.uint8)
+    f, src = compiled("#pragma parallel for simd\nfor i in range(n):\n    c[i] = a[i] + b[i]", c=a8.copy(), a=a8, b=a8, n=64)
+    assert f.default_spec.vec == 16 and "appy::vload<unsigned char, 16>" in body_of(src) and ".sf" in body_of(src)
+    a16 = np.zeros(64, np.float16)
+    g, src = compiled("#pragma parallel for simd\nfor i in range(n):\n    c[i] = a[i] * 2", c=a16.copy(), a=a16, n=64)
+    assert g.default_spec.vec == 8 and "appy::vstore<_Float16, 8>" in body_of(src)
+    # the widest element decides: a byte mask next to float32 data keeps 4 elements per lane
+    m = np.zeros(64, bool)
+    x = np.zeros(64, np.float32)
+    h, _ = compiled("#pragma parallel for simd\nfor i in range(n):\n    c[i] = x[i] if m[i] else 0.0", c=x.copy(), x=x, m=m, n=64)
+    assert h.default_spec.vec == 4
