@@ -295,6 +295,22 @@ class CompiledLoop:
     def _elem_sizes(self):
         return list(self._indexed_arrays().values()) or [4]
 
+    def _simd_elem_sizes(self):
+        """Element sizes of the arrays that ``simd`` loops walk with their own
+        variable in the contiguous dimension (what a team streams; the per-row
+        result ``y[i]`` does not count)."""
+        sizes = []
+        for lp in ast.walk(self.analysis.outer):
+            if not (isinstance(lp, ast.For) and lp is not self.analysis.outer
+                    and "simd" in (getattr(lp, "pragma", None) or {}) and isinstance(lp.target, ast.Name)):
+                continue
+            for n in ast.walk(lp):
+                if (isinstance(n, ast.Subscript) and isinstance(n.value, ast.Name) and n.value.id in self.analysis.arrays):
+                    last = n.slice.elts[-1] if isinstance(n.slice, ast.Tuple) else n.slice
+                    if any(isinstance(x, ast.Name) and x.id == lp.target.id for x in ast.walk(last)):
+                        sizes.append(self.analysis.arrays[n.value.id].ty.size)
+        return sizes
+
     def _default_spec(self) -> Spec:
         a = self.analysis
         widest = max(self._elem_sizes())
@@ -307,6 +323,11 @@ class CompiledLoop:
             # with or without `simd`: iterations of a parallel loop are independent, and
             # lanes handle control flow on their own, so both forms take the vector shape
             return Spec("flat", block=256, vec=v, unroll=2)
+        # teams: 16 bytes per lane of the widest element the simd loops stream, at most 8
+        # elements (int8 GEMV 16384^2: 0.33 of peak with 2 elements per lane, 0.74 with 8)
+        inner = self._simd_elem_sizes()
+        if inner:
+            v = max(1, min(8, 16 // max(inner)))
         return Spec("team", block=256, vec=v, width=64)
 
     def kernel_for(self, spec: Spec) -> Kernel:
