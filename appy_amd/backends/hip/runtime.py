@@ -12,7 +12,7 @@ import threading
 _LIB_NAME = "libappy_hip.so"
 _PKG_ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 
 class Props(C.Structure):

@@ -24,7 +24,9 @@
 extern "C" {
 #endif
 
-#define APPY_HIP_ABI_VERSION 1
+/* 2: page-locked host memory, streams and graphs, appy_hip_rtc_version (additions only:
+ * every entry point of version 1 is unchanged). */
+#define APPY_HIP_ABI_VERSION 2
 
 typedef struct appy_hip_props {
     char     name[128];        /* marketing name */
