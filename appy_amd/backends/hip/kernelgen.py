@@ -606,6 +606,9 @@ class KernelBuilder:
         arr = self.a.arrays.get(tgt.value.id)
         if arr is None:
             raise Unsupported(f"`{tgt.value.id}` is subscripted but is not an array argument")
+        shared_update = self._shared_update(st)
+        if shared_update is not None:
+            return self._atomic_update(st, arr, *shared_update)
         vc, vt = self.ex.emit(st.value)
         if key in self.store_subst:
             lv, _lty = self.store_subst[key]
@@ -626,6 +629,58 @@ class KernelBuilder:
             self.w(store)
         # a later read of the same element in this iteration goes to memory again
         self.ex.load_subst.pop(key, None)
+
+    def _shared_update(self, st: ast.Assign):
+        """``X[idx] = X[idx] op e`` on an element that other iterations of the
+        parallel loop may update as well (no index is the parallel variable plus a
+        constant: ``hist[bin[i]] += 1``, ``colsum[j] += A[i, j]``): returns
+        ``(op, e)`` - such an update has to be atomic.  None for updates of
+        elements that belong to the iteration, and for plain stores."""
+        tgt = st.targets[0]
+        if any(_var_offset(e, self.a.var) is not None for e in _elts(tgt)):
+            return None
+        key = ast.unparse(tgt)
+        val = st.value
+        if isinstance(val, ast.BinOp) and isinstance(val.op, (ast.Add, ast.Sub, ast.Mult)):
+            if ast.unparse(val.left) == key:
+                other = val.right
+            elif ast.unparse(val.right) == key and not isinstance(val.op, ast.Sub):
+                other = val.left
+            else:
+                return None
+            op = {ast.Add: "+", ast.Sub: "-", ast.Mult: "*"}[type(val.op)]
+        elif (isinstance(val, ast.Call) and isinstance(val.func, ast.Name) and val.func.id in ("max", "min")
+              and len(val.args) == 2 and any(ast.unparse(a) == key for a in val.args)):
+            other = val.args[1] if ast.unparse(val.args[0]) == key else val.args[0]
+            op = val.func.id
+        else:
+            return None
+        if any(isinstance(n, ast.Subscript) and ast.unparse(n) == key for n in ast.walk(other)):
+            return None
+        return op, other
+
+    def _atomic_update(self, st, arr: ArrayParam, op: str, other):
+        if arr.ty.size < 4:
+            raise Unsupported(f"`{ast.unparse(st.targets[0])}` is updated by several iterations of the parallel loop; "
+                              f"atomic updates of {arr.ty.name} elements are not supported")
+        oc, ot = self.ex.emit(other)
+        val = cast(oc, ot, arr.ty)
+        if op == "-":
+            op, val = "+", f"(-{val})"
+        tgt = st.targets[0]
+        if self.spec.checked:
+            idx = self.ex.index_code(arr, tgt, check=False)
+            guard = f"if ({self.ex.inside_code(arr, tgt)}) "
+            tail = f" else appy::report(__oob, {self.ex.site(tgt)});"
+        else:
+            idx, guard, tail = self.ex.index_code(arr, tgt), "", ""
+        arr.loaded = True
+        upd = f"{guard}appy::atomic_combine<{_OPS[op]}, {arr.elem_c}>::run(&{cname(arr.name)}[{idx}], {val});{tail}"
+        if self.mode == "team":
+            self.w(f"if ({self._leader()}) {{ {upd} }}")
+        else:
+            self.w(upd)
+        self.ex.load_subst.pop(ast.unparse(tgt), None)
 
     def _store_value(self, vc, vt, arr: ArrayParam):
         if arr.ty.is_bool:
@@ -697,7 +752,10 @@ class KernelBuilder:
                         loads[key] = (arr, n)
                 else:
                     top = any(isinstance(t, ast.Assign) and t.targets[0] is n for t in body)
-                    if ok and top and not skips:
+                    owner = next((t for t in body if isinstance(t, ast.Assign) and t.targets[0] is n), None)
+                    if owner is not None and self._shared_update(owner) is not None:
+                        blocked.add(arr.name)       # updated atomically, element by element
+                    elif ok and top and not skips:
                         stores[key] = (arr, n)
                     else:
                         blocked.add(arr.name)
@@ -898,6 +956,8 @@ class KernelBuilder:
         el = _elts(tgt)
         if not (isinstance(el[-1], ast.Name) and el[-1].id == c) or any(_uses_name(e, c) for e in el[:-1]):
             return None
+        if not any(_var_offset(e, self.a.var) is not None for e in el):
+            return None     # a row that other outer iterations update as well cannot live in registers
         key = ast.unparse(tgt)
         arr_name = tgt.value.id
         val = st.value

@@ -427,3 +427,20 @@ def test_small_element_types_move_16_bytes_per_lane_too():
     x = np.zeros(64, np.float32)
     h, _ = compiled("#pragma parallel for simd\nfor i in range(n):\n    c[i] = x[i] if m[i] else 0.0", c=x.copy(), x=x, m=m, n=64)
     assert h.default_spec.vec == 4
+
+
+def test_updates_of_elements_shared_between_iterations_are_atomic():
+    h = np.zeros(16, np.int64)
+    b = np.zeros(64, np.int32)
+    w = np.zeros(64, np.float32)
+    f, src = compiled("#pragma parallel for simd\nfor i in range(n):\n    hist[b[i]] += 1\n    top[0, b[i]] = max(top[0, b[i]], w[i])\n"
+                      "    own[i] += w[i]\n", hist=h, b=b, w=w, top=np.zeros((1, 16), np.float32), own=w.copy(), n=64)
+    k = body_of(src)
+    assert "appy::atomic_combine<appy::OpAdd, long long>::run(&hist[" in k
+    assert "appy::atomic_combine<appy::OpMax, float>::run(&top[" in k
+    assert "atomic_combine<appy::OpAdd, float>" not in k and "vstore<float, 2>(own" in k     # own[i] belongs to the iteration
+    g, src = compiled("#pragma parallel for\nfor i in range(n):\n    #pragma simd\n    for j in range(m):\n        col[j] -= A[i, j]\n",
+                      col=np.zeros(32), A=np.zeros((8, 32)), n=8, m=32)
+    assert "appy::atomic_combine<appy::OpAdd, double>::run(&col[" in body_of(src) and "(-" in body_of(src)
+    with pytest.raises(NotImplementedError, match="atomic updates of int16"):
+        compiled("#pragma parallel for simd\nfor i in range(n):\n    hist[b[i]] += 1\n", hist=np.zeros(16, np.int16), b=b, n=64)

@@ -394,3 +394,43 @@ def test_check_bounds_reports_instead_of_faulting(gpu):
         shifted_store(a, out)
     checked(data, indptr, indices, x, y2)            # the runtime is fine afterwards
     assert np.allclose(y1, y2, rtol=1e-5, atol=1e-5)
+
+
+def test_updates_shared_between_iterations_are_atomic(gpu):
+    """Histograms and sums that several iterations of the parallel loop feed
+    (no index is the loop variable itself) are updated atomically; the reference's
+    guide describes ``a[j] += b[i, j]`` under ``prange(i)`` as a reduction with
+    regard to ``i`` (docs/source/developer.rst, "Reduction Detection")."""
+    import appy_amd as appy
+    from appy_amd import prange
+
+    @appy.jit
+    def histogram(bins, weights, hist, wsum, wmax):
+        #pragma parallel for simd
+        for i in range(bins.shape[0]):
+            hist[bins[i]] += 1
+            wsum[bins[i]] += weights[i]
+            wmax[bins[i]] = max(wmax[bins[i]], weights[i])
+
+    @appy.jit
+    def column_sums(a, b):
+        for i in prange(b.shape[0]):
+            for j in range(b.shape[1]):
+                a[j] += b[i, j]
+
+    rng = np.random.default_rng(17)
+    n, nb = 1_000_003, 97
+    bins = rng.integers(0, nb, n).astype(np.int32)
+    weights = rng.random(n)
+    hist, wsum, wmax = np.zeros(nb, np.int64), np.zeros(nb), np.full(nb, -1.0)
+    histogram(bins, weights, hist, wsum, wmax)
+    assert np.array_equal(hist, np.bincount(bins, minlength=nb))
+    assert np.allclose(wsum, np.bincount(bins, weights=weights, minlength=nb), rtol=1e-11)
+    ref_max = np.full(nb, -1.0)
+    np.maximum.at(ref_max, bins, weights)
+    assert np.array_equal(wmax, ref_max)
+
+    b = rng.standard_normal((700, 333)).astype(np.float32)
+    a = np.zeros(333, np.float32)
+    column_sums(a, b)
+    assert np.allclose(a, b.sum(axis=0, dtype=np.float64), rtol=1e-4, atol=1e-3)
