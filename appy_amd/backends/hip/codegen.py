@@ -499,7 +499,7 @@ class CompiledLoop:
             if trip >= 128 * v and n_outer * 32 * 16 < TEAM_BYTES_IN_FLIGHT:
                 w = 64
         block = d.block
-        if n_outer * 32 < DEFAULT_CUS * 256 and trip >= 64 * v * 32:
+        if self.analysis.multi_wave_ok and n_outer * 32 < DEFAULT_CUS * 256 and trip >= 64 * v * 32:
             # few, very long rows: wavefront teams would leave most of the chip idle,
             # so a whole workgroup takes each row (the more lanes the fewer rows there are)
             block = 1024 if n_outer <= DEFAULT_CUS else 256

@@ -246,6 +246,24 @@ def _has_simd_loop(stmts) -> bool:
 class LoopAnalysis:
     """Facts about a loop nest that do not depend on the launch shape."""
 
+    def _leader_store_reloaded(self) -> bool:
+        shared_out = set()
+        for n in ast.walk(self.outer):
+            if isinstance(n, ast.For) and n is not self.outer and "simd" in (getattr(n, "pragma", None) or {}):
+                shared_out.update(id(x) for x in ast.walk(n))
+        for st in ast.walk(self.outer):
+            if not (isinstance(st, ast.Assign) and id(st) not in shared_out):
+                continue
+            t = st.targets[0]
+            if not (isinstance(t, ast.Subscript) and isinstance(t.value, ast.Name) and t.value.id in self.arrays):
+                continue
+            mine = {id(x) for x in ast.walk(st)}
+            for n in ast.walk(self.outer):
+                if (isinstance(n, ast.Subscript) and isinstance(n.ctx, ast.Load) and isinstance(n.value, ast.Name)
+                        and n.value.id == t.value.id and id(n) not in mine):
+                    return True
+        return False
+
     def _find_strip(self):
         """``{id(loop): {scalar: op}}`` for the inner loops that a *strip* kernel
         shares out between wavefronts, or None if the loop nest does not suit that
@@ -374,7 +392,13 @@ class LoopAnalysis:
             isinstance(n, ast.Subscript) and _uses_name(_elts(n)[-1], self.var)
             for lp in nested for st in lp.body for n in ast.walk(st))
 
-        self.strip = self._find_strip()
+        # Shapes whose team spans several wavefronts (strips, workgroup teams) run statements
+        # outside the shared-out loops on every wavefront but store from one of them only.
+        # An array stored that way and read by another statement would need a barrier between
+        # the two (the other wavefronts may read too early or too late), so such loop nests
+        # keep to teams inside one wavefront, where program order is enough.
+        self.multi_wave_ok = not self._leader_store_reloaded()
+        self.strip = self._find_strip() if self.multi_wave_ok else None
 
         # reductions of the parallel loop: constant-subscript elements of arrays
         self.outer_reductions = []

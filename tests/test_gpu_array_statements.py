@@ -201,3 +201,32 @@ def test_jacobi_1d(gpu):
     rng = np.random.default_rng(7)
     got, ref = both(jacobi_1d, 10, rng.random(4001), rng.random(4001))
     assert close(got, ref, atol=0)
+
+
+def gram_schmidt_step_reading_back(Q, A, R, k):
+    #pragma parallel for
+    for j in range(k + 1, A.shape[1]):
+        R[k, j] = np.sum(Q[:, k] * A[:, j])        # stored by one lane of the team ...
+        A[:, j] -= Q[:, k] * R[k, j]               # ... and read back by all of them
+
+
+def test_value_stored_by_the_team_leader_and_read_back_by_the_team(gpu):
+    """The read-after-write pattern of docs/metal_simd_memory_hazards.md:38-60 in its
+    natural form: correct on teams inside one wavefront, which is what such loop
+    nests are kept to (no strip, no workgroup team)."""
+    from appy_amd.backends.hip import codegen as cg
+
+    rng = np.random.default_rng(14)
+    A = rng.standard_normal((900, 70))
+    Q = rng.standard_normal((900, 70))
+    R = np.zeros((70, 70))
+    k = 3
+    ref_R = R.copy()
+    ref_R[k, k + 1:] = Q[:, k] @ A[:, k + 1:]
+    ref_A = A.copy()
+    ref_A[:, k + 1:] -= np.outer(Q[:, k], ref_R[k, k + 1:])
+    appy.jit(gram_schmidt_step_reading_back)(Q, A, R, k)
+    assert np.allclose(R, ref_R, rtol=1e-12, atol=1e-12) and np.allclose(A, ref_A, rtol=1e-11, atol=1e-11)
+    loop = [v[0] for kk, v in cg.code_cache.items() if kk[-1] == "gram_schmidt_step_reading_back"][-1]
+    assert loop.analysis.strip is None and not loop.analysis.multi_wave_ok
+    assert loop.last_launch.spec.kind == "team" and loop.last_launch.spec.width <= 64
