@@ -245,6 +245,34 @@ class _ReduceCalls(ast.NodeTransformer):
         return node
 
 
+def _refuse_shifted_self_reference(tgt, dim, lo, value, ctx: _Ctx):
+    """``A[i, 1:] = f(A[i, :-1])``: NumPy evaluates the right-hand side before it
+    stores anything; a loop whose iterations run side by side on the same row
+    cannot (an element is overwritten by one lane while another still has to
+    read its old value - the reference documents the same limit,
+    docs/metal_simd_memory_hazards.md, "Slice with index offset").  Refused
+    rather than computed wrongly."""
+    if not isinstance(tgt.value, ast.Name):
+        return
+    t_elts = tgt.slice.elts if isinstance(tgt.slice, ast.Tuple) else [tgt.slice]
+    others = [ast.unparse(e) for k, e in enumerate(t_elts) if k != dim]
+    for n in ast.walk(value):
+        if not (isinstance(n, ast.Subscript) and isinstance(n.value, ast.Name) and n.value.id == tgt.value.id):
+            continue
+        sl = _slices_of(n)
+        n_elts = n.slice.elts if isinstance(n.slice, ast.Tuple) else [n.slice]
+        if len(sl) != 1 or sl[0][0] != dim or len(n_elts) != len(t_elts):
+            continue
+        if [ast.unparse(e) for k, e in enumerate(n_elts) if k != dim] != others:
+            continue
+        n_lo, _ = _bounds(n, dim, sl[0][1], ctx)
+        if ast.unparse(n_lo) != ast.unparse(lo):
+            raise RuntimeError(
+                f"`{ast.unparse(tgt)}` is updated from `{ast.unparse(n)}`, the same row at another offset: "
+                "the elements cannot be updated side by side in place; write the result to another array"
+            )
+
+
 def _lower_assign(st: ast.Assign, ctx: _Ctx):
     out = []
     # 1. reductions inside the right-hand side become scalar temporaries
@@ -265,6 +293,7 @@ def _lower_assign(st: ast.Assign, ctx: _Ctx):
     c = ctx.fresh("c")
     dim, s = sl[0]
     lo, hi = _bounds(tgt, dim, s, ctx)
+    _refuse_shifted_self_reference(tgt, dim, lo, st.value, ctx)
     new_tgt = copy.deepcopy(tgt)
     idx = _offset(lo, c)
     if isinstance(new_tgt.slice, ast.Tuple):

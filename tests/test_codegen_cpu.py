@@ -444,3 +444,12 @@ def test_updates_of_elements_shared_between_iterations_are_atomic():
     assert "appy::atomic_combine<appy::OpAdd, double>::run(&col[" in body_of(src) and "(-" in body_of(src)
     with pytest.raises(NotImplementedError, match="atomic updates of int16"):
         compiled("#pragma parallel for simd\nfor i in range(n):\n    hist[b[i]] += 1\n", hist=np.zeros(16, np.int16), b=b, n=64)
+
+
+def test_in_place_slice_update_from_a_shifted_slice_of_the_same_row_is_refused():
+    A = np.zeros((8, 16))
+    B = np.zeros((8, 16))
+    with pytest.raises(RuntimeError, match="another offset"):
+        compiled("#pragma parallel for\nfor i in range(n):\n    A[i, 1:] = 0.5 * (A[i, :-1] + B[i, :-1])\n", A=A, B=B, n=8)
+    # same offsets, other rows, other arrays: fine
+    compiled("#pragma parallel for\nfor i in range(1, n):\n    A[i, 1:] = A[i, 1:] + A[i - 1, :-1] + B[i, :-1]\n", A=A, B=B, n=8)
