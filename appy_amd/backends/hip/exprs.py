@@ -130,7 +130,11 @@ class ExprEmitter:
         m = getattr(self, "e_" + type(node).__name__, None)
         if m is None:
             raise NotImplementedError(f"Expression not supported in a kernel: {ast.unparse(node)}")
-        return m(node)
+        code, ty = m(node)
+        if isinstance(node, (ast.BinOp, ast.UnaryOp)) and ty.is_int and ty.size < 4:
+            # C++ computes 8- and 16-bit integers as `int`; NumPy wraps in the operands' type
+            code = f"(({ty.c})({code}))"
+        return code, ty
 
     def e_Constant(self, node):
         v = node.value
@@ -333,6 +337,11 @@ class ExprEmitter:
             if sym is None:
                 raise NotImplementedError(f"Comparison not supported in a kernel: {ast.unparse(node)}")
             t = T.promote(lt, rt)
+            if t.is_int and lt.weak != rt.weak and (lt.is_int or lt.is_bool) and (rt.is_int or rt.is_bool) \
+                    and t.name != "uint64":
+                # a Python integer next to a typed one is compared by value (`u8 > -2` is true), not
+                # squeezed into the other operand's type first
+                t = T.I64
             parts.append(f"({cast(lc, lt, t)} {sym} {cast(rc, rt, t)})")
             lc, lt = rc, rt
         return ("(" + " && ".join(parts) + ")" if len(parts) > 1 else parts[0]), T.BOOL

@@ -434,3 +434,86 @@ def test_updates_shared_between_iterations_are_atomic(gpu):
     a = np.zeros(333, np.float32)
     column_sums(a, b)
     assert np.allclose(a, b.sum(axis=0, dtype=np.float64), rtol=1e-4, atol=1e-3)
+
+
+def _random_expression(rng, depth, leaves):
+    if depth == 0 or rng.random() < 0.25:
+        return leaves[rng.integers(len(leaves))]
+    kind = rng.integers(0, 10)
+    a = _random_expression(rng, depth - 1, leaves)
+    b = _random_expression(rng, depth - 1, leaves)
+    if kind <= 2:
+        return f"({a} {['+', '-', '*'][kind]} {b})"
+    if kind == 3:
+        return f"({a} / (abs({b}) + 1))"
+    if kind == 4:
+        return f"({a} // (abs({b}) + 1))"
+    if kind == 5:
+        return f"({a} % (abs({b}) + 2))"
+    if kind == 6:
+        return f"({a} if {_random_expression(rng, depth - 1, leaves)} > {b} else {b})"
+    if kind == 7:
+        return f"{['min', 'max'][rng.integers(2)]}({a}, {b})"
+    if kind == 8:
+        return f"abs({a})"
+    return f"(-{a})"
+
+
+@pytest.mark.parametrize("seed", range(60))
+def test_random_expressions_type_and_value_like_numpy(gpu, seed):
+    """Random expression trees over arrays of five dtypes, NumPy scalars and Python
+    scalars: the kernel must produce the dtype and the values that NumPy's own
+    evaluation of the same expression over the arrays gives (NEP 50 promotion,
+    floor division and modulo with Python's sign rules, true division)."""
+    import appy_amd as appy
+
+    rng = np.random.default_rng(1000 + seed)
+    n = 4099
+    env = {
+        "f": rng.uniform(-4, 4, n).astype(np.float32),
+        "d": rng.uniform(-4, 4, n),
+        "k": rng.integers(-20, 20, n).astype(np.int32),
+        "l": rng.integers(-20, 20, n).astype(np.int64),
+        "u": rng.integers(0, 9, n).astype(np.uint8),
+        "s32": np.float32(1.5), "w": 3, "z": 0.75,
+    }
+    # the builtins keep Python scalars Python scalars (weak), as they do in the un-jitted loop
+    plain = (int, float)
+    env["abs"] = lambda x: abs(x) if isinstance(x, plain) else np.abs(x)
+    env["min"] = lambda x, y: min(x, y) if isinstance(x, plain) and isinstance(y, plain) else np.minimum(x, y)
+    env["max"] = lambda x, y: max(x, y) if isinstance(x, plain) and isinstance(y, plain) else np.maximum(x, y)
+    env["h"] = rng.integers(-300, 300, n).astype(np.int16)
+    leaves = ["f[i]", "d[i]", "k[i]", "l[i]", "u[i]", "h[i]", "s32", "w", "z", "2", "0.5",
+              "(k[i] & 7)", "(l[i] >> 1)", "(u[i] << 2)", "(h[i] ^ k[i])", "(u[i] * u[i])", "(h[i] * h[i])"]
+    expr = _random_expression(rng, 3, leaves)
+    vec_expr = expr.replace("[i]", "")
+    # `x if c else y` on arrays is np.where(c, x, y)
+    import ast as _ast
+
+    class _Where(_ast.NodeTransformer):
+        def visit_IfExp(self, node):
+            self.generic_visit(node)
+            return _ast.Call(func=_ast.Attribute(value=_ast.Name(id="np", ctx=_ast.Load()), attr="where", ctx=_ast.Load()),
+                             args=[node.test, node.body, node.orelse], keywords=[])
+
+    tree = _ast.fix_missing_locations(_Where().visit(_ast.parse(vec_expr, mode="eval")))
+    with np.errstate(all="ignore"):
+        ref = eval(compile(tree, "<ref>", "eval"), {"np": np}, env)
+    ref = np.broadcast_to(np.asarray(ref), (n,)) if np.ndim(ref) == 0 else ref
+    if ref.dtype == np.float16:
+        pytest.skip("float16 result")
+    out = np.zeros(n, dtype=ref.dtype)
+    src = (f"def kernel(f, d, k, l, u, h, s32, w, z, out):\n    #pragma parallel for simd\n"
+           f"    for i in range(out.shape[0]):\n        out[i] = {expr}\n")
+    import linecache
+
+    name = f"<random_expr_{seed}>"
+    linecache.cache[name] = (len(src), None, src.splitlines(True), name)
+    ns = {}
+    exec(compile(src, name, "exec"), {"np": np, "abs": abs, "min": min, "max": max}, ns)
+    fn = appy.jit(ns["kernel"])
+    fn(env["f"], env["d"], env["k"], env["l"], env["u"], env["h"], env["s32"], env["w"], env["z"], out)
+    if ref.dtype.kind == "f":
+        assert np.allclose(out, ref, rtol=2e-6 if ref.dtype == np.float32 else 1e-13, atol=1e-6, equal_nan=True), expr
+    else:
+        assert np.array_equal(out, ref), expr
