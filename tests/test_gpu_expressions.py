@@ -484,9 +484,11 @@ def test_random_expressions_type_and_value_like_numpy(gpu, seed):
     env["max"] = lambda x, y: max(x, y) if isinstance(x, plain) and isinstance(y, plain) else np.maximum(x, y)
     env["h"] = rng.integers(-300, 300, n).astype(np.int16)
     leaves = ["f[i]", "d[i]", "k[i]", "l[i]", "u[i]", "h[i]", "s32", "w", "z", "2", "0.5",
-              "(k[i] & 7)", "(l[i] >> 1)", "(u[i] << 2)", "(h[i] ^ k[i])", "(u[i] * u[i])", "(h[i] * h[i])"]
+              "(k[i] & 7)", "(l[i] >> 1)", "(u[i] << 2)", "(h[i] ^ k[i])", "(u[i] * u[i])", "(h[i] * h[i])",
+              "np.sqrt(abs(f[i]))", "np.exp(k[i] * 0.1)", "np.floor(d[i])", "np.tanh(f[i])", "np.sqrt(l[i] * l[i])",
+              "np.float32(w)", "np.int32(d[i])"]
     expr = _random_expression(rng, 3, leaves)
-    vec_expr = expr.replace("[i]", "")
+    vec_expr = expr.replace("[i]", "").replace("np.int32(d)", "d.astype(np.int32)")
     # `x if c else y` on arrays is np.where(c, x, y)
     import ast as _ast
 
@@ -499,6 +501,8 @@ def test_random_expressions_type_and_value_like_numpy(gpu, seed):
     tree = _ast.fix_missing_locations(_Where().visit(_ast.parse(vec_expr, mode="eval")))
     with np.errstate(all="ignore"):
         ref = eval(compile(tree, "<ref>", "eval"), {"np": np}, env)
+    if isinstance(ref, (int, float)):
+        pytest.skip("an expression of Python scalars only")
     ref = np.broadcast_to(np.asarray(ref), (n,)) if np.ndim(ref) == 0 else ref
     if ref.dtype == np.float16:
         pytest.skip("float16 result")
@@ -514,6 +518,72 @@ def test_random_expressions_type_and_value_like_numpy(gpu, seed):
     fn = appy.jit(ns["kernel"])
     fn(env["f"], env["d"], env["k"], env["l"], env["u"], env["h"], env["s32"], env["w"], env["z"], out)
     if ref.dtype.kind == "f":
-        assert np.allclose(out, ref, rtol=2e-6 if ref.dtype == np.float32 else 1e-13, atol=1e-6, equal_nan=True), expr
+        # float32 exp / tanh are good to an ulp or two, which later float64 arithmetic carries along
+        loose = ref.dtype == np.float32 or "np.exp" in expr or "np.tanh" in expr
+        assert np.allclose(out, ref, rtol=3e-6 if loose else 1e-13, atol=1e-5 if loose else 1e-6, equal_nan=True), expr
     else:
         assert np.array_equal(out, ref), expr
+
+
+def _random_program(rng):
+    """A loop body with temporaries, a branch and an inner simd reduction."""
+    # (no unsigned operands here: a temporary that is uint8 on one path and float on another wraps
+    #  on negation in the interpreter, while a kernel variable has one type, the join of both)
+    arr = ["f[i]", "d[i]", "k[i]", "A[i, 0]"]
+    temps = []
+    lines = []
+
+    def leaf_pool():
+        return arr + temps + ["w", "z", "s32", "2", "0.25"]
+
+    for t in range(int(rng.integers(2, 5))):
+        lines.append(f"t{t} = {_random_expression(rng, 2, leaf_pool())}")
+        temps.append(f"t{t}")
+    cond = f"{_random_expression(rng, 1, leaf_pool())} > {_random_expression(rng, 1, leaf_pool())}"
+    tgt = temps[int(rng.integers(len(temps)))]
+    lines.append(f"if {cond}:")
+    lines.append(f"    {tgt} = {_random_expression(rng, 2, leaf_pool())}")
+    if rng.random() < 0.5:
+        lines.append("else:")
+        lines.append(f"    {temps[int(rng.integers(len(temps)))]} = {_random_expression(rng, 1, leaf_pool())}")
+    red = ["+", "max", "min"][int(rng.integers(3))]
+    init = {"+": "0.0", "max": "-1e30", "min": "1e30"}[red]
+    inner = _random_expression(rng, 2, ["A[i, j]", "v[j]", "f[i]", "k[i]", "z"] + temps)
+    lines.append(f"s = {init}")
+    lines.append("#pragma simd")
+    lines.append("for j in range(A.shape[1]):")
+    lines.append(f"    s += {inner}" if red == "+" else f"    s = {red}(s, {inner})")
+    lines.append(f"out[i] = s + {_random_expression(rng, 1, temps + ['f[i]'])}")
+    return lines
+
+
+@pytest.mark.parametrize("seed", range(50))
+def test_random_programs_against_the_interpreter(gpu, seed):
+    """Random loop bodies (temporaries that change type, a branch, an inner simd
+    reduction) run by the interpreter statement by statement and by the kernel."""
+    import linecache
+
+    import appy_amd as appy
+
+    rng = np.random.default_rng(5000 + seed)
+    n, m = 67, 45
+    args = {
+        "f": rng.uniform(-2, 2, n).astype(np.float32), "d": rng.uniform(-2, 2, n),
+        "k": rng.integers(-9, 9, n).astype(np.int32), "u": rng.integers(0, 9, n).astype(np.uint8),
+        "A": rng.uniform(-1, 1, (n, m)).astype(np.float32), "v": rng.uniform(-1, 1, m),
+        "s32": np.float32(1.5), "w": 3, "z": 0.75,
+    }
+    body = _random_program(rng)
+    src = ("def kernel(f, d, k, u, A, v, s32, w, z, out):\n    #pragma parallel for\n    for i in range(out.shape[0]):\n"
+           + "".join(f"        {ln}\n" for ln in body))
+    name = f"<random_program_{seed}>"
+    linecache.cache[name] = (len(src), None, src.splitlines(True), name)
+    ns = {}
+    exec(compile(src, name, "exec"), {"np": np}, ns)
+    ref = np.zeros(n)
+    with np.errstate(all="ignore"):
+        ns["kernel"](*args.values(), ref)
+    out = np.zeros(n)
+    appy.jit(ns["kernel"])(*args.values(), out)
+    scale = np.maximum(1.0, np.abs(ref))
+    assert np.all(np.abs(out - ref) <= 2e-4 * scale * m), "\n".join(body)
