@@ -230,3 +230,63 @@ def test_value_stored_by_the_team_leader_and_read_back_by_the_team(gpu):
     loop = [v[0] for kk, v in cg.code_cache.items() if kk[-1] == "gram_schmidt_step_reading_back"][-1]
     assert loop.analysis.strip is None and not loop.analysis.multi_wave_ok
     assert loop.last_launch.spec.kind == "team" and loop.last_launch.spec.width <= 64
+
+
+def _slice(rng, length, size):
+    """Text of a slice of ``length`` elements inside an axis of ``size``, in one of NumPy's spellings."""
+    lo = int(rng.integers(0, size - length + 1))
+    hi = lo + length
+    forms = [f"{lo}:{hi}"]
+    if lo == 0:
+        forms.append(f":{hi}")
+    if hi == size:
+        forms.append(f"{lo}:")
+    if lo == 0 and hi == size:
+        forms.append(":")
+    if hi < size:
+        forms.append(f"{lo}:{hi - size}")          # negative upper bound
+    return forms[int(rng.integers(len(forms)))]
+
+
+@pytest.mark.parametrize("seed", range(30))
+def test_random_slice_statements_against_numpy(gpu, seed):
+    """Random 1-D array statements inside a parallel loop (row slices, column
+    slices, whole 1-D arrays, reductions of slice products, in-place operators),
+    executed by NumPy and by the kernels."""
+    import linecache
+
+    rng = np.random.default_rng(9000 + seed)
+    n, m = 23, 61
+    L = int(rng.integers(1, m + 1))
+    Lc = int(rng.integers(1, n + 1))
+    args = {"A": rng.standard_normal((n, m)), "B": rng.standard_normal((n, m)), "C": rng.standard_normal((n, m)),
+            "v": rng.standard_normal(m), "r": np.zeros(n), "alpha": 1.25}
+    row_ops = [
+        f"A[i, {_slice(rng, L, m)}] = B[i, {_slice(rng, L, m)}] * alpha + v[{_slice(rng, L, m)}]",
+        f"A[i, {_slice(rng, L, m)}] += B[i, {_slice(rng, L, m)}] * C[i, {_slice(rng, L, m)}]",
+        f"A[i, {_slice(rng, L, m)}] = np.maximum(B[i, {_slice(rng, L, m)}], 0.0) - alpha",
+        f"r[i] = np.sum(B[i, {_slice(rng, L, m)}] * C[i, {_slice(rng, L, m)}]) + alpha",
+        f"r[i] = B[i, {_slice(rng, L, m)}] @ v[{_slice(rng, L, m)}]",
+        f"r[i] = np.max(B[i, {_slice(rng, L, m)}]) - np.min(C[i, {_slice(rng, L, m)}])",
+        "A[i, :] = v * alpha - B[i, :]",
+        f"s = np.sum(C[i, {_slice(rng, L, m)}])\n            A[i, {_slice(rng, L, m)}] -= s * B[i, {_slice(rng, L, m)}]",
+    ]
+    col_ops = [
+        f"A[{_slice(rng, Lc, n)}, j] = B[{_slice(rng, Lc, n)}, j] + alpha",
+        f"v[j] = B[{_slice(rng, Lc, n)}, j] @ C[{_slice(rng, Lc, n)}, j]",
+        f"A[{_slice(rng, Lc, n)}, j] *= C[{_slice(rng, Lc, n)}, j]",
+    ]
+    pick = lambda ops, k: "\n            ".join(ops[int(x)] for x in rng.choice(len(ops), size=k, replace=False))  # noqa: E731
+    src = ("def kernel(A, B, C, v, r, alpha):\n"
+           "    #pragma parallel for\n    for i in range(A.shape[0]):\n            " + pick(row_ops, 2) + "\n"
+           "    #pragma parallel for\n    for j in range(A.shape[1]):\n            " + pick(col_ops, 1) + "\n")
+    name = f"<random_slices_{seed}>"
+    linecache.cache[name] = (len(src), None, src.splitlines(True), name)
+    ns = {}
+    exec(compile(src, name, "exec"), {"np": np}, ns)
+    ref = {k: (x.copy() if isinstance(x, np.ndarray) else x) for k, x in args.items()}
+    got = {k: (x.copy() if isinstance(x, np.ndarray) else x) for k, x in args.items()}
+    ns["kernel"](**ref)
+    appy.jit(ns["kernel"])(**got)
+    for key in ("A", "v", "r"):
+        assert np.allclose(got[key], ref[key], rtol=1e-12, atol=1e-12), (key, src)
