@@ -439,3 +439,49 @@ def test_repeated_calls_on_gpu_tensors_replay_the_staged_launch(gpu):
     assert torch.equal(c, a * 2.0 + b)
     with pytest.raises(IndexError):
         scaled_add(a, b[:10], c, 2.0)                         # host checks still run for new shapes
+
+
+_INNER_STATEMENTS = [
+    "t = A[i, j] * 2.0\n            B[i, j] = t + x[j]",
+    "B[i, j] = B[i, j - 1] + A[i, j]",                       # carried through B
+    "s += A[i, j] * x[j]",
+    "s = s * 0.5 + A[i, j]",                                 # carried scalar, not a reduction
+    "y[i] += A[i, j]",
+    "y[i] = max(y[i], A[i, j])",
+    "B[i, p[j]] = A[i, j]",                                  # scatter through a permutation
+    "if A[i, j] > 0.0:\n                s += A[i, j]",
+    "c[j] += A[i, j]",                                       # every outer iteration feeds c[j]
+    "B[i, j] = A[i, j] + s",                                 # reads the running value of s
+    "t = A[i, j]\n            B[i, j] = t * t\n            s += t",
+    "B[i, j] = x[p[j]] * A[i, j]",                           # gather
+    "u = x[j]\n            B[i, j] = u",
+]
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_prange_nests_agree_with_the_interpreter(gpu, seed):
+    """Random inner loops under ``prange`` (independent ones, carried ones,
+    reductions, scatters, gathers): whatever the compiler decides to spread over
+    lanes, the result must be the interpreter's."""
+    import linecache
+
+    rng = np.random.default_rng(7000 + seed)
+    n, m = 19, 83
+    k = int(rng.integers(1, 4))
+    body = "\n            ".join(_INNER_STATEMENTS[int(x)] for x in rng.choice(len(_INNER_STATEMENTS), size=k, replace=False))
+    lo = int(rng.integers(0, 2))
+    src = ("def kernel(A, B, x, y, c, p, out):\n    for i in prange(A.shape[0]):\n        s = 0.0\n        t = 0.0\n        u = 0.0\n"
+           f"        for j in range({lo if 'j - 1' not in body else 1}, A.shape[1]):\n            {body}\n"
+           "        out[i] = s + t + u\n")
+    name = f"<random_prange_{seed}>"
+    linecache.cache[name] = (len(src), None, src.splitlines(True), name)
+    ns = {}
+    exec(compile(src, name, "exec"), {"np": np, "prange": appy.prange}, ns)
+    base = {"A": rng.standard_normal((n, m)), "B": rng.standard_normal((n, m)), "x": rng.standard_normal(m),
+            "y": rng.standard_normal(n), "c": np.zeros(m), "p": rng.permutation(m).astype(np.int32), "out": np.zeros(n)}
+    ref = {key: v.copy() for key, v in base.items()}
+    got = {key: v.copy() for key, v in base.items()}
+    ns["kernel"](**ref)
+    appy.jit(ns["kernel"])(**got)
+    for key in ("B", "y", "c", "out"):
+        assert np.allclose(got[key], ref[key], rtol=1e-10, atol=1e-10), (key, src)
