@@ -328,3 +328,44 @@ def test_launches_from_several_threads(k):
     for t in threads:
         t.join()
     assert not errors, errors
+
+
+_FLAT_SPECS = [dict(block=b, vec=v, unroll=u, stream_loads=nt, stream_stores=nt)
+               for b, v, u, nt in ((64, 1, 1, False), (256, 2, 4, False), (1024, 4, 2, True), (512, 1, 8, False), (128, 4, 1, True))]
+_TEAM_SPECS = [dict(block=b, vec=v, width=w, stream_loads=nt)
+               for b, v, w, nt in ((256, 1, 1, False), (256, 4, 2, False), (64, 2, 64, True), (512, 4, 16, False),
+                                   (1024, 1, 1024, False), (256, 4, 256, True), (128, 2, 8, False))]
+
+
+@pytest.mark.parametrize("spec", _FLAT_SPECS, ids=lambda s: "b{block}v{vec}u{unroll}".format(**s))
+def test_flat_kernels_give_the_same_results_in_every_launch_shape(gpu, spec):
+    k = selfcheck.kernels(hip_spec=spec)
+    a, b = wl.vec_add(70_001)
+    assert np.array_equal(k.vec_add(a, b), vo.vec_add(a, b))
+    A, M = wl.reduce_inputs(333_337)
+    ref, budget = vo.vector_sum(A)
+    assert abs(k.vector_sum(A) - ref) <= TOL * budget
+    ref, budget = vo.masked_sum(A, M)
+    assert abs(k.masked_sum(A, M) - ref) <= TOL * budget
+    c = np.empty_like(a)
+    k.copy(a, c)
+    assert np.array_equal(a, c)
+
+
+@pytest.mark.parametrize("spec", _TEAM_SPECS, ids=lambda s: "b{block}v{vec}w{width}".format(**s))
+def test_team_kernels_give_the_same_results_in_every_launch_shape(gpu, spec):
+    k = selfcheck.kernels(hip_spec=spec)
+    Am, x = wl.gemv(301, 1237)
+    ref, budget = vo.gemv(Am, x)
+    ok, worst = vo.within_budget(k.gemv(Am, x), ref, budget, TOL)
+    assert ok, worst
+    data, indptr, indices, xs = wl.spmv_powerlaw(3000, 3000, clip=700)
+    ref, budget = vo.spmv_csr(data, indptr, indices, xs, (3000, 3000))
+    ok, worst = vo.within_budget(k.spmv(data, indptr, indices, xs, 3000, 3000), ref, budget, TOL)
+    assert ok, worst
+    data, indptr, indices, B = wl.spmm(500, 400, 128)
+    ref, budget = vo.spmm_csr(data, indptr, indices, B, (500, 400))
+    Y = np.empty((500, 128), dtype=np.float32)
+    k.spmm(data, indptr, indices, B, Y, 500)
+    ok, worst = vo.within_budget(Y, ref, budget, TOL)
+    assert ok, worst
