@@ -369,3 +369,13 @@ def test_team_kernels_give_the_same_results_in_every_launch_shape(gpu, spec):
     k.spmm(data, indptr, indices, B, Y, 500)
     ok, worst = vo.within_budget(Y, ref, budget, TOL)
     assert ok, worst
+
+
+@pytest.mark.parametrize("block,unroll", [(64, 1), (128, 4), (256, 8), (512, 2), (1024, 8)])
+def test_strip_kernel_gives_the_same_results_for_every_workgroup_size(gpu, block, unroll):
+    k = selfcheck.kernels(hip_spec=dict(kind="strip", block=block, vec=1, unroll=unroll, stream_loads=block == 256))
+    Am, _ = wl.gemv(777, 333)
+    yv = Am[:, 1].copy()
+    ref, budget = vo.gemv(Am.T, yv)
+    ok, worst = vo.within_budget(k.gemv_columns(Am, yv), ref, budget, TOL)
+    assert ok, worst
