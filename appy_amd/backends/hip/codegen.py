@@ -809,6 +809,8 @@ class Launch:
             g.launches += 1
             g.keepalive.extend(self.keepalive)
             for m, _dptr, _host, stored, _name in self.mirrored:
+                if m not in g.used_mirrors:
+                    g.used_mirrors.append(m)
                 if stored and m not in g.stored_mirrors:
                     g.stored_mirrors.append(m)
 
@@ -845,6 +847,8 @@ class Launch:
                         original[...] = host
             waited = bool(self.temps)
             for m, dptr, host, stored, _name in self.mirrored:
+                if m.resident:
+                    m.stream, m.busy = self.stream, True
                 if not stored:
                     continue
                 if m.resident:

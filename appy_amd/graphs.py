@@ -43,6 +43,7 @@ class graph:
         self.exec = 0
         self.launches = 0          # kernels recorded
         self.stored_mirrors = []   # resident host arrays the recorded kernels store to
+        self.used_mirrors = []     # resident host arrays the recorded kernels touch at all
         self.keepalive = []        # tensors whose memory the graph refers to
 
     # ---- capture ----------------------------------------------------------------------
@@ -85,9 +86,10 @@ class graph:
             raise RuntimeError("the graph has not been captured")
         s = self.stream if stream is None else int(stream)
         rt.graph_launch(self.exec, s)
+        for m in self.used_mirrors:
+            m.stream, m.busy = s, True
         for m in self.stored_mirrors:
             m.device_dirty = True
-            m.stream = s
 
     def synchronize(self):
         rt.sync(self.stream)
@@ -101,6 +103,7 @@ class graph:
             self.stream = 0
         self.keepalive = []
         self.stored_mirrors = []
+        self.used_mirrors = []
 
     def __del__(self):
         try:

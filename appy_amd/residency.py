@@ -39,7 +39,7 @@ class Mirror:
     """HBM buffer paired with the host bytes [addr, addr + nbytes)."""
 
     __slots__ = ("addr", "nbytes", "dptr", "pinned", "resident", "device_dirty", "host_dirty", "keep", "depth",
-                 "stream")
+                 "stream", "busy")
 
     def __init__(self, addr: int, nbytes: int, pinned: bool, keep=None):
         self.addr = addr
@@ -51,7 +51,8 @@ class Mirror:
         self.host_dirty = False     # the host bytes changed since the last upload (resident mode)
         self.keep = keep            # keeps an ordinary array alive while its address is registered
         self.depth = 0              # nested `resident` blocks
-        self.stream = 0             # stream of the last launch that stored to the mirror
+        self.stream = 0             # stream of the last launch that used the mirror
+        self.busy = False           # a launch on `stream` may still be using the mirror
 
     def device_ptr(self) -> int:
         if not self.dptr:
@@ -65,7 +66,8 @@ class Mirror:
 
     def download(self) -> None:
         if self.nbytes and self.dptr:
-            rt.memcpy_d2h(self.addr, self.dptr, self.nbytes, self.stream)
+            rt.memcpy_d2h(self.addr, self.dptr, self.nbytes, self.stream)   # waits for the stream
+            self.busy = False
         self.device_dirty = False
 
 
@@ -100,6 +102,8 @@ def unregister(addr: int) -> None:
             del _bases[i]
         if m.dptr:
             try:
+                if m.busy:
+                    rt.sync(m.stream)   # the buffer goes back to the pool: nothing may still be reading it
                 rt.free(m.dptr)
             except Exception:
                 pass    # interpreter shutdown: the library may be gone already
