@@ -96,7 +96,9 @@ int appy_hip_occupancy(void* func, int block_threads, size_t dynamic_lds_bytes,
  * (appy/backends/triton/passes/host_passes/gen_data_movement.py:25-87) for
  * NumPy / CPU-tensor arguments.  Buffers come from a size-bucketed pool so a
  * repeated call does not pay hipMalloc/hipFree; appy_hip_pool_trim releases
- * everything the pool holds. */
+ * everything the pool holds.  appy_hip_free does not wait for the GPU: the
+ * block may be handed out again at once, so synchronise the streams that still
+ * use it first (appy_hip_memcpy_d2h and appy_hip_sync do). */
 int appy_hip_malloc(size_t nbytes, void** dptr_out);
 int appy_hip_free(void* dptr);
 int appy_hip_pool_trim(void);
