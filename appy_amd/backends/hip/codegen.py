@@ -263,6 +263,9 @@ class CompiledLoop:
             self._strip_trip_code = compile(ast.Expression(body=ast.fix_missing_locations(
                 ast.BinOp(left=_copy(hi), op=ast.Sub(), right=_copy(lo)))), "<trip>", "eval")
         self.kernels = {}   # Spec -> Kernel
+        self._overwrite_codes = {
+            name: (None if node is None else compile(ast.Expression(body=ast.fix_missing_locations(_copy(node))), "<n>", "eval"))
+            for name, node in a.overwritten.items()}
         self._replays = {}  # call identity -> Launch that can simply be launched again
         # scalars that no host-side decision looks at (range of the loop, inner trip counts,
         # row extents): a replayed launch may carry new values of these
@@ -597,6 +600,19 @@ class CompiledLoop:
                 self._replays.clear()
             self._replays[key] = plan
 
+    def overwrites(self, name, lo, hi, env, shape) -> bool:
+        """True if this launch stores every element of array ``name`` (so that its
+        previous contents need not travel to the device)."""
+        if name not in self._overwrite_codes or lo != 0 or hi != shape[0]:
+            return False
+        code = self._overwrite_codes[name]
+        if code is None:
+            return len(shape) == 1
+        try:
+            return len(shape) == 2 and int(eval(code, _HOST_EVAL_GLOBALS, env)) == shape[1]
+        except Exception:
+            return False
+
     def _replay_key(self, args):
         """Identity of a call whose arrays all live on the GPU already; None for
         any other call (host arrays are copied per call, captures record)."""
@@ -648,6 +664,7 @@ class Launch:
         self.loop = loop
         a = loop.analysis
         self.lo, self.hi = lo, hi
+        self.env = env
         self.temps = []          # (dptr, host ndarray (contiguous), original, stored)
         self.mirrored = []       # (mirror, dptr, host ndarray, stored): arguments with a standing HBM mirror
         self.oob = 0             # checked kernels: device word that receives the report
@@ -775,7 +792,7 @@ class Launch:
             if m.resident:
                 if m.host_dirty:
                     m.upload(self.stream)
-            elif nbytes:
+            elif nbytes and not (stored and self.loop.overwrites(name, self.lo, self.hi, self.env, host.shape)):
                 rt.memcpy_h2d(m.device_ptr() + off, host.ctypes.data, nbytes, self.stream)
             dptr = m.device_ptr() + off
             self.mirrored.append((m, dptr, host, stored, name))
@@ -785,7 +802,7 @@ class Launch:
         self._no_capture(name, "it is a host array that would be copied per launch (use GPU tensors, or NumPy "
                                "arrays inside `with appy.resident(...)`; `shared()` scalars cannot be captured)")
         dptr = rt.malloc(max(nbytes, 1))
-        if nbytes:
+        if nbytes and not (stored and self.loop.overwrites(name, self.lo, self.hi, self.env, host.shape)):
             rt.memcpy_h2d(dptr, host.ctypes.data, nbytes, self.stream)
         self.temps.append((dptr, host, original, stored, name))
         self.ptr[name] = dptr

@@ -246,6 +246,40 @@ def _has_simd_loop(stmts) -> bool:
 class LoopAnalysis:
     """Facts about a loop nest that do not depend on the launch shape."""
 
+    def _fully_overwritten(self):
+        """Arrays of which the loop stores every element it covers without reading any:
+        ``X[i] = e`` (1-D) or ``for j in range(0, n): X[i, j] = e`` (2-D rows) as
+        unconditional statements of the body.  ``{name: None}`` for the 1-D form,
+        ``{name: extent node of the inner loop}`` for the row form.  When the outer
+        range then spans the whole first dimension (and the inner loop the second),
+        a host copy of such an array need not be uploaded before the launch."""
+        if skips_iterations(self.outer.body):
+            return {}
+        out = {}
+        loaded = {n.value.id for n in ast.walk(self.outer)
+                  if isinstance(n, ast.Subscript) and isinstance(n.ctx, ast.Load) and isinstance(n.value, ast.Name)}
+        for st in self.outer.body:
+            if isinstance(st, ast.Assign) and isinstance(st.targets[0], ast.Subscript):
+                t = st.targets[0]
+                el = _elts(t)
+                if (isinstance(t.value, ast.Name) and t.value.id in self.arrays and t.value.id not in loaded
+                        and len(el) == 1 and isinstance(el[0], ast.Name) and el[0].id == self.var):
+                    out[t.value.id] = None
+            elif (isinstance(st, ast.For) and isinstance(st.target, ast.Name) and not st.orelse
+                  and isinstance(st.iter.args[0], ast.Constant) and st.iter.args[0].value == 0
+                  and not skips_iterations(st.body)):
+                jv = st.target.id
+                for inner in st.body:
+                    if not (isinstance(inner, ast.Assign) and isinstance(inner.targets[0], ast.Subscript)):
+                        continue
+                    t = inner.targets[0]
+                    el = _elts(t)
+                    if (isinstance(t.value, ast.Name) and t.value.id in self.arrays and t.value.id not in loaded
+                            and len(el) == 2 and isinstance(el[0], ast.Name) and el[0].id == self.var
+                            and isinstance(el[1], ast.Name) and el[1].id == jv):
+                        out[t.value.id] = st.iter.args[1]
+        return out
+
     def _leader_store_reloaded(self) -> bool:
         shared_out = set()
         for n in ast.walk(self.outer):
@@ -391,6 +425,8 @@ class LoopAnalysis:
         self.lane_loops_strided = self.lane_loops and any(
             isinstance(n, ast.Subscript) and _uses_name(_elts(n)[-1], self.var)
             for lp in nested for st in lp.body for n in ast.walk(st))
+
+        self.overwritten = self._fully_overwritten()
 
         # Shapes whose team spans several wavefronts (strips, workgroup teams) run statements
         # outside the shared-out loops on every wavefront but store from one of them only.

@@ -379,3 +379,44 @@ def test_strip_kernel_gives_the_same_results_for_every_workgroup_size(gpu, block
     ref, budget = vo.gemv(Am.T, yv)
     ok, worst = vo.within_budget(k.gemv_columns(Am, yv), ref, budget, TOL)
     assert ok, worst
+
+
+def test_arrays_that_a_launch_overwrites_completely_are_not_uploaded(gpu, monkeypatch):
+    """``c[i] = ...`` over the whole of ``c``: its old contents stay on the host.
+    As soon as the range leaves elements out, or the loop reads the array, it
+    is uploaded as before (the untouched elements must survive)."""
+    import appy_amd as appy
+    from appy_amd.backends.hip import runtime as rt
+
+    uploads = []
+    real = rt.memcpy_h2d
+    monkeypatch.setattr(rt, "memcpy_h2d", lambda dst, src, n, stream=0: (uploads.append(n), real(dst, src, n, stream))[1])
+
+    @appy.jit
+    def fill(a, c, start):
+        #pragma parallel for simd
+        for i in range(start, a.shape[0]):
+            c[i] = a[i] * 2.0
+
+    @appy.jit
+    def rows(A, C):
+        #pragma parallel for
+        for i in range(A.shape[0]):
+            C[i, :] = A[i, :] + 1.0
+
+    a = np.arange(5000.0)
+    c = np.full(5000, -1.0)
+    fill(a, c, 0)
+    assert np.array_equal(c, 2.0 * a) and uploads == [a.nbytes]            # only `a` travelled up
+    uploads.clear()
+    c[:] = -1.0
+    fill(a, c, 3)
+    assert np.array_equal(c[3:], 2.0 * a[3:]) and (c[:3] == -1.0).all() and uploads == [a.nbytes, c.nbytes]
+    uploads.clear()
+    A = np.arange(600.0).reshape(20, 30)
+    C = np.full((20, 30), -1.0)
+    rows(A, C)
+    assert np.array_equal(C, A + 1.0) and uploads == [A.nbytes]
+    uploads.clear()
+    rows(A[:, :20], C[:, :20])                                             # packed copies of views: same rule
+    assert np.array_equal(C[:, :20], A[:, :20] + 1.0) and len(uploads) == 1
