@@ -925,11 +925,14 @@ def _copy(node):
 def codegen(loop_source, loop_name, val_map, options):
     key = (loop_source, loop_name, _signature(val_map), options.get("hip_spec") and repr(options.get("hip_spec")),
            options.get("hip_max_blocks"), bool(options.get("check_bounds")), options.get("fn_name"))
-    hit = code_cache.get(key)
+    # `clear_cache=True` regenerates the loop on every call instead of using the cached kernel
+    # (reference: appy/backends/metal/codegen.py:23)
+    fresh = bool(options.get("clear_cache"))
+    hit = None if fresh else code_cache.get(key)
     if hit is not None:
         return hit
     with _cache_lock:
-        hit = code_cache.get(key)
+        hit = None if fresh else code_cache.get(key)
         if hit is not None:
             return hit
         f = CompiledLoop(loop_source, loop_name, val_map, options)

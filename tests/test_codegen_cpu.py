@@ -453,3 +453,12 @@ def test_in_place_slice_update_from_a_shifted_slice_of_the_same_row_is_refused()
         compiled("#pragma parallel for\nfor i in range(n):\n    A[i, 1:] = 0.5 * (A[i, :-1] + B[i, :-1])\n", A=A, B=B, n=8)
     # same offsets, other rows, other arrays: fine
     compiled("#pragma parallel for\nfor i in range(1, n):\n    A[i, 1:] = A[i, 1:] + A[i - 1, :-1] + B[i, :-1]\n", A=A, B=B, n=8)
+
+
+def test_clear_cache_option_regenerates_the_loop():
+    a = np.zeros(8, np.float32)
+    src = "#pragma parallel for simd\nfor i in range(n):\n    a[i] = 1.0"
+    f1, _ = cg.codegen(src, "kernel_loop_1", {"a": a, "n": 8}, {})
+    f2, _ = cg.codegen(src, "kernel_loop_1", {"a": a, "n": 8}, {})
+    f3, _ = cg.codegen(src, "kernel_loop_1", {"a": a, "n": 8}, {"clear_cache": True})
+    assert f1 is f2 and f3 is not f1
