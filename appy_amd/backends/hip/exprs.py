@@ -157,6 +157,15 @@ class ExprEmitter:
     def e_Attribute(self, node):
         if isinstance(node.value, ast.Name) and node.value.id in _MATH_MODULE_NAMES and node.attr in _CONSTANTS:
             return T.float_literal(_CONSTANTS[node.attr], T.F64), T.WEAK_FLOAT
+        if isinstance(node.value, ast.Name) and node.value.id in self.arrays:
+            arr = self.arrays[node.value.id]
+            if node.attr == "ndim":
+                return f"{arr.ndim}LL", T.WEAK_INT
+            if node.attr == "size":
+                for d in range(arr.ndim):
+                    self.shape_scalars.add((arr.name, d))
+                dims = [cname(f"{arr.name}_shape_{d}") for d in range(arr.ndim)] or ["1LL"]
+                return "(" + " * ".join(dims) + ")", T.WEAK_INT
         raise NotImplementedError(f"Attribute not supported in a kernel: {ast.unparse(node)}")
 
     # ---- memory -----------------------------------------------------------------
@@ -329,6 +338,12 @@ class ExprEmitter:
         raise NotImplementedError(f"Operator not supported in a kernel: {ast.unparse(node)}")
 
     def e_Compare(self, node):
+        if (len(node.ops) == 1 and isinstance(node.ops[0], (ast.In, ast.NotIn))
+                and isinstance(node.comparators[0], (ast.Tuple, ast.List, ast.Set)) and node.comparators[0].elts):
+            # `x in (1, 2, 3)`: one of the values equals x
+            tests = [ast.Compare(left=node.left, ops=[ast.Eq()], comparators=[e]) for e in node.comparators[0].elts]
+            code, ty = self.e_BoolOp(ast.BoolOp(op=ast.Or(), values=tests))
+            return (f"(!{code})" if isinstance(node.ops[0], ast.NotIn) else code), ty
         parts = []
         lc, lt = self.emit(node.left)
         for op, right in zip(node.ops, node.comparators):
@@ -428,6 +443,15 @@ class ExprEmitter:
             return truth(c, t), T.BOOL
         if name == "pow" and len(args) == 2:
             return self.e_BinOp(ast.BinOp(left=args[0], op=ast.Pow(), right=args[1]))
+        if name == "len" and len(args) == 1 and isinstance(args[0], ast.Name) and args[0].id in self.arrays:
+            self.shape_scalars.add((args[0].id, 0))
+            return cname(f"{args[0].id}_shape_0"), T.WEAK_INT
+        if name == "round" and len(args) == 1:       # Python's round(): half to even, an int
+            c, t = self.emit(args[0])
+            if not t.is_float:
+                return c, t
+            fn = "rintf" if t.name == "float32" else "rint"
+            return f"((long long){fn}({c}))", T.WEAK_INT
         if name in _UNARY_MATH and len(args) == 1:        # `from math import sqrt`
             return self._float_fn(_UNARY_MATH[name], [self.emit(args[0])])
         raise ValueError(f"Unknown function: {name}")
@@ -474,4 +498,49 @@ class ExprEmitter:
             if not t.is_float:
                 return "false", T.BOOL
             return f"(__builtin_{attr}({c}) != 0)", T.BOOL
+        if attr == "isfinite" and len(args) == 1:
+            c, t = self.emit(args[0])
+            if not t.is_float:
+                return "true", T.BOOL
+            return f"(__builtin_isfinite({c}) != 0)", T.BOOL
+        # the rest are spelled through operators and functions that exist already
+        P = ast.parse
+        call = lambda fn, *xs: ast.Call(func=P(fn, mode="eval").body, args=list(xs), keywords=[])   # noqa: E731
+        num = lambda v: ast.Constant(value=v)                                                          # noqa: E731
+        if attr == "clip" and len(args) == 3:
+            return self._minmax("min", call("min", call("max", args[0], args[1]), args[2]))
+        if attr in ("mod", "remainder") and len(args) == 2:
+            return self.e_BinOp(ast.BinOp(left=args[0], op=ast.Mod(), right=args[1]))
+        if attr == "floor_divide" and len(args) == 2:
+            return self.e_BinOp(ast.BinOp(left=args[0], op=ast.FloorDiv(), right=args[1]))
+        if attr in ("divide", "true_divide") and len(args) == 2:
+            return self.e_BinOp(ast.BinOp(left=args[0], op=ast.Div(), right=args[1]))
+        if attr in ("add", "subtract", "multiply") and len(args) == 2:
+            op = {"add": ast.Add(), "subtract": ast.Sub(), "multiply": ast.Mult()}[attr]
+            return self.e_BinOp(ast.BinOp(left=args[0], op=op, right=args[1]))
+        if attr == "negative" and len(args) == 1:
+            return self.e_UnaryOp(ast.UnaryOp(op=ast.USub(), operand=args[0]))
+        if attr == "reciprocal" and len(args) == 1:
+            return self.e_BinOp(ast.BinOp(left=num(1.0), op=ast.Div(), right=args[0]))
+        if attr in ("deg2rad", "radians", "rad2deg", "degrees") and len(args) == 1:
+            f = math.pi / 180.0 if attr in ("deg2rad", "radians") else 180.0 / math.pi
+            if is_math:
+                c, t = self.emit(args[0])
+                return f"({cast(c, t, T.F64)} * {T.float_literal(f, T.F64)})", T.WEAK_FLOAT
+            c, t = self.emit(args[0])
+            ft = T.to_float(t)
+            return f"({cast(c, t, ft)} * {T.float_literal(f, ft.strong() if not ft.weak else T.F64)})", ft
+        if attr in ("round", "around", "round_") and len(args) == 1 and not is_math:
+            return self._module_call(mod, "rint", call("np.rint", args[0]))   # half to even, like NumPy
+        if attr == "sign" and len(args) == 1:
+            c, t = self.emit(args[0])
+            if t.is_bool or t.kind == "u":
+                return f"(({t.c})(({c}) != 0))", t
+            zero = "0" if t.is_int else T.float_literal(0.0, t if not t.weak else T.F64)
+            return f"(({t.c})((({c}) > {zero}) - (({c}) < {zero})))", t
+        if attr == "heaviside" and len(args) == 2:
+            test_neg = ast.Compare(left=args[0], ops=[ast.Lt()], comparators=[num(0.0)])
+            test_zero = ast.Compare(left=args[0], ops=[ast.Eq()], comparators=[num(0.0)])
+            return self.e_IfExp(ast.IfExp(test=test_neg, body=num(0.0),
+                                          orelse=ast.IfExp(test=test_zero, body=args[1], orelse=num(1.0))))
         raise ValueError(f"Unknown function: {mod}.{attr}")

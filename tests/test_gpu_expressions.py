@@ -587,3 +587,37 @@ def test_random_programs_against_the_interpreter(gpu, seed):
     appy.jit(ns["kernel"])(*args.values(), out)
     scale = np.maximum(1.0, np.abs(ref))
     assert np.all(np.abs(out - ref) <= 2e-4 * scale * m), "\n".join(body)
+
+
+def test_more_numpy_functions_and_builtins(gpu):
+    import appy_amd as appy
+
+    @appy.jit
+    def many(d, k, o1, o2, o3, o4, flags):
+        #pragma parallel for simd
+        for i in range(d.shape[0]):
+            o1[i] = np.clip(d[i], -0.5, 0.75) + np.sign(d[i]) + np.heaviside(d[i], 0.5) + np.reciprocal(d[i] + 3.0)
+            o2[i] = np.mod(d[i], 0.7) + np.remainder(k[i], 5) + np.floor_divide(d[i], 0.3) + np.copysign(2.0, d[i])
+            o3[i] = np.round(d[i] * 3.0) + round(d[i] * 5.0) + np.deg2rad(d[i]) + np.rad2deg(d[i]) + np.negative(d[i])
+            o4[i] = len(d) + d.size + d.ndim + np.multiply(d[i], 2.0) - np.subtract(d[i], 1.0) + np.divide(k[i], 4)
+            flags[i] = np.isfinite(d[i]) and (k[i] in (1, 2, 3) or k[i] not in (0, 4, 5, 6, 7))
+
+    rng = np.random.default_rng(44)
+    n = 10_007
+    d = rng.uniform(-2, 2, n)
+    d[::97] = 0.0
+    d[5] = np.inf
+    k = rng.integers(-3, 9, n).astype(np.int32)
+    o1, o2, o3, o4 = (np.zeros(n) for _ in range(4))
+    flags = np.zeros(n, bool)
+    many(d, k, o1, o2, o3, o4, flags)
+    with np.errstate(all="ignore"):
+        r1 = np.clip(d, -0.5, 0.75) + np.sign(d) + np.heaviside(d, 0.5) + np.reciprocal(d + 3.0)
+        r2 = np.mod(d, 0.7) + np.remainder(k, 5) + np.floor_divide(d, 0.3) + np.copysign(2.0, d)
+        r3 = np.round(d * 3.0) + np.rint(d * 5.0) + np.deg2rad(d) + np.rad2deg(d) + np.negative(d)
+        r4 = n + n + 1 + np.multiply(d, 2.0) - np.subtract(d, 1.0) + np.divide(k, 4)
+    rf = np.isfinite(d) & (np.isin(k, (1, 2, 3)) | ~np.isin(k, (0, 4, 5, 6, 7)))
+    fin = np.isfinite(d)
+    for got, ref in ((o1, r1), (o2, r2), (o3, r3), (o4, r4)):
+        assert np.allclose(got[fin], ref[fin], rtol=1e-12, atol=1e-12)
+    assert np.array_equal(flags, rf)
