@@ -43,17 +43,71 @@ class _Normalise(ast.NodeTransformer):
     (reference: appy/frontend/rewrite_tuple_assign.py:4-17,
     rewrite_aug_assign.py:5-20, rewrite_range.py:4-27)."""
 
+    _tmp = 0
+
     def visit_Assign(self, node):
         self.generic_visit(node)
+        if len(node.targets) > 1:
+            # a = b = e  ->  a = e; b = a   (targets are assigned from left to right)
+            first, rest = node.targets[0], node.targets[1:]
+            out = self.visit_Assign(ast.copy_location(ast.Assign(targets=[first], value=node.value), node))
+            out = out if isinstance(out, list) else [out]
+            src_ = copy.deepcopy(first)
+            for n in ast.walk(src_):
+                if hasattr(n, "ctx"):
+                    n.ctx = ast.Load()
+            for t in rest:
+                more = self.visit_Assign(ast.copy_location(ast.Assign(targets=[t], value=copy.deepcopy(src_)), node))
+                out.extend(more if isinstance(more, list) else [more])
+            return out
         if isinstance(node.value, ast.Tuple):
             tgt = node.targets[0]
             assert isinstance(tgt, ast.Tuple) and len(tgt.elts) == len(node.value.elts), (
                 "a tuple on the right-hand side needs a tuple of the same length on the left"
             )
-            return [
-                ast.copy_location(ast.Assign(targets=[t], value=v), node)
-                for t, v in zip(tgt.elts, node.value.elts)
-            ]
+            written = {ast.unparse(t) for t in tgt.elts}
+            reads_a_target = any(
+                isinstance(n, (ast.Name, ast.Subscript)) and ast.unparse(n) in written
+                for v in node.value.elts[1:] for n in ast.walk(v))
+            if not reads_a_target:
+                return [
+                    ast.copy_location(ast.Assign(targets=[t], value=v), node)
+                    for t, v in zip(tgt.elts, node.value.elts)
+                ]
+            # `p, q = q, p`: the right-hand side is evaluated in full before anything is stored
+            out, temps = [], []
+            for v in node.value.elts:
+                _Normalise._tmp += 1
+                name = f"__appy_t{_Normalise._tmp}"
+                temps.append(name)
+                out.append(ast.copy_location(ast.Assign(targets=[ast.Name(id=name, ctx=ast.Store())], value=v), node))
+            for t, name in zip(tgt.elts, temps):
+                out.append(ast.copy_location(ast.Assign(targets=[t], value=ast.Name(id=name, ctx=ast.Load())), node))
+            return out
+        return node
+
+    def visit_AnnAssign(self, node):
+        self.generic_visit(node)
+        if node.value is None:
+            return None                     # a bare annotation declares nothing a kernel needs
+        return self.visit_Assign(ast.copy_location(ast.Assign(targets=[node.target], value=node.value), node))
+
+    def visit_Assert(self, node):
+        return None                         # as under `python -O`: kernels carry no assertions
+
+    def visit_Subscript(self, node):
+        self.generic_visit(node)
+        inner = node.value
+        if (isinstance(inner, ast.Subscript) and isinstance(inner.value, ast.Name)
+                and not isinstance(node.slice, (ast.Slice, ast.Tuple))
+                and not isinstance(inner.slice, ast.Slice)
+                and not (isinstance(inner.slice, ast.Tuple) and any(isinstance(e, ast.Slice) for e in inner.slice.elts))
+                and not (isinstance(inner.value, ast.Attribute))):
+            # A[r][c] is A[r, c]
+            first = list(inner.slice.elts) if isinstance(inner.slice, ast.Tuple) else [inner.slice]
+            return ast.copy_location(
+                ast.Subscript(value=inner.value, slice=ast.Tuple(elts=first + [node.slice], ctx=ast.Load()), ctx=node.ctx),
+                node)
         return node
 
     def visit_AugAssign(self, node):

@@ -621,3 +621,36 @@ def test_more_numpy_functions_and_builtins(gpu):
     for got, ref in ((o1, r1), (o2, r2), (o3, r3), (o4, r4)):
         assert np.allclose(got[fin], ref[fin], rtol=1e-12, atol=1e-12)
     assert np.array_equal(flags, rf)
+
+
+def test_statement_forms_of_ordinary_python(gpu):
+    """Swapping tuple assignments (right-hand side first), chained targets,
+    annotated assignments, asserts (dropped), ``A[r][c]``, ``elif`` chains."""
+    import appy_amd as appy
+
+    @appy.jit
+    def forms(d, a, A, out, cls):
+        #pragma parallel for simd
+        for i in range(d.shape[0]):
+            assert d[i] == d[i]
+            p = q = d[i] * 2.0
+            r: float = a[i]
+            p, r = r, p + q                     # r becomes 4 d[i], p becomes a[i]
+            p, q = q, p                         # swap: p = 2 d[i], q = a[i]
+            out[i] = p * 100.0 + q * 10.0 + r + A[i % 4][i % 5]
+            if d[i] > 1.0:
+                cls[i] = 2
+            elif d[i] > 0.0:
+                cls[i] = 1
+            else:
+                cls[i] = 0
+
+    rng = np.random.default_rng(51)
+    n = 5003
+    d, a = rng.uniform(-2, 2, n), rng.uniform(-2, 2, n)
+    A = rng.uniform(-1, 1, (4, 5))
+    out, cls = np.zeros(n), np.zeros(n, np.int64)
+    forms(d, a, A, out, cls)
+    i = np.arange(n)
+    assert np.allclose(out, 2 * d * 100.0 + a * 10.0 + 4 * d + A[i % 4, i % 5], rtol=1e-13, atol=1e-12)
+    assert np.array_equal(cls, np.where(d > 1.0, 2, np.where(d > 0.0, 1, 0)))
