@@ -119,6 +119,10 @@ def analyse(loop: ast.For, outer: ast.For) -> _Verdict:
             if isinstance(n, _BLOCKERS) or (isinstance(n, ast.Call) and not isinstance(n.func, (ast.Name, ast.Attribute))):
                 v.ok = False
                 return v
+            if isinstance(n, ast.stmt) and not isinstance(n, (ast.Assign, ast.AugAssign, ast.If, ast.Pass)) and not (
+                    isinstance(n, ast.Expr) and isinstance(n.value, ast.Constant)):
+                v.ok = False            # a kind of statement this analysis does not model (annotated assignment, ...)
+                return v
 
     # ---- assignments: scalars and array stores -------------------------------------
     scalar_kinds = {}            # name -> set of ops (None = plain)
