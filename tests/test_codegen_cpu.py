@@ -462,3 +462,27 @@ def test_clear_cache_option_regenerates_the_loop():
     f2, _ = cg.codegen(src, "kernel_loop_1", {"a": a, "n": 8}, {})
     f3, _ = cg.codegen(src, "kernel_loop_1", {"a": a, "n": 8}, {"clear_cache": True})
     assert f1 is f2 and f3 is not f1
+
+
+def test_generated_code_objects_hold_no_packed_fp32_instructions():
+    """Kernels are compiled with the packed-fp32 feature switched off; the ISA of a
+    float-heavy generated kernel (own code object) must show none of those forms."""
+    import os
+    import re
+    import subprocess
+    import tempfile
+
+    objdump = "/opt/rocm/llvm/bin/llvm-objdump"
+    if not os.path.exists(objdump):
+        pytest.skip("llvm-objdump not found")
+    x = np.zeros(64, np.float32)
+    src = ("#pragma parallel for simd\nfor i in range(n):\n    xi = x[i]\n    x3 = xi * xi * xi\n"
+           "    y[i] = 0.5 * xi * (1 + 0.044715 * x3) + xi * 2.0 + x3 * 3.0 + z[i] * xi\n")
+    f, _ = compiled(src, x=x, y=x.copy(), z=x.copy(), n=64)
+    with tempfile.NamedTemporaryFile(suffix=".co") as fh:
+        fh.write(f.kernels[f.default_spec].code)
+        fh.flush()
+        isa = subprocess.run([objdump, "-d", fh.name], capture_output=True, text=True, check=True).stdout
+    assert "v_mul_f32" in isa or "v_fma" in isa or "v_add_f32" in isa
+    assert not re.search(r"v_pk_(add|mul|fma)_f32", isa)
+    assert "global_load_dwordx4" in isa and "global_store_dwordx4" in isa
