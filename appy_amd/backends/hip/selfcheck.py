@@ -98,6 +98,16 @@ def spmv(A_data, A_indptr, A_indices, x, M, N):
     return y
 
 
+def gather_dot(v, idx, x):
+    """Calibration loop: one coalesced stream of (value, index) pairs and one 4-byte
+    gather per pair, i.e. the memory behaviour of CSR SpMV without its row structure."""
+    s = 0.0
+    #pragma parallel for simd shared(s)
+    for i in range(v.shape[0]):
+        s += v[i] * x[idx[i]]
+    return s
+
+
 def spmm(A_data, A_indptr, A_indices, B, y, M):
     #pragma parallel for
     for i in range(M):
@@ -107,7 +117,7 @@ def spmm(A_data, A_indptr, A_indices, B, y, M):
             y[i, :] += A_data[k] * B[A_indices[k], :]
 
 
-_RAW = (vec_add, copy, vector_sum, masked_sum, gemv, gemv_columns, spmv, spmm)
+_RAW = (vec_add, copy, vector_sum, masked_sum, gemv, gemv_columns, spmv, spmm, gather_dot)
 _cache = {}
 
 
@@ -149,6 +159,7 @@ def compile_all_patterns() -> int:
     k.gemv_columns(A, x[:8].copy())
     k.spmv(data, indptr, indices, x[:8].copy(), 8, 8)
     k.spmm(data, indptr, indices, B, Y, 8)
+    k.gather_dot(data, indices, x[:8].copy())
     count = 0
     for key in set(cg.code_cache) - before:
         loop, _src = cg.code_cache[key]

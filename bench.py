@@ -53,7 +53,7 @@ def parse_args():
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=50)
     p.add_argument("--warmup", type=int, default=5)
-    p.add_argument("--workloads", default="vector_sum,masked_sum,copy,vec_add,gemv,gemv_columns,spmv_uniform,spmv_powerlaw,spmv_powerlaw16,spmm",
+    p.add_argument("--workloads", default="vector_sum,masked_sum,copy,vec_add,gemv,gemv_columns,gather,spmv_uniform,spmv_powerlaw,spmv_powerlaw16,spmm",
                    help="comma separated subset; vector_sum is always run (headline)")
     p.add_argument("--scale", type=float, default=1.0, help="shrink every size by this factor (debugging)")
     p.add_argument("--no-cpu-baseline", action="store_true")
@@ -328,8 +328,34 @@ def main():
         vals = {"A_data": data_d, "A_indptr": indptr_d, "A_indices": indices_d, "x": x_d, "y": y_d, "M": m}
         nbytes = 8 * nnz + 4 * (m + 1) + 4 * ncol + 4 * m
         results[name] = run.measure(loop, vals, nbytes, K, W)
-        results[name].update({"nnz": int(nnz), "rows": m, "mean_row": float(nnz) / m, "max_row": int(lens.max().item())})
+        results[name].update({"nnz": int(nnz), "rows": m, "mean_row": float(nnz) / m, "max_row": int(lens.max().item()),
+                              "giga_nnz_per_s": nnz / results[name]["kernel_ms"] / 1e6})
+        if "gather" in results:
+            results[name]["frac_of_gather_rate"] = results[name]["giga_nnz_per_s"] / results["gather"]["giga_gathers_per_s"]
         log(name, results[name], parity[name])
+
+    # ---------------- calibration: the gather rate of the device ---------------------------------
+    # s += v[i] * x[idx[i]] over 2^26 (value, index) pairs with uniformly random indices into
+    # 2^22 floats: the memory behaviour of the uniform SpMV (8 streamed bytes and one 4-byte
+    # gather from a 16 MiB vector per non-zero) without its row structure.  What this loop
+    # reaches is what the machine gives a CSR SpMV over such a matrix.
+    if "gather" in want:
+        ng, nx = shrink(1 << 26), shrink(1 << 22)
+        gx = torch.Generator(device="cuda"); gx.manual_seed(43)
+        v_d = torch.randn(ng, generator=gx, device="cuda", dtype=torch.float32)
+        idx_d = torch.randint(0, nx, (ng,), generator=gx, device="cuda", dtype=torch.int32)
+        xg_d = torch.randn(nx, generator=gx, device="cuda", dtype=torch.float32)
+        before = set(cg.code_cache)
+        got = k.gather_dot(v_d, idx_d, xg_d)
+        loop = run.loop_of(before)
+        ref, budget = vo.gather_dot(v_d.cpu().numpy(), idx_d.cpu().numpy(), xg_d.cpu().numpy())
+        parity["gather"] = {"abs_err": abs(got - ref), "bound": vo.TOL * budget, "ok": abs(got - ref) <= vo.TOL * budget}
+        vals = {"s": s_d, "v": v_d, "idx": idx_d, "x": xg_d, "v_shape_0": ng}
+        results["gather"] = run.measure(loop, vals, 8 * ng + 4 * nx + 8, K, W, clear=s_d)
+        results["gather"]["giga_gathers_per_s"] = ng / results["gather"]["kernel_ms"] / 1e6
+        log("gather", results["gather"], parity["gather"])
+        del v_d, idx_d, xg_d
+        torch.cuda.empty_cache()
 
     spmv_case.loop = None
     if "spmv_uniform" in want:

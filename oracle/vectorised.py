@@ -60,6 +60,13 @@ def spmm_csr(data, indptr, indices, B, shape):
     return np.asarray(C), np.asarray(budget)
 
 
+def gather_dot(v, idx, x):
+    """s += v[i] * x[idx[i]]: the inner loop of examples/03-spmv.py:12-13 over one flat
+    stream of (value, index) pairs (used to calibrate the gather rate)."""
+    terms = np.asarray(v, dtype=np.float64) * np.asarray(x, dtype=np.float64)[np.asarray(idx)]
+    return float(terms.sum()), float(np.abs(terms).sum())
+
+
 def within_budget(out, value, budget, tol=TOL):
     """max over outputs of |out - value| / (tol * budget) <= 1 (outputs whose
     budget is zero must be exact)."""

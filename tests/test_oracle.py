@@ -53,6 +53,19 @@ def test_masked_sum_masks_and_complement():
     assert abs(np.corrcoef(A, M)[0, 1]) < 0.05
 
 
+def test_gather_dot_is_a_one_row_spmv():
+    rng = np.random.default_rng(31)
+    v = rng.standard_normal(501).astype(np.float32)
+    x = rng.standard_normal(64).astype(np.float32)
+    idx = rng.integers(0, 64, 501).astype(np.int32)
+    val, budget = vo.gather_dot(v, idx, x)
+    assert val == pytest.approx(math.fsum(float(v[i]) * float(x[idx[i]]) for i in range(501)), rel=1e-13)
+    assert budget == pytest.approx(math.fsum(abs(float(v[i]) * float(x[idx[i]])) for i in range(501)), rel=1e-13)
+    # identity permutation: a plain dot product; a constant index picks one element of x
+    assert vo.gather_dot(x, np.arange(64), x)[0] == pytest.approx(float(x.astype(np.float64) @ x.astype(np.float64)), rel=1e-14)
+    assert vo.gather_dot(v, np.full(501, 7), x)[0] == pytest.approx(float(x[7]) * vo.vector_sum(v)[0], rel=1e-12)
+
+
 def test_gemv_unit_vectors_identity_linearity_loop():
     A, x = wl.gemv(37, 53)
     val, budget = vo.gemv(A, x)
