@@ -37,6 +37,7 @@ MEASURED_TRAFFIC = {
     "vec_add": int((65549.0 * 2.000 + 65536.0 * 0.999) * 1024),
     "gemv": int((524558.6 * 2.000 + 64.0 * 0.999) * 1024),
     "gemv_columns": int((524558.5 * 2.000 + 64.0 * 0.999) * 1024),
+    "gather": int((3422204.6 * 2.000 + 6.0 * 0.999) * 1024),
     "spmv_uniform": int((3442392.1 * 2.000 + 18589.0 * 0.999) * 1024),
     "spmv_powerlaw": int((21322939.7 * 2.000 + 37060.8 * 0.999) * 1024),
     "spmm": int((8641723.2 * 2.000 + 524288.0 * 0.999) * 1024),
