@@ -219,6 +219,110 @@ def reduction_operand(assign: ast.Assign):
     return a
 
 
+def _as_addition(assign: ast.Assign) -> None:
+    """``t = t - e`` becomes ``t = t + (-e)`` (the same value in IEEE and in wrapping
+    integer arithmetic), so that a running difference is a ``+`` reduction."""
+    val = assign.value
+    if (isinstance(val, ast.BinOp) and isinstance(val.op, ast.Sub) and len(assign.targets) == 1
+            and isinstance(val.left, (ast.Name, ast.Subscript))
+            and ast.unparse(val.left) == ast.unparse(assign.targets[0])):
+        assign.value = ast.BinOp(left=val.left, op=ast.Add(), right=ast.UnaryOp(op=ast.USub(), operand=val.right))
+
+
+def _element_reduction(st, loop_var: str, assigned: set, body):
+    """For ``X[idx] = X[idx] op e`` / ``X[idx] = max(X[idx], e)`` at the top level of a
+    simd loop, with ``idx`` the same in every iteration and ``X`` touched nowhere else in
+    the loop: the operator; otherwise None."""
+    if not (isinstance(st, ast.Assign) and len(st.targets) == 1):
+        return None
+    tgt = st.targets[0]
+    if not (isinstance(tgt, ast.Subscript) and isinstance(tgt.value, ast.Name)) or is_scalar_location(tgt):
+        return None
+    idx = tgt.slice.elts if isinstance(tgt.slice, ast.Tuple) else [tgt.slice]
+    for e in idx:
+        if isinstance(e, ast.Slice):
+            return None
+        for n in ast.walk(e):
+            if isinstance(n, ast.Name) and (n.id == loop_var or n.id in assigned):
+                return None
+            if isinstance(n, ast.Subscript):
+                return None                 # an index read from memory: keep to the simple case
+    key = ast.unparse(tgt)
+    val = st.value
+    same = lambda e: isinstance(e, ast.Subscript) and ast.unparse(e) == key   # noqa: E731
+    if isinstance(val, ast.BinOp) and isinstance(val.op, (ast.Add, ast.Mult)) and same(val.left) != same(val.right):
+        op, other = ("+" if isinstance(val.op, ast.Add) else "*"), (val.right if same(val.left) else val.left)
+    elif (isinstance(val, ast.Call) and isinstance(val.func, ast.Name) and val.func.id in ("max", "min")
+          and len(val.args) == 2 and not val.keywords and same(val.args[0]) != same(val.args[1])):
+        op, other = val.func.id, (val.args[1] if same(val.args[0]) else val.args[0])
+    else:
+        return None
+    # the array may appear in the loop only as the two mentions of this statement
+    mentions = sum(1 for b in body for n in ast.walk(b) if isinstance(n, ast.Name) and n.id == tgt.value.id)
+    if mentions != 2 or any(isinstance(n, ast.Name) and n.id == tgt.value.id for n in ast.walk(other)):
+        return None
+    return op, other
+
+
+def _hoist_element_reductions(tree: ast.Module) -> None:
+    """A ``simd`` loop inside a parallel loop that accumulates into one array element
+    (``y[i] += A[i, j] * x[j]`` under ``for j``) carries a dependence through memory that
+    its lanes would race on.  Such an element becomes a scalar around the loop::
+
+        __appy_e1 = y[i]
+        #pragma simd
+        for j in ...: __appy_e1 = __appy_e1 + A[i, j] * x[j]
+        y[i] = __appy_e1
+
+    which the reduction detection below then treats like any local accumulator."""
+    counter = [0]
+
+    def block(stmts, inside_parallel):
+        out = []
+        for st in stmts:
+            if isinstance(st, ast.For):
+                pragma = getattr(st, "pragma", None) or {}
+                var = st.target.id if isinstance(st.target, ast.Name) else ""
+                if inside_parallel and "simd" in pragma and "parallel_for" not in pragma:
+                    for a in st.body:
+                        if isinstance(a, ast.Assign):
+                            _as_addition(a)
+                    assigned = {n.targets[0].id for b in st.body for n in ast.walk(b)
+                                if isinstance(n, ast.Assign) and isinstance(n.targets[0], ast.Name)}
+                    pre, post = [], []
+                    for k, a in enumerate(list(st.body)):
+                        found = _element_reduction(a, var, assigned, st.body)
+                        if found is None:
+                            continue
+                        op, other = found
+                        counter[0] += 1
+                        name = f"__appy_e{counter[0]}"
+                        tgt = a.targets[0]
+                        read = copy.deepcopy(tgt)
+                        read.ctx = ast.Load()
+                        pre.append(ast.copy_location(ast.Assign(targets=[ast.Name(id=name, ctx=ast.Store())], value=read), st))
+                        acc = ast.Name(id=name, ctx=ast.Load())
+                        if op in ("+", "*"):
+                            value = ast.BinOp(left=acc, op=ast.Add() if op == "+" else ast.Mult(), right=other)
+                        else:
+                            value = ast.Call(func=ast.Name(id=op, ctx=ast.Load()), args=[acc, other], keywords=[])
+                        st.body[k] = ast.copy_location(ast.Assign(targets=[ast.Name(id=name, ctx=ast.Store())], value=value), a)
+                        post.append(ast.copy_location(
+                            ast.Assign(targets=[copy.deepcopy(tgt)], value=ast.Name(id=name, ctx=ast.Load())), st))
+                    out.extend(pre + [st] + post)
+                    continue
+                st.body = block(st.body, inside_parallel or "parallel_for" in pragma)
+            else:
+                for f in ("body", "orelse"):
+                    sub = getattr(st, f, None)
+                    if isinstance(sub, list) and sub and isinstance(sub[0], ast.stmt):
+                        setattr(st, f, block(sub, inside_parallel))
+            out.append(st)
+        return out
+
+    tree.body = block(tree.body, False)
+
+
 def _assignments_in(node):
     for n in ast.walk(node):
         if isinstance(n, ast.Assign):
@@ -242,6 +346,7 @@ def _mark_all(tree: ast.Module) -> None:
         for a in _assignments_in(loop):
             tgt = a.targets[0]
             if is_scalar_location(tgt):
+                _as_addition(a)
                 ops_of.setdefault(ast.unparse(tgt), set()).add(reduction_operator(a))
         found = {}
         for a in _assignments_in(loop):
@@ -292,6 +397,7 @@ def build(loop_source: str) -> ast.Module:
     check_structure(tree)
     tree = _Normalise().visit(tree)
     tree.body, _ = _attach_pragmas(tree.body, None)
+    _hoist_element_reductions(tree)
     _mark_all(tree)
     ast.fix_missing_locations(tree)
     return tree

@@ -295,3 +295,34 @@ def f(data, indptr, indices, B, C):
     # loops under a pragma are left as the programmer wrote them
     kept = loop_text("def f(A, y):\n    #pragma parallel for\n    for i in range(A.shape[0]):\n        for j in range(A.shape[1]):\n            A[i, j] = 0\n")
     assert "#pragma simd" not in kept
+
+
+def test_ir_simd_loops_accumulating_into_one_element_use_a_scalar():
+    """`y[i] += ...` under an inner simd loop carries a dependence through memory; the
+    element is accumulated in a scalar around the loop (the reference's detection only knows
+    names and literal subscripts, appy/frontend/reduction_detection.py:12-13)."""
+    tree = loop_ir.build(
+        "#pragma parallel for\nfor i in range(n):\n    y[i] = 0.0\n    #pragma simd\n"
+        "    for j in range(m):\n        y[i] += A[i, j] * x[j]\n        z[i] = max(z[i], A[i, j])\n        w[i] -= x[j]")
+    body = loop_ir.outer_loop(tree).body
+    text = [ast.unparse(s) for s in body]
+    assert text[:4] == ["y[i] = 0.0", "__appy_e1 = y[i]", "__appy_e2 = z[i]", "__appy_e3 = w[i]"]
+    assert text[5:] == ["y[i] = __appy_e1", "z[i] = __appy_e2", "w[i] = __appy_e3"]
+    inner = body[4]
+    assert [ast.unparse(s) for s in inner.body] == [
+        "__appy_e1 = __appy_e1 + A[i, j] * x[j]", "__appy_e2 = max(__appy_e2, A[i, j])", "__appy_e3 = __appy_e3 + -x[j]"]
+    assert inner.pragma["reduction"] == "+:__appy_e1,max:__appy_e2,+:__appy_e3"
+    # an element that depends on the loop variable, or an array the loop also reads elsewhere, is left alone
+    tree = loop_ir.build(
+        "#pragma parallel for\nfor i in range(n):\n    #pragma simd\n    for j in range(m):\n"
+        "        y[j] += A[i, j]\n        v[i] += v[j]")
+    inner = loop_ir.outer_loop(tree).body[0]
+    assert [ast.unparse(s) for s in inner.body] == ["y[j] = y[j] + A[i, j]", "v[i] = v[i] + v[j]"]
+
+
+def test_ir_running_difference_is_a_sum_reduction():
+    tree = loop_ir.build(
+        "#pragma parallel for\nfor i in range(n):\n    s = 0.0\n    #pragma simd\n"
+        "    for j in range(m):\n        s -= A[i, j]\n    y[i] = s")
+    inner = loop_ir.outer_loop(tree).body[1]
+    assert ast.unparse(inner.body[0]) == "s = s + -A[i, j]" and inner.pragma["reduction"] == "+:s"

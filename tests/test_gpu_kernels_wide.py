@@ -540,3 +540,50 @@ def test_strip_loops_inside_a_sequential_loop_with_uniform_bounds(gpu):
     assert np.allclose(A, ref, rtol=1e-12, atol=1e-12)
     loop = [v[0] for kk, v in cg.code_cache.items() if kk[-1] == "repeated_column_smoothing"][-1]
     assert loop.last_launch.spec.kind == "strip"
+
+
+@appy.jit
+def rows_into_elements(A, x, y, z, w):
+    #pragma parallel for
+    for i in range(A.shape[0]):
+        y[i] = 0.5
+        #pragma simd
+        for j in range(A.shape[1]):
+            y[i] += A[i, j] * x[j]
+            z[i] = max(z[i], A[i, j])
+            w[i] -= x[j]
+
+
+@appy.jit
+def running_differences(a, A, y):
+    s = 10.0
+    #pragma parallel for simd shared(s)
+    for i in range(a.shape[0]):
+        s -= a[i]
+    #pragma parallel for
+    for i in range(A.shape[0]):
+        t = 1.0
+        #pragma simd
+        for j in range(A.shape[1]):
+            t -= A[i, j]
+        y[i] = t
+    return s
+
+
+@pytest.mark.parametrize("shape", [(37, 83), (300, 1000), (5, 20000)])
+def test_simd_loops_that_accumulate_into_an_array_element(gpu, shape):
+    """`y[i] += ...` inside a simd loop: one element is updated by every iteration of the
+    loop, so it is accumulated in a register and stored once (a lane-parallel
+    read-modify-write of `y[i]` would lose updates)."""
+    rng = np.random.default_rng(11)
+    A, x = rng.standard_normal(shape), rng.standard_normal(shape[1])
+    y, z, w = np.zeros(shape[0]), np.full(shape[0], 0.25), rng.standard_normal(shape[0])
+    w0 = w.copy()
+    rows_into_elements(A, x, y, z, w)
+    assert np.allclose(y, 0.5 + A @ x)
+    assert np.array_equal(z, np.maximum(0.25, A.max(axis=1)))
+    assert np.allclose(w, w0 - x.sum())
+    a = rng.standard_normal(100_003)
+    s = running_differences(a, A, y)
+    assert s == pytest.approx(10.0 - a.sum(), rel=1e-12)
+    assert np.allclose(y, 1.0 - A.sum(axis=1))
