@@ -70,7 +70,6 @@ def rewrite_loops(fn, **options):
     new_source = ast.unparse(tree)
     if options["verbose_static_rewrite"]:
         print("[Static Rewrite] new code:\n", new_source)
-    code = compile(new_source, filename=f"<appy:{fn.__name__}>", mode="exec")
     import numpy
 
     g = fn.__globals__
@@ -78,10 +77,46 @@ def rewrite_loops(fn, **options):
     # The stub is spelled `appy._kernel_launch`; make that name resolve even if
     # the caller imported this package under another name.
     g.setdefault("appy", sys.modules[__name__])
-    namespace = {}
-    exec(code, g, namespace)
-    new_fn = namespace[fn.__name__]
+    free = fn.__code__.co_freevars
+    if free and fn.__closure__:
+        new_fn = _with_closure(fn, new_source, g)
+    else:
+        namespace = {}
+        exec(compile(new_source, filename=f"<appy:{fn.__name__}>", mode="exec"), g, namespace)
+        new_fn = namespace[fn.__name__]
     new_fn.__appy_source__ = new_source
+    return new_fn
+
+
+def _with_closure(fn, new_source, g):
+    """The rewritten function bound to the cells ``fn`` closes over, so that names of
+    an enclosing function (constants, helper functions defined next to the kernel)
+    stay visible, late binding included.  The loops have become strings, so each free
+    variable is mentioned once at the top of the body: that keeps it a free variable of
+    the new code object and puts it into the ``locals()`` the launch stub looks names up in."""
+    import types
+
+    free = fn.__code__.co_freevars
+    tree = ast.parse(new_source)
+    fdef = next(n for n in tree.body if isinstance(n, (ast.FunctionDef, ast.AsyncFunctionDef)) and n.name == fn.__name__)
+    mention = ast.Expr(value=ast.Tuple(elts=[ast.Name(id=v, ctx=ast.Load()) for v in free], ctx=ast.Load()))
+    at = 1 if (fdef.body and isinstance(fdef.body[0], ast.Expr) and isinstance(fdef.body[0].value, ast.Constant)
+               and isinstance(fdef.body[0].value.value, str)) else 0
+    fdef.body.insert(at, mention)
+    factory = ast.FunctionDef(
+        name="__appy_factory", args=ast.arguments(posonlyargs=[], args=[], kwonlyargs=[], kw_defaults=[], defaults=[]),
+        body=[ast.Assign(targets=[ast.Name(id=v, ctx=ast.Store()) for v in free], value=ast.Constant(value=None)),
+              fdef, ast.Return(value=ast.Name(id=fn.__name__, ctx=ast.Load()))],
+        decorator_list=[])
+    module = ast.fix_missing_locations(ast.Module(body=[factory], type_ignores=[]))
+    namespace = {}
+    exec(compile(module, filename=f"<appy:{fn.__name__}>", mode="exec"), g, namespace)
+    shell = namespace["__appy_factory"]()
+    cells = dict(zip(free, fn.__closure__))
+    new_fn = types.FunctionType(shell.__code__, g, fn.__name__, shell.__defaults__,
+                                tuple(cells[v] for v in shell.__code__.co_freevars))
+    new_fn.__kwdefaults__ = shell.__kwdefaults__
+    new_fn.__dict__.update(shell.__dict__)
     return new_fn
 
 

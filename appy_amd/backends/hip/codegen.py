@@ -47,6 +47,23 @@ _HOST_EVAL_GLOBALS = {"__builtins__": {"min": min, "max": max, "abs": abs, "int"
                                        "round": round, "bool": bool}}
 _device_header = None
 
+
+class _ShapeView:
+    """What host-side bound expressions may ask of an array argument: ``len(a)``,
+    ``a.shape``, ``a.size``, ``a.ndim`` (never its elements)."""
+
+    __slots__ = ("shape", "ndim", "size")
+
+    def __init__(self, a):
+        self.shape = tuple(int(d) for d in a.shape)
+        self.ndim = len(self.shape)
+        self.size = int(np.prod(self.shape, dtype=np.int64))
+
+    def __len__(self):
+        if not self.shape:
+            raise TypeError("len() of a 0-d array")
+        return self.shape[0]
+
 # Hardware facts used by the launch heuristics (MI355X: 256 CUs in 8 XCDs,
 # 256 MiB of memory-side cache in front of the HBM3E).
 DEFAULT_CUS = 256
@@ -274,6 +291,9 @@ class CompiledLoop:
             if isinstance(n, ast.For):
                 for arg in n.iter.args:
                     steering.update(x.id for x in ast.walk(arg) if isinstance(x, ast.Name))
+        # bounds that ask an array for its length or shape (`range(len(a) // 2)`) are given
+        # shape-only stand-ins of the arrays when they are evaluated on the host
+        self._bounds_name_arrays = bool(steering & set(a.arrays))
         self._value_only = [i for i, k in enumerate(self.arg_names)
                             if k in a.scalars and k not in steering and k not in a.assigned]
         self._value_only_set = set(self._value_only)
@@ -646,6 +666,9 @@ class CompiledLoop:
         env = {k: v for k, v in vals.items() if k not in a.arrays}
         env["np"] = np
         env["math"] = math
+        if self._bounds_name_arrays:
+            for k in a.arrays:
+                env[k] = _ShapeView(vals[k])
         lo = int(eval(self._lo_code, _HOST_EVAL_GLOBALS, env))
         hi = int(eval(self._hi_code, _HOST_EVAL_GLOBALS, env))
         if hi <= lo:

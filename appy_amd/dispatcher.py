@@ -31,13 +31,30 @@ def _resolve_backend(name):
     raise NotImplementedError("Unknown backend:" + str(name))
 
 
+def _by_value(v):
+    """A 0-d array or tensor (``np.array(2.0)``, ``torch.tensor(2.0)``, the result of a
+    ``.sum()``) enters a kernel as the scalar it holds, in its own dtype."""
+    if isinstance(v, np.ndarray):
+        return v[()]
+    host = v.detach().cpu()
+    try:
+        return host.numpy()[()]
+    except TypeError:           # a dtype NumPy does not have (bfloat16)
+        return host.item()
+
+
 def build_val_map(loop_source, local_scope, global_scope):
     val_map = {}
     for k in used_names(loop_source):      # locals shadow globals; no copy of either scope
         if k in local_scope:
-            val_map[k] = local_scope[k]
+            v = local_scope[k]
         elif k in global_scope:
-            val_map[k] = global_scope[k]
+            v = global_scope[k]
+        else:
+            continue
+        if getattr(v, "ndim", 1) == 0 and not isinstance(v, np.generic) and hasattr(v, "dtype"):
+            v = _by_value(v)
+        val_map[k] = v
     val_map.setdefault("np", np)
     val_map.setdefault("math", math)
     return val_map

@@ -326,3 +326,24 @@ def test_ir_running_difference_is_a_sum_reduction():
         "    for j in range(m):\n        s -= A[i, j]\n    y[i] = s")
     inner = loop_ir.outer_loop(tree).body[1]
     assert ast.unparse(inner.body[0]) == "s = s + -A[i, j]" and inner.pragma["reduction"] == "+:s"
+
+
+def test_decorated_functions_keep_their_closure():
+    """Free variables of the decorated function stay bound to the enclosing scope's cells
+    (late binding included); the reference executes the rewritten source at module level,
+    where such names are lost (appy/__init__.py:60-64)."""
+    def make(k):
+        @appy.jit(dry_run=True)
+        def f(a, out, beta=1.0):
+            """doc"""
+            #pragma parallel for simd
+            for i in range(a.shape[0]):
+                out[i] = k * a[i] + beta
+        return f
+
+    a, out = np.arange(10.0), np.zeros(10)
+    f = make(2.5)
+    f(a, out)
+    assert np.array_equal(out, 2.5 * a + 1.0)
+    f(a, out, beta=2.0)
+    assert np.array_equal(out, 2.5 * a + 2.0) and f.__name__ == "f"
