@@ -154,6 +154,19 @@ class _SimdRanges(ast.NodeTransformer):
         return node
 
 
+class _InnerPranges(ast.NodeTransformer):
+    """A ``prange`` loop inside a loop that already is a kernel promises independent
+    iterations and nothing more: inside the kernel it is a ``range`` loop (which the
+    vectoriser may then spread over lanes)."""
+
+    def visit_For(self, node):
+        self.generic_visit(node)
+        if _is_prange_loop(node):
+            node.iter.func = ast.Name(id="range", ctx=ast.Load())
+            node.iter.keywords = [k for k in node.iter.keywords if k.arg not in ("parallel", "shared")]
+        return node
+
+
 def prange_reductions(loop: ast.For):
     """Scalars that a ``prange`` loop without a pragma reduces across its
     iterations (reference behaviour as documented for ``appy.prange``,
@@ -227,6 +240,7 @@ class _LoopOutliner:
             loop.iter.func = ast.Name(id="range", ctx=ast.Load())
             loop.iter.keywords = []
         loop = _SimdRanges().visit(copy.deepcopy(loop))
+        loop.body = [_InnerPranges().visit(st) for st in loop.body]
         if pragma:
             shared = shared_names(pragma)
             if shared:

@@ -485,3 +485,19 @@ def test_random_prange_nests_agree_with_the_interpreter(gpu, seed):
     appy.jit(ns["kernel"])(**got)
     for key in ("B", "y", "c", "out"):
         assert np.allclose(got[key], ref[key], rtol=1e-10, atol=1e-10), (key, src)
+
+
+@appy.jit
+def nested_pranges(A, B):
+    for i in appy.prange(A.shape[0]):
+        for j in appy.prange(A.shape[1]):
+            B[i, j] = A[i, j] * 2 + i
+
+
+def test_prange_inside_prange_is_a_range_loop_of_the_kernel(gpu):
+    A = np.random.default_rng(3).standard_normal((41, 300))
+    B = np.zeros_like(A)
+    nested_pranges(A, B)
+    assert np.array_equal(B, A * 2 + np.arange(41)[:, None])
+    assert "for j in range(A_shape_1)" in nested_pranges.__appy_source__
+    assert "#pragma simd" in nested_pranges.__appy_source__        # and the vectoriser sees it
