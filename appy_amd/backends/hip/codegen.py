@@ -71,6 +71,10 @@ MALL_BYTES = 256 << 20
 REDUCTION_WINDOW_BYTES = 6 << 20
 CACHED_REDUCTION_WINDOW_BYTES = 4 << 20
 TEAM_BYTES_IN_FLIGHT = 8.0e6
+# staged launches kept per loop for exact repeats of a call; a host loop that launches once
+# per row or per time step (`for i in range(n): <kernel using i in a bound>`) cycles through
+# n of them
+REPLAY_CACHE_ENTRIES = 2048
 
 
 def device_header() -> str:
@@ -84,16 +88,13 @@ def device_header() -> str:
 # ---------------------------------------------------------------------------
 # classification of run-time values
 # ---------------------------------------------------------------------------
-def _kind(v) -> str:
-    return f"{type(v).__module__}.{type(v).__name__}"
-
-
 def is_numpy_array(v) -> bool:
-    return _kind(v) == "numpy.ndarray"
+    return isinstance(v, np.ndarray)
 
 
 def is_torch_tensor(v) -> bool:
-    return _kind(v) == "torch.Tensor" or (type(v).__module__.startswith("torch") and hasattr(v, "data_ptr"))
+    # without importing torch: its tensors (and their subclasses) are what has `data_ptr`
+    return not isinstance(v, np.ndarray) and hasattr(v, "data_ptr") and type(v).__module__.startswith("torch")
 
 
 def _torch_np_dtype(t):
@@ -616,8 +617,10 @@ class CompiledLoop:
             return
         plan.run()
         if key is not None and plan.replayable():
-            if len(self._replays) >= 64:
-                self._replays.clear()
+            if len(self._replays) >= REPLAY_CACHE_ENTRIES:
+                # drop the older half (dicts keep insertion order)
+                for old in list(self._replays)[:REPLAY_CACHE_ENTRIES // 2]:
+                    del self._replays[old]
             self._replays[key] = plan
 
     def overwrites(self, name, lo, hi, env, shape) -> bool:
@@ -705,12 +708,13 @@ class Launch:
         self.stream = 0
         device = 0
         # -- device and stream: PyTorch's when a GPU tensor takes part
-        gpu_tensors = [v for v in arrays.values() if is_torch_tensor(v) and v.device.type == "cuda"]
-        if gpu_tensors:
-            import torch
-
-            device = gpu_tensors[0].device.index or 0
-            self.stream = _current_raw_stream(device)
+        on_gpu = {}
+        for name, v in arrays.items():
+            if not isinstance(v, np.ndarray) and v.is_cuda:
+                if not on_gpu:
+                    device = v.device.index or 0
+                    self.stream = _current_raw_stream(device)
+                on_gpu[name] = True
         self.capture = graphs.current()
         if self.capture is not None:
             # the launch is recorded into the graph's stream, not executed
@@ -729,21 +733,24 @@ class Launch:
             arr = a.arrays[name]
             if not (arr.loaded or arr.stored):
                 continue
-            if is_numpy_array(v):
+            if isinstance(v, np.ndarray):
                 host = v if v.flags["C_CONTIGUOUS"] else np.ascontiguousarray(v)
                 self._stage_host(name, host, v, arr.stored)
-            elif v.device.type == "cuda":
+            elif name in on_gpu:
                 t = v
-                if t.ndim >= 1 and t.numel() > 1 and t.stride(-1) != 1:
+                strides = t.stride()
+                if strides and strides[-1] != 1 and t.numel() > 1:
                     self._no_capture(name, "its last dimension is not contiguous (it would be repacked per launch)")
                     t = v.contiguous()
+                    strides = t.stride()
                     self.keepalive_copies = True
                     if arr.stored:
                         self.keepalive.append(("copy_back", v, t))
                 self.keepalive.append(t)
-                self.ptr[name] = t.data_ptr()
-                self.strides[name] = [t.stride(d) for d in range(t.ndim)]
-                extents.append((name, t.data_ptr(), t.numel() * t.element_size(), arr.stored))
+                dptr = t.data_ptr()
+                self.ptr[name] = dptr
+                self.strides[name] = strides
+                extents.append((name, dptr, t.numel() * t.element_size(), arr.stored))
             else:
                 # CPU tensor: same path as NumPy through a shared-memory view
                 self._no_capture(name, "it is a CPU tensor (it would be copied per launch)")

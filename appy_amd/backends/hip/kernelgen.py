@@ -281,10 +281,46 @@ class LoopAnalysis:
         return out
 
     def _leader_store_reloaded(self) -> bool:
-        shared_out = set()
-        for n in ast.walk(self.outer):
-            if isinstance(n, ast.For) and n is not self.outer and "simd" in (getattr(n, "pragma", None) or {}):
-                shared_out.update(id(x) for x in ast.walk(n))
+        """True if some wavefront of a multi-wavefront team could read an array element
+        on the wrong side of a store that only the leading wavefront issues.
+
+        Statements outside the shared-out loops run on every wavefront, their stores on
+        one.  A store to ``X`` is harmless when every other load of ``X`` in the loop nest
+        (a) comes earlier in program order, (b) shares no sequential loop with the store
+        (no later iteration reads after it) and (c) stands inside a shared-out loop, whose
+        closing barrier every wavefront passes after its loads and before the store
+        (in-place updates such as ``B[i, j] = alpha * (B[i, j] + sum_k A[k, i] * B[k, j])``).
+        Anything else counts as a reload."""
+        shared_out = set()          # ids of the nodes inside shared-out loops
+        spread = [n for n in ast.walk(self.outer)
+                  if isinstance(n, ast.For) and n is not self.outer and "simd" in (getattr(n, "pragma", None) or {})]
+        if not spread:
+            parts = _find_strip_parts(self.outer.body, self.var)
+            if parts is not None:
+                spread = [parts[1]]
+        for lp in spread:
+            shared_out.update(id(x) for x in ast.walk(lp))
+
+        order, loops_of = {}, {}    # id(node) -> position of its statement; -> enclosing inner loops
+        counter = [0]
+
+        def number(stmts, chain):
+            for st in stmts:
+                counter[0] += 1
+                here = counter[0]
+                if isinstance(st, (ast.For, ast.While, ast.If)):
+                    header = [st.iter] if isinstance(st, ast.For) else [st.test]
+                    for h in header:
+                        for x in ast.walk(h):
+                            order[id(x)], loops_of[id(x)] = here, chain
+                    inner = chain + (id(st),) if isinstance(st, (ast.For, ast.While)) else chain
+                    number(st.body, inner)
+                    number(st.orelse, inner)
+                else:
+                    for x in ast.walk(st):
+                        order[id(x)], loops_of[id(x)] = here, chain
+
+        number(self.outer.body, ())
         for st in ast.walk(self.outer):
             if not (isinstance(st, ast.Assign) and id(st) not in shared_out):
                 continue
@@ -295,7 +331,10 @@ class LoopAnalysis:
             for n in ast.walk(self.outer):
                 if (isinstance(n, ast.Subscript) and isinstance(n.ctx, ast.Load) and isinstance(n.value, ast.Name)
                         and n.value.id == t.value.id and id(n) not in mine):
-                    return True
+                    earlier = order.get(id(n), 1 << 60) < order.get(id(st), -1)
+                    apart = not (set(loops_of.get(id(n), ())) & set(loops_of.get(id(st), ())))
+                    if not (earlier and apart and id(n) in shared_out):
+                        return True
         return False
 
     def _find_strip(self):
@@ -321,7 +360,8 @@ class LoopAnalysis:
             return not any(isinstance(n, stop) for st in stmts for n in ast.walk(st))
 
         def has_simd(node):
-            return any(isinstance(n, ast.For) and "simd" in (getattr(n, "pragma", None) or {}) for n in ast.walk(node))
+            return any(isinstance(n, ast.For) and n is not self.outer and "simd" in (getattr(n, "pragma", None) or {})
+                       for n in ast.walk(node))
 
         def walk(stmts) -> bool:
             if skips_iterations(stmts):

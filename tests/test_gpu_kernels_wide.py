@@ -587,3 +587,55 @@ def test_simd_loops_that_accumulate_into_an_array_element(gpu, shape):
     s = running_differences(a, A, y)
     assert s == pytest.approx(10.0 - a.sum(), rel=1e-12)
     assert np.allclose(y, 1.0 - A.sum(axis=1))
+
+
+@appy.jit
+def trmm_row_by_row(alpha, A, B):
+    for i in range(B.shape[0]):
+        #pragma parallel for simd
+        for j in range(B.shape[1]):
+            s = 0.0
+            for k in range(i + 1, A.shape[0]):
+                s += A[k, i] * B[k, j]
+            B[i, j] = alpha * (B[i, j] + s)
+    return B
+
+
+@appy.jit
+def trmm_column_by_column(alpha, A, B):
+    #pragma parallel for
+    for j in range(B.shape[1]):
+        for i in range(B.shape[0]):
+            s = 0.0
+            #pragma simd
+            for k in range(i + 1, A.shape[0]):
+                s += A[k, i] * B[k, j]
+            B[i, j] = alpha * (B[i, j] + s)
+    return B
+
+
+def test_trmm_in_place_updates(gpu):
+    """The triangular product of the reference's NPBench tests
+    (tests/integration/triton/npbench/test_trmm.py:20-38), in the two race-free orders:
+    one launch per row with the columns in parallel (an in-place update whose loads all
+    precede its store: runs as a strip), and one launch with the columns in parallel around
+    the row loop (a stored row is read by later rows: single-wavefront teams)."""
+    from appy_amd.backends.hip import codegen as cg
+
+    M, N = 150, 200
+    A = np.fromfunction(lambda i, j: ((i * j) % M) / M, (M, M), dtype=np.float64)
+    np.fill_diagonal(A, 1.0)
+    B = np.fromfunction(lambda i, j: ((N + i - j) % N) / N, (M, N), dtype=np.float64)
+    want = B.copy()
+    for i in range(M):
+        want[i, :] += A[i + 1:, i] @ want[i + 1:, :]
+    want *= 1.5
+    got = trmm_row_by_row(1.5, A, B.copy())
+    assert np.allclose(got, want, atol=1e-6)
+    loop = next(v[0] for k, v in cg.code_cache.items() if k[-1] == "trmm_row_by_row")
+    assert loop.analysis.strip is not None and loop.analysis.multi_wave_ok
+    assert loop.choose_spec(N, dict(i=0, A_shape_0=M, alpha=1.5), dict(A=A, B=B)).kind == "strip"
+    got = trmm_column_by_column(1.5, A, B.copy())
+    assert np.allclose(got, want, atol=1e-6)
+    loop = next(v[0] for k, v in cg.code_cache.items() if k[-1] == "trmm_column_by_column")
+    assert not loop.analysis.multi_wave_ok
