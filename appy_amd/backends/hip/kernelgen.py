@@ -111,8 +111,9 @@ class OuterReduction:
     op: str
     array: str
     index: int
-    ty: Ty
+    ty: Ty               # type of the register accumulators (at least 32 bits wide)
     acc: str             # register name
+    elem_ty: Ty = None   # type of the array element the totals are combined into
 
 
 @dataclass
@@ -487,10 +488,16 @@ class LoopAnalysis:
                     and node.value.id in self.arrays and isinstance(node.slice, ast.Constant)
                     and type(node.slice.value) is int and self.arrays[node.value.id].ndim == 1):
                 arr = self.arrays[node.value.id]
+                acc_ty = arr.ty
                 if arr.ty.size < 4:
-                    raise Unsupported(f"Reduction into a {arr.ty.name} element is not supported: {key}")
+                    # 8- and 16-bit elements: registers and cross-lane steps work on 32 bits; sums
+                    # wrap to the element type at the end exactly as they would have step by step
+                    acc_ty = T.F32 if arr.ty.is_float else (T.Ty("uint32") if arr.ty.kind == "u" else T.I32)
+                if arr.ty.is_bool:
+                    op = {"+": "max", "*": "min"}.get(op, op)       # NumPy's bool arithmetic: or / and
                 self.outer_reductions.append(
-                    OuterReduction(key, op, arr.name, node.slice.value, arr.ty, f"__acc{len(self.outer_reductions)}")
+                    OuterReduction(key, op, arr.name, node.slice.value, acc_ty, f"__acc{len(self.outer_reductions)}",
+                                   arr.ty)
                 )
 
         # accesses indexed directly by the parallel loop variable: checked on
@@ -509,6 +516,27 @@ class LoopAnalysis:
                     off = _var_offset(e, self.var)
                     if off is not None and (n.value.id, d, off) not in into:
                         into.append((n.value.id, d, off))
+
+
+def _partial_type(ty: Ty) -> Ty:
+    """Type of the per-lane partial results of a reduction: registers and cross-lane
+    steps are 32 or 64 bits wide, so 16-bit floats accumulate in float32 (rounded once,
+    when the team combines) and 8/16-bit integers and flags in 32-bit integers (sums wrap
+    to the narrow type at the end exactly as they would have step by step)."""
+    if ty.size >= 4:
+        return ty
+    if ty.is_float:
+        return T.F32
+    return Ty("uint32") if ty.kind == "u" else T.I32
+
+
+def _partial_identity(op: str, ty: Ty, pty: Ty) -> str:
+    """Neutral element of ``op`` over ``ty``, written in the partial type ``pty``."""
+    if pty == ty or ty.is_float:
+        return T.identity_literal(op, pty)
+    if ty.is_bool:
+        return "0" if op in ("max", "+") else "1"
+    return f"(({pty.c}){T.identity_literal(op, ty)})"
 
 
 def _find_strip_parts(body, var):
@@ -694,10 +722,16 @@ class KernelBuilder:
         if not (isinstance(tgt, ast.Subscript) and isinstance(tgt.value, ast.Name)):
             raise Unsupported(f"Assignment target not supported in a kernel: {ast.unparse(tgt)}")
         key = ast.unparse(tgt)
-        if red_op and key in self.red_by_key and self.red_by_key[key].op == red_op:
+        if red_op and key in self.red_by_key and self.red_by_key[key].op in (
+                red_op, {"+": "max", "*": "min"}.get(red_op) if self.red_by_key[key].elem_ty.is_bool else red_op):
             r = self.red_by_key[key]
             oc, ot = self.ex.emit(loop_ir.reduction_operand(st))
-            upd = f"{r.acc} = {_OPS[r.op]}::f<{r.ty.c}>({r.acc}, {cast(oc, ot, r.ty)});"
+            if r.elem_ty.is_int and ot.is_float:
+                raise TypeError(
+                    f"`{key}` is an integer ({r.elem_ty.name}) but accumulates {ot.name} values, which would be "
+                    f"truncated one by one: start the shared scalar as a float (`0.0`)")
+            operand = f"(int)({truth(oc, ot)})" if r.elem_ty.is_bool else cast(oc, ot, r.ty)
+            upd = f"{r.acc} = {_OPS[r.op]}::f<{r.ty.c}>({r.acc}, {operand});"
             if self.mode == "team":
                 self.w(f"if ({self._leader()}) {{ {upd} }}")
             else:
@@ -760,11 +794,12 @@ class KernelBuilder:
         return op, other
 
     def _atomic_update(self, st, arr: ArrayParam, op: str, other):
-        if arr.ty.size < 4:
-            raise Unsupported(f"`{ast.unparse(st.targets[0])}` is updated by several iterations of the parallel loop; "
-                              f"atomic updates of {arr.ty.name} elements are not supported")
         oc, ot = self.ex.emit(other)
-        val = cast(oc, ot, arr.ty)
+        if arr.ty.is_bool:
+            op = {"+": "max", "*": "min"}.get(op, op)
+            val = f"(unsigned char)({truth(oc, ot)})"
+        else:
+            val = cast(oc, ot, arr.ty)
         if op == "-":
             op, val = "+", f"(-{val})"
         tgt = st.targets[0]
@@ -989,10 +1024,9 @@ class KernelBuilder:
             if ty is None:
                 raise NameError(f"reduction variable `{name}` has no value before the loop")
             p = self.fresh(f"part_{name}_")
-            if ty.is_float and ty.size < 4:
-                ty = T.F32      # lanes accumulate 16-bit floats in float32; rounded once when the team combines
-            self.partials[name] = (p, ty)
-            self.w(f"{ty.c} {p} = {T.identity_literal(op, ty)};")
+            pty = _partial_type(ty)
+            self.partials[name] = (p, pty)
+            self.w(f"{pty.c} {p} = {_partial_identity(op, ty, pty)};")
         saved_mode = self.mode
         self.mode = "lane"
         saved_depth, self.seq_depth = self.seq_depth, 0
@@ -1029,8 +1063,6 @@ class KernelBuilder:
             self.w("__syncthreads();")
         for name, op in reds.items():
             p, ty = self.partials[name]
-            if ty.size < 4:
-                raise Unsupported(f"Reduction variable `{name}` of type {ty.name} is not supported")
             vty = self.ex.locals.get(name, ty)
             total = self._team_total(op, ty, p)
             self.w(f"{cname(name)} = {cast(_OPS[op] + '::f<' + ty.c + '>(' + cast(cname(name), vty, ty) + ', ' + total + ')', ty, vty)};")
@@ -1415,13 +1447,11 @@ class KernelBuilder:
             ty = self.ex.locals.get(name)
             if ty is None:
                 raise NameError(f"reduction variable `{name}` has no value before the loop")
-            pty = T.F32 if (ty.is_float and ty.size < 4) else ty
-            if pty.size < 4:
-                raise Unsupported(f"Reduction variable `{name}` of type {ty.name} is not supported")
+            pty = _partial_type(ty)
             p = self.fresh(f"part_{name}_")
             typed[name] = (p, pty)
             self.partials[name] = (p, pty)
-            self.w(f"{pty.c} {p} = {T.identity_literal(op, pty)};")
+            self.w(f"{pty.c} {p} = {_partial_identity(op, ty, pty)};")
         saved_mode, self.mode = self.mode, "lane"
         saved_depth, self.seq_depth = self.seq_depth, 0
         saved_stream = set(self.ex.stream_arrays)
@@ -1554,10 +1584,9 @@ class KernelBuilder:
             if ty is None:
                 raise NameError(f"reduction variable `{name}` has no value before the loop")
             p = self.fresh(f"part_{name}_")
-            if ty.is_float and ty.size < 4:
-                ty = T.F32      # lanes accumulate 16-bit floats in float32; rounded once when the team combines
-            self.partials[name] = (p, ty)
-            self.w(f"{ty.c} {p} = {T.identity_literal(op, ty)};")
+            pty = _partial_type(ty)
+            self.partials[name] = (p, pty)
+            self.w(f"{pty.c} {p} = {_partial_identity(op, ty, pty)};")
         jt = self.fresh("jt")
         self.w(f"for (appy::i64 {jt} = {lo_v}; {jt} < {hi_v}; {jt} += {TILE}) {{")
         self.ind += 1
@@ -1621,8 +1650,6 @@ class KernelBuilder:
         self.w("}")
         for name, op in reds.items():
             p, ty = self.partials[name]
-            if ty.size < 4:
-                raise Unsupported(f"Reduction variable `{name}` of type {ty.name} is not supported")
             vty = self.ex.locals.get(name, ty)
             total = self._team_total(op, ty, p)
             self.w(f"{cname(name)} = {cast(_OPS[op] + '::f<' + ty.c + '>(' + cast(cname(name), vty, ty) + ', ' + total + ')', ty, vty)};")
@@ -1633,13 +1660,26 @@ class KernelBuilder:
     def _epilogue(self):
         B = self.spec.block
         for r in self.a.outer_reductions:
-            ident = T.identity_literal(r.op, r.ty)
+            ident = self._outer_identity(r)
+            elem_c = self.a.arrays[r.array].elem_c
+            total = "__tot" if r.elem_ty == r.ty else (
+                "(unsigned char)(__tot != 0)" if r.elem_ty.is_bool else cast("__tot", r.ty, r.elem_ty))
             self.w("{")
             self.ind += 1
             self.w(f"const {r.ty.c} __tot = appy::block_reduce<{_OPS[r.op]}, {B}, {r.ty.c}>({r.acc}, {ident});")
-            self.w(f"if (threadIdx.x == 0) appy::atomic_combine<{_OPS[r.op]}, {r.ty.c}>::run(&{cname(r.array)}[{r.index}], __tot);")
+            self.w(f"if (threadIdx.x == 0) appy::atomic_combine<{_OPS[r.op]}, {elem_c}>::run(&{cname(r.array)}[{r.index}], {total});")
             self.ind -= 1
             self.w("}")
+
+    @staticmethod
+    def _outer_identity(r: OuterReduction) -> str:
+        """Neutral element of the element type, written in the accumulator type (the
+        smallest int8 for a maximum over int8 values held in 32-bit registers)."""
+        if r.elem_ty == r.ty:
+            return T.identity_literal(r.op, r.ty)
+        if r.elem_ty.is_bool:
+            return "0" if r.op == "max" else "1"
+        return f"(({r.ty.c}){T.identity_literal(r.op, r.elem_ty)})"
 
     # ---- parameters -----------------------------------------------------------------
     def _params(self):
@@ -1680,7 +1720,7 @@ class KernelBuilder:
         self.partials = {}
         self.lds_plan = None
         for r in self.a.outer_reductions:
-            self.w(f"{r.ty.c} {r.acc} = {T.identity_literal(r.op, r.ty)};")
+            self.w(f"{r.ty.c} {r.acc} = {self._outer_identity(r)};")
         if self.spec.kind == "flat":
             self._body_flat()
         elif self.spec.kind == "strip":

@@ -270,12 +270,58 @@ __device__ __forceinline__ void atomic_cas_combine(T* p, T v) {
     }
 }
 
+// 8- and 16-bit elements: compare-and-swap on the aligned 32-bit word that holds the element
+// (device allocations are whole multiples of four bytes, so the word is inside the allocation).
+template <int N>
+struct small_uint_of;
+template <>
+struct small_uint_of<1> {
+    typedef unsigned char type;
+};
+template <>
+struct small_uint_of<2> {
+    typedef unsigned short type;
+};
+
 template <typename Op, typename T>
+__device__ __forceinline__ void atomic_subword_combine(T* p, T v) {
+    typedef typename small_uint_of<sizeof(T)>::type U;
+    const unsigned long long addr = reinterpret_cast<unsigned long long>(p);
+    unsigned int* word = reinterpret_cast<unsigned int*>(addr & ~3ull);
+    const unsigned int shift = static_cast<unsigned int>(addr & 3ull) * 8u;
+    const unsigned int mask = (sizeof(T) == 1 ? 0xFFu : 0xFFFFu) << shift;
+    unsigned int seen = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    for (;;) {
+        const T cur = __builtin_bit_cast(T, static_cast<U>((seen & mask) >> shift));
+        const T next = Op::f(cur, v);
+        const unsigned int want = (seen & ~mask) | (static_cast<unsigned int>(__builtin_bit_cast(U, next)) << shift);
+        if (want == seen) return;
+        if (__hip_atomic_compare_exchange_strong(word, &seen, want, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                                 __HIP_MEMORY_SCOPE_AGENT))
+            return;
+    }
+}
+
+template <typename Op, typename T, int N = sizeof(T)>
 struct atomic_combine {
     __device__ static __forceinline__ void run(T* p, T v) { atomic_cas_combine<Op, T>(p, v); }
 };
+template <typename Op, typename T>
+struct atomic_combine<Op, T, 1> {
+    __device__ static __forceinline__ void run(T* p, T v) { atomic_subword_combine<Op, T>(p, v); }
+};
+template <typename Op, typename T>
+struct atomic_combine<Op, T, 2> {
+    __device__ static __forceinline__ void run(T* p, T v) { atomic_subword_combine<Op, T>(p, v); }
+};
 template <typename T>
-struct atomic_combine<OpAdd, T> {  // hardware add for 32/64-bit integers, float and double
+struct atomic_combine<OpAdd, T, 4> {  // hardware add for 32/64-bit integers, float and double
+    __device__ static __forceinline__ void run(T* p, T v) {
+        __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+};
+template <typename T>
+struct atomic_combine<OpAdd, T, 8> {
     __device__ static __forceinline__ void run(T* p, T v) {
         __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }

@@ -60,6 +60,20 @@ class _Normalise(ast.NodeTransformer):
                 more = self.visit_Assign(ast.copy_location(ast.Assign(targets=[t], value=copy.deepcopy(src_)), node))
                 out.extend(more if isinstance(more, list) else [more])
             return out
+        if (isinstance(node.value, ast.BoolOp) and len(node.value.values) == 2
+                and isinstance(node.targets[0], (ast.Name, ast.Subscript))):
+            # `found = found or e` / `ok = ok and e`: a flag folded over the iterations is the
+            # maximum / minimum of truth values
+            key = ast.unparse(node.targets[0])
+            a, b = node.value.values
+            if (ast.unparse(a) == key) != (ast.unparse(b) == key):
+                mine, other = (a, b) if ast.unparse(a) == key else (b, a)
+                fn = "max" if isinstance(node.value.op, ast.Or) else "min"
+                node.value = ast.Call(
+                    func=ast.Name(id=fn, ctx=ast.Load()),
+                    args=[mine, ast.Call(func=ast.Name(id="bool", ctx=ast.Load()), args=[other], keywords=[])],
+                    keywords=[])
+                return node
         if isinstance(node.value, ast.Tuple):
             tgt = node.targets[0]
             assert isinstance(tgt, ast.Tuple) and len(tgt.elts) == len(node.value.elts), (

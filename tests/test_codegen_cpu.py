@@ -442,8 +442,11 @@ def test_updates_of_elements_shared_between_iterations_are_atomic():
     g, src = compiled("#pragma parallel for\nfor i in range(n):\n    #pragma simd\n    for j in range(m):\n        col[j] -= A[i, j]\n",
                       col=np.zeros(32), A=np.zeros((8, 32)), n=8, m=32)
     assert "appy::atomic_combine<appy::OpAdd, double>::run(&col[" in body_of(src) and "(-" in body_of(src)
-    with pytest.raises(NotImplementedError, match="atomic updates of int16"):
-        compiled("#pragma parallel for simd\nfor i in range(n):\n    hist[b[i]] += 1\n", hist=np.zeros(16, np.int16), b=b, n=64)
+    # 8- and 16-bit elements: compare-and-swap on the 32-bit word that holds the element
+    h16, src = compiled("#pragma parallel for simd\nfor i in range(n):\n    hist[b[i]] += 1\n    seen[b[i]] = seen[b[i]] or True\n",
+                        hist=np.zeros(16, np.int16), seen=np.zeros(16, bool), b=b, n=64)
+    assert "appy::atomic_combine<appy::OpAdd, short>::run(&hist[" in body_of(src)
+    assert "appy::atomic_combine<appy::OpMax, unsigned char>::run(&seen[" in body_of(src)
 
 
 def test_in_place_slice_update_from_a_shifted_slice_of_the_same_row_is_refused():
