@@ -131,6 +131,17 @@ def jit(fn=None, **options):
     return jit_with_args
 
 
+def shader(fn=None, **options):
+    """Shader-style kernels (one function body per work-item) are an experiment of the
+    reference's Metal and Numba back ends (reference: appy/__init__.py:84-92); the HIP
+    execution path runs annotated loops only."""
+    raise NotImplementedError("shader functions are not part of the HIP execution path; annotate a loop with "
+                              "`#pragma parallel for` instead")
+
+
+cpu_shader = shader
+
+
 # ---- names usable inside annotated functions -------------------------------
 def vidx(start, stepsize, bound=None):
     """Slice of at most ``stepsize`` indices from ``start``, clipped at
