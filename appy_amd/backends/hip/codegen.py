@@ -159,7 +159,7 @@ def compile_source(text: str, name: str) -> bytes:
     if d:
         h = hashlib.sha256()
         h.update(text.encode())
-        h.update(repr(rt.BASE_COMPILE_OPTIONS).encode())
+        h.update(repr(rt.BASE_COMPILE_OPTIONS + rt.extra_compile_options()).encode())
         h.update(ARCH.encode())
         h.update(str(rt.rtc_version()).encode())
         path = os.path.join(d, h.hexdigest() + ".co")

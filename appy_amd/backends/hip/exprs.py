@@ -290,8 +290,9 @@ class ExprEmitter:
                 t = T.WEAK_INT if t.weak else T.from_dtype(np.int8)
             a, b = cast(lc, lt, t), cast(rc, rt, t)
             if t.is_float:
-                fl = "floorf" if t.name == "float32" else "floor"
-                return f"{fl}({a} / {b})", t
+                if t.size == 2:     # 16-bit floats: computed in float32, rounded once
+                    return cast(f"appy::floordiv_float({cast(lc, lt, T.F32)}, {cast(rc, rt, T.F32)})", T.F32, t), t
+                return f"appy::floordiv_float({a}, {b})", t
             if t.kind == "u":
                 return f"({a} / {b})", t
             return f"appy::floordiv_int<{t.c}>({a}, {b})", t
@@ -301,8 +302,8 @@ class ExprEmitter:
                 t = T.WEAK_INT if t.weak else T.from_dtype(np.int8)
             a, b = cast(lc, lt, t), cast(rc, rt, t)
             if t.is_float:
-                if t.size == 2:
-                    raise NotImplementedError(f"{t.name} modulo")
+                if t.size == 2:     # 16-bit floats: computed in float32, rounded once
+                    return cast(f"appy::mod_float({cast(lc, lt, T.F32)}, {cast(rc, rt, T.F32)})", T.F32, t), t
                 return f"appy::mod_float({a}, {b})", t
             if t.kind == "u":
                 return f"({a} % {b})", t

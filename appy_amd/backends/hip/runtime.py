@@ -173,12 +173,23 @@ BASE_COMPILE_OPTIONS = (
     "-ffp-contract=off",
     "-munsafe-fp-atomics",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # no 8-bit dot-product instructions: the compiler's fold of byte multiply-add chains into
+    # v_dot4_u32_u8 rewrote `u * u + max(u, u * u)` (uint8) as `dot4((u, u, 0, 0), (u, u, 0, 0)) + u`,
+    # a different value, and crashed in instruction selection on the 16-byte form of the same loop
+    "-Xclang", "-target-feature", "-Xclang", "-dot7-insts",
+    "-Xclang", "-target-feature", "-Xclang", "-dot1-insts",
 )
+
+
+def extra_compile_options() -> tuple:
+    """Options appended to every hiprtc compilation: ``APPY_HIP_EXTRA_COMPILE_OPTIONS``
+    (space separated)."""
+    return tuple(os.environ.get("APPY_HIP_EXTRA_COMPILE_OPTIONS", "").split())
 
 
 def compile_to_code_object(source: str, name: str, arch: str = "gfx950", extra_opts=()) -> bytes:
     """HIP C++ text -> code object bytes (works without a GPU)."""
-    opts = [o.encode() for o in (*BASE_COMPILE_OPTIONS, *extra_opts)]
+    opts = [o.encode() for o in (*BASE_COMPILE_OPTIONS, *extra_opts, *extra_compile_options())]
     arr = (C.c_char_p * len(opts))(*opts)
     code = _vp()
     size = C.c_size_t(0)

@@ -101,14 +101,41 @@ __device__ __forceinline__ T mod_int(T a, T b) {
     return ((r != 0) && ((r < 0) != (b < 0))) ? r + b : r;
 }
 
+// Floating-point `%` and `//` follow NumPy's (and CPython's) divmod: the remainder comes from
+// fmod, which is exact, and the quotient is derived from it, so that a / b rounding up to
+// a whole number does not push the floor one too high.
 __device__ __forceinline__ float mod_float(float a, float b) {
     float r = fmodf(a, b);
-    return ((r != 0.0f) && ((r < 0.0f) != (b < 0.0f))) ? r + b : r;
+    if (r != 0.0f) return ((r < 0.0f) != (b < 0.0f)) ? r + b : r;
+    return (b == 0.0f) ? r : copysignf(0.0f, b);
 }
 
 __device__ __forceinline__ double mod_float(double a, double b) {
     double r = fmod(a, b);
-    return ((r != 0.0) && ((r < 0.0) != (b < 0.0))) ? r + b : r;
+    if (r != 0.0) return ((r < 0.0) != (b < 0.0)) ? r + b : r;
+    return (b == 0.0) ? r : copysign(0.0, b);
+}
+
+__device__ __forceinline__ float floordiv_float(float a, float b) {
+    if (b == 0.0f) return a / b;
+    const float r = fmodf(a, b);
+    float div = (a - r) / b;
+    if (r != 0.0f && ((b < 0.0f) != (r < 0.0f))) div -= 1.0f;
+    if (div == 0.0f) return copysignf(0.0f, a / b);
+    float q = floorf(div);
+    if (div - q > 0.5f) q += 1.0f;
+    return q;
+}
+
+__device__ __forceinline__ double floordiv_float(double a, double b) {
+    if (b == 0.0) return a / b;
+    const double r = fmod(a, b);
+    double div = (a - r) / b;
+    if (r != 0.0 && ((b < 0.0) != (r < 0.0))) div -= 1.0;
+    if (div == 0.0) return copysign(0.0, a / b);
+    double q = floor(div);
+    if (div - q > 0.5) q += 1.0;
+    return q;
 }
 
 template <typename T>

@@ -489,3 +489,26 @@ def test_generated_code_objects_hold_no_packed_fp32_instructions():
     assert "v_mul_f32" in isa or "v_fma" in isa or "v_add_f32" in isa
     assert not re.search(r"v_pk_(add|mul|fma)_f32", isa)
     assert "global_load_dwordx4" in isa and "global_store_dwordx4" in isa
+
+
+def test_byte_multiply_add_chains_are_not_folded_into_dot_products():
+    """Kernels are compiled without the 8-bit dot-product instructions: the compiler's fold of
+    `u * u + max(u, u * u)` over uint8 into v_dot4_u32_u8 computed another value (and the
+    16-byte form of the loop crashed instruction selection).  The loop must compile and its ISA
+    must keep the maximum."""
+    import os
+    import subprocess
+    import tempfile
+
+    objdump = "/opt/rocm/llvm/bin/llvm-objdump"
+    if not os.path.exists(objdump):
+        pytest.skip("llvm-objdump not found")
+    u = np.zeros(64, np.uint8)
+    src = "#pragma parallel for simd\nfor i in range(n):\n    out[i] = (-(u[i] * u[i])) - max((u[i] * u[i]), u[i])\n"
+    for dt in (np.uint8, np.float64):
+        f, _ = compiled(src, u=u, out=np.zeros(64, dt), n=64)
+        with tempfile.NamedTemporaryFile(suffix=".co") as fh:
+            fh.write(f.kernels[f.default_spec].code)
+            fh.flush()
+            isa = subprocess.run([objdump, "-d", fh.name], capture_output=True, text=True, check=True).stdout
+        assert "v_dot4" not in isa and "v_max_u" in isa

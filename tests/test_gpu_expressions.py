@@ -654,3 +654,22 @@ def test_statement_forms_of_ordinary_python(gpu):
     i = np.arange(n)
     assert np.allclose(out, 2 * d * 100.0 + a * 10.0 + 4 * d + A[i % 4, i % 5], rtol=1e-13, atol=1e-12)
     assert np.array_equal(cls, np.where(d > 1.0, 2, np.where(d > 0.0, 1, 0)))
+
+
+def test_uint8_square_plus_maximum_regression(gpu):
+    """`-(u * u) - max(u * u, u)` over uint8: the compiler once folded the byte multiply-add
+    chain into a dot-product instruction that computed `-(2 u*u + u)`."""
+    import appy_amd as appy
+
+    @appy.jit
+    def kernel(u, out):
+        #pragma parallel for simd
+        for i in range(out.shape[0]):
+            out[i] = (-(u[i] * u[i])) - max((u[i] * u[i]), u[i])
+
+    u = np.random.default_rng(7).integers(0, 256, 100_003).astype(np.uint8)
+    want = (-(u * u)) - np.maximum(u * u, u)
+    for dt in (np.uint8, np.int32, np.float64):
+        out = np.zeros(u.size, dt)
+        kernel(u, out)
+        assert np.array_equal(out, want.astype(dt))
