@@ -639,3 +639,156 @@ def test_trmm_in_place_updates(gpu):
     assert np.allclose(got, want, atol=1e-6)
     loop = next(v[0] for k, v in cg.code_cache.items() if k[-1] == "trmm_column_by_column")
     assert not loop.analysis.multi_wave_ok
+
+
+# ---- further NPBench kernels in the reference's loop style (polybench covariance / correlation /
+# heat-3d / doitgen, deep-learning softmax): column walks under triangular loops, 3-D stencils,
+# 4-D arrays addressed through a flattened parallel index, slices of 3-D arrays -------------------
+@appy.jit
+def covariance(data, cov, mean):
+    #pragma parallel for
+    for j in range(data.shape[1]):
+        s = 0.0
+        for k in range(data.shape[0]):
+            s += data[k, j]
+        mean[j] = s / data.shape[0]
+    #pragma parallel for
+    for k in range(data.shape[0]):
+        data[k, :] -= mean[:]
+    #pragma parallel for
+    for i in range(data.shape[1]):
+        for j in range(i, data.shape[1]):
+            s = 0.0
+            #pragma simd
+            for k in range(data.shape[0]):
+                s += data[k, i] * data[k, j]
+            cov[i, j] = cov[j, i] = s / (data.shape[0] - 1.0)
+def covariance_ref(data, cov, mean):
+    mean[:] = data.mean(axis=0); data -= mean
+    cov[:] = data.T @ data / (data.shape[0] - 1.0)
+
+@appy.jit
+def heat_3d(T, A, B):
+    for t in range(1, T):
+        #pragma parallel for
+        for i in range(1, A.shape[0] - 1):
+            for j in range(1, A.shape[1] - 1):
+                #pragma simd
+                for k in range(1, A.shape[2] - 1):
+                    B[i, j, k] = (0.125 * (A[i + 1, j, k] - 2.0 * A[i, j, k] + A[i - 1, j, k]) + 0.125 * (A[i, j + 1, k] - 2.0 * A[i, j, k] + A[i, j - 1, k])
+                                  + 0.125 * (A[i, j, k + 1] - 2.0 * A[i, j, k] + A[i, j, k - 1]) + A[i, j, k])
+        #pragma parallel for
+        for i in range(1, A.shape[0] - 1):
+            for j in range(1, A.shape[1] - 1):
+                #pragma simd
+                for k in range(1, A.shape[2] - 1):
+                    A[i, j, k] = (0.125 * (B[i + 1, j, k] - 2.0 * B[i, j, k] + B[i - 1, j, k]) + 0.125 * (B[i, j + 1, k] - 2.0 * B[i, j, k] + B[i, j - 1, k])
+                                  + 0.125 * (B[i, j, k + 1] - 2.0 * B[i, j, k] + B[i, j, k - 1]) + B[i, j, k])
+def heat_3d_ref(T, A, B):
+    for t in range(1, T):
+        B[1:-1, 1:-1, 1:-1] = (0.125 * (A[2:, 1:-1, 1:-1] - 2.0 * A[1:-1, 1:-1, 1:-1] + A[:-2, 1:-1, 1:-1]) + 0.125 * (A[1:-1, 2:, 1:-1] - 2.0 * A[1:-1, 1:-1, 1:-1] + A[1:-1, :-2, 1:-1]) + 0.125 * (A[1:-1, 1:-1, 2:] - 2.0 * A[1:-1, 1:-1, 1:-1] + A[1:-1, 1:-1, 0:-2]) + A[1:-1, 1:-1, 1:-1])
+        A[1:-1, 1:-1, 1:-1] = (0.125 * (B[2:, 1:-1, 1:-1] - 2.0 * B[1:-1, 1:-1, 1:-1] + B[:-2, 1:-1, 1:-1]) + 0.125 * (B[1:-1, 2:, 1:-1] - 2.0 * B[1:-1, 1:-1, 1:-1] + B[1:-1, :-2, 1:-1]) + 0.125 * (B[1:-1, 1:-1, 2:] - 2.0 * B[1:-1, 1:-1, 1:-1] + B[1:-1, 1:-1, 0:-2]) + B[1:-1, 1:-1, 1:-1])
+
+@appy.jit
+def softmax4(x, out):
+    #pragma parallel for
+    for n in range(x.shape[0] * x.shape[1] * x.shape[2]):
+        a = n // (x.shape[1] * x.shape[2])
+        b = (n // x.shape[2]) % x.shape[1]
+        c = n % x.shape[2]
+        m = -1e30
+        #pragma simd
+        for k in range(x.shape[3]):
+            m = max(m, x[a, b, c, k])
+        s = 0.0
+        #pragma simd
+        for k in range(x.shape[3]):
+            s += np.exp(x[a, b, c, k] - m)
+        #pragma simd
+        for k in range(x.shape[3]):
+            out[a, b, c, k] = np.exp(x[a, b, c, k] - m) / s
+def softmax4_ref(x, out):
+    e = np.exp(x - x.max(axis=-1, keepdims=True)); out[:] = e / e.sum(axis=-1, keepdims=True)
+
+@appy.jit
+def softmax_slices(x, out):
+    #pragma parallel for
+    for i in range(x.shape[0]):
+        for j in range(x.shape[1]):
+            m = np.max(x[i, j, :])
+            s = np.sum(np.exp(x[i, j, :] - m))
+            out[i, j, :] = np.exp(x[i, j, :] - m) / s
+def softmax_slices_ref(x, out):
+    e = np.exp(x - x.max(axis=-1, keepdims=True)); out[:] = e / e.sum(axis=-1, keepdims=True)
+
+@appy.jit
+def correlation(data, corr, mean, std):
+    #pragma parallel for
+    for j in range(data.shape[1]):
+        s = 0.0
+        q = 0.0
+        for k in range(data.shape[0]):
+            s += data[k, j]
+        mu = s / data.shape[0]
+        for k in range(data.shape[0]):
+            q += (data[k, j] - mu) ** 2
+        sd = math.sqrt(q / data.shape[0])
+        mean[j] = mu
+        std[j] = 1.0 if sd <= 0.1 else sd
+    #pragma parallel for
+    for k in range(data.shape[0]):
+        data[k, :] = (data[k, :] - mean[:]) / (math.sqrt(data.shape[0]) * std[:])
+    #pragma parallel for
+    for i in range(data.shape[1]):
+        corr[i, i] = 1.0
+        for j in range(i + 1, data.shape[1]):
+            s = 0.0
+            #pragma simd
+            for k in range(data.shape[0]):
+                s += data[k, i] * data[k, j]
+            corr[i, j] = s
+            corr[j, i] = s
+def correlation_ref(data, corr, mean, std):
+    mean[:] = data.mean(axis=0); sd = data.std(axis=0); sd[sd <= 0.1] = 1.0; std[:] = sd
+    data -= mean; data /= math.sqrt(data.shape[0]) * std
+    corr[:] = data.T @ data; np.fill_diagonal(corr, 1.0)
+
+@appy.jit
+def doitgen(A, C4, tmp):
+    #pragma parallel for
+    for n in range(A.shape[0] * A.shape[1]):
+        r = n // A.shape[1]
+        q = n % A.shape[1]
+        for p in range(A.shape[2]):
+            s = 0.0
+            #pragma simd
+            for k in range(A.shape[2]):
+                s += A[r, q, k] * C4[k, p]
+            tmp[r, q, p] = s
+        #pragma simd
+        for p in range(A.shape[2]):
+            A[r, q, p] = tmp[r, q, p]
+def doitgen_ref(A, C4, tmp):
+    tmp[:] = A @ C4; A[:] = tmp
+
+
+def test_more_npbench_kernels(gpu):
+    rng = np.random.default_rng(0)
+
+    def check(fn, ref, *args, tol=1e-9):
+        mine = [a.copy() if hasattr(a, "copy") else a for a in args]
+        ref(*args)
+        fn(*mine)
+        for got, want in zip(mine, args):
+            if hasattr(got, "shape"):
+                assert np.allclose(got, want, rtol=tol, atol=tol), fn.__name__
+
+    N, M = 130, 90
+    check(covariance, covariance_ref, rng.random((N, M)), np.zeros((M, M)), np.zeros(M))
+    check(correlation, correlation_ref, rng.random((N, M)), np.zeros((M, M)), np.zeros(M), np.zeros(M))
+    check(heat_3d, heat_3d_ref, 5, rng.random((20, 22, 70)), rng.random((20, 22, 70)))
+    x = rng.standard_normal((3, 4, 17, 65))
+    check(softmax4, softmax4_ref, x, np.zeros_like(x))
+    x3 = rng.standard_normal((7, 17, 65))
+    check(softmax_slices, softmax_slices_ref, x3, np.zeros_like(x3))
+    check(doitgen, doitgen_ref, rng.random((6, 5, 40)), rng.random((40, 40)), np.zeros((6, 5, 40)))
