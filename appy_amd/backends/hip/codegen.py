@@ -75,6 +75,9 @@ TEAM_BYTES_IN_FLIGHT = 8.0e6
 # per row or per time step (`for i in range(n): <kernel using i in a bound>`) cycles through
 # n of them
 REPLAY_CACHE_ENTRIES = 2048
+# a parallel loop with fewer iterations than this, whose body is one independent sequential loop,
+# runs the two loops as one iteration space (one wavefront per iteration would not fill 256 CUs)
+COLLAPSE_BELOW_ROWS = 8192
 
 
 def device_header() -> str:
@@ -271,6 +274,11 @@ class CompiledLoop:
         a = self.analysis
         self._lo_code = compile(ast.Expression(body=ast.fix_missing_locations(_copy(a.lo_node))), "<lo>", "eval")
         self._hi_code = compile(ast.Expression(body=ast.fix_missing_locations(_copy(a.hi_node))), "<hi>", "eval")
+        self._collapse_codes = None
+        if a.collapse is not None:
+            self._collapse_codes = tuple(
+                compile(ast.Expression(body=ast.fix_missing_locations(_copy(x))), "<inner bound>", "eval")
+                for x in a.collapse.iter.args[:2])
         self._simd_loops = self._collect_simd_loops()
         self._row_extent_code = self._find_row_extent()
         self._strip_trip_code = None
@@ -508,6 +516,9 @@ class CompiledLoop:
                 if -(-ext // (w * ve)) <= 8:
                     return Spec("team", block=d.block, vec=ve, width=w, restrict=restrict,
                                 stream_loads=False, extent=ext)
+        nj = self.collapse_count(n_outer, env)
+        if nj:
+            n_outer *= nj       # the pairs (i, j) are the rows from here on
         trip, uniform = self._estimate_trip(env, arrays, n_outer)
         if trip < 2 * v:
             v = 1
@@ -528,7 +539,19 @@ class CompiledLoop:
             # so a whole workgroup takes each row (the more lanes the fewer rows there are)
             block = 1024 if n_outer <= DEFAULT_CUS else 256
             w = block
-        return Spec("team", block=block, vec=v, width=w, restrict=restrict, stream_loads=stream)
+        return Spec("team", block=block, vec=v, width=w, restrict=restrict, stream_loads=stream, collapse=bool(nj))
+
+    def collapse_count(self, n_outer, env) -> int:
+        """Trip count of the sequential loop that may be collapsed into the parallel loop,
+        when that is possible and worth it for ``n_outer`` parallel iterations; else 0."""
+        if self._collapse_codes is None or n_outer >= COLLAPSE_BELOW_ROWS or self.options.get("check_bounds"):
+            return 0
+        try:
+            lo = int(eval(self._collapse_codes[0], _HOST_EVAL_GLOBALS, env))
+            hi = int(eval(self._collapse_codes[1], _HOST_EVAL_GLOBALS, env))
+        except Exception:
+            return 0
+        return hi - lo if hi - lo >= 2 else 0
 
     def row_hint(self, n_outer, env, arrays):
         """(expected inner trip count, same for every row?) for grid sizing."""
@@ -804,6 +827,8 @@ class Launch:
                 val = hi
             setattr(st, fname, val)
         self.args = st
+        if spec.collapse:
+            n_outer *= max(1, loop.collapse_count(n_outer, env))
         self.grid = (loop.grid_for(spec, n_outer, kernel=self.kernel,
                                    row_hint=loop.row_hint(n_outer, env, arrays)), 1, 1)
         self.block = (spec.block, 1, 1)

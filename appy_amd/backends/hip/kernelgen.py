@@ -68,6 +68,8 @@ class Spec:
     checked: bool = False        # every subscript is compared with the extents; violations are reported
     hoist_guarded: bool = True   # flat only: loads the source guards with a condition may be issued
                                  # unconditionally (the host has checked that they stay inside their arrays)
+    collapse: bool = False       # team only: the parallel loop and the sequential loop that is its whole body
+                                 # run as one iteration space (the analysis has shown the inner iterations independent)
 
     def __post_init__(self):
         def pow2(n):
@@ -85,6 +87,8 @@ class Spec:
             raise ValueError(f"team width must be a power of two up to 64, or the whole workgroup, got {self.width}")
         if self.checked and (self.vec != 1 or self.unroll != 1 or self.extent or self.lds_tile):
             raise ValueError("a bounds-checked kernel takes one element per access (vec = unroll = 1, no row extent, no LDS tile)")
+        if self.collapse and (self.kind != "team" or self.lds_tile):
+            raise ValueError("only team kernels without an LDS tile collapse their two outer loops")
         if self.extent < 0 or self.lds_tile < 0 or self.lds_tile % 4 or self.lds_tile > 16384:
             raise ValueError("row extent / LDS tile out of range (tile: multiple of 4, at most 16384 elements)")
 
@@ -92,7 +96,7 @@ class Spec:
         return (f"{self.kind}_b{self.block}_v{self.vec}_u{self.unroll}_w{self.width}"
                 f"{'_r' if self.restrict else ''}{'_nt' if self.stream_loads else ''}"
                 f"{'_e' + str(self.extent) if self.extent else ''}{'_nts' if self.stream_stores else ''}"
-                f"{'_lds' + str(self.lds_tile) if self.lds_tile else ''}{'' if self.hoist_guarded else '_g'}{'_chk' if self.checked else ''}")
+                f"{'_lds' + str(self.lds_tile) if self.lds_tile else ''}{'' if self.hoist_guarded else '_g'}{'_chk' if self.checked else ''}{'_c2' if self.collapse else ''}")
 
 
 @dataclass
@@ -338,6 +342,86 @@ class LoopAnalysis:
                         return True
         return False
 
+    def _find_collapse(self):
+        """The sequential loop ``for j in range(lo, hi)`` that is the whole body of the
+        parallel loop, if its iterations are provably independent - then the pairs (i, j)
+        may run as one parallel iteration space (3-D stencils written as `parallel i / for j
+        / simd k`, row operations on 3-D arrays): with few `i` the chip would otherwise hold
+        one team per `i` and nothing else.  None if the nest is not of that form.
+
+        Independence as checked here: the bounds of the loop do not depend on `i` or on
+        anything the nest assigns; every scalar the loop assigns is a temporary of one
+        iteration (assigned before it is read); every array it stores to is indexed by
+        `j + c` in one dimension, the same for all its stores, and loaded - if at all -
+        with `j + c` in that dimension too, so that iteration `j` only ever touches its
+        own slab; nothing leaves the loop early."""
+        body = self.outer.body
+        if len(body) != 1 or not isinstance(body[0], ast.For) or "simd" in self.pragma:
+            return None
+        loop = body[0]
+        if getattr(loop, "pragma", None) or loop.orelse or not isinstance(loop.target, ast.Name):
+            return None
+        it = loop.iter
+        if not (isinstance(it, ast.Call) and isinstance(it.func, ast.Name) and it.func.id == "range" and len(it.args) == 3):
+            return None
+        j = loop.target.id
+        if j == self.var or loop_ir.reductions_of(self.outer):
+            return None
+        assigned = set(self.assigned) | set(self.loop_vars)
+        for a in it.args[:2]:
+            for n in ast.walk(a):
+                if isinstance(n, ast.Name) and (n.id in assigned or n.id in self.arrays):
+                    return None
+                if isinstance(n, (ast.Subscript, ast.Call)):
+                    return None
+        # nothing may leave the loop early or skip the rest of an iteration of it
+        def leaves(stmts):
+            for st in stmts:
+                if isinstance(st, (ast.Break, ast.Continue)):
+                    return True
+                if isinstance(st, ast.If) and (leaves(st.body) or leaves(st.orelse)):
+                    return True
+            return False
+        if leaves(loop.body) or any(isinstance(n, ast.While) for n in ast.walk(loop)):
+            return None
+        # scalars: temporaries of one iteration
+        names = []
+        for n in ast.walk(loop):
+            if isinstance(n, ast.Assign) and isinstance(n.targets[0], ast.Name) and n.targets[0].id not in names:
+                names.append(n.targets[0].id)
+            elif isinstance(n, ast.For) and n is not loop and n.target.id not in names:
+                names.append(n.target.id)
+        if j in names or self.var in names:
+            return None
+        for name in names:
+            first = next((st for st in loop.body if _uses_name(st, name)), None)
+            if isinstance(first, ast.For) and first.target.id == name and not any(_uses_name(a, name) for a in first.iter.args):
+                continue
+            if not (isinstance(first, ast.Assign) and isinstance(first.targets[0], ast.Name)
+                    and first.targets[0].id == name and not _uses_name(first.value, name)):
+                return None
+        # arrays: iteration j stays inside its own slab of everything the loop stores to
+        slab = {}       # array -> (dimension, offset)
+        for n in ast.walk(loop):
+            if isinstance(n, ast.Assign) and isinstance(n.targets[0], ast.Subscript):
+                t = n.targets[0]
+                if not (isinstance(t.value, ast.Name) and t.value.id in self.arrays):
+                    return None
+                where = [(d, _var_offset(e, j)) for d, e in enumerate(_elts(t)) if _var_offset(e, j) is not None]
+                if len(where) != 1 or slab.setdefault(t.value.id, where[0]) != where[0]:
+                    return None
+        if not slab:
+            return None
+        for n in ast.walk(loop):
+            if isinstance(n, ast.Subscript) and isinstance(n.value, ast.Name) and n.value.id in slab:
+                d, off = slab[n.value.id]
+                idx = _elts(n)
+                if d >= len(idx) or _var_offset(idx[d], j) != off:
+                    return None
+                if any(_uses_name(e, j) for k, e in enumerate(idx) if k != d):
+                    return None
+        return loop
+
     def _find_strip(self):
         """``{id(loop): {scalar: op}}`` for the inner loops that a *strip* kernel
         shares out between wavefronts, or None if the loop nest does not suit that
@@ -476,6 +560,7 @@ class LoopAnalysis:
         # keep to teams inside one wavefront, where program order is enough.
         self.multi_wave_ok = not self._leader_store_reloaded()
         self.strip = self._find_strip() if self.multi_wave_ok else None
+        self.collapse = self._find_collapse() if self.kind == "team" else None
 
         # reductions of the parallel loop: constant-subscript elements of arrays
         self.outer_reductions = []
@@ -1313,9 +1398,18 @@ class KernelBuilder:
     def _iteration(self, idx_code: str):
         self.w("{")
         self.ind += 1
-        self.w(f"const appy::i64 {cname(self.a.var)} = {idx_code};")
-        self._declare_locals()
-        self.iteration_body(self.a.outer.body)
+        if self.spec.collapse:
+            # idx_code counts the pairs (i, j) from zero, j fastest
+            inner = self.a.collapse
+            self.w(f"const appy::i64 {cname(self.a.var)} = __lo + ({idx_code}) / __nj;")
+            self.w(f"const appy::i64 {cname(inner.target.id)} = __jlo + ({idx_code}) % __nj;")
+            self.ex.locals[inner.target.id] = T.WEAK_INT
+            self._declare_locals()
+            self.iteration_body(inner.body)
+        else:
+            self.w(f"const appy::i64 {cname(self.a.var)} = {idx_code};")
+            self._declare_locals()
+            self.iteration_body(self.a.outer.body)
         self.ind -= 1
         self.w("}")
 
@@ -1541,6 +1635,20 @@ class KernelBuilder:
         self.lds_plan = self._find_lds_plan()
         self.w(f"const int __lane = threadIdx.x & {W - 1};")
         self.w(f"const appy::i64 __team = threadIdx.x / {W};")
+        if self.spec.collapse:
+            if self.a.collapse is None or self.lds_plan is not None:
+                raise Unsupported("the loop nest does not suit the collapsed shape")
+            jlo, jhi = self._range_args(self.a.collapse)
+            self.w(f"const appy::i64 __jlo = {jlo};")
+            self.w(f"const appy::i64 __nj = ({jhi}) > __jlo ? ({jhi}) - __jlo : 0;")
+            self.w(f"for (appy::i64 __c = blockIdx.x * {tpb}LL + __team; __c < (__hi - __lo) * __nj; __c += gridDim.x * {tpb}LL) {{")
+            self.ind += 1
+            self.mode = "team"
+            self._iteration("__c")
+            self.mode = "lane"
+            self.ind -= 1
+            self.w("}")
+            return
         if self.lds_plan is None:
             self.w(f"for (appy::i64 __i = __lo + blockIdx.x * {tpb}LL + __team; __i < __hi; __i += gridDim.x * {tpb}LL) {{")
             self.ind += 1

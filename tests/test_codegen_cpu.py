@@ -512,3 +512,42 @@ def test_byte_multiply_add_chains_are_not_folded_into_dot_products():
             fh.flush()
             isa = subprocess.run([objdump, "-d", fh.name], capture_output=True, text=True, check=True).stdout
         assert "v_dot4" not in isa and "v_max_u" in isa
+
+
+def test_independent_inner_loops_collapse_into_the_parallel_loop():
+    """`parallel i / for j / simd k` with few `i`: when the `j` iterations are provably
+    independent the pairs (i, j) become the iteration space of the team kernel."""
+    A, B = np.zeros((20, 22, 70)), np.zeros((20, 22, 70))
+    env = dict(A_shape_0=20, A_shape_1=22, A_shape_2=70)
+    stencil = ("#pragma parallel for\nfor i in range(1, A_shape_0 - 1):\n    for j in range(1, A_shape_1 - 1):\n"
+               "        #pragma simd\n        for k in range(1, A_shape_2 - 1):\n"
+               "            B[i, j, k] = A[i, j, k - 1] + A[i, j + 1, k] + A[i - 1, j, k]\n")
+    f, _ = compiled(stencil, A=A, B=B, **env)
+    assert f.analysis.collapse is not None
+    spec = f.choose_spec(18, dict(env), dict(A=A, B=B))
+    assert spec.kind == "team" and spec.collapse
+    k = body_of(f.kernel_for(spec).src.text)
+    assert "__c < (__hi - __lo) * __nj" in k and "const appy::i64 i = __lo + (__c) / __nj;" in k
+    assert "const appy::i64 j = __jlo + (__c) % __nj;" in k and "for (appy::i64 j" not in k
+    # many parallel iterations: nothing to gain
+    assert not f.choose_spec(20000, dict(env, A_shape_0=20002), dict(A=A, B=B)).collapse
+
+    def collapsible(body, **extra):
+        src = "#pragma parallel for\nfor i in range(n):\n    for j in range(m):\n" + body
+        g, _ = compiled(src, A=A, B=B, y=np.zeros((20, 22)), n=20, m=22, p=70, **extra)
+        return g.analysis.collapse is not None
+
+    simd = "        #pragma simd\n        for k in range(p):\n"
+    assert collapsible("        s = 0.0\n" + simd + "            s += A[i, j, k]\n        y[i, j] = s\n")
+    # a value carried from one j to the next
+    assert not collapsible("        s = y[i, 0]\n" + simd + "            s += A[i, j, k]\n        y[i, 0] = s\n")
+    # the loop reads a slab that another j writes
+    assert not collapsible(simd + "            A[i, j, k] = A[i, j - 1, k] + 1.0\n")
+    # a scalar that lives across iterations of j
+    assert not collapsible(simd + "            B[i, j, k] = A[i, j, k] + t\n        t = t + 1.0\n", t=0.5)
+    # leaving the loop early
+    assert not collapsible("        if y[i, j] > 0:\n            break\n" + simd + "            B[i, j, k] = A[i, j, k]\n")
+    # bounds that depend on the parallel variable
+    src = "#pragma parallel for\nfor i in range(n):\n    for j in range(i):\n" + simd + "            B[i, j, k] = A[i, j, k]\n"
+    g, _ = compiled(src, A=A, B=B, n=20, p=70)
+    assert g.analysis.collapse is None
