@@ -302,7 +302,7 @@ class LoopAnalysis:
         if not spread:
             parts = _find_strip_parts(self.outer.body, self.var)
             if parts is not None:
-                spread = [parts[1]]
+                spread = [lp for lp, _ops in parts]
         for lp in spread:
             shared_out.update(id(x) for x in ast.walk(lp))
 
@@ -482,10 +482,10 @@ class LoopAnalysis:
             parts = _find_strip_parts(body, self.var)
             if parts is None:
                 return None
-            _pre, loop, _post, ops = parts
-            for st in loop.body:
-                st.reduce = ops[st.targets[0].id]
-            spread[id(loop)] = ops
+            for loop, ops in parts:
+                for st in loop.body:
+                    st.reduce = ops[st.targets[0].id]
+                spread[id(loop)] = ops
         if not spread:
             return None
         # profitability: down the columns, never along a row of a matrix
@@ -625,46 +625,44 @@ def _partial_identity(op: str, ty: Ty, pty: Ty) -> str:
 
 
 def _find_strip_parts(body, var):
-    """``(pre, loop, post, {scalar: op})`` if the body of a parallel loop is
-    scalar set-up, then ONE sequential loop that only folds values into scalars
-    with a reduction operator (``s += A[j, i] * y[j]``) and never looks at the
-    running value, then anything without loops: a column reduction written
-    without ``simd``.  None otherwise."""
-    loops = [k for k, st in enumerate(body) if isinstance(st, (ast.For, ast.While))]
-    if len(loops) != 1 or not isinstance(body[loops[0]], ast.For):
+    """``[(loop, {scalar: op}), ...]`` if the body of a parallel loop is scalar set-up,
+    then sequential loops that only fold values into scalars with a reduction operator
+    (``s += A[j, i] * y[j]``) and never look at the running value, with nothing but scalar
+    assignments between them (``mu = s / n``), then anything without loops: column
+    reductions written without ``simd``.  None otherwise."""
+    at = [k for k, st in enumerate(body) if isinstance(st, (ast.For, ast.While))]
+    if not at or not all(isinstance(body[k], ast.For) for k in at):
         return None
-    k = loops[0]
-    pre, loop, post = body[:k], body[k], body[k + 1:]
-    if loop.orelse or not isinstance(loop.target, ast.Name):
-        return None
-    pragma = getattr(loop, "pragma", None) or {}
-    if pragma:
-        return None
-    for st in pre + post:
-        if any(isinstance(n, (ast.For, ast.While, ast.Break, ast.Continue)) for n in ast.walk(st)):
+    found = []
+    for k in at:
+        loop = body[k]
+        if loop.orelse or not isinstance(loop.target, ast.Name) or (getattr(loop, "pragma", None) or {}):
             return None
-    for st in loop.body:    # `continue` ends one iteration of the inner loop, wherever that runs
-        if any(isinstance(n, (ast.For, ast.While, ast.Break)) for n in ast.walk(st)):
+        for st in loop.body:    # `continue` ends one iteration of the inner loop, wherever that runs
+            if any(isinstance(n, (ast.For, ast.While, ast.Break)) for n in ast.walk(st)):
+                return None
+        ops = {}
+        for st in loop.body:
+            if not (isinstance(st, ast.Assign) and isinstance(st.targets[0], ast.Name)):
+                return None
+            op = loop_ir.reduction_operator(st)
+            name = st.targets[0].id
+            if op is None or ops.setdefault(name, op) != op:
+                return None
+        for name in ops:    # the running value is not looked at inside the loop
+            if any(_uses_name(loop_ir.reduction_operand(s2), name) for s2 in loop.body):
+                return None
+        if not ops or any(_uses_name(a, n) for a in loop.iter.args for n in ops):
             return None
-    for st in pre:      # run by every wavefront of the strip: values only, no effects
-        if not (isinstance(st, ast.Assign) and isinstance(st.targets[0], ast.Name)):
+        found.append((loop, ops))
+    for k, st in enumerate(body):
+        if k in at:
+            continue
+        if any(isinstance(n, (ast.Break, ast.Continue)) for n in ast.walk(st)):
             return None
-    ops = {}
-    for st in loop.body:
-        if not (isinstance(st, ast.Assign) and isinstance(st.targets[0], ast.Name)):
-            return None
-        op = loop_ir.reduction_operator(st)
-        name = st.targets[0].id
-        if op is None or ops.setdefault(name, op) != op:
-            return None
-    for name in ops:    # the running value is not looked at inside the loop
-        if any(_uses_name(loop_ir.reduction_operand(s2), name) for s2 in loop.body):
-            return None
-    if not ops:
-        return None
-    if any(_uses_name(a, n) for a in loop.iter.args for n in ops):
-        return None
-    return pre, loop, post, ops
+        if k < at[-1] and not (isinstance(st, ast.Assign) and isinstance(st.targets[0], ast.Name)):
+            return None     # run by every wavefront of the strip: values only, no effects
+    return found
 
 
 class KernelBuilder:
