@@ -503,7 +503,10 @@ class CompiledLoop:
             return Spec("flat", block=d.block, vec=d.vec, unroll=d.unroll, restrict=restrict, stream_loads=stream)
         stream = self._bytes_touched(arrays) > MALL_BYTES
         v = d.vec
-        if self._row_extent_code is not None:
+        # (arguments that share memory could carry a dependence from one j to the next that the
+        #  analysis, which reasons by array name, cannot see)
+        nj = self.collapse_count(n_outer, env) if restrict else 0
+        if self._row_extent_code is not None and not nj:
             try:
                 ext = int(eval(self._row_extent_code, _HOST_EVAL_GLOBALS, env))
             except Exception:
@@ -516,7 +519,6 @@ class CompiledLoop:
                 if -(-ext // (w * ve)) <= 8:
                     return Spec("team", block=d.block, vec=ve, width=w, restrict=restrict,
                                 stream_loads=False, extent=ext)
-        nj = self.collapse_count(n_outer, env)
         if nj:
             n_outer *= nj       # the pairs (i, j) are the rows from here on
         trip, uniform = self._estimate_trip(env, arrays, n_outer)
@@ -718,6 +720,8 @@ class Launch:
         self.mirrored = []       # (mirror, dptr, host ndarray, stored): arguments with a standing HBM mirror
         self.oob = 0             # checked kernels: device word that receives the report
         self.keepalive_copies = False   # a non-contiguous tensor was repacked for this launch
+        self.staged_twice = {}   # (address, bytes, strides, dtype) of a staged host array -> (index in temps, uploaded?)
+        self.aliases = []        # (name, dptr, bytes, stored) of host arrays that share the copy of another name
         self.keepalive = []
         # -- bounds of accesses indexed by the parallel loop variable (host check, before any device work)
         for name, dim, off in a.bound_checks:
@@ -782,6 +786,7 @@ class Launch:
                 self._stage_host(name, host, v if tc is v else ("tensor", v, tc), arr.stored)
         for dptr, host, _orig, stored, name in self.temps:
             extents.append((name, dptr, host.nbytes, stored))
+        extents.extend(self.aliases)
         for _m, dptr, host, stored, name in self.mirrored:
             extents.append((name, dptr, host.nbytes, stored))
         restrict = not _overlaps(extents)
@@ -856,10 +861,25 @@ class Launch:
             return
         self._no_capture(name, "it is a host array that would be copied per launch (use GPU tensors, or NumPy "
                                "arrays inside `with appy.resident(...)`; `shared()` scalars cannot be captured)")
-        dptr = rt.malloc(max(nbytes, 1))
-        if nbytes and not (stored and self.loop.overwrites(name, self.lo, self.hi, self.env, host.shape)):
-            rt.memcpy_h2d(dptr, host.ctypes.data, nbytes, self.stream)
-        self.temps.append((dptr, host, original, stored, name))
+        skip_upload = bool(stored and self.loop.overwrites(name, self.lo, self.hi, self.env, host.shape))
+        key = (host.ctypes.data, nbytes, host.strides, host.dtype.str)
+        twin = self.staged_twice.get(key) if nbytes else None
+        if twin is not None:
+            # the same host array under a second name: one device copy serves both, so that what
+            # the kernel stores through one name is what it loads through the other
+            k, uploaded = twin
+            dptr, host0, original0, stored0, name0 = self.temps[k]
+            if not uploaded and not skip_upload:
+                rt.memcpy_h2d(dptr, host.ctypes.data, nbytes, self.stream)
+                self.staged_twice[key] = (k, True)
+            self.temps[k] = (dptr, host0, original0, stored0 or stored, name0)
+            self.aliases.append((name, dptr, nbytes, stored))
+        else:
+            dptr = rt.malloc(max(nbytes, 1))
+            if nbytes and not skip_upload:
+                rt.memcpy_h2d(dptr, host.ctypes.data, nbytes, self.stream)
+            self.staged_twice[key] = (len(self.temps), not skip_upload)
+            self.temps.append((dptr, host, original, stored, name))
         self.ptr[name] = dptr
         self.strides[name] = [s // host.itemsize for s in host.strides]
 

@@ -792,3 +792,44 @@ def test_more_npbench_kernels(gpu):
     x3 = rng.standard_normal((7, 17, 65))
     check(softmax_slices, softmax_slices_ref, x3, np.zeros_like(x3))
     check(doitgen, doitgen_ref, rng.random((6, 5, 40)), rng.random((40, 40)), np.zeros((6, 5, 40)))
+
+
+@appy.jit
+def shift_planes(A, B):
+    #pragma parallel for
+    for i in range(A.shape[0]):
+        for j in range(1, A.shape[1]):
+            #pragma simd
+            for k in range(A.shape[2]):
+                B[i, j, k] = A[i, j - 1, k] + 1.0
+
+
+def test_collapsed_nests_keep_sequential_meaning_when_arguments_alias(gpu):
+    """`B[i, j] = A[i, j - 1] + 1` is independent across j for two arrays and a running sum
+    along j when both names are one array: the collapsed shape is only taken when the
+    arguments do not share memory."""
+    from appy_amd.backends.hip import codegen as cg
+
+    rng = np.random.default_rng(12)
+    A = rng.random((6, 40, 50))
+    B = np.zeros_like(A)
+    shift_planes(A, B)
+    assert np.array_equal(B[:, 1:], A[:, :-1] + 1.0) and not B[:, 0].any()
+    loop = next(v[0] for k, v in cg.code_cache.items() if k[-1] == "shift_planes")
+    assert loop.last_launch.spec.collapse
+    C = A.copy()
+    shift_planes(C, C)                          # one array under both names
+    assert not loop.last_launch.spec.collapse
+    want = A.copy()
+    for j in range(1, 40):
+        want[:, j] = want[:, j - 1] + 1.0
+    assert np.allclose(C, want)
+    # degenerate trip counts of the inner loop
+    one = rng.random((5, 1, 8))
+    out = np.full_like(one, -1.0)
+    shift_planes(one, out)
+    assert np.all(out == -1.0)
+    two = rng.random((5, 2, 8))
+    out = np.zeros_like(two)
+    shift_planes(two, out)
+    assert np.array_equal(out[:, 1], two[:, 0] + 1.0)
