@@ -342,6 +342,36 @@ class LoopAnalysis:
                         return True
         return False
 
+    def _find_reread(self) -> set:
+        """Arrays that one iteration of the parallel loop reads more than once: loaded in two
+        or more ``simd`` loops, or in a ``simd`` loop inside a sequential loop whose variable
+        the subscript does not use.  Such data should stay in the caches between the passes."""
+        seen = {}
+        out = set()
+
+        def visit(stmts, seq_vars):
+            for st in stmts:
+                if isinstance(st, ast.For):
+                    if "simd" in (getattr(st, "pragma", None) or {}):
+                        for n in ast.walk(st):
+                            if (isinstance(n, ast.Subscript) and isinstance(n.ctx, ast.Load) and isinstance(n.value, ast.Name)
+                                    and n.value.id in self.arrays):
+                                name = n.value.id
+                                if seen.setdefault(name, id(st)) != id(st):
+                                    out.add(name)
+                                if any(not _uses_name(n, v) for v in seq_vars):
+                                    out.add(name)
+                    else:
+                        inner = seq_vars + [st.target.id]
+                        visit(st.body, inner)
+                        visit(st.orelse, inner)
+                elif isinstance(st, (ast.If, ast.While)):
+                    visit(st.body, seq_vars)
+                    visit(st.orelse, seq_vars)
+
+        visit(self.outer.body, [])
+        return out
+
     def _find_collapse(self):
         """The sequential loop ``for j in range(lo, hi)`` that is the whole body of the
         parallel loop, if its iterations are provably independent - then the pairs (i, j)
@@ -561,6 +591,7 @@ class LoopAnalysis:
         self.multi_wave_ok = not self._leader_store_reloaded()
         self.strip = self._find_strip() if self.multi_wave_ok else None
         self.collapse = self._find_collapse() if self.kind == "team" else None
+        self.reread = self._find_reread()
 
         # reductions of the parallel loop: constant-subscript elements of arrays
         self.outer_reductions = []
@@ -1043,6 +1074,8 @@ class KernelBuilder:
             return False
         if self.spec.kind == "flat":
             return True
+        if isinstance(sub.value, ast.Name) and sub.value.id in self.a.reread:
+            return False        # the iteration comes back to this data (softmax: max, sum, write): keep it cached
         return self.bounds_vary or any(_uses_name(e, self.a.var) for e in _elts(sub))
 
     def vector_body(self, body, var: str, base_code: str, V: int, loads, stores, declare_locals=False, extra=None):

@@ -551,3 +551,17 @@ def test_independent_inner_loops_collapse_into_the_parallel_loop():
     src = "#pragma parallel for\nfor i in range(n):\n    for j in range(i):\n" + simd + "            B[i, j, k] = A[i, j, k]\n"
     g, _ = compiled(src, A=A, B=B, n=20, p=70)
     assert g.analysis.collapse is None
+
+
+def test_rows_that_an_iteration_reads_twice_are_not_loaded_non_temporally():
+    from appy_amd.backends.hip.kernelgen import Spec
+
+    x = np.zeros((8, 64), np.float32)
+    src = ("#pragma parallel for\nfor i in range(n):\n    m = -1e30\n    #pragma simd\n    for k in range(p):\n"
+           "        m = max(m, x[i, k])\n    s = 0.0\n    #pragma simd\n    for k in range(p):\n"
+           "        s += np.exp(x[i, k] - m)\n    #pragma simd\n    for k in range(p):\n        out[i, k] = w[i, k] / s\n")
+    f, _ = compiled(src, x=x, w=x.copy(), out=x.copy(), n=8, p=64)
+    assert f.analysis.reread == {"x"}
+    k = body_of(f.kernel_for(Spec("team", block=256, vec=4, width=16, stream_loads=True)).src.text)
+    assert "appy::vload<float, 4>(x +" in k and "vload_stream<float, 4>(x +" not in k
+    assert "appy::vload_stream<float, 4>(w +" in k          # read once: streams past the caches
