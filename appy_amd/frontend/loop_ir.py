@@ -314,6 +314,14 @@ def _hoist_element_reductions(tree: ast.Module) -> None:
                         tgt = a.targets[0]
                         read = copy.deepcopy(tgt)
                         read.ctx = ast.Load()
+                        # `y[i] = 0.0` right before the loop: the accumulator starts from that literal
+                        # instead of reading the element back
+                        prev = out[-1] if out else None
+                        if (not pre and isinstance(prev, ast.Assign) and len(prev.targets) == 1
+                                and ast.unparse(prev.targets[0]) == ast.unparse(tgt)
+                                and isinstance(prev.value, ast.Constant) and type(prev.value.value) in (int, float)
+                                and float(prev.value.value).is_integer()):
+                            read = ast.Constant(value=prev.value.value)
                         pre.append(ast.copy_location(ast.Assign(targets=[ast.Name(id=name, ctx=ast.Store())], value=read), st))
                         acc = ast.Name(id=name, ctx=ast.Load())
                         if op in ("+", "*"):

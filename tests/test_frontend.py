@@ -306,7 +306,8 @@ def test_ir_simd_loops_accumulating_into_one_element_use_a_scalar():
         "    for j in range(m):\n        y[i] += A[i, j] * x[j]\n        z[i] = max(z[i], A[i, j])\n        w[i] -= x[j]")
     body = loop_ir.outer_loop(tree).body
     text = [ast.unparse(s) for s in body]
-    assert text[:4] == ["y[i] = 0.0", "__appy_e1 = y[i]", "__appy_e2 = z[i]", "__appy_e3 = w[i]"]
+    # (the literal stored just before the loop is where the first accumulator starts)
+    assert text[:4] == ["y[i] = 0.0", "__appy_e1 = 0.0", "__appy_e2 = z[i]", "__appy_e3 = w[i]"]
     assert text[5:] == ["y[i] = __appy_e1", "z[i] = __appy_e2", "w[i] = __appy_e3"]
     inner = body[4]
     assert [ast.unparse(s) for s in inner.body] == [
