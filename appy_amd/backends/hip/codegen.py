@@ -188,11 +188,23 @@ class Kernel:
 
     def __init__(self, src: KernelSource):
         self.src = src
-        self.code = compile_source(src.text, src.name)
+        self._code = None
+        self._compile_lock = threading.Lock()
         self._funcs = {}   # device -> function handle
         fields = [(f"f{i}", p.ctype) for i, p in enumerate(src.params)]
         self.ArgStruct = type("Args" + src.name, (C.Structure,), {"_fields_": fields})
         self._field_names = [f for f, _ in fields]
+
+    @property
+    def code(self) -> bytes:
+        """The code object, compiled when first asked for: a loop is generated in its default
+        shape when it is first seen, but the launch may pick another shape, and hiprtc takes a
+        few hundred milliseconds per variant."""
+        if self._code is None:
+            with self._compile_lock:
+                if self._code is None:
+                    self._code = compile_source(self.src.text, self.src.name)
+        return self._code
 
     def function(self, device: int):
         f = self._funcs.get(device)
@@ -1011,6 +1023,8 @@ def codegen(loop_source, loop_name, val_map, options):
         if hit is not None:
             return hit
         f = CompiledLoop(loop_source, loop_name, val_map, options)
+        if options.get("dry_run"):
+            f.kernels[f.default_spec].code      # nothing will be launched: compile now, so that errors surface
         code_cache[key] = (f, f.code_src)
     if options.get("dump_code"):
         print(f"--- Dumped code for loop {loop_name} ---")

@@ -165,10 +165,10 @@ def compile_all_patterns() -> int:
         loop, _src = cg.code_cache[key]
         count += len(loop.kernels)
         if loop.analysis.strip is not None:
-            loop.kernel_for(Spec("strip", block=1024, vec=1, unroll=8, stream_loads=True))
+            loop.kernel_for(Spec("strip", block=1024, vec=1, unroll=8, stream_loads=True)).code
             count += 1
         if loop.analysis.kind == "team":
             for w in (1, 4, 16, 64):
-                loop.kernel_for(Spec("team", block=256, vec=loop.default_spec.vec, width=w))
+                loop.kernel_for(Spec("team", block=256, vec=loop.default_spec.vec, width=w)).code
                 count += 1
     return count
