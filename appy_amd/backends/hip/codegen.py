@@ -286,6 +286,8 @@ class CompiledLoop:
         a = self.analysis
         self._lo_code = compile(ast.Expression(body=ast.fix_missing_locations(_copy(a.lo_node))), "<lo>", "eval")
         self._hi_code = compile(ast.Expression(body=ast.fix_missing_locations(_copy(a.hi_node))), "<hi>", "eval")
+        self._affine_check_codes = [(name, dim, text, compile(text, "<subscript>", "eval"))
+                                    for name, dim, text in a.affine_checks]
         self._collapse_codes = None
         if a.collapse is not None:
             self._collapse_codes = tuple(
@@ -743,6 +745,18 @@ class Launch:
                     f"{loop.loop_name}: `{name}` has extent {ext} in dimension {dim} but the loop "
                     f"range [{lo}, {hi}) indexes it at offset {off:+d}"
                 )
+
+        for name, dim, text, code in loop._affine_check_codes:
+            ext = arrays[name].shape[dim]
+            try:
+                ends = [int(eval(code, _HOST_EVAL_GLOBALS, {**env, a.var: x})) for x in (lo, hi - 1)]
+            except Exception:
+                continue        # not computable on the host: left to the kernel
+            if min(ends) < 0 or max(ends) >= ext:
+                raise IndexError(
+                    f"{loop.loop_name}: `{name}` has extent {ext} in dimension {dim} but over the loop range "
+                    f"[{lo}, {hi}) its subscript `{text}` runs from {min(ends)} to {max(ends)} "
+                    f"(negative subscripts other than literals count as outside)")
 
         self.stream = 0
         device = 0

@@ -159,6 +159,29 @@ def _var_offset(node, var: str):
     return None
 
 
+def _affine_in(node, var: str, scalars) -> bool:
+    """True if ``node`` is an affine expression of the loop variable ``var`` with integer
+    constants and by-value scalars as coefficients (``2 * i + 1``, ``n - 1 - i``, ``-i``) and
+    does mention ``var``: its extreme values over a range are taken at the ends of the range."""
+    def walk(n):
+        """(is affine, mentions var)"""
+        if isinstance(n, ast.Constant):
+            return type(n.value) is int, False
+        if isinstance(n, ast.Name):
+            return (n.id == var or n.id in scalars), n.id == var
+        if isinstance(n, ast.UnaryOp) and isinstance(n.op, (ast.USub, ast.UAdd)):
+            return walk(n.operand)
+        if isinstance(n, ast.BinOp) and isinstance(n.op, (ast.Add, ast.Sub, ast.Mult)):
+            (la, lv), (ra, rv) = walk(n.left), walk(n.right)
+            if not (la and ra) or (isinstance(n.op, ast.Mult) and lv and rv):
+                return False, False
+            return True, lv or rv
+        return False, False
+
+    ok, uses = walk(node)
+    return ok and uses
+
+
 def guarded_nodes(stmts) -> set:
     """ids of the subscripts that the program evaluates only under a condition:
     in the arms of ``a if c else b``, after the first operand of ``and`` / ``or``
@@ -624,6 +647,10 @@ class LoopAnalysis:
         # their array.
         self.bound_checks = []
         self.guarded_checks = []
+        # other affine subscripts of the parallel variable (`a[2 * i]`, `a[n - 1 - i]`, `a[-i]`):
+        # (array, dimension, expression); the host evaluates them at both ends of the range
+        self.affine_checks = []
+        fixed_scalars = {k for k, p in self.scalars.items() if k not in self.assigned and p.ty.kind in "iub"}
         guarded = guarded_nodes(self.outer.body)
         for n in ast.walk(self.outer):
             if isinstance(n, ast.Subscript) and isinstance(n.value, ast.Name) and n.value.id in self.arrays:
@@ -632,6 +659,11 @@ class LoopAnalysis:
                     off = _var_offset(e, self.var)
                     if off is not None and (n.value.id, d, off) not in into:
                         into.append((n.value.id, d, off))
+                    elif (off is None and id(n) not in guarded and not isinstance(e, ast.Slice)
+                          and _affine_in(e, self.var, fixed_scalars)):
+                        item = (n.value.id, d, ast.unparse(e))
+                        if item not in self.affine_checks:
+                            self.affine_checks.append(item)
 
 
 def _partial_type(ty: Ty) -> Ty:

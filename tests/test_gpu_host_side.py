@@ -201,3 +201,36 @@ def test_zero_dimensional_arrays_and_tensors_are_scalars(gpu):
     assert torch.equal(ot, 2 * at)
     scale(at, ot, at.max())                         # a 0-d GPU tensor: its value is fetched
     assert torch.equal(ot, 99 * at) and ot.dtype == torch.float32
+
+
+def test_affine_subscripts_of_the_parallel_variable_are_checked_on_the_host(gpu):
+    @appy.jit
+    def reverse(a, out, n):
+        #pragma parallel for simd
+        for i in range(n):
+            out[i] = a[n - 1 - i]
+
+    @appy.jit
+    def every_other(a, out, n):
+        #pragma parallel for simd
+        for i in range(n):
+            out[i] = a[2 * i]
+
+    @appy.jit
+    def from_the_end(a, out, n):
+        #pragma parallel for simd
+        for i in range(n):
+            out[i] = a[-i]
+
+    a = np.arange(100.0)
+    out = np.zeros(100)
+    reverse(a, out, 100)
+    assert np.array_equal(out, a[::-1])
+    every_other(a, out, 50)
+    assert np.array_equal(out[:50], a[::2])
+    with pytest.raises(IndexError, match=r"subscript `2 \* i` runs from 0 to 198"):
+        every_other(a, out, 100)
+    with pytest.raises(IndexError, match="runs from -99 to 0"):
+        from_the_end(a, out, 100)
+    with pytest.raises(IndexError, match="runs from 0 to 100"):
+        reverse(a, np.zeros(101), 101)
