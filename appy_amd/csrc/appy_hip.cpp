@@ -175,17 +175,33 @@ Stager& stager(int device) {
     return *it->second;
 }
 
+void stager_release(Stager& st) {
+    for (auto& lane : st.lanes) {
+        for (int r = 0; r < kRing; ++r) {
+            if (lane.done[r]) (void)hipEventDestroy(lane.done[r]);
+            if (lane.pinned[r]) (void)hipHostFree(lane.pinned[r]);
+            lane.done[r] = nullptr;
+            lane.pinned[r] = nullptr;
+        }
+        if (lane.stream) (void)hipStreamDestroy(lane.stream);
+        lane.stream = nullptr;
+    }
+}
+
 hipError_t stager_prepare(Stager& st) {
     if (st.ready) return hipSuccess;
+    hipError_t e = hipSuccess;
     for (auto& lane : st.lanes) {
-        hipError_t e = hipStreamCreateWithFlags(&lane.stream, hipStreamNonBlocking);
-        if (e != hipSuccess) return e;
-        for (int r = 0; r < kRing; ++r) {
+        e = hipStreamCreateWithFlags(&lane.stream, hipStreamNonBlocking);   // default priority
+        for (int r = 0; r < kRing && e == hipSuccess; ++r) {
             e = hipHostMalloc(reinterpret_cast<void**>(&lane.pinned[r]), kChunk, hipHostMallocDefault);
-            if (e != hipSuccess) return e;
-            e = hipEventCreateWithFlags(&lane.done[r], hipEventDisableTiming);
-            if (e != hipSuccess) return e;
+            if (e == hipSuccess) e = hipEventCreateWithFlags(&lane.done[r], hipEventDisableTiming);
         }
+        if (e != hipSuccess) break;
+    }
+    if (e != hipSuccess) {
+        stager_release(st);     // a partial set-up is of no use: give back what it took
+        return e;
     }
     st.ready = true;
     return hipSuccess;
@@ -254,6 +270,7 @@ hipError_t staged_copy(void* dev, void* host, size_t n, bool to_device, hipStrea
     per = (per + 4095) & ~size_t(4095);
     hipError_t results[kLanes];
     std::thread workers[kLanes];
+    bool inline_slices[kLanes] = {};
     int used = 0;
     for (int t = 0; t < kLanes; ++t) {
         results[t] = hipSuccess;
@@ -265,12 +282,26 @@ hipError_t staged_copy(void* dev, void* host, size_t n, bool to_device, hipStrea
         StageLane* lane = &st.lanes[t];
         hipError_t* out = &results[t];
         if (t == 0) continue;   // the calling thread takes the first slice itself, below
-        workers[t] = std::thread([=] { *out = stage_slice(*lane, device, d, h, m, to_device); });
+        try {
+            workers[t] = std::thread([=] { *out = stage_slice(*lane, device, d, h, m, to_device); });
+        } catch (...) {
+            // no thread to be had: the calling thread copies this slice too (no exception may
+            // cross the C boundary)
+            inline_slices[t] = true;
+        }
         used = t;
     }
     results[0] = stage_slice(st.lanes[0], device, static_cast<char*>(dev), static_cast<char*>(host),
                              std::min(per, n), to_device);
-    for (int t = 1; t <= used; ++t) workers[t].join();
+    for (int t = 1; t <= used; ++t) {
+        if (inline_slices[t]) {
+            const size_t o = per * size_t(t);
+            results[t] = stage_slice(st.lanes[t], device, static_cast<char*>(dev) + o, static_cast<char*>(host) + o,
+                                     std::min(per, n - o), to_device);
+        } else {
+            workers[t].join();
+        }
+    }
     for (int t = 0; t < kLanes; ++t)
         if (results[t] != hipSuccess) return results[t];
     return hipSuccess;
