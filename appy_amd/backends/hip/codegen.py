@@ -306,6 +306,8 @@ class CompiledLoop:
         self._overwrite_codes = {
             name: (None if node is None else compile(ast.Expression(body=ast.fix_missing_locations(_copy(node))), "<n>", "eval"))
             for name, node in a.overwritten.items()}
+        self._scratch = {}  # (device, stream) -> (device pointer, bytes): partial results of two-phase launches
+        self._scratch_retired = []
         self._replays = {}  # call identity -> Launch that can simply be launched again
         # scalars that no host-side decision looks at (range of the loop, inner trip counts,
         # row extents): a replayed launch may carry new values of these
@@ -485,8 +487,15 @@ class CompiledLoop:
                     block //= 2
                 # eight row segments in flight per wavefront; matrices beyond the memory-side
                 # cache are read non-temporally (16384^2 float32: 0.84 of peak against 0.72)
-                return Spec("strip", block=block, vec=1, unroll=8, restrict=restrict,
+                spec = Spec("strip", block=block, vec=1, unroll=8, restrict=restrict,
                             stream_loads=self._bytes_touched(arrays) > MALL_BYTES)
+                if (self.analysis.strip_split is not None and strips * 2 <= DEFAULT_CUS
+                        and trip >= 64 * (block // 64) and not self.options.get("check_bounds")):
+                    # few columns, many rows: one workgroup per strip would leave the chip idle
+                    # (2^20 x 64 floats: 4.8 ms), so several workgroups share the rows of a strip
+                    # and a second, small kernel finishes the body on their partial results
+                    spec = dataclasses.replace(spec, phase=1)
+                return spec
         if d.kind == "flat":
             stream = self._bytes_touched(arrays) > MALL_BYTES
             if self.analysis.lane_loops and not self.analysis.outer_reductions:
@@ -556,6 +565,36 @@ class CompiledLoop:
             block = 1024 if n_outer <= DEFAULT_CUS else 256
             w = block
         return Spec("team", block=block, vec=v, width=w, restrict=restrict, stream_loads=stream, collapse=bool(nj))
+
+    def strip_parts(self, spec: Spec, n_outer: int, env) -> int:
+        """Workgroups per strip of a two-phase strip launch: one workgroup of 1024 lanes per CU
+        in all (2^20 x 64 floats: 79 us with 128 workgroups, 98 with 256, 156 with 512 - the
+        finishing kernel walks the parts of a column one after the other), each part at least
+        four rows per wavefront long."""
+        strips = -(-n_outer // 64)
+        try:
+            trip = int(eval(self._strip_trip_code, _HOST_EVAL_GLOBALS, env))
+        except Exception:
+            trip = 0
+        nw = spec.block // 64
+        parts = min(DEFAULT_CUS // max(1, strips), max(1, trip // (4 * nw)), 1024)
+        return max(1, parts)
+
+    def scratch(self, device: int, stream: int, nbytes: int) -> int:
+        """Device memory for partial results of two-phase launches of this loop: one buffer per
+        device and stream, kept for the life of the loop (launches on one stream follow one
+        another, so they may share it; it only ever grows)."""
+        key = (device, stream)
+        have = self._scratch.get(key)
+        if have is None or have[1] < nbytes:
+            if have is not None:
+                # launches in flight (or recorded in a graph) may still name the smaller buffer:
+                # it is kept, not freed; doubling bounds what is kept to less than the final size
+                self._scratch_retired.append(have[0])
+                nbytes = max(nbytes, 2 * have[1])
+            have = (rt.malloc(nbytes), nbytes)
+            self._scratch[key] = have
+        return have[0]
 
     def collapse_count(self, n_outer, env) -> int:
         """Trip count of the sequential loop that may be collapsed into the parallel loop,
@@ -829,9 +868,32 @@ class Launch:
                     break
         self.kernel = loop.kernel_for(spec)
         self.spec = spec
-        st = self.kernel.ArgStruct()
+        self.second = None           # (kernel, argument block, grid, block) of the finishing kernel of a two-phase launch
+        self.nsplit = 1
+        self.scratch_ptr = 0
+        if spec.phase == 1:
+            self.nsplit = loop.strip_parts(spec, n_outer, env)
+            reds = len(a.strip[id(a.strip_split)])
+            self.scratch_ptr = loop.scratch(device, self.stream, reds * self.nsplit * n_outer * 8)
         self.scalar_fields = {}      # by-value scalar -> field of the argument block
-        for fname, p in zip(self.kernel._field_names, self.kernel.src.params):
+        self.args = self._argument_block(self.kernel, vals, arrays, lo, hi)
+        if spec.phase == 1:
+            fin = loop.kernel_for(dataclasses.replace(spec, block=64, phase=2))
+            strips = -(-n_outer // 64)
+            self.second = (fin, self._argument_block(fin, vals, arrays, lo, hi), (strips, 1, 1), (64, 1, 1))
+            self.grid = (strips * self.nsplit, 1, 1)
+        else:
+            if spec.collapse:
+                n_outer *= max(1, loop.collapse_count(n_outer, env))
+            self.grid = (loop.grid_for(spec, n_outer, kernel=self.kernel,
+                                       row_hint=loop.row_hint(n_outer, env, arrays)), 1, 1)
+        self.block = (spec.block, 1, 1)
+        loop.last_launch = self
+
+    def _argument_block(self, kernel, vals, arrays, lo, hi):
+        loop = self.loop
+        st = kernel.ArgStruct()
+        for fname, p in zip(kernel._field_names, kernel.src.params):
             if p.role == "array":
                 val = self.ptr[p.source]
             elif p.role == "stride":
@@ -852,18 +914,16 @@ class Launch:
                 self.oob = rt.malloc(4)
                 rt.memset_async(self.oob, 0, 4, self.stream)
                 val = self.oob
+            elif p.role == "scratch":
+                val = self.scratch_ptr
+            elif p.role == "nsplit":
+                val = self.nsplit
             elif p.role == "lo":
                 val = lo
             else:
                 val = hi
             setattr(st, fname, val)
-        self.args = st
-        if spec.collapse:
-            n_outer *= max(1, loop.collapse_count(n_outer, env))
-        self.grid = (loop.grid_for(spec, n_outer, kernel=self.kernel,
-                                   row_hint=loop.row_hint(n_outer, env, arrays)), 1, 1)
-        self.block = (spec.block, 1, 1)
-        loop.last_launch = self
+        return st
 
     def _stage_host(self, name, host, original, stored):
         nbytes = host.nbytes
@@ -911,7 +971,8 @@ class Launch:
 
     def replayable(self) -> bool:
         """True if nothing but the kernel launch happens when this call is repeated."""
-        return not (self.temps or self.mirrored or self.keepalive_copies or self.oob or self.capture is not None)
+        return not (self.temps or self.mirrored or self.keepalive_copies or self.oob or self.capture is not None
+                    or self.second is not None)
 
     def _no_capture(self, name, why):
         if self.capture is not None:
@@ -922,6 +983,9 @@ class Launch:
 
     def launch_only(self):
         rt.launch(self.function(), self.grid, self.block, self.args, self.stream)
+        if self.second is not None:
+            fin, args, grid, block = self.second
+            rt.launch(fin.function(self.device), grid, block, args, self.stream)
         g = self.capture
         if g is not None:
             g.launches += 1

@@ -68,6 +68,9 @@ class Spec:
     checked: bool = False        # every subscript is compared with the extents; violations are reported
     hoist_guarded: bool = True   # flat only: loads the source guards with a condition may be issued
                                  # unconditionally (the host has checked that they stay inside their arrays)
+    phase: int = 0               # strip only: 1 = partial results of the shared-out loop over one part of its range
+                                 # (the grid holds several workgroups per strip), 2 = the rest of the body on
+                                 # those partial results; 0 = the whole loop nest in one kernel
     collapse: bool = False       # team only: the parallel loop and the sequential loop that is its whole body
                                  # run as one iteration space (the analysis has shown the inner iterations independent)
 
@@ -87,6 +90,8 @@ class Spec:
             raise ValueError(f"team width must be a power of two up to 64, or the whole workgroup, got {self.width}")
         if self.checked and (self.vec != 1 or self.unroll != 1 or self.extent or self.lds_tile):
             raise ValueError("a bounds-checked kernel takes one element per access (vec = unroll = 1, no row extent, no LDS tile)")
+        if self.phase not in (0, 1, 2) or (self.phase and self.kind != "strip"):
+            raise ValueError("only strip kernels run in two phases")
         if self.collapse and (self.kind != "team" or self.lds_tile):
             raise ValueError("only team kernels without an LDS tile collapse their two outer loops")
         if self.extent < 0 or self.lds_tile < 0 or self.lds_tile % 4 or self.lds_tile > 16384:
@@ -96,7 +101,7 @@ class Spec:
         return (f"{self.kind}_b{self.block}_v{self.vec}_u{self.unroll}_w{self.width}"
                 f"{'_r' if self.restrict else ''}{'_nt' if self.stream_loads else ''}"
                 f"{'_e' + str(self.extent) if self.extent else ''}{'_nts' if self.stream_stores else ''}"
-                f"{'_lds' + str(self.lds_tile) if self.lds_tile else ''}{'' if self.hoist_guarded else '_g'}{'_chk' if self.checked else ''}{'_c2' if self.collapse else ''}")
+                f"{'_lds' + str(self.lds_tile) if self.lds_tile else ''}{'' if self.hoist_guarded else '_g'}{'_chk' if self.checked else ''}{'_c2' if self.collapse else ''}{'_p' + str(self.phase) if self.phase else ''}")
 
 
 @dataclass
@@ -365,6 +370,23 @@ class LoopAnalysis:
                         return True
         return False
 
+    def _find_strip_split(self):
+        """The one shared-out loop of a strip, if the loop nest can run in two phases:
+        partial results of that loop over parts of its range (several workgroups per strip,
+        for matrices with few columns and many rows), then the rest of the body.  That needs
+        a single shared-out loop with reductions, directly in the body of the parallel loop,
+        and nothing but scalar assignments in front of it (they are run by both phases)."""
+        if not self.strip or len(self.strip) != 1:
+            return None
+        body = self.outer.body
+        at = next((k for k, st in enumerate(body) if isinstance(st, ast.For) and id(st) in self.strip), None)
+        if at is None or not self.strip[id(body[at])]:
+            return None
+        for st in body[:at]:
+            if not (isinstance(st, ast.Assign) and isinstance(st.targets[0], ast.Name)):
+                return None
+        return body[at]
+
     def _find_reread(self) -> set:
         """Arrays that one iteration of the parallel loop reads more than once: loaded in two
         or more ``simd`` loops, or in a ``simd`` loop inside a sequential loop whose variable
@@ -614,6 +636,7 @@ class LoopAnalysis:
         self.multi_wave_ok = not self._leader_store_reloaded()
         self.strip = self._find_strip() if self.multi_wave_ok else None
         self.collapse = self._find_collapse() if self.kind == "team" else None
+        self.strip_split = self._find_strip_split()
         self.reread = self._find_reread()
 
         # reductions of the parallel loop: constant-subscript elements of arrays
@@ -1575,16 +1598,32 @@ class KernelBuilder:
         self.w("const int __lane = threadIdx.x & 63;")
         self.w("const int __wave = threadIdx.x >> 6;")
         self.w(f"__shared__ double __strip_slots[{NW}][64];   // one slot per wavefront and lane, any 4- or 8-byte type")
-        self.w("for (appy::i64 __s = blockIdx.x; __lo + __s * 64 < __hi; __s += gridDim.x) {")
+        body = self.a.outer.body
+        if self.spec.phase:
+            if self.a.strip_split is None:
+                raise Unsupported("the loop nest does not suit the two-phase strip shape")
+        if self.spec.phase == 1:
+            # __nsplit workgroups per strip, each with its part of the shared-out loop's range;
+            # the grid holds exactly strips x __nsplit workgroups
+            self.w("const appy::i64 __chunk = blockIdx.x % __nsplit;")
+            self.w("for (appy::i64 __s = blockIdx.x / __nsplit; __lo + __s * 64 < __hi; __s += gridDim.x / __nsplit) {")
+            body = body[:body.index(self.a.strip_split) + 1]
+        else:
+            self.w("for (appy::i64 __s = blockIdx.x; __lo + __s * 64 < __hi; __s += gridDim.x) {")
         self.ind += 1
         self.w("const bool __active = __lo + __s * 64 + __lane < __hi;")
         self.w(f"const appy::i64 {cname(var)} = __active ? __lo + __s * 64 + __lane : __hi - 1;")
         self._declare_locals()
         self.mode = "team"
-        self.block(self.a.outer.body)
+        self.block(body)
         self.mode = "lane"
         self.ind -= 1
         self.w("}")
+
+    def _scratch_slot(self, r: int, chunk: str, pty: Ty) -> str:
+        """Partial result number ``r`` of part ``chunk`` of this lane's column (8-byte slots)."""
+        var = cname(self.a.var)
+        return f"*reinterpret_cast<{pty.c}*>(__scratch + (({r} * __nsplit + {chunk}) * (__hi - __lo) + ({var} - __lo)))"
 
     def strip_spread_loop(self, st: ast.For):
         """A loop of a strip kernel whose iterations are dealt to the wavefronts."""
@@ -1609,6 +1648,36 @@ class KernelBuilder:
             typed[name] = (p, pty)
             self.partials[name] = (p, pty)
             self.w(f"{pty.c} {p} = {_partial_identity(op, ty, pty)};")
+        if self.spec.phase == 2:
+            # The loop has run already (phase 1): pick up the partial results of its parts.  The
+            # loop is still walked, into a buffer that is thrown away, because its statements
+            # decide the types of the variables they assign - both phases must agree on those.
+            kept, self.lines = self.lines, []
+            saved_mode, self.mode = self.mode, "lane"
+            saved_depth, self.seq_depth = self.seq_depth, 0
+            self.iteration_body(st.body)
+            self.mode, self.seq_depth = saved_mode, saved_depth
+            self.lines = kept
+            for r, (name, (p, pty)) in enumerate(typed.items()):
+                op = _OPS[ops[name]]
+                vty = self.ex.locals[name]
+                self.w("if (__active) {")
+                self.w("    #pragma unroll 16")
+                self.w(f"    for (appy::i64 __c = 0; __c < __nsplit; ++__c) "
+                       f"{p} = {op}::f<{pty.c}>({p}, {self._scratch_slot(r, '__c', pty)});")
+                self.w("}")
+                self.w(f"{cname(name)} = {cast(op + '::f<' + pty.c + '>(' + cast(cname(name), vty, pty) + ', ' + p + ')', pty, vty)};")
+            self.partials = saved_partials
+            self.ind -= 1
+            self.w("}")
+            return
+        if self.spec.phase == 1:
+            part = self.fresh("part")
+            self.w(f"const appy::i64 {part} = ({hi_v} - {lo_v} + __nsplit - 1) / __nsplit;")
+            lo_c, hi_c = self.fresh("lo"), self.fresh("hi")
+            self.w(f"const appy::i64 {lo_c} = {lo_v} + __chunk * {part};")
+            self.w(f"const appy::i64 {hi_c} = ({lo_c} + {part}) < {hi_v} ? ({lo_c} + {part}) : {hi_v};")
+            lo_v, hi_v = lo_c, hi_c
         saved_mode, self.mode = self.mode, "lane"
         saved_depth, self.seq_depth = self.seq_depth, 0
         saved_stream = set(self.ex.stream_arrays)
@@ -1647,7 +1716,11 @@ class KernelBuilder:
             t = self.fresh("tot")
             self.w(f"{pty.c} {t} = {slot}[__lane];")
             self.w(f"for (int __w = 1; __w < {NW}; ++__w) {t} = {op}::f<{pty.c}>({t}, {slot}[__w * 64 + __lane]);")
-            self.w(f"{cname(name)} = {cast(op + '::f<' + pty.c + '>(' + cast(cname(name), vty, pty) + ', ' + t + ')', pty, vty)};")
+            if self.spec.phase == 1:
+                r = list(typed).index(name)
+                self.w(f"if (__wave == 0 && __active) {self._scratch_slot(r, '__chunk', pty)} = {t};")
+            else:
+                self.w(f"{cname(name)} = {cast(op + '::f<' + pty.c + '>(' + cast(cname(name), vty, pty) + ', ' + t + ')', pty, vty)};")
             self.w("__syncthreads();   // the slots are free again")
         self.ind -= 1
         self.w("}")
@@ -1876,6 +1949,9 @@ class KernelBuilder:
             params.append(Param(nm, f"const appy::i64 {nm}", C.c_int64, "shape", arr, dim))
         if self.spec.checked:
             params.append(Param("__oob", "int* __oob", C.c_void_p, "oob"))
+        if self.spec.phase:
+            params.append(Param("__scratch", "double* __scratch", C.c_void_p, "scratch"))
+            params.append(Param("__nsplit", "const appy::i64 __nsplit", C.c_int64, "nsplit"))
         params.append(Param("__lo", "const appy::i64 __lo", C.c_int64, "lo"))
         params.append(Param("__hi", "const appy::i64 __hi", C.c_int64, "hi"))
         return params

@@ -141,3 +141,34 @@ def test_replay_is_faster_than_launching_one_by_one(gpu):
     replay = time.perf_counter() - t0
     print(f"\n{2 * steps} launches: eager {eager * 1e3:.2f} ms, one graph replay {replay * 1e3:.2f} ms")
     assert replay < eager
+
+
+@appy.jit
+def column_sums(A, out):
+    #pragma parallel for
+    for j in range(A.shape[1]):
+        s = 0.0
+        for i in range(A.shape[0]):
+            s += A[i, j]
+        out[j] = s
+
+
+def test_two_phase_launches_are_captured_with_both_kernels(gpu):
+    """A tall matrix with few columns runs as two kernels with a scratch buffer between them;
+    a captured launch replays both and keeps using the buffer it was recorded with."""
+    import torch
+
+    A = torch.rand(300_000, 24, device="cuda", dtype=torch.float64)
+    out = torch.zeros(24, device="cuda", dtype=torch.float64)
+    column_sums(A, out)                               # compiled and loaded before the capture
+    assert torch.allclose(out, A.sum(dim=0))
+    out.zero_()
+    with appy.graph() as g:
+        column_sums(A, out)
+    assert not out.any()
+    for replay in range(3):
+        A.mul_(1.5)
+        column_sums(A[:1000], torch.zeros_like(out))  # eager launches of the same loop in between
+        g.launch()
+        g.synchronize()
+        assert torch.allclose(out, A.sum(dim=0)), replay

@@ -833,3 +833,66 @@ def test_collapsed_nests_keep_sequential_meaning_when_arguments_alias(gpu):
     out = np.zeros_like(two)
     shift_planes(two, out)
     assert np.array_equal(out[:, 1], two[:, 0] + 1.0)
+
+
+@appy.jit
+def tall_column_stats(A, total, top, scaled, w):
+    #pragma parallel for
+    for j in range(A.shape[1]):
+        bias = w * 2.0
+        s = 0.0
+        m = -1e30
+        for i in range(A.shape[0]):
+            s += A[i, j]
+            m = max(m, A[i, j])
+        total[j] = s
+        top[j] = m
+        scaled[j] = (s + bias) / A.shape[0]
+
+
+@appy.jit
+def tall_column_dot(A, y, x):
+    #pragma parallel for
+    for j in range(A.shape[1]):
+        s = 0.0
+        #pragma simd
+        for i in range(A.shape[0]):
+            s += A[i, j] * y[i]
+        x[j] = s
+
+
+@pytest.mark.parametrize("shape,dtype", [((200_003, 20), np.float64), ((100_000, 64), np.float32),
+                                         ((50_001, 257), np.float32), ((70_000, 3), np.int32)])
+def test_tall_matrices_with_few_columns_run_as_two_phase_strips(gpu, shape, dtype):
+    """Few columns, many rows: several workgroups share the rows of a strip (partial sums
+    and maxima in a scratch buffer), a second small kernel runs the rest of the body."""
+    from appy_amd.backends.hip import codegen as cg
+
+    rng = np.random.default_rng(21)
+    A = (rng.standard_normal(shape) * 10).astype(dtype)
+    n, m = shape
+    total, top, scaled = np.zeros(m, dtype), np.zeros(m, dtype), np.zeros(m, np.float64)
+    tall_column_stats(A, total, top, scaled, 0.25)
+    loop = next(v[0] for k, v in cg.code_cache.items() if k[-1] == "tall_column_stats"
+                and v[0].analysis.arrays["A"].ty.name == np.dtype(dtype).name)
+    assert loop.last_launch.spec.phase == 1 and loop.last_launch.second is not None
+    want = A.sum(axis=0, dtype=np.float64)
+    if np.dtype(dtype).kind == "f":
+        assert np.allclose(total, want, rtol=1e-4 if dtype == np.float32 else 1e-11, atol=1e-2 if dtype == np.float32 else 1e-7)
+        assert np.allclose(scaled, (want + 0.5) / n, rtol=1e-4 if dtype == np.float32 else 1e-11, atol=1e-6)
+    else:
+        assert np.array_equal(total, want.astype(dtype))
+    assert np.array_equal(top, A.max(axis=0))
+    # twice in a row (the scratch buffer is reused), then on a smaller matrix
+    tall_column_stats(A, total, top, scaled, 0.25)
+    assert np.array_equal(top, A.max(axis=0))
+    B = A[: n // 3].copy()
+    tall_column_stats(B, total, top, scaled, 0.25)
+    assert np.array_equal(top, B.max(axis=0))
+    if np.dtype(dtype).kind == "f":
+        y = rng.standard_normal(n).astype(dtype)
+        x = np.zeros(m, dtype)
+        tall_column_dot(A, y, x)
+        ref = A.astype(np.float64).T @ y.astype(np.float64)
+        budget = np.abs(A.astype(np.float64)).T @ np.abs(y.astype(np.float64))
+        assert np.all(np.abs(x - ref) <= (1e-5 if dtype == np.float32 else 1e-12) * budget + 1e-30)

@@ -243,11 +243,11 @@ def test_repeated_calls_reuse_pooled_buffers(gpu):
     k0.vec_add(a, b)
     used, cached = ctypes.c_uint64(), ctypes.c_uint64()
     rt.check(rt.lib().appy_hip_pool_stats(ctypes.byref(used), ctypes.byref(cached)))
-    first = cached.value
+    first, held = cached.value, used.value      # (held: scratch buffers that loops of earlier tests keep)
     for _ in range(5):
         assert np.array_equal(k0.vec_add(a, b), a + b)
     rt.check(rt.lib().appy_hip_pool_stats(ctypes.byref(used), ctypes.byref(cached)))
-    assert used.value == 0 and cached.value == first          # nothing leaked, nothing newly allocated
+    assert used.value == held and cached.value == first       # nothing leaked, nothing newly allocated
 
 
 @pytest.mark.parametrize("n", [1, 1000, 4099, (1 << 22) + 7])
