@@ -564,7 +564,20 @@ class CompiledLoop:
             # so a whole workgroup takes each row (the more lanes the fewer rows there are)
             block = 1024 if n_outer <= DEFAULT_CUS else 256
             w = block
+            if (self.analysis.team_split is not None and n_outer * 2 <= DEFAULT_CUS and not nj
+                    and trip >= 8 * block * v and not self.options.get("check_bounds")):
+                # fewer rows than half the CUs: several workgroups share a row (4 x 2^24 floats
+                # added elementwise: 3.4 ms with one workgroup per row), partial results of
+                # reductions meet in a second, small kernel
+                return Spec("team", block=block, vec=v, width=w, restrict=restrict, stream_loads=stream, phase=1)
         return Spec("team", block=block, vec=v, width=w, restrict=restrict, stream_loads=stream, collapse=bool(nj))
+
+    def team_parts(self, spec: Spec, n_outer: int, env, arrays) -> int:
+        """Workgroups per row of a two-phase team launch: two workgroups per CU in all, each
+        part at least four vector steps per lane long."""
+        trip, _uniform = self._estimate_trip(env, arrays, n_outer)
+        parts = min(2 * DEFAULT_CUS // max(1, n_outer), int(trip // (4 * spec.block * spec.vec)), 1024)
+        return max(1, parts)
 
     def strip_parts(self, spec: Spec, n_outer: int, env) -> int:
         """Workgroups per strip of a two-phase strip launch: one workgroup of 1024 lanes per CU
@@ -871,17 +884,26 @@ class Launch:
         self.second = None           # (kernel, argument block, grid, block) of the finishing kernel of a two-phase launch
         self.nsplit = 1
         self.scratch_ptr = 0
-        if spec.phase == 1:
+        if spec.phase == 1 and spec.kind == "strip":
             self.nsplit = loop.strip_parts(spec, n_outer, env)
             reds = len(a.strip[id(a.strip_split)])
             self.scratch_ptr = loop.scratch(device, self.stream, reds * self.nsplit * n_outer * 8)
+        elif spec.phase == 1:
+            self.nsplit = loop.team_parts(spec, n_outer, env, arrays)
+            reds = len(loop_ir.reductions_of(a.team_split))
+            self.scratch_ptr = loop.scratch(device, self.stream, max(1, reds) * self.nsplit * n_outer * 8)
         self.scalar_fields = {}      # by-value scalar -> field of the argument block
         self.args = self._argument_block(self.kernel, vals, arrays, lo, hi)
-        if spec.phase == 1:
+        if spec.phase == 1 and spec.kind == "strip":
             fin = loop.kernel_for(dataclasses.replace(spec, block=64, phase=2))
             strips = -(-n_outer // 64)
             self.second = (fin, self._argument_block(fin, vals, arrays, lo, hi), (strips, 1, 1), (64, 1, 1))
             self.grid = (strips * self.nsplit, 1, 1)
+        elif spec.phase == 1:
+            if a.split_needs_finish():
+                fin = loop.kernel_for(dataclasses.replace(spec, block=64, width=64, phase=2))
+                self.second = (fin, self._argument_block(fin, vals, arrays, lo, hi), (n_outer, 1, 1), (64, 1, 1))
+            self.grid = (n_outer * self.nsplit, 1, 1)
         else:
             if spec.collapse:
                 n_outer *= max(1, loop.collapse_count(n_outer, env))

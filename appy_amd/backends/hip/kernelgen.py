@@ -68,9 +68,9 @@ class Spec:
     checked: bool = False        # every subscript is compared with the extents; violations are reported
     hoist_guarded: bool = True   # flat only: loads the source guards with a condition may be issued
                                  # unconditionally (the host has checked that they stay inside their arrays)
-    phase: int = 0               # strip only: 1 = partial results of the shared-out loop over one part of its range
-                                 # (the grid holds several workgroups per strip), 2 = the rest of the body on
-                                 # those partial results; 0 = the whole loop nest in one kernel
+    phase: int = 0               # strips and workgroup teams: 1 = the shared-out loop over one part of its range,
+                                 # partial results to a scratch buffer (the grid holds several workgroups per strip
+                                 # or row), 2 = the rest of the body on those partial results; 0 = one kernel
     collapse: bool = False       # team only: the parallel loop and the sequential loop that is its whole body
                                  # run as one iteration space (the analysis has shown the inner iterations independent)
 
@@ -90,8 +90,10 @@ class Spec:
             raise ValueError(f"team width must be a power of two up to 64, or the whole workgroup, got {self.width}")
         if self.checked and (self.vec != 1 or self.unroll != 1 or self.extent or self.lds_tile):
             raise ValueError("a bounds-checked kernel takes one element per access (vec = unroll = 1, no row extent, no LDS tile)")
-        if self.phase not in (0, 1, 2) or (self.phase and self.kind != "strip"):
-            raise ValueError("only strip kernels run in two phases")
+        if self.phase not in (0, 1, 2) or (self.phase and not (
+                self.kind == "strip" or (self.kind == "team" and self.width in (64, self.block)
+                                         and not self.extent and not self.lds_tile and not self.collapse))):
+            raise ValueError("only strip kernels and teams of a whole wavefront or workgroup run in two phases")
         if self.collapse and (self.kind != "team" or self.lds_tile):
             raise ValueError("only team kernels without an LDS tile collapse their two outer loops")
         if self.extent < 0 or self.lds_tile < 0 or self.lds_tile % 4 or self.lds_tile > 16384:
@@ -387,6 +389,32 @@ class LoopAnalysis:
                 return None
         return body[at]
 
+    def _find_team_split(self):
+        """The one ``simd`` loop of a team nest, if the nest can run in two phases (few,
+        very long rows: several workgroups share a row): a single ``simd`` loop, directly in
+        the body of the parallel loop, with nothing but scalar assignments in front of it."""
+        if self.kind != "team" or not self.multi_wave_ok:
+            return None
+        loops = [n for n in ast.walk(self.outer)
+                 if isinstance(n, ast.For) and n is not self.outer and "simd" in (getattr(n, "pragma", None) or {})]
+        if len(loops) != 1 or not any(loops[0] is st for st in self.outer.body):
+            return None
+        body = self.outer.body
+        at = next(k for k, st in enumerate(body) if st is loops[0])
+        for st in body[:at]:
+            if not (isinstance(st, ast.Assign) and isinstance(st.targets[0], ast.Name)):
+                return None
+        for key in loop_ir.reductions_of(loops[0]):
+            if not key.isidentifier():
+                return None
+        return loops[0]
+
+    def split_needs_finish(self) -> bool:
+        """True if the two-phase form of a team nest needs its second kernel (the loop
+        reduces into scalars, or statements follow it)."""
+        loop = self.team_split
+        return bool(loop_ir.reductions_of(loop)) or self.outer.body[-1] is not loop
+
     def _find_reread(self) -> set:
         """Arrays that one iteration of the parallel loop reads more than once: loaded in two
         or more ``simd`` loops, or in a ``simd`` loop inside a sequential loop whose variable
@@ -637,6 +665,7 @@ class LoopAnalysis:
         self.strip = self._find_strip() if self.multi_wave_ok else None
         self.collapse = self._find_collapse() if self.kind == "team" else None
         self.strip_split = self._find_strip_split()
+        self.team_split = self._find_team_split()
         self.reread = self._find_reread()
 
         # reductions of the parallel loop: constant-subscript elements of arrays
@@ -1198,6 +1227,33 @@ class KernelBuilder:
             pty = _partial_type(ty)
             self.partials[name] = (p, pty)
             self.w(f"{pty.c} {p} = {_partial_identity(op, ty, pty)};")
+        if self.spec.phase == 2:
+            # the loop has run (phase 1); it is walked into a buffer that is thrown away, for the
+            # types of the variables it assigns, and its partial results are picked up
+            kept, self.lines = self.lines, []
+            saved_mode, self.mode = self.mode, "lane"
+            saved_depth, self.seq_depth = self.seq_depth, 0
+            self.iteration_body(st.body)
+            self.mode, self.seq_depth = saved_mode, saved_depth
+            self.lines = kept
+            for r, (name, op) in enumerate(reds.items()):
+                p, pty = self.partials[name]
+                vty = self.ex.locals.get(name, pty)
+                self.w("#pragma unroll 16")
+                self.w(f"for (appy::i64 __c = 0; __c < __nsplit; ++__c) "
+                       f"{p} = {_OPS[op]}::f<{pty.c}>({p}, {self._scratch_slot(r, '__c', pty)});")
+                self.w(f"{cname(name)} = {cast(_OPS[op] + '::f<' + pty.c + '>(' + cast(cname(name), vty, pty) + ', ' + p + ')', pty, vty)};")
+            self.partials = saved_partials
+            self.ind -= 1
+            self.w("}")
+            return
+        if self.spec.phase == 1:
+            part = self.fresh("part")
+            self.w(f"const appy::i64 {part} = ({hi_v} - {lo_v} + __nsplit - 1) / __nsplit;")
+            lo_c, hi_c = self.fresh("lo"), self.fresh("hi")
+            self.w(f"const appy::i64 {lo_c} = {lo_v} + __chunk * {part};")
+            self.w(f"const appy::i64 {hi_c} = ({lo_c} + {part}) < {hi_v} ? ({lo_c} + {part}) : {hi_v};")
+            lo_v, hi_v = lo_c, hi_c
         saved_mode = self.mode
         self.mode = "lane"
         saved_depth, self.seq_depth = self.seq_depth, 0
@@ -1232,11 +1288,16 @@ class KernelBuilder:
                           for b in st.body for n in ast.walk(b)):
             # a team of several wavefronts: what one of them stored is read by the others only after this
             self.w("__syncthreads();")
-        for name, op in reds.items():
+        for r, (name, op) in enumerate(reds.items()):
             p, ty = self.partials[name]
             vty = self.ex.locals.get(name, ty)
             total = self._team_total(op, ty, p)
-            self.w(f"{cname(name)} = {cast(_OPS[op] + '::f<' + ty.c + '>(' + cast(cname(name), vty, ty) + ', ' + total + ')', ty, vty)};")
+            if self.spec.phase == 1:
+                t = self.fresh("tot")
+                self.w(f"const {ty.c} {t} = {total};")
+                self.w(f"if ({self._leader()}) {self._scratch_slot(r, '__chunk', ty)} = {t};")
+            else:
+                self.w(f"{cname(name)} = {cast(_OPS[op] + '::f<' + ty.c + '>(' + cast(cname(name), vty, ty) + ', ' + total + ')', ty, vty)};")
         self.partials = saved_partials
         self.ind -= 1
         self.w("}")
@@ -1481,10 +1542,14 @@ class KernelBuilder:
             init = f" = {cname(name)}__arg" if name in self.shadowed else " = 0"
             self.w(f"{ty.c} {cname(name)}{init};")
 
-    def _iteration(self, idx_code: str):
+    def _iteration(self, idx_code: str, body=None):
         self.w("{")
         self.ind += 1
-        if self.spec.collapse:
+        if body is not None:
+            self.w(f"const appy::i64 {cname(self.a.var)} = {idx_code};")
+            self._declare_locals()
+            self.iteration_body(body)
+        elif self.spec.collapse:
             # idx_code counts the pairs (i, j) from zero, j fastest
             inner = self.a.collapse
             self.w(f"const appy::i64 {cname(self.a.var)} = __lo + ({idx_code}) / __nj;")
@@ -1771,6 +1836,26 @@ class KernelBuilder:
         self.lds_plan = self._find_lds_plan()
         self.w(f"const int __lane = threadIdx.x & {W - 1};")
         self.w(f"const appy::i64 __team = threadIdx.x / {W};")
+        if self.spec.phase:
+            if self.a.team_split is None or self.lds_plan is not None:
+                raise Unsupported("the loop nest does not suit the two-phase team shape")
+            self.mode = "team"
+            if self.spec.phase == 1:
+                # __nsplit workgroups per row, each with its part of the simd loop's range
+                self.w("const appy::i64 __chunk = blockIdx.x % __nsplit;")
+                self.w(f"for (appy::i64 __i = __lo + (blockIdx.x / __nsplit) * {tpb}LL + __team; __i < __hi; "
+                       f"__i += (gridDim.x / __nsplit) * {tpb}LL) {{")
+                self.ind += 1
+                body = self.a.outer.body
+                self._iteration("__i", body[:body.index(self.a.team_split) + 1])
+            else:
+                self.w(f"for (appy::i64 __i = __lo + blockIdx.x * {tpb}LL + __team; __i < __hi; __i += gridDim.x * {tpb}LL) {{")
+                self.ind += 1
+                self._iteration("__i")
+            self.mode = "lane"
+            self.ind -= 1
+            self.w("}")
+            return
         if self.spec.collapse:
             if self.a.collapse is None or self.lds_plan is not None:
                 raise Unsupported("the loop nest does not suit the collapsed shape")

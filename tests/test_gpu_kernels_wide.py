@@ -896,3 +896,65 @@ def test_tall_matrices_with_few_columns_run_as_two_phase_strips(gpu, shape, dtyp
         ref = A.astype(np.float64).T @ y.astype(np.float64)
         budget = np.abs(A.astype(np.float64)).T @ np.abs(y.astype(np.float64))
         assert np.all(np.abs(x - ref) <= (1e-5 if dtype == np.float32 else 1e-12) * budget + 1e-30)
+
+
+@appy.jit
+def few_long_rows(A, B, C, y, z, scale):
+    #pragma parallel for
+    for i in range(A.shape[0]):
+        #pragma simd
+        for j in range(A.shape[1]):
+            C[i, j] = A[i, j] + B[i, j]
+    #pragma parallel for
+    for i in range(A.shape[0]):
+        f = scale[i] * 2.0
+        s = 0.0
+        m = -1e30
+        #pragma simd
+        for j in range(A.shape[1]):
+            s += A[i, j] * f
+            m = max(m, B[i, j])
+        y[i] = s + 1.0
+        z[i] = m
+
+
+@appy.jit
+def csr_rows(data, indptr, indices, x, y):
+    #pragma parallel for
+    for i in range(y.shape[0]):
+        start, end = indptr[i], indptr[i + 1]
+        s = 0.0
+        #pragma simd
+        for k in range(start, end):
+            s += data[k] * x[indices[k]]
+        y[i] = s
+
+
+@pytest.mark.parametrize("shape", [(1, 1_000_003), (3, 400_001), (40, 70_000)])
+def test_few_very_long_rows_are_shared_by_several_workgroups(gpu, shape):
+    """Fewer rows than half the CUs, each very long: several workgroups take parts of a row;
+    elementwise loops need nothing more, reductions meet in a finishing kernel."""
+    from appy_amd.backends.hip import codegen as cg
+
+    rng = np.random.default_rng(31)
+    A, B = rng.standard_normal(shape), rng.standard_normal(shape)
+    C = np.zeros(shape)
+    y, z, scale = np.zeros(shape[0]), np.zeros(shape[0]), rng.random(shape[0])
+    few_long_rows(A, B, C, y, z, scale)
+    loops = [v[0] for k, v in cg.code_cache.items() if k[-1] == "few_long_rows"]
+    assert all(lp.last_launch.spec.phase == 1 for lp in loops)
+    assert sorted(lp.last_launch.second is not None for lp in loops) == [False, True]
+    assert np.array_equal(C, A + B)
+    assert np.allclose(y, (A * (scale[:, None] * 2.0)).sum(axis=1) + 1.0, rtol=1e-11, atol=1e-8)
+    assert np.array_equal(z, B.max(axis=1))
+    # CSR rows whose bounds are read per row: two long rows and an empty one
+    n = 300_000
+    data, x = rng.standard_normal(2 * n), rng.standard_normal(1000)
+    indices = rng.integers(0, 1000, 2 * n).astype(np.int32)
+    indptr = np.array([0, n, n, 2 * n], dtype=np.int64)
+    out = np.zeros(3)
+    csr_rows(data, indptr, indices, x, out)
+    want = [np.dot(data[:n], x[indices[:n]]), 0.0, np.dot(data[n:], x[indices[n:]])]
+    assert np.allclose(out, want, rtol=1e-10, atol=1e-7)
+    loop = next(v[0] for k, v in cg.code_cache.items() if k[-1] == "csr_rows")
+    assert loop.last_launch.spec.phase == 1
