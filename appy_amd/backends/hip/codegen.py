@@ -887,7 +887,7 @@ class Launch:
         if spec.phase == 1 and spec.kind == "strip":
             self.nsplit = loop.strip_parts(spec, n_outer, env)
             reds = len(a.strip[id(a.strip_split)])
-            self.scratch_ptr = loop.scratch(device, self.stream, reds * self.nsplit * n_outer * 8)
+            self.scratch_ptr = loop.scratch(device, self.stream, max(1, reds) * self.nsplit * n_outer * 8)
         elif spec.phase == 1:
             self.nsplit = loop.team_parts(spec, n_outer, env, arrays)
             reds = len(loop_ir.reductions_of(a.team_split))
@@ -895,9 +895,10 @@ class Launch:
         self.scalar_fields = {}      # by-value scalar -> field of the argument block
         self.args = self._argument_block(self.kernel, vals, arrays, lo, hi)
         if spec.phase == 1 and spec.kind == "strip":
-            fin = loop.kernel_for(dataclasses.replace(spec, block=64, phase=2))
             strips = -(-n_outer // 64)
-            self.second = (fin, self._argument_block(fin, vals, arrays, lo, hi), (strips, 1, 1), (64, 1, 1))
+            if a.strip_split_needs_finish():
+                fin = loop.kernel_for(dataclasses.replace(spec, block=64, phase=2))
+                self.second = (fin, self._argument_block(fin, vals, arrays, lo, hi), (strips, 1, 1), (64, 1, 1))
             self.grid = (strips * self.nsplit, 1, 1)
         elif spec.phase == 1:
             if a.split_needs_finish():

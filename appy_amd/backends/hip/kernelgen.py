@@ -382,7 +382,7 @@ class LoopAnalysis:
             return None
         body = self.outer.body
         at = next((k for k, st in enumerate(body) if isinstance(st, ast.For) and id(st) in self.strip), None)
-        if at is None or not self.strip[id(body[at])]:
+        if at is None:
             return None
         for st in body[:at]:
             if not (isinstance(st, ast.Assign) and isinstance(st.targets[0], ast.Name)):
@@ -414,6 +414,10 @@ class LoopAnalysis:
         reduces into scalars, or statements follow it)."""
         loop = self.team_split
         return bool(loop_ir.reductions_of(loop)) or self.outer.body[-1] is not loop
+
+    def strip_split_needs_finish(self) -> bool:
+        loop = self.strip_split
+        return bool(self.strip[id(loop)]) or self.outer.body[-1] is not loop
 
     def _find_reread(self) -> set:
         """Arrays that one iteration of the parallel loop reads more than once: loaded in two
@@ -587,7 +591,8 @@ class LoopAnalysis:
                 return None
             for loop, ops in parts:
                 for st in loop.body:
-                    st.reduce = ops[st.targets[0].id]
+                    if isinstance(st.targets[0], ast.Name):
+                        st.reduce = ops[st.targets[0].id]
                 spread[id(loop)] = ops
         if not spread:
             return None
@@ -741,10 +746,12 @@ def _partial_identity(op: str, ty: Ty, pty: Ty) -> str:
 
 def _find_strip_parts(body, var):
     """``[(loop, {scalar: op}), ...]`` if the body of a parallel loop is scalar set-up,
-    then sequential loops that only fold values into scalars with a reduction operator
-    (``s += A[j, i] * y[j]``) and never look at the running value, with nothing but scalar
-    assignments between them (``mu = s / n``), then anything without loops: column
-    reductions written without ``simd``.  None otherwise."""
+    then sequential loops with independent iterations - they fold values into scalars with
+    a reduction operator (``s += A[j, i] * y[j]``) without looking at the running value,
+    and / or store to arrays, each iteration inside its own slab (``C[j, i] = A[j, i] * f[i]``:
+    the loop variable, plus a constant, in one dimension of every subscript of that array) -
+    with nothing but scalar assignments between them (``mu = s / n``), then anything without
+    loops: column reductions and column updates written without ``simd``.  None otherwise."""
     at = [k for k, st in enumerate(body) if isinstance(st, (ast.For, ast.While))]
     if not at or not all(isinstance(body[k], ast.For) for k in at):
         return None
@@ -757,17 +764,38 @@ def _find_strip_parts(body, var):
             if any(isinstance(n, (ast.For, ast.While, ast.Break)) for n in ast.walk(st)):
                 return None
         ops = {}
+        k_var = loop.target.id
+        slab = {}           # array stored in the loop -> (dimension, offset) of the loop variable in its subscripts
+        folds = []
         for st in loop.body:
-            if not (isinstance(st, ast.Assign) and isinstance(st.targets[0], ast.Name)):
+            if not isinstance(st, ast.Assign):
                 return None
-            op = loop_ir.reduction_operator(st)
-            name = st.targets[0].id
-            if op is None or ops.setdefault(name, op) != op:
+            tgt = st.targets[0]
+            if isinstance(tgt, ast.Name):
+                op = loop_ir.reduction_operator(st)
+                if op is None or ops.setdefault(tgt.id, op) != op:
+                    return None
+                folds.append(st)
+            elif isinstance(tgt, ast.Subscript) and isinstance(tgt.value, ast.Name):
+                # a store: iterations are independent when each one stays in its own slab of the array
+                where = [(d, _var_offset(e, k_var)) for d, e in enumerate(_elts(tgt)) if _var_offset(e, k_var) is not None]
+                if len(where) != 1 or slab.setdefault(tgt.value.id, where[0]) != where[0]:
+                    return None
+            else:
                 return None
         for name in ops:    # the running value is not looked at inside the loop
-            if any(_uses_name(loop_ir.reduction_operand(s2), name) for s2 in loop.body):
+            if any(_uses_name(loop_ir.reduction_operand(s2), name) for s2 in folds):
                 return None
-        if not ops or any(_uses_name(a, n) for a in loop.iter.args for n in ops):
+            if any(_uses_name(s2.value, name) for s2 in loop.body if s2 not in folds):
+                return None
+        for n in ast.walk(loop):
+            if isinstance(n, ast.Subscript) and isinstance(n.value, ast.Name) and n.value.id in slab:
+                d, off = slab[n.value.id]
+                idx = _elts(n)
+                if d >= len(idx) or _var_offset(idx[d], k_var) != off or any(
+                        _uses_name(e, k_var) for q, e in enumerate(idx) if q != d):
+                    return None
+        if not (ops or slab) or any(_uses_name(a, n) for a in loop.iter.args for n in ops):
             return None
         found.append((loop, ops))
     for k, st in enumerate(body):

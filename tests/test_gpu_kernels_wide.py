@@ -958,3 +958,34 @@ def test_few_very_long_rows_are_shared_by_several_workgroups(gpu, shape):
     assert np.allclose(out, want, rtol=1e-10, atol=1e-7)
     loop = next(v[0] for k, v in cg.code_cache.items() if k[-1] == "csr_rows")
     assert loop.last_launch.spec.phase == 1
+
+
+@appy.jit
+def shifted_column_updates(A, f, C, D):
+    #pragma parallel for
+    for j in range(A.shape[1]):
+        w = f[j] * 2.0
+        for i in range(1, A.shape[0]):
+            C[i, j] = A[i, j] * w + A[i - 1, j]
+            D[i - 1, j] = A[i, j] - w
+
+
+@pytest.mark.parametrize("shape", [(3, 5000), (700, 300), (100_000, 48), (300_000, 5)])
+def test_column_updates_written_without_simd(gpu, shape):
+    """A sequential loop down the columns that only stores, each iteration to its own row of
+    the arrays it stores to: shared out between the wavefronts of a strip like a reduction
+    loop (and between workgroups when the matrix is tall and narrow); with few rows one lane
+    per column walks them."""
+    from appy_amd.backends.hip import codegen as cg
+
+    rng = np.random.default_rng(41)
+    A, f = rng.standard_normal(shape), rng.standard_normal(shape[1])
+    C, D = np.zeros(shape), np.zeros(shape)
+    shifted_column_updates(A, f, C, D)
+    assert np.array_equal(C[1:], A[1:] * (f * 2.0) + A[:-1]) and not C[0].any()
+    assert np.array_equal(D[:-1], A[1:] - f * 2.0) and not D[-1].any()
+    loop = next(v[0] for k, v in cg.code_cache.items() if k[-1] == "shifted_column_updates")
+    spec = loop.last_launch.spec
+    assert loop.analysis.strip is not None
+    assert spec.kind == ("flat" if shape[0] < 64 else "strip")
+    assert spec.phase == (1 if shape[0] >= 100_000 else 0) and loop.last_launch.second is None
