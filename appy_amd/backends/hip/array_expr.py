@@ -26,6 +26,10 @@ import ast
 import copy
 
 _REDUCERS = {"sum": "+", "max": "max", "min": "min", "amax": "max", "amin": "min", "prod": "*"}
+# further NumPy functions of one 1-D operand (two for the products) that come down to reductions
+_DERIVED = ("mean", "average", "var", "std", "any", "all", "count_nonzero", "dot", "inner", "vdot", "argmax", "argmin")
+# methods of an array expression that mean the function of the same name
+_METHODS = ("sum", "max", "min", "prod", "mean", "var", "std", "any", "all", "dot", "argmax", "argmin")
 
 
 def _is_array(val) -> bool:
@@ -68,10 +72,9 @@ def _has_vector_part(node, ctx: _Ctx) -> bool:
             and isinstance(n.func, ast.Attribute)
             and isinstance(n.func.value, ast.Name)
             and n.func.value.id in ("np", "numpy")
-            and n.func.attr in _REDUCERS
-            and len(n.args) == 1
-            and isinstance(n.args[0], ast.Name)
-            and ctx.ndim(n.args[0].id) == 1
+            and (n.func.attr in _REDUCERS or n.func.attr in _DERIVED)
+            and 1 <= len(n.args) <= 2
+            and all(isinstance(a, ast.Name) and ctx.ndim(a.id) == 1 for a in n.args)
         ):
             return True
     return False
@@ -117,6 +120,48 @@ def _offset(lo, c: str):
     if isinstance(lo, ast.Constant) and lo.value == 0:
         return idx
     return ast.BinOp(left=copy.deepcopy(lo), op=ast.Add(), right=idx)
+
+
+class _Canonical(ast.NodeTransformer):
+    """Spellings that mean an array expression without showing a slice: ``A[i]`` of a 2-D
+    array is the row ``A[i, :]``; ``E.sum()`` is ``np.sum(E)``, ``E.astype(T)`` is ``T(E)``
+    element by element, for an array expression ``E``."""
+
+    def __init__(self, ctx: _Ctx):
+        self.ctx = ctx
+
+    def visit_Subscript(self, node):
+        self.generic_visit(node)
+        if isinstance(node.value, ast.Name):
+            nd = self.ctx.ndim(node.value.id)
+            elts = list(node.slice.elts) if isinstance(node.slice, ast.Tuple) else [node.slice]
+            if nd is not None and 0 < len(elts) < nd and not any(isinstance(e, ast.Constant) and e.value is Ellipsis for e in elts):
+                elts += [ast.Slice(lower=None, upper=None, step=None) for _ in range(nd - len(elts))]
+                node.slice = ast.Tuple(elts=elts, ctx=ast.Load())
+        return node
+
+    def visit_Call(self, node):
+        self.generic_visit(node)
+        f = node.func
+        # `axis=0` / `axis=-1` on a 1-D operand says nothing
+        if (isinstance(f, ast.Attribute) and (f.attr in _REDUCERS or f.attr in _DERIVED or f.attr in _METHODS)
+                and len(node.keywords) == 1 and node.keywords[0].arg == "axis"
+                and isinstance(node.keywords[0].value, (ast.Constant, ast.UnaryOp))
+                and ast.literal_eval(node.keywords[0].value) in (0, -1)):
+            node.keywords = []
+        if (isinstance(f, ast.Attribute) and isinstance(f.value, ast.Name) and f.value.id in ("np", "numpy")
+                and f.attr in ("zeros_like", "ones_like") and len(node.args) == 1 and not node.keywords
+                and (_has_vector_part(node.args[0], self.ctx)
+                     or (isinstance(node.args[0], ast.Name) and self.ctx.ndim(node.args[0].id) == 1))):
+            return ast.Constant(value=0 if f.attr == "zeros_like" else 1)
+        if isinstance(f, ast.Attribute) and not (isinstance(f.value, ast.Name) and f.value.id in ("np", "numpy", "math")):
+            vec = _has_vector_part(f.value, self.ctx) or (isinstance(f.value, ast.Name) and self.ctx.ndim(f.value.id) == 1)
+            if vec and f.attr in _METHODS and not node.keywords:
+                np_fn = ast.Attribute(value=ast.Name(id="np", ctx=ast.Load()), attr=f.attr, ctx=ast.Load())
+                return ast.Call(func=np_fn, args=[f.value] + node.args, keywords=[])
+            if vec and f.attr == "astype" and len(node.args) == 1 and not node.keywords:
+                return ast.Call(func=node.args[0], args=[f.value], keywords=[])
+        return node
 
 
 class _Scalarise(ast.NodeTransformer):
@@ -194,14 +239,19 @@ class _ReduceCalls(ast.NodeTransformer):
         self.ctx = ctx
         self.prologue = []
 
-    def _reduce(self, op: str, vec_expr):
+    def _reduce(self, op: str, vec_expr, init=None, indexed=None):
         r = self.ctx.fresh("r")
         c = self.ctx.fresh("c")
         sc = _Scalarise(self.ctx, c)
         elem = sc.visit(copy.deepcopy(vec_expr))
         if sc.first_extent is None:
             raise RuntimeError(f"Reduction over a non-array expression: {ast.unparse(vec_expr)}")
-        if op == "+":
+        self.last_extent = sc.first_extent
+        if indexed is not None:
+            elem = indexed(elem, c, sc.first_extent)
+        if init is not None:
+            pass
+        elif op == "+":
             init = ast.Constant(value=0)
         elif op == "*":
             init = ast.Constant(value=1)
@@ -219,20 +269,67 @@ class _ReduceCalls(ast.NodeTransformer):
         self.prologue.append(_simd_loop(c, sc.first_extent, [upd], reduction=(op, r)))
         return ast.Name(id=r, ctx=ast.Load())
 
+    def _is_vec(self, node):
+        return _has_vector_part(node, self.ctx) or self._is_vec_name(node)
+
     def visit_Call(self, node):
         f = node.func
-        if (
-            isinstance(f, ast.Attribute)
-            and isinstance(f.value, ast.Name)
-            and f.value.id in ("np", "numpy")
-            and f.attr in _REDUCERS
-            and len(node.args) == 1
-            and (_has_vector_part(node.args[0], self.ctx) or self._is_vec_name(node.args[0]))
-        ):
+        is_np = isinstance(f, ast.Attribute) and isinstance(f.value, ast.Name) and f.value.id in ("np", "numpy")
+        if is_np and f.attr in _REDUCERS and len(node.args) == 1 and not node.keywords and self._is_vec(node.args[0]):
             inner = self.visit(node.args[0])  # nested reductions first
             return self._reduce(_REDUCERS[f.attr], inner)
+        if is_np and f.attr in _DERIVED and node.args and not node.keywords and all(self._is_vec(a) for a in node.args):
+            return self._derived(f.attr, [self.visit(a) for a in node.args], node)
+        if (isinstance(f, ast.Name) and f.id == "len" and len(node.args) == 1 and _has_vector_part(node.args[0], self.ctx)):
+            sc = _Scalarise(self.ctx, "__none")
+            sc.visit(copy.deepcopy(node.args[0]))
+            return sc.first_extent
         self.generic_visit(node)
         return node
+
+    def _derived(self, fn: str, args, node):
+        """``np.mean`` / ``var`` / ``std`` / ``any`` / ``all`` / ``count_nonzero`` / ``dot`` of
+        1-D array expressions, spelled through sum / max / min reductions."""
+        P = lambda text: ast.parse(text, mode="eval").body      # noqa: E731
+        if fn in ("dot", "inner", "vdot"):
+            if len(args) != 2:
+                raise RuntimeError(f"np.{fn} takes two 1-D operands here: {ast.unparse(node)}")
+            return self._reduce("+", ast.BinOp(left=args[0], op=ast.Mult(), right=args[1]))
+        if len(args) != 1:
+            raise RuntimeError(f"np.{fn} takes one 1-D operand here: {ast.unparse(node)}")
+        e = args[0]
+        if fn in ("mean", "average"):
+            total = self._reduce("+", e, init=ast.Constant(value=0.0))
+            return ast.BinOp(left=total, op=ast.Div(), right=copy.deepcopy(self.last_extent))
+        if fn in ("var", "std"):
+            total = self._reduce("+", e, init=ast.Constant(value=0.0))
+            n = self.last_extent
+            mean = ast.BinOp(left=total, op=ast.Div(), right=copy.deepcopy(n))
+            m = self.ctx.fresh("r")
+            self.prologue.append(ast.Assign(targets=[ast.Name(id=m, ctx=ast.Store())], value=mean))
+            dev = ast.BinOp(left=copy.deepcopy(e), op=ast.Sub(), right=ast.Name(id=m, ctx=ast.Load()))
+            sq = self._reduce("+", ast.BinOp(left=dev, op=ast.Mult(), right=copy.deepcopy(dev)), init=ast.Constant(value=0.0))
+            var = ast.BinOp(left=sq, op=ast.Div(), right=copy.deepcopy(n))
+            return var if fn == "var" else ast.BinOp(left=var, op=ast.Pow(), right=ast.Constant(value=0.5))
+        if fn in ("argmax", "argmin"):
+            # the extreme value first, then the smallest position that holds it
+            best = self._reduce("max" if fn == "argmax" else "min", e)
+            b = self.ctx.fresh("r")
+            self.prologue.append(ast.Assign(targets=[ast.Name(id=b, ctx=ast.Store())], value=best))
+
+            def position(elem, c, extent):
+                hit = ast.Compare(left=elem, ops=[ast.Eq()], comparators=[ast.Name(id=b, ctx=ast.Load())])
+                return ast.IfExp(test=hit, body=ast.Name(id=c, ctx=ast.Load()), orelse=copy.deepcopy(extent))
+
+            first = self._reduce("min", e, init=ast.Constant(value=2 ** 62), indexed=position)
+            return first
+        truth = ast.Call(func=ast.Name(id="bool", ctx=ast.Load()), args=[e], keywords=[])
+        if fn == "any":
+            return self._reduce("max", truth, init=ast.Constant(value=False))
+        if fn == "all":
+            return self._reduce("min", truth, init=ast.Constant(value=True))
+        assert fn == "count_nonzero"
+        return self._reduce("+", ast.Call(func=ast.Name(id="int", ctx=ast.Load()), args=[truth], keywords=[]))
 
     def _is_vec_name(self, node):
         return isinstance(node, ast.Name) and self.ctx.ndim(node.id) == 1
@@ -311,7 +408,10 @@ def _lower_assign(st: ast.Assign, ctx: _Ctx):
 
 def _lower_block(stmts, ctx: _Ctx):
     out = []
+    canon = _Canonical(ctx)
     for st in stmts:
+        if isinstance(st, ast.Assign):
+            st = canon.visit(st)
         if isinstance(st, ast.Assign) and (
             _has_vector_part(st, ctx)
         ):

@@ -565,3 +565,24 @@ def test_rows_that_an_iteration_reads_twice_are_not_loaded_non_temporally():
     k = body_of(f.kernel_for(Spec("team", block=256, vec=4, width=16, stream_loads=True)).src.text)
     assert "appy::vload<float, 4>(x +" in k and "vload_stream<float, 4>(x +" not in k
     assert "appy::vload_stream<float, 4>(w +" in k          # read once: streams past the caches
+
+
+def test_rows_without_slices_and_reductions_spelled_as_methods_are_lowered_to_simd_loops():
+    import ast
+
+    from appy_amd.backends.hip import array_expr
+    from appy_amd.frontend import loop_ir
+
+    A, x, out = np.zeros((4, 9)), np.zeros(9), np.zeros(4)
+    src = ("#pragma parallel for\nfor i in range(n):\n    B[i] = A[i] * 2\n    out[i] = A[i].mean() + np.dot(A[i], x)\n"
+           "    k[i] = np.argmax(A[i, :])\n")
+    tree, shapes = array_expr.transform(loop_ir.build(src), dict(A=A, B=A.copy(), x=x, out=out, k=np.zeros(4, np.int64), n=4, np=np))
+    text = ast.unparse(tree)
+    assert "B[i, __c1] = A[i, __c1] * 2" in text                       # the row, element by element
+    assert "__r2 = __r2 + A[i, __c3]" in text and "/ A_shape_1" in text     # mean = sum / extent
+    assert "A[i, __c5] * x[__c5]" in text                               # np.dot of two 1-D operands
+    assert "max(__r" in text and "if A[i, __c" in text and "== __r" in text      # argmax: the maximum, then its first position
+    assert ("A", 1) in shapes
+    # and the whole nest compiles
+    f, _ = compiled(src, A=A, B=A.copy(), x=x, out=out, k=np.zeros(4, np.int64), n=4)
+    assert f.analysis.kind == "team"

@@ -290,3 +290,50 @@ def test_random_slice_statements_against_numpy(gpu, seed):
     appy.jit(ns["kernel"])(**got)
     for key in ("A", "v", "r"):
         assert np.allclose(got[key], ref[key], rtol=1e-12, atol=1e-12), (key, src)
+
+
+_MORE_FORMS = {
+    "implicit row": "B[i] = A[i] * 2",
+    "np.dot of rows": "out[i] = np.dot(A[i], x)",
+    "matmul of a row": "out[i] = A[i] @ x",
+    "sum method": "out[i] = A[i].sum()",
+    "mean": "out[i] = np.mean(A[i, :])",
+    "centre with the mean method": "B[i, :] = A[i, :] - A[i, :].mean()",
+    "std and var": "out[i] = np.std(A[i, :]) + np.var(A[i, 2:])",
+    "argmax and argmin": "out[i] = np.argmax(A[i, :]) - A[i].argmin()",
+    "max and min methods": "out[i] = A[i, :].max() - A[i, :].min()",
+    "sum of a product, as a method": "out[i] = (A[i, :] * x).sum()",
+    "any": "out[i] = np.any(A[i, :] > 2.5)",
+    "all": "out[i] = np.all(A[i, :] > -2.0)",
+    "count_nonzero": "out[i] = np.count_nonzero(A[i, :] > 0)",
+    "dot of two rows": "out[i] = np.dot(A[i, :], A[(i + 1) % A.shape[0], :])",
+    "axis keyword": "out[i] = A[i, :].mean(axis=0) + np.sum(A[i], axis=-1)",
+    "astype": "B[i, :] = A[i, :].astype(np.float32)",
+    "zeros_like and ones_like": "B[i, :] = np.zeros_like(A[i, :]) + np.ones_like(x) * 3",
+    "len of a slice": "out[i] = len(A[i, 3:]) + len(x)",
+    "norm": "out[i] = np.sqrt(np.sum(A[i] ** 2))",
+}
+
+
+@pytest.mark.parametrize("name", sorted(_MORE_FORMS))
+def test_more_numpy_spellings_of_row_expressions(gpu, name):
+    """Rows without a slice (`A[i]` of a 2-D array), reductions as methods, and the NumPy
+    functions that come down to sum / max / min reductions, inside `prange` loops as the
+    reference's guide promises for "common NumPy array operations, slicing, and indexing"
+    (docs/source/high-level.rst:48-50); each against the same loop run by NumPy."""
+    import linecache
+
+    body = _MORE_FORMS[name]
+    src = f"def f(A, B, x, out):\n    for i in appy.prange(A.shape[0]):\n        {body}\n"
+    fname = f"<row_forms_{name}>"
+    linecache.cache[fname] = (len(src), None, src.splitlines(True), fname)
+    ns = {}
+    exec(compile(src, fname, "exec"), {"np": np, "appy": appy}, ns)
+    rng = np.random.default_rng(5)
+    A, B, x, out = rng.standard_normal((23, 61)), rng.standard_normal((23, 61)), rng.standard_normal(61), np.zeros(23)
+    want = [v.copy() for v in (A, B, x, out)]
+    ns["f"](*want)
+    got = [A, B, x, out]
+    appy.jit(ns["f"])(*got)
+    for g, w in zip(got, want):
+        assert np.allclose(g, w, rtol=1e-9, atol=1e-9)
