@@ -294,7 +294,7 @@ class ExprEmitter:
                     return cast(f"appy::floordiv_float({cast(lc, lt, T.F32)}, {cast(rc, rt, T.F32)})", T.F32, t), t
                 return f"appy::floordiv_float({a}, {b})", t
             if t.kind == "u":
-                return f"({a} / {b})", t
+                return f"appy::div_unsigned<{t.c}>({a}, {b})", t
             return f"appy::floordiv_int<{t.c}>({a}, {b})", t
         if isinstance(op, ast.Mod):
             t = T.promote(lt, rt)
@@ -306,7 +306,7 @@ class ExprEmitter:
                     return cast(f"appy::mod_float({cast(lc, lt, T.F32)}, {cast(rc, rt, T.F32)})", T.F32, t), t
                 return f"appy::mod_float({a}, {b})", t
             if t.kind == "u":
-                return f"({a} % {b})", t
+                return f"appy::mod_unsigned<{t.c}>({a}, {b})", t
             return f"appy::mod_int<{t.c}>({a}, {b})", t
         if isinstance(op, ast.Pow):
             t = T.promote(lt, rt)

@@ -88,8 +88,10 @@ __device__ __forceinline__ i64 at(i64 idx, i64 extent, int site, int* oob) {
 }
 
 // ---- Python arithmetic that differs from C ------------------------------------
+// (integer division by zero gives 0, as NumPy's floor_divide and remainder do)
 template <typename T>
 __device__ __forceinline__ T floordiv_int(T a, T b) {
+    if (b == 0) return 0;
     T q = a / b;
     T r = a % b;
     return ((r != 0) && ((r < 0) != (b < 0))) ? q - 1 : q;
@@ -97,8 +99,19 @@ __device__ __forceinline__ T floordiv_int(T a, T b) {
 
 template <typename T>
 __device__ __forceinline__ T mod_int(T a, T b) {
+    if (b == 0) return 0;
     T r = a % b;
     return ((r != 0) && ((r < 0) != (b < 0))) ? r + b : r;
+}
+
+template <typename T>
+__device__ __forceinline__ T div_unsigned(T a, T b) {
+    return b == 0 ? (T)0 : (T)(a / b);
+}
+
+template <typename T>
+__device__ __forceinline__ T mod_unsigned(T a, T b) {
+    return b == 0 ? (T)0 : (T)(a % b);
 }
 
 // Floating-point `%` and `//` follow NumPy's (and CPython's) divmod: the remainder comes from

@@ -459,7 +459,7 @@ def _random_expression(rng, depth, leaves):
     return f"(-{a})"
 
 
-@pytest.mark.parametrize("seed", list(range(60)) + [230, 246])      # the last two: float `//`, uint8 multiply-add chains
+@pytest.mark.parametrize("seed", list(range(60)) + [230, 246, 1320])      # the last three: float `//`, uint8 multiply-add chains, integer division by zero
 def test_random_expressions_type_and_value_like_numpy(gpu, seed):
     """Random expression trees over arrays of five dtypes, NumPy scalars and Python
     scalars: the kernel must produce the dtype and the values that NumPy's own
