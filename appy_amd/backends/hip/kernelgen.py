@@ -387,7 +387,17 @@ class LoopAnalysis:
         for st in body[:at]:
             if not (isinstance(st, ast.Assign) and isinstance(st.targets[0], ast.Name)):
                 return None
+        if not self._set_up_is_repeatable(body[:at], body[at]):
+            return None
         return body[at]
+
+    def _set_up_is_repeatable(self, pre, loop) -> bool:
+        """The statements in front of a split loop are run by every workgroup that takes a part
+        of the loop, and again by the finishing kernel: they must not read what the loop stores."""
+        stored = {n.targets[0].value.id for n in ast.walk(loop)
+                  if isinstance(n, ast.Assign) and isinstance(n.targets[0], ast.Subscript)
+                  and isinstance(n.targets[0].value, ast.Name)}
+        return not any(isinstance(n, ast.Name) and n.id in stored for st in pre for n in ast.walk(st))
 
     def _find_team_split(self):
         """The one ``simd`` loop of a team nest, if the nest can run in two phases (few,
@@ -407,6 +417,8 @@ class LoopAnalysis:
         for key in loop_ir.reductions_of(loops[0]):
             if not key.isidentifier():
                 return None
+        if not self._set_up_is_repeatable(body[:at], loops[0]):
+            return None
         return loops[0]
 
     def split_needs_finish(self) -> bool:
@@ -1167,6 +1179,24 @@ class KernelBuilder:
             return f"appy::team_reduce<{_OPS[op]}, {W}, {ty.c}>({partial})"
         return f"appy::workgroup_reduce_all<{_OPS[op]}, {self.spec.block}, {ty.c}>({partial}, {T.identity_literal(op, ty)})"
 
+    def _stores_what_others_read(self, loop: ast.For) -> bool:
+        """True if ``loop`` stores to an array that statements outside it load: in a team of
+        several wavefronts those statements run on every wavefront, so the wavefronts must
+        have passed them before any of them starts storing."""
+        stored = {n.targets[0].value.id for n in ast.walk(loop)
+                  if isinstance(n, ast.Assign) and isinstance(n.targets[0], ast.Subscript)
+                  and isinstance(n.targets[0].value, ast.Name)}
+        if not stored:
+            return False
+        # (loads inside other shared-out loops are kept apart by the barriers those loops end in)
+        inside = {id(n) for lp in ast.walk(self.a.outer)
+                  if isinstance(lp, ast.For) and lp is not self.a.outer
+                  and ("simd" in (getattr(lp, "pragma", None) or {}) or (self.a.strip and id(lp) in self.a.strip))
+                  for n in ast.walk(lp)}
+        inside |= {id(n) for n in ast.walk(loop)}
+        return any(isinstance(n, ast.Subscript) and isinstance(n.ctx, ast.Load) and isinstance(n.value, ast.Name)
+                   and n.value.id in stored and id(n) not in inside for n in ast.walk(self.a.outer))
+
     def _leader(self) -> str:
         """Condition under which a team-level statement has its side effect."""
         if self.spec.kind == "strip":
@@ -1289,6 +1319,8 @@ class KernelBuilder:
         outer_locals = set(self.a.assigned) | {self.a.var}
         self.bounds_vary = any(_uses_name(b, n) for b in st.iter.args[:2] for n in outer_locals)
         loads, stores = self._vector_accesses(st.body, var) if V > 1 else ({}, {})
+        if W > 64 and self._stores_what_others_read(st):
+            self.w("__syncthreads();   // every wavefront has read what it needs of the arrays this loop stores to")
         if V > 1 and (loads or stores):
             nv = self.fresh("nv")
             q = self.fresh("q")
@@ -1781,6 +1813,8 @@ class KernelBuilder:
                     if (isinstance(n, ast.Subscript) and isinstance(n.value, ast.Name) and n.value.id in self.a.arrays
                             and _uses_name(n, var) and _uses_name(n, self.a.var)):
                         self.ex.stream_arrays.add(n.value.id)
+        if self._stores_what_others_read(st):
+            self.w("__syncthreads();   // every wavefront has read what it needs of the arrays this loop stores to")
         # lanes past the end of the range skip the loop as a whole (its bounds stay wavefront-uniform,
         # which keeps the unrolled loads of a step in flight together); the barriers are outside
         self.w("if (__active) {")

@@ -586,3 +586,35 @@ def test_rows_without_slices_and_reductions_spelled_as_methods_are_lowered_to_si
     # and the whole nest compiles
     f, _ = compiled(src, A=A, B=A.copy(), x=x, out=out, k=np.zeros(4, np.int64), n=4)
     assert f.analysis.kind == "team"
+
+
+def test_two_phase_shapes_need_set_up_statements_that_can_be_repeated():
+    """Statements in front of a split loop run once per part and again in the finishing kernel;
+    a nest whose set-up reads what the loop stores keeps to one kernel."""
+    A = np.zeros((4, 100000))
+    rows = "#pragma parallel for\nfor i in range(n):\n    f = {first}\n    #pragma simd\n    for j in range(m):\n        C[i, j] = A[i, j] * f\n"
+    f, _ = compiled(rows.format(first="A[i, 0]"), A=A, C=A.copy(), n=4, m=100000)
+    assert f.analysis.team_split is not None
+    f, _ = compiled(rows.format(first="C[i, 0]"), A=A, C=A.copy(), n=4, m=100000)
+    assert f.analysis.team_split is None
+    cols = "#pragma parallel for\nfor j in range(m):\n    f = {first}\n    for i in range(n):\n        C[i, j] = A[i, j] * f\n"
+    f, _ = compiled(cols.format(first="A[0, j]"), A=A, C=A.copy(), n=4, m=100000)
+    assert f.analysis.strip_split is not None
+    f, _ = compiled(cols.format(first="C[0, j]"), A=A, C=A.copy(), n=4, m=100000)
+    assert f.analysis.strip is not None and f.analysis.strip_split is None
+
+
+def test_store_loops_of_multi_wavefront_teams_wait_for_the_set_up_reads():
+    from appy_amd.backends.hip.kernelgen import Spec
+
+    A = np.zeros((100, 256))
+    cols = "#pragma parallel for\nfor j in range(m):\n    f = {first}\n    for i in range(n):\n        C[i, j] = A[i, j] * f\n"
+    f, _ = compiled(cols.format(first="C[0, j]"), A=A, C=A.copy(), n=100, m=256)
+    k = body_of(f.kernel_for(Spec("strip", block=256, vec=1, unroll=8)).src.text)
+    assert k.index("f = C[") < k.index("__syncthreads();   // every wavefront has read") < k.index("C[i * C_stride_0 + j] =")
+    f, _ = compiled(cols.format(first="A[0, j]"), A=A, C=A.copy(), n=100, m=256)
+    assert "every wavefront has read" not in f.kernel_for(Spec("strip", block=256, vec=1, unroll=8)).src.text
+    rows = "#pragma parallel for\nfor i in range(n):\n    f = C[i, 0]\n    #pragma simd\n    for j in range(m):\n        C[i, j] = A[i, j] * f\n"
+    g, _ = compiled(rows, A=A, C=A.copy(), n=100, m=256)
+    assert "every wavefront has read" in g.kernel_for(Spec("team", block=256, vec=2, width=256)).src.text
+    assert "every wavefront has read" not in g.kernel_for(Spec("team", block=256, vec=2, width=64)).src.text
