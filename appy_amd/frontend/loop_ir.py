@@ -233,6 +233,19 @@ def reduction_operand(assign: ast.Assign):
     return a
 
 
+def _inner_parallel_loops_are_simd(tree: ast.Module) -> None:
+    """``#pragma parallel for`` on a loop inside the loop that becomes the kernel promises
+    independent iterations, which is what ``simd`` asks for: the inner loop is spread over
+    the lanes of the team that runs the outer iteration."""
+    outer = outer_loop(tree)
+    for n in ast.walk(outer):
+        if isinstance(n, ast.For) and n is not outer:
+            pragma = getattr(n, "pragma", None)
+            if pragma and "parallel_for" in pragma:
+                del pragma["parallel_for"]
+                pragma["simd"] = True
+
+
 def _as_addition(assign: ast.Assign) -> None:
     """``t = t - e`` becomes ``t = t + (-e)`` (the same value in IEEE and in wrapping
     integer arithmetic), so that a running difference is a ``+`` reduction."""
@@ -419,6 +432,7 @@ def build(loop_source: str) -> ast.Module:
     check_structure(tree)
     tree = _Normalise().visit(tree)
     tree.body, _ = _attach_pragmas(tree.body, None)
+    _inner_parallel_loops_are_simd(tree)
     _hoist_element_reductions(tree)
     _mark_all(tree)
     ast.fix_missing_locations(tree)

@@ -348,3 +348,10 @@ def test_decorated_functions_keep_their_closure():
     assert np.array_equal(out, 2.5 * a + 1.0)
     f(a, out, beta=2.0)
     assert np.array_equal(out, 2.5 * a + 2.0) and f.__name__ == "f"
+
+
+def test_ir_parallel_for_on_an_inner_loop_counts_as_simd():
+    tree = loop_ir.build(
+        "#pragma parallel for\nfor i in range(n):\n    #pragma parallel for\n    for j in range(m):\n        B[i, j] = A[i, j] + 1")
+    outer = loop_ir.outer_loop(tree)
+    assert dict(outer.pragma) == {"parallel_for": True} and dict(outer.body[0].pragma) == {"simd": True}
