@@ -242,6 +242,11 @@ class _LoopOutliner:
         loop = _SimdRanges().visit(copy.deepcopy(loop))
         loop.body = [_InnerPranges().visit(st) for st in loop.body]
         if pragma:
+            if not re.search(r"\bsimd\b", pragma):
+                # inner loops without annotations of their own: those that are provably independent
+                # and walk the contiguous dimension are spread over lanes, as the reference's guide
+                # says of loops whose `simd` was not spelled out (docs/source/legacy.rst:6)
+                auto_simd.vectorise_inner_loops(loop)
             shared = shared_names(pragma)
             if shared:
                 loop = _NameToElement0(shared).visit(copy.deepcopy(loop))
