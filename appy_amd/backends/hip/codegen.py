@@ -1005,10 +1005,15 @@ class Launch:
         return self.kernel.function(self.device)
 
     def launch_only(self):
-        rt.launch(self.function(), self.grid, self.block, self.args, self.stream)
-        if self.second is not None:
+        if self.second is None:
+            rt.launch(self.function(), self.grid, self.block, self.args, self.stream)
+        else:
+            # both kernels share the loop's scratch buffer for this stream: they are queued as a
+            # pair, so that another thread's pair for the same loop cannot come between them
             fin, args, grid, block = self.second
-            rt.launch(fin.function(self.device), grid, block, args, self.stream)
+            with self.loop._lock:
+                rt.launch(self.function(), self.grid, self.block, self.args, self.stream)
+                rt.launch(fin.function(self.device), grid, block, args, self.stream)
         g = self.capture
         if g is not None:
             g.launches += 1
