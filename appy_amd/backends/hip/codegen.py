@@ -598,16 +598,17 @@ class CompiledLoop:
         device and stream, kept for the life of the loop (launches on one stream follow one
         another, so they may share it; it only ever grows)."""
         key = (device, stream)
-        have = self._scratch.get(key)
-        if have is None or have[1] < nbytes:
-            if have is not None:
-                # launches in flight (or recorded in a graph) may still name the smaller buffer:
-                # it is kept, not freed; doubling bounds what is kept to less than the final size
-                self._scratch_retired.append(have[0])
-                nbytes = max(nbytes, 2 * have[1])
-            have = (rt.malloc(nbytes), nbytes)
-            self._scratch[key] = have
-        return have[0]
+        with self._lock:
+            have = self._scratch.get(key)
+            if have is None or have[1] < nbytes:
+                if have is not None:
+                    # launches in flight (or recorded in a graph) may still name the smaller buffer:
+                    # it is kept, not freed; doubling bounds what is kept to less than the final size
+                    self._scratch_retired.append(have[0])
+                    nbytes = max(nbytes, 2 * have[1])
+                have = (rt.malloc(nbytes), nbytes)
+                self._scratch[key] = have
+            return have[0]
 
     def collapse_count(self, n_outer, env) -> int:
         """Trip count of the sequential loop that may be collapsed into the parallel loop,
