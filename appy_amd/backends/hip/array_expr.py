@@ -290,7 +290,6 @@ class _ReduceCalls(ast.NodeTransformer):
     def _derived(self, fn: str, args, node):
         """``np.mean`` / ``var`` / ``std`` / ``any`` / ``all`` / ``count_nonzero`` / ``dot`` of
         1-D array expressions, spelled through sum / max / min reductions."""
-        P = lambda text: ast.parse(text, mode="eval").body      # noqa: E731
         if fn in ("dot", "inner", "vdot"):
             if len(args) != 2:
                 raise RuntimeError(f"np.{fn} takes two 1-D operands here: {ast.unparse(node)}")

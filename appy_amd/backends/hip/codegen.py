@@ -33,7 +33,7 @@ from . import dtypes as T
 from . import runtime as rt
 from ... import graphs, residency
 from .exprs import ArrayParam, ScalarParam
-from .kernelgen import KernelBuilder, KernelSource, LoopAnalysis, Spec, Unsupported
+from .kernelgen import KernelBuilder, KernelSource, LoopAnalysis, Spec, Unsupported  # noqa: F401 - Unsupported is part of this module's interface
 
 ARCH = "gfx950"
 _HEADER_PATH = os.path.join(os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__)))), "csrc", "appy_device.h")

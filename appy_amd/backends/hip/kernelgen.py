@@ -2125,7 +2125,7 @@ class KernelBuilder:
 
     def build(self, header: str) -> KernelSource:
         # names of shapes produced by array-statement lowering act as scalars
-        for it in range(8):
+        for _pass in range(8):
             self.dirty = False
             self._emit_body()
             if not self.dirty:
