@@ -113,6 +113,27 @@ class Runner:
         }
 
 
+def _blas_threads():
+    """Threads NumPy's BLAS may use (only `A @ x` of the per-kernel CPU figures is multi-threaded)."""
+    try:
+        from threadpoolctl import threadpool_info
+
+        return max([p.get("num_threads", 1) for p in threadpool_info() if p.get("user_api") == "blas"] or [1])
+    except Exception:
+        return int(os.environ.get("OMP_NUM_THREADS", "0")) or None
+
+
+def _cpu_model():
+    try:
+        with open("/proc/cpuinfo") as fh:
+            for line in fh:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return None
+
+
 def cpu_time(fn, reps=3):
     """Best wall time of ``fn`` over ``reps`` runs, seconds."""
     best = 1e30
@@ -201,6 +222,7 @@ def main():
             "sample": f"oracle A.sum(dtype=float64) over all N={n} float32, best of 3 ({best * 1e3:.1f} ms); "
                       f"literal interpreter loop on the first {m} elements: {lit:.0f} ns/element",
             "host_cpus": os.cpu_count(), "affinity": len(os.sched_getaffinity(0)),
+            "blas_threads": _blas_threads(), "cpu_model": _cpu_model(),
         }
         log("cpu_baseline", cpu_baseline)
 
