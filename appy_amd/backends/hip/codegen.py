@@ -610,6 +610,22 @@ class CompiledLoop:
                 self._scratch[key] = have
             return have[0]
 
+    def release(self):
+        """Give back the device memory this loop holds (scratch buffers of two-phase launches),
+        once the launches that use it have finished."""
+        with self._lock:
+            held, self._scratch, self._scratch_retired = (
+                [(k, p) for k, (p, _n) in self._scratch.items()] + [(None, p) for p in self._scratch_retired], {}, [])
+        try:
+            for key, _ptr in held:
+                if key is not None:
+                    _ensure_device(key[0])
+                    rt.sync(key[1])
+            for _key, ptr in held:
+                rt.free(ptr)
+        except Exception:           # the runtime may be shutting down
+            pass
+
     def collapse_count(self, n_outer, env) -> int:
         """Trip count of the sequential loop that may be collapsed into the parallel loop,
         when that is possible and worth it for ``n_outer`` parallel iterations; else 0."""
@@ -1129,6 +1145,9 @@ def codegen(loop_source, loop_name, val_map, options):
         hit = None if fresh else code_cache.get(key)
         if hit is not None:
             return hit
+        stale = code_cache.get(key)
+        if stale is not None:
+            stale[0].release()          # `clear_cache`: the loop object of the previous call goes away
         f = CompiledLoop(loop_source, loop_name, val_map, options)
         if options.get("dry_run"):
             f.kernels[f.default_spec].code      # nothing will be launched: compile now, so that errors surface

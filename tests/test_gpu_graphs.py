@@ -172,3 +172,37 @@ def test_two_phase_launches_are_captured_with_both_kernels(gpu):
         g.launch()
         g.synchronize()
         assert torch.allclose(out, A.sum(dim=0)), replay
+
+
+def test_loops_regenerated_on_every_call_give_their_scratch_memory_back(gpu):
+    """`clear_cache=True` builds a new loop object per call; the scratch buffer of the one it
+    replaces returns to the pool."""
+    import ctypes
+
+    import torch
+
+    from appy_amd.backends.hip import runtime as rt
+
+    fresh = appy.jit(_plain_column_sums, clear_cache=True)
+    A = torch.rand(200_000, 8, device="cuda", dtype=torch.float64)
+    out = torch.zeros(8, device="cuda", dtype=torch.float64)
+    fresh(A, out)
+    torch.cuda.synchronize()
+    used, cached = ctypes.c_uint64(), ctypes.c_uint64()
+    rt.check(rt.lib().appy_hip_pool_stats(ctypes.byref(used), ctypes.byref(cached)))
+    held = used.value
+    for _ in range(3):
+        fresh(A, out)
+        assert torch.allclose(out, A.sum(dim=0))
+    torch.cuda.synchronize()
+    rt.check(rt.lib().appy_hip_pool_stats(ctypes.byref(used), ctypes.byref(cached)))
+    assert used.value == held
+
+
+def _plain_column_sums(A, out):
+    #pragma parallel for
+    for j in range(A.shape[1]):
+        s = 0.0
+        for i in range(A.shape[0]):
+            s += A[i, j]
+        out[j] = s
