@@ -12,6 +12,7 @@ from __future__ import annotations
 import ast
 import builtins as _builtins
 import inspect
+import os
 import sys
 import textwrap
 
@@ -54,6 +55,9 @@ def _reduction_result(buffer, start):
 def set_default_options(options):
     for key, val in _DEFAULT_OPTIONS:
         options.setdefault(key, val)
+    if os.environ.get("APPY_HIP_CHECK_BOUNDS") == "1":
+        # a whole program under device-side index checks, without touching its decorators
+        options.setdefault("check_bounds", True)
 
 
 def rewrite_loops(fn, **options):
