@@ -806,6 +806,20 @@ class Launch:
         self.staged_twice = {}   # (address, bytes, strides, dtype) of a staged host array -> (index in temps, uploaded?)
         self.aliases = []        # (name, dptr, bytes, stored) of host arrays that share the copy of another name
         self.keepalive = []
+        try:
+            self._stage(vals, arrays)
+        except BaseException:
+            # nothing is launched: staging buffers taken so far go back to the pool
+            for dptr, *_ in self.temps:
+                rt.free(dptr)
+            self.temps = []
+            if self.oob:
+                rt.free(self.oob)
+                self.oob = 0
+            raise
+
+    def _stage(self, vals, arrays):
+        loop, a, env, lo, hi = self.loop, self.loop.analysis, self.env, self.lo, self.hi
         # -- bounds of accesses indexed by the parallel loop variable (host check, before any device work)
         for name, dim, off in a.bound_checks:
             ext = arrays[name].shape[dim]
