@@ -154,6 +154,9 @@ def main():
     import numpy as np
     import torch
 
+    import __graft_entry__
+
+    __graft_entry__.ensure_built()      # loads what is built; builds only if nothing is
     from appy_amd.backends.hip import codegen as cg
     from appy_amd.backends.hip import runtime as rt
     from appy_amd.backends.hip import selfcheck

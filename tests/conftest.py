@@ -12,6 +12,13 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
 
 
+def pytest_sessionstart(session):
+    """The tests load the library that is built; it is built here only if there is none."""
+    import __graft_entry__
+
+    __graft_entry__.ensure_built()
+
+
 def _gpu_count():
     try:
         from appy_amd.backends.hip import runtime as rt
