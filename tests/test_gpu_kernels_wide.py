@@ -989,3 +989,75 @@ def test_column_updates_written_without_simd(gpu, shape):
     assert loop.analysis.strip is not None
     assert spec.kind == ("flat" if shape[0] < 64 else "strip")
     assert spec.phase == (1 if shape[0] >= 100_000 else 0) and loop.last_launch.second is None
+
+
+@appy.jit
+def shape_rowstats(A, y, z):
+    #pragma parallel for
+    for i in range(A.shape[0]):
+        s = 0.0
+        m = -1e30
+        #pragma simd
+        for j in range(A.shape[1]):
+            s += A[i, j]
+            m = max(m, A[i, j])
+        y[i] = s
+        z[i] = m
+
+
+@appy.jit
+def shape_colstats(A, y, z):
+    #pragma parallel for
+    for j in range(A.shape[1]):
+        s = 0.0
+        m = -1e30
+        for i in range(A.shape[0]):
+            s += A[i, j]
+            m = max(m, A[i, j])
+        y[j] = s
+        z[j] = m
+
+
+@appy.jit
+def shape_rowscale(A, f, C):
+    #pragma parallel for
+    for i in range(A.shape[0]):
+        #pragma simd
+        for j in range(A.shape[1]):
+            C[i, j] = A[i, j] * f[i] + 1.0
+
+
+@appy.jit
+def shape_colscale(A, f, C):
+    #pragma parallel for
+    for j in range(A.shape[1]):
+        for i in range(A.shape[0]):
+            C[i, j] = A[i, j] * f[j] + 1.0
+
+
+_EDGE_SHAPES = [(1, 200_000), (2, 65_537), (127, 8193), (128, 8192), (129, 4095), (1023, 1025), (4096, 257),
+                (8193, 63), (32_769, 64), (65_536, 3), (200_000, 1), (63, 32_768), (64, 32_767), (3, 3)]
+
+
+@pytest.mark.parametrize("shape", _EDGE_SHAPES)
+def test_row_and_column_loops_over_shapes_at_the_edges_of_the_launch_heuristics(gpu, shape):
+    """The same four loops (row and column reductions, row and column updates) over matrices of
+    every aspect ratio, with extents at and next to the thresholds where the launch picks another
+    kernel shape (teams of a wavefront or a workgroup, strips, one or two phases, flat)."""
+    n, m = shape
+    for dt in (np.float32, np.float64):
+        rng = np.random.default_rng(n * 31 + m)
+        A = rng.standard_normal(shape).astype(dt)
+        tol = dict(rtol=1e-3, atol=1e-2) if dt == np.float32 else dict(rtol=1e-9, atol=1e-9)
+        y, z = np.zeros(n, dt), np.zeros(n, dt)
+        shape_rowstats(A, y, z)
+        assert np.allclose(y, A.sum(axis=1, dtype=np.float64), **tol) and np.array_equal(z, A.max(axis=1))
+        y, z = np.zeros(m, dt), np.zeros(m, dt)
+        shape_colstats(A, y, z)
+        assert np.allclose(y, A.sum(axis=0, dtype=np.float64), **tol) and np.array_equal(z, A.max(axis=0))
+        f, C = rng.standard_normal(n).astype(dt), np.zeros_like(A)
+        shape_rowscale(A, f, C)
+        assert np.array_equal(C, A * f[:, None] + dt(1.0))
+        f, C = rng.standard_normal(m).astype(dt), np.zeros_like(A)
+        shape_colscale(A, f, C)
+        assert np.array_equal(C, A * f[None, :] + dt(1.0))
