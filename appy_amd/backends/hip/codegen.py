@@ -78,6 +78,8 @@ REPLAY_CACHE_ENTRIES = 2048
 # a parallel loop with fewer iterations than this, whose body is one independent sequential loop,
 # runs the two loops as one iteration space (one wavefront per iteration would not fill 256 CUs)
 COLLAPSE_BELOW_ROWS = 8192
+# vector steps of a row that a lane keeps in registers between the simd loops of an iteration
+ROW_CACHE_STEPS = 16
 
 
 def device_header() -> str:
@@ -288,6 +290,11 @@ class CompiledLoop:
         self._hi_code = compile(ast.Expression(body=ast.fix_missing_locations(_copy(a.hi_node))), "<hi>", "eval")
         self._affine_check_codes = [(name, dim, text, compile(text, "<subscript>", "eval"))
                                     for name, dim, text in a.affine_checks]
+        self._row_cache_codes = None
+        if a.row_cache is not None:
+            self._row_cache_codes = [
+                tuple(compile(ast.Expression(body=ast.fix_missing_locations(_copy(b))), "<row bound>", "eval") for b in pair)
+                for pair in a.row_cache[2]]
         self._collapse_codes = None
         if a.collapse is not None:
             self._collapse_codes = tuple(
@@ -570,7 +577,30 @@ class CompiledLoop:
                 # added elementwise: 3.4 ms with one workgroup per row), partial results of
                 # reductions meet in a second, small kernel
                 return Spec("team", block=block, vec=v, width=w, restrict=restrict, stream_loads=stream, phase=1)
-        return Spec("team", block=block, vec=v, width=w, restrict=restrict, stream_loads=stream, collapse=bool(nj))
+        steps = 0
+        if self._row_cache_codes is not None and not nj and v > 1 and not self.options.get("check_bounds"):
+            # the rows that several simd loops of an iteration read stay in registers when every
+            # lane takes a whole, small number of vector steps of them
+            try:
+                spans = {(int(eval(lo, _HOST_EVAL_GLOBALS, env)), int(eval(hi, _HOST_EVAL_GLOBALS, env)))
+                         for lo, hi in self._row_cache_codes}
+            except Exception:
+                spans = set()
+            ext = 0
+            if len(spans) == 1:
+                (lo_, hi_), = spans
+                ext = hi_ - lo_
+            shapes = [(w, block)]
+            if w == 64 and self.analysis.multi_wave_ok:
+                # rows too long for one wavefront's registers: a workgroup takes each row
+                shapes += [(256, 256), (1024, 1024)]
+            for cw, cb in shapes:
+                most = ROW_CACHE_STEPS if cb <= 256 else ROW_CACHE_STEPS // 2     # registers per lane halve at 1024 lanes
+                if ext > 0 and ext % (cw * v) == 0 and ext // (cw * v) <= most:
+                    steps, w, block = ext // (cw * v), cw, cb
+                    break
+        return Spec("team", block=block, vec=v, width=w, restrict=restrict, stream_loads=stream, collapse=bool(nj),
+                    row_steps=steps)
 
     def team_parts(self, spec: Spec, n_outer: int, env, arrays) -> int:
         """Workgroups per row of a two-phase team launch: two workgroups per CU in all, each

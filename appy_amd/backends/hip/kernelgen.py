@@ -71,6 +71,8 @@ class Spec:
     phase: int = 0               # strips and workgroup teams: 1 = the shared-out loop over one part of its range,
                                  # partial results to a scratch buffer (the grid holds several workgroups per strip
                                  # or row), 2 = the rest of the body on those partial results; 0 = one kernel
+    row_steps: int = 0           # team only: every lane takes exactly this many vector steps of the rows that several
+                                 # simd loops of one iteration read; those rows stay in registers between the loops
     collapse: bool = False       # team only: the parallel loop and the sequential loop that is its whole body
                                  # run as one iteration space (the analysis has shown the inner iterations independent)
 
@@ -94,6 +96,9 @@ class Spec:
                 self.kind == "strip" or (self.kind == "team" and self.width in (64, self.block)
                                          and not self.extent and not self.lds_tile and not self.collapse))):
             raise ValueError("only strip kernels and teams of a whole wavefront or workgroup run in two phases")
+        if self.row_steps and (self.kind != "team" or self.phase or self.extent or self.lds_tile or self.vec < 2
+                               or not 1 <= self.row_steps <= 16 or self.checked):
+            raise ValueError("rows are kept in registers by plain team kernels only, for 1 to 16 vector steps per lane")
         if self.collapse and (self.kind != "team" or self.lds_tile):
             raise ValueError("only team kernels without an LDS tile collapse their two outer loops")
         if self.extent < 0 or self.lds_tile < 0 or self.lds_tile % 4 or self.lds_tile > 16384:
@@ -103,7 +108,7 @@ class Spec:
         return (f"{self.kind}_b{self.block}_v{self.vec}_u{self.unroll}_w{self.width}"
                 f"{'_r' if self.restrict else ''}{'_nt' if self.stream_loads else ''}"
                 f"{'_e' + str(self.extent) if self.extent else ''}{'_nts' if self.stream_stores else ''}"
-                f"{'_lds' + str(self.lds_tile) if self.lds_tile else ''}{'' if self.hoist_guarded else '_g'}{'_chk' if self.checked else ''}{'_c2' if self.collapse else ''}{'_p' + str(self.phase) if self.phase else ''}")
+                f"{'_lds' + str(self.lds_tile) if self.lds_tile else ''}{'' if self.hoist_guarded else '_g'}{'_chk' if self.checked else ''}{'_c2' if self.collapse else ''}{'_p' + str(self.phase) if self.phase else ''}{'_rc' + str(self.row_steps) if self.row_steps else ''}")
 
 
 @dataclass
@@ -461,6 +466,40 @@ class LoopAnalysis:
         visit(self.outer.body, [])
         return out
 
+    def _find_row_cache(self):
+        """``(loops, arrays, bounds)`` when an iteration of the parallel loop walks the same rows
+        in several ``simd`` loops (soft-max: maximum, sum, quotient; layer norm: mean, variance,
+        result): simd loops directly in the body whose bounds do not depend on the iteration
+        (``bounds`` lists the distinct ones), and arrays that two or more of them load and none of the nest stores.  With
+        few enough vector steps per lane those rows can stay in registers between the loops."""
+        if self.kind != "team":
+            return None
+        loops = [st for st in self.outer.body
+                 if isinstance(st, ast.For) and "simd" in (getattr(st, "pragma", None) or {}) and isinstance(st.target, ast.Name)]
+        if len(loops) < 2:
+            return None
+        blocked = set(self.assigned) | set(self.loop_vars) | {self.var} | set(self.arrays)
+        loops = [lp for lp in loops
+                 if not any(isinstance(n, ast.Name) and n.id in blocked for b in lp.iter.args[:2] for n in ast.walk(b))]
+        if len(loops) < 2:
+            return None
+        # bounds that read differently (the row length of one array, then of another) may still
+        # be equal: the launch evaluates them all and keeps rows in registers only if they are
+        bounds = {}
+        for lp in loops:
+            lo, hi = lp.iter.args[:2]
+            bounds.setdefault((ast.unparse(lo), ast.unparse(hi)), (lo, hi))
+        seen, arrays = {}, set()
+        for lp in loops:
+            for n in ast.walk(lp):
+                if (isinstance(n, ast.Subscript) and isinstance(n.ctx, ast.Load) and isinstance(n.value, ast.Name)
+                        and n.value.id in self.arrays and n.value.id not in self.stored):
+                    if seen.setdefault(n.value.id, id(lp)) != id(lp):
+                        arrays.add(n.value.id)
+        if not arrays:
+            return None
+        return {id(lp) for lp in loops}, arrays, list(bounds.values())
+
     def _find_collapse(self):
         """The sequential loop ``for j in range(lo, hi)`` that is the whole body of the
         parallel loop, if its iterations are provably independent - then the pairs (i, j)
@@ -684,6 +723,7 @@ class LoopAnalysis:
         self.strip_split = self._find_strip_split()
         self.team_split = self._find_team_split()
         self.reread = self._find_reread()
+        self.row_cache = self._find_row_cache()
 
         # reductions of the parallel loop: constant-subscript elements of arrays
         self.outer_reductions = []
@@ -1226,7 +1266,8 @@ class KernelBuilder:
             return False        # the iteration comes back to this data (softmax: max, sum, write): keep it cached
         return self.bounds_vary or any(_uses_name(e, self.a.var) for e in _elts(sub))
 
-    def vector_body(self, body, var: str, base_code: str, V: int, loads, stores, declare_locals=False, extra=None):
+    def vector_body(self, body, var: str, base_code: str, V: int, loads, stores, declare_locals=False, extra=None,
+                    cached=None):
         """Emit V consecutive iterations starting at ``base_code``: vector
         loads first, the V scalar bodies, vector stores last."""
         regs = {}
@@ -1235,6 +1276,13 @@ class KernelBuilder:
             r = self.fresh(f"ld_{arr.name}_")
             regs[key] = r
             ld = "vload_stream" if self._streamed(sub) else "vload"
+            slot = (cached or {}).get(key)
+            if slot is not None:
+                name, fill = slot
+                if fill:
+                    self.w(f"{name}[__k] = appy::{ld}<{arr.elem_c}, {V}>({self._addr(arr, sub, var, base_code)});")
+                self.w(f"const appy::vec<{arr.elem_c}, {V}>::type {r} = {name}[__k];")
+                continue
             self.w(f"const appy::vec<{arr.elem_c}, {V}>::type {r} = "
                    f"appy::{ld}<{arr.elem_c}, {V}>({self._addr(arr, sub, var, base_code)});")
         sregs = {}
@@ -1327,7 +1375,26 @@ class KernelBuilder:
         loads, stores = self._vector_accesses(st.body, var) if V > 1 else ({}, {})
         if W > 64 and self._stores_what_others_read(st):
             self.w("__syncthreads();   // every wavefront has read what it needs of the arrays this loop stores to")
-        if V > 1 and (loads or stores):
+        in_registers = (self.spec.row_steps and self.a.row_cache is not None and id(st) in self.a.row_cache[0]
+                        and V > 1 and (loads or stores))
+        if in_registers:
+            # the host has checked that the loop is exactly row_steps x W x V long: no tail; rows
+            # that other loops of the iteration read as well are loaded once and kept
+            cached = {}
+            for key, (arr, sub) in loads.items():
+                rk = self._row_key(sub, var)
+                if rk in self.rc_slots:
+                    cached[key] = (self.rc_slots[rk], rk not in self.rc_filled)
+            base = self.fresh("j")
+            self.w("#pragma unroll")
+            self.w(f"for (int __k = 0; __k < {self.spec.row_steps}; ++__k) {{")
+            self.ind += 1
+            self.w(f"const appy::i64 {base} = {lo_v} + ((appy::i64)__lane + (appy::i64)__k * {W}) * {V};")
+            self.vector_body(st.body, var, base, V, loads, stores, cached=cached)
+            self.ind -= 1
+            self.w("}")
+            self.rc_filled.update(self._row_key(sub, var) for key, (arr, sub) in loads.items() if key in cached)
+        elif V > 1 and (loads or stores):
             nv = self.fresh("nv")
             q = self.fresh("q")
             self.w(f"const appy::i64 {nv} = ({hi_v} - {lo_v}) / {V};")
@@ -1342,11 +1409,12 @@ class KernelBuilder:
             start = f"{lo_v} + {nv} * {V} + __lane"
         else:
             start = f"{lo_v} + __lane"
-        self.w(f"for (appy::i64 {cname(var)} = {start}; {cname(var)} < {hi_v}; {cname(var)} += {W}) {{")
-        self.ind += 1
-        self.iteration_body(st.body)
-        self.ind -= 1
-        self.w("}")
+        if not in_registers:
+            self.w(f"for (appy::i64 {cname(var)} = {start}; {cname(var)} < {hi_v}; {cname(var)} += {W}) {{")
+            self.ind += 1
+            self.iteration_body(st.body)
+            self.ind -= 1
+            self.w("}")
         self.mode = saved_mode
         self.seq_depth = saved_depth
         self.bounds_vary = saved_vary
@@ -1626,9 +1694,35 @@ class KernelBuilder:
         else:
             self.w(f"const appy::i64 {cname(self.a.var)} = {idx_code};")
             self._declare_locals()
+            self._declare_row_cache(self.a.outer.body)
             self.iteration_body(self.a.outer.body)
         self.ind -= 1
         self.w("}")
+
+    def _row_key(self, sub: ast.Subscript, var: str) -> str:
+        """A subscript with the loop variable blanked out: the same element of the row,
+        whatever the loop that touches it calls its variable."""
+        node = ast.parse(ast.unparse(sub), mode="eval").body
+        for n in ast.walk(node):
+            if isinstance(n, ast.Name) and n.id == var:
+                n.id = "__step"
+        return ast.unparse(node)
+
+    def _declare_row_cache(self, body):
+        self.rc_slots, self.rc_filled = {}, set()
+        if not self.spec.row_steps or self.a.row_cache is None:
+            return
+        loops, arrays, _bounds = self.a.row_cache
+        V = self.spec.vec
+        for st in body:
+            if isinstance(st, ast.For) and id(st) in loops:
+                loads, _stores = self._vector_accesses(st.body, st.target.id)
+                for _key, (arr, sub) in loads.items():
+                    rk = self._row_key(sub, st.target.id)
+                    if arr.name in arrays and rk not in self.rc_slots:
+                        slot = f"__rc{len(self.rc_slots)}"
+                        self.rc_slots[rk] = slot
+                        self.w(f"appy::vec<{arr.elem_c}, {V}>::type {slot}[{self.spec.row_steps}];   // {ast.unparse(sub)}")
 
     def _body_flat(self):
         s = self.spec
@@ -2119,6 +2213,7 @@ class KernelBuilder:
         self.store_subst = {}
         self.partials = {}
         self.lds_plan = None
+        self.rc_slots, self.rc_filled = {}, set()
         for r in self.a.outer_reductions:
             self.w(f"{r.ty.c} {r.acc} = {self._outer_identity(r)};")
         if self.spec.kind == "flat":

@@ -618,3 +618,35 @@ def test_store_loops_of_multi_wavefront_teams_wait_for_the_set_up_reads():
     g, _ = compiled(rows, A=A, C=A.copy(), n=100, m=256)
     assert "every wavefront has read" in g.kernel_for(Spec("team", block=256, vec=2, width=256)).src.text
     assert "every wavefront has read" not in g.kernel_for(Spec("team", block=256, vec=2, width=64)).src.text
+
+
+def test_rows_that_several_simd_loops_read_stay_in_registers():
+    """Soft-max and layer-norm nests: when a row is a whole, small number of vector steps per
+    lane, the first simd loop loads it into registers and the later ones read it from there."""
+    x = np.zeros((64, 1024), np.float32)
+    g = np.zeros(1024, np.float32)
+    src = ("#pragma parallel for\nfor i in range(n):\n    s = 0.0\n    #pragma simd\n    for j in range(d):\n        s += x[i, j]\n"
+           "    mu = s / d\n    v = 0.0\n    #pragma simd\n    for j in range(d):\n        v += (x[i, j] - mu) * (x[i, j] - mu)\n"
+           "    r = 1.0 / np.sqrt(v / d + 1e-5)\n    #pragma simd\n    for k in range(x_shape_1):\n"
+           "        out[i, k] = (x[i, k] - mu) * r * g[k]\n")
+    env = dict(n=64, d=1024, x_shape_1=1024)
+    f, _ = compiled(src, x=x, g=g, out=x.copy(), **env)
+    assert f.analysis.row_cache is not None and f.analysis.row_cache[1] == {"x"}
+    assert len(f.analysis.row_cache[2]) == 2            # two spellings of the bounds, compared at the launch
+    spec = f.choose_spec(64, dict(env), dict(x=x, g=g, out=x))
+    assert spec.kind == "team" and spec.width == 64 and spec.row_steps == 4 and spec.tag().endswith("_rc4")
+    k = body_of(f.kernel_for(spec).src.text)
+    assert k.count("appy::vload<float, 4>(x +") == 1 and k.count("__rc0[__k] = ") == 1
+    assert k.count(" = __rc0[__k];") == 3 and "appy::vload<float, 4>(g +" in k
+    assert "for (int __k = 0; __k < 4; ++__k)" in k
+    # a row that is not a whole number of steps, or too many of them: the loops as before
+    assert f.choose_spec(64, dict(env, d=1000, x_shape_1=1000), dict(x=x, g=g, out=x)).row_steps == 0
+    assert f.choose_spec(64, dict(env, d=1024, x_shape_1=512), dict(x=x, g=g, out=x)).row_steps == 0
+    # rows too long for a wavefront's registers go to a workgroup each
+    long = f.choose_spec(4096, dict(env, n=4096, d=8192, x_shape_1=8192), dict(x=np.zeros((4096, 8192), np.float32), g=g, out=x))
+    assert long.row_steps == 8 and long.width == long.block == 256
+    # a row that the nest stores to is read from memory every time
+    upd = ("#pragma parallel for\nfor i in range(n):\n    s = 0.0\n    #pragma simd\n    for j in range(d):\n        s += x[i, j]\n"
+           "    #pragma simd\n    for j in range(d):\n        x[i, j] = x[i, j] / s\n")
+    h, _ = compiled(upd, x=x, n=64, d=1024)
+    assert h.analysis.row_cache is None

@@ -1061,3 +1061,71 @@ def test_row_and_column_loops_over_shapes_at_the_edges_of_the_launch_heuristics(
         f, C = rng.standard_normal(m).astype(dt), np.zeros_like(A)
         shape_colscale(A, f, C)
         assert np.array_equal(C, A * f[None, :] + dt(1.0))
+
+
+# rows that several simd loops of an iteration read (layer norm, RMS norm, soft-max over 2-D
+# rows): kept in registers when a row is a whole, small number of vector steps per lane, read
+# again from memory otherwise - both against NumPy in float64
+@appy.jit
+def layer_norm_rows(x, g, b, out, eps):
+    #pragma parallel for
+    for i in range(x.shape[0]):
+        s = 0.0
+        #pragma simd
+        for j in range(x.shape[1]):
+            s += x[i, j]
+        mu = s / x.shape[1]
+        v = 0.0
+        #pragma simd
+        for j in range(x.shape[1]):
+            v += (x[i, j] - mu) * (x[i, j] - mu)
+        r = 1.0 / np.sqrt(v / x.shape[1] + eps)
+        #pragma simd
+        for j in range(x.shape[1]):
+            out[i, j] = (x[i, j] - mu) * r * g[j] + b[j]
+
+
+@appy.jit
+def rms_norm_rows(x, g, out, eps):
+    for i in appy.prange(x.shape[0]):
+        r = 1.0 / np.sqrt(np.mean(x[i] * x[i]) + eps)
+        out[i] = x[i] * r * g
+
+
+@appy.jit
+def softmax_rows(x, out):
+    for i in appy.prange(x.shape[0]):
+        m = np.max(x[i])
+        out[i] = np.exp(x[i] - m) / np.sum(np.exp(x[i] - m))
+
+
+@pytest.mark.parametrize("n,d", [(300, 512), (1000, 1024), (257, 4096), (600, 8192), (3, 32768), (40, 16384),
+                                 (300, 1000), (33, 4100), (5000, 256), (7, 1024)])
+def test_rows_read_by_several_simd_loops(gpu, n, d):
+    from appy_amd.backends.hip import codegen as cg
+
+    rng = np.random.default_rng(n * 7 + d)
+    x = (rng.standard_normal((n, d)) * 3 + 1).astype(np.float32)
+    g, b = rng.random(d, dtype=np.float32) + 0.5, rng.random(d, dtype=np.float32)
+    x64 = x.astype(np.float64)
+    mu, var = x64.mean(axis=1, keepdims=True), x64.var(axis=1, keepdims=True)
+    out = np.zeros_like(x)
+    layer_norm_rows(x, g, b, out, 1e-5)
+    np.testing.assert_allclose(out, (x64 - mu) / np.sqrt(var + 1e-5) * g + b, rtol=2e-4, atol=2e-4)
+    loop = next(v[0] for k, v in cg.code_cache.items() if k[-1] == "layer_norm_rows")
+    spec = loop.last_launch.spec
+    if (n, d) in ((300, 512), (1000, 1024), (257, 4096), (600, 8192), (5000, 256)):
+        assert spec.row_steps == d // (spec.width * spec.vec) > 0, spec.tag()
+    if d in (1000, 4100):
+        assert spec.row_steps == 0, spec.tag()
+    out = np.zeros_like(x)
+    rms_norm_rows(x, g, out, 1e-5)
+    np.testing.assert_allclose(out, x64 / np.sqrt((x64 * x64).mean(axis=1, keepdims=True) + 1e-5) * g, rtol=2e-4, atol=2e-4)
+    out = np.zeros_like(x)
+    softmax_rows(x, out)
+    e = np.exp(x64 - x64.max(axis=1, keepdims=True))
+    np.testing.assert_allclose(out, e / e.sum(axis=1, keepdims=True), rtol=2e-4, atol=1e-7)
+    # the result written over the input: every lane has read its part of the row before it stores
+    y = x.copy()
+    layer_norm_rows(y, g, b, y, 1e-5)
+    np.testing.assert_allclose(y, (x64 - mu) / np.sqrt(var + 1e-5) * g + b, rtol=2e-4, atol=2e-4)
