@@ -578,7 +578,8 @@ class CompiledLoop:
                 # reductions meet in a second, small kernel
                 return Spec("team", block=block, vec=v, width=w, restrict=restrict, stream_loads=stream, phase=1)
         steps = 0
-        if self._row_cache_codes is not None and not nj and v > 1 and not self.options.get("check_bounds"):
+        if (self._row_cache_codes is not None and bool(nj) == (self.analysis.collapse is not None) and v > 1
+                and not self.options.get("check_bounds")):
             # the rows that several simd loops of an iteration read stay in registers when every
             # lane takes a whole, small number of vector steps of them
             try:

@@ -474,7 +474,10 @@ class LoopAnalysis:
         few enough vector steps per lane those rows can stay in registers between the loops."""
         if self.kind != "team":
             return None
-        loops = [st for st in self.outer.body
+        # (in a nest whose `for j` can be collapsed into the parallel loop, the loops of that body:
+        #  they share a row only when the pairs (i, j) are the iterations)
+        body = self.outer.body if self.collapse is None else self.collapse.body
+        loops = [st for st in body
                  if isinstance(st, ast.For) and "simd" in (getattr(st, "pragma", None) or {}) and isinstance(st.target, ast.Name)]
         if len(loops) < 2:
             return None
@@ -1690,6 +1693,7 @@ class KernelBuilder:
             self.w(f"const appy::i64 {cname(inner.target.id)} = __jlo + ({idx_code}) % __nj;")
             self.ex.locals[inner.target.id] = T.WEAK_INT
             self._declare_locals()
+            self._declare_row_cache(inner.body)
             self.iteration_body(inner.body)
         else:
             self.w(f"const appy::i64 {cname(self.a.var)} = {idx_code};")
@@ -1712,6 +1716,8 @@ class KernelBuilder:
         self.rc_slots, self.rc_filled = {}, set()
         if not self.spec.row_steps or self.a.row_cache is None:
             return
+        if bool(self.spec.collapse) != (self.a.collapse is not None):
+            return      # the loops sit under a sequential loop here: nothing outlives one pass of it
         loops, arrays, _bounds = self.a.row_cache
         V = self.spec.vec
         for st in body:

@@ -1129,3 +1129,30 @@ def test_rows_read_by_several_simd_loops(gpu, n, d):
     y = x.copy()
     layer_norm_rows(y, g, b, y, 1e-5)
     np.testing.assert_allclose(y, (x64 - mu) / np.sqrt(var + 1e-5) * g + b, rtol=2e-4, atol=2e-4)
+
+
+@appy.jit
+def softmax_planes(x, out):
+    #pragma parallel for
+    for i in range(x.shape[0]):
+        for j in range(x.shape[1]):
+            m = np.max(x[i, j, :])
+            s = np.sum(np.exp(x[i, j, :] - m))
+            out[i, j, :] = np.exp(x[i, j, :] - m) / s
+
+
+def test_collapsed_nests_keep_rows_in_registers_too(gpu):
+    """`parallel i / for j / three simd loops over x[i, j, :]`: the pairs (i, j) are the
+    iterations, and each keeps its row in registers when the row length allows."""
+    from appy_amd.backends.hip import codegen as cg
+
+    rng = np.random.default_rng(77)
+    for shape in ((6, 50, 512), (3, 7, 2048), (5, 9, 500)):
+        x = (rng.standard_normal(shape) * 4).astype(np.float32)
+        out = np.zeros_like(x)
+        softmax_planes(x, out)
+        x64 = x.astype(np.float64)
+        e = np.exp(x64 - x64.max(axis=-1, keepdims=True))
+        np.testing.assert_allclose(out, e / e.sum(axis=-1, keepdims=True), rtol=2e-4, atol=1e-7)
+        spec = next(v[0] for k, v in cg.code_cache.items() if k[-1] == "softmax_planes").last_launch.spec
+        assert spec.collapse and bool(spec.row_steps) == (shape[2] % 512 == 0), spec.tag()
