@@ -1425,6 +1425,11 @@ class KernelBuilder:
                           for b in st.body for n in ast.walk(b)):
             # a team of several wavefronts: what one of them stored is read by the others only after this
             self.w("__syncthreads();")
+        elif 1 < W <= 64 and any(isinstance(n, ast.Subscript) and isinstance(n.value, ast.Name) and n.value.id in self.a.stored
+                                 for b in st.body for n in ast.walk(b)):
+            # lanes of one wavefront: the loop touches an array that the nest stores to, and another
+            # lane may touch the same elements in a later loop (slices that overlap, shifted reads)
+            self.w("appy::wave_fence();")
         for r, (name, op) in enumerate(reds.items()):
             p, ty = self.partials[name]
             vty = self.ex.locals.get(name, ty)
@@ -1568,6 +1573,8 @@ class KernelBuilder:
         for t in range(nv):
             guard = "" if full[t] else f"if ({bases[t]} < {E}LL) "
             self.w(f"{guard}appy::vstore<{arr.elem_c}, {V}>({self._addr(arr, tgt, c, bases[t])}, {accs[t]});")
+        if 1 < W <= 64:
+            self.w("appy::wave_fence();     // the row is stored: later loops of the team may read other lanes' elements")
         self.ind -= 1
         self.w("}")
         return k - i + 1
@@ -1666,6 +1673,8 @@ class KernelBuilder:
         self.ind -= 1
         self.w("}")
         self.mode, self.seq_depth = saved_mode, saved_depth
+        if 1 < W <= 64:
+            self.w("appy::wave_fence();     // the row is stored: later loops of the team may read other lanes' elements")
         self.ind -= 1
         self.w("}")
         return True

@@ -232,6 +232,17 @@ __device__ __forceinline__ T team_reduce(T v) {
     return v;
 }
 
+// Between two loops that the lanes of one wavefront share: what any lane stored in the first is
+// visible to every lane in the second, and nothing of the second is started before the first is
+// through.  The hardware runs the lanes in lockstep; this keeps the compiler from moving one
+// lane's loads and stores of the second loop over those of the first when it can prove that
+// lane's own addresses distinct (the overlap is between lanes).  No instruction is generated.
+__device__ __forceinline__ void wave_fence() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 // Workgroup reduction: wavefront butterfly, one LDS slot per wavefront, then a
 // butterfly over the slots.  Must be reached by every thread of the workgroup.
 // The total is returned in every lane of wavefront 0 (only).

@@ -40,6 +40,7 @@ _spmm_kernel_loop_1(
                     }
                 }
                 appy::vstore<float, 4>(y + (i * y_stride_0 + ((0LL + __lane) * 4)), __acc1);
+                appy::wave_fence();     // the row is stored: later loops of the team may read other lanes' elements
             }
         }
     }

@@ -650,3 +650,27 @@ def test_rows_that_several_simd_loops_read_stay_in_registers():
            "    #pragma simd\n    for j in range(d):\n        x[i, j] = x[i, j] / s\n")
     h, _ = compiled(upd, x=x, n=64, d=1024)
     assert h.analysis.row_cache is None
+
+
+def test_simd_loops_of_a_wavefront_team_are_fenced_when_they_touch_stored_arrays():
+    """Two simd loops of an iteration may touch the same elements from different lanes (slices
+    that overlap): the compiler sees only each lane's own, distinct addresses and could reorder
+    them across the loops, so a wavefront-scope fence separates the loops."""
+    from appy_amd.backends.hip.kernelgen import Spec
+
+    A = np.zeros((23, 61))
+    src = ("#pragma parallel for\nfor i in range(n):\n    #pragma simd\n    for j in range(16):\n        A[i, 18 + j] = B[i, 24 + j] - alpha\n"
+           "    #pragma simd\n    for j in range(16):\n        A[i, 12 + j] = B[i, 44 + j] * alpha\n")
+    f, _ = compiled(src, A=A, B=A.copy(), n=23, alpha=1.25)
+    k = body_of(f.kernel_for(Spec("team", block=256, vec=2, width=4)).src.text)
+    assert k.count("appy::wave_fence();") == 2
+    assert k.index("A + (i * A_stride_0 + (18LL") < k.index("appy::wave_fence();") < k.index("A + (i * A_stride_0 + (12LL")
+    # one lane per iteration: program order; several wavefronts: a workgroup barrier
+    assert "wave_fence" not in f.kernel_for(Spec("team", block=256, vec=2, width=1)).src.text.split('extern "C"')[1]
+    wide = body_of(f.kernel_for(Spec("team", block=256, vec=2, width=256)).src.text)
+    assert "wave_fence" not in wide and "__syncthreads();" in wide
+    # loops that only read arrays nothing stores to need none
+    src = ("#pragma parallel for\nfor i in range(n):\n    s = 0.0\n    #pragma simd\n    for j in range(m):\n        s += B[i, j]\n"
+           "    t = 0.0\n    #pragma simd\n    for j in range(m):\n        t += B[i, j] * B[i, j]\n    y[i] = s * t\n")
+    g, _ = compiled(src, B=A, y=np.zeros(23), n=23, m=61)
+    assert "wave_fence();" not in body_of(g.kernel_for(Spec("team", block=256, vec=2, width=16)).src.text)

@@ -337,3 +337,37 @@ def test_more_numpy_spellings_of_row_expressions(gpu, name):
     appy.jit(ns["f"])(*got)
     for g, w in zip(got, want):
         assert np.allclose(g, w, rtol=1e-9, atol=1e-9)
+
+
+def test_overlapping_row_slices_stored_by_two_statements_keep_program_order(gpu):
+    """The second statement overwrites part of what the first stored, from other lanes of the
+    team; with rows short enough for fully unrolled loops the order must still hold."""
+    @appy.jit
+    def kernel(A, B, v, alpha):
+        #pragma parallel for
+        for i in range(A.shape[0]):
+            A[i, 18:34] = np.maximum(B[i, 24:40], 0.0) - alpha
+            A[i, 12:-33] = B[i, 44:-1] * alpha + v[41:-4]
+
+    @appy.jit
+    def shifted(A, B, out):
+        #pragma parallel for
+        for i in range(A.shape[0]):
+            A[i, :-1] = B[i, 1:] * 2.0
+            out[i, 1:] = A[i, :-1] + A[i, 0]
+
+    rng = np.random.default_rng(5173)
+    for m in (61, 64, 65, 128, 257):
+        A, B, v = rng.standard_normal((23, m)), rng.standard_normal((23, m)), rng.standard_normal(m)
+        ref = A.copy()
+        ref[:, 18:34] = np.maximum(B[:, 24:40], 0.0) - 1.25
+        ref[:, 12:m - 33] = B[:, 44:m - 1] * 1.25 + v[41:m - 4]
+        got = A.copy()
+        kernel(got, B, v, 1.25)
+        assert np.array_equal(got, ref), m
+        ref, out_ref = A.copy(), np.zeros_like(A)
+        ref[:, :-1] = B[:, 1:] * 2.0
+        out_ref[:, 1:] = ref[:, :-1] + ref[:, :1]
+        got, out = A.copy(), np.zeros_like(A)
+        shifted(got, B, out)
+        assert np.array_equal(got, ref) and np.array_equal(out, out_ref), m
