@@ -579,7 +579,8 @@ class CompiledLoop:
                 return Spec("team", block=block, vec=v, width=w, restrict=restrict, stream_loads=stream, phase=1)
         steps = 0
         if (self._row_cache_codes is not None and bool(nj) == (self.analysis.collapse is not None) and v > 1
-                and not self.options.get("check_bounds")):
+                and restrict and not self.options.get("check_bounds")):
+            # (arguments that share memory: a row that no loop stores to by name may still change)
             # the rows that several simd loops of an iteration read stay in registers when every
             # lane takes a whole, small number of vector steps of them
             try:

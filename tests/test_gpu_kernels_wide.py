@@ -1156,3 +1156,39 @@ def test_collapsed_nests_keep_rows_in_registers_too(gpu):
         np.testing.assert_allclose(out, e / e.sum(axis=-1, keepdims=True), rtol=2e-4, atol=1e-7)
         spec = next(v[0] for k, v in cg.code_cache.items() if k[-1] == "softmax_planes").last_launch.spec
         assert spec.collapse and bool(spec.row_steps) == (shape[2] % 512 == 0), spec.tag()
+
+
+@appy.jit
+def normalise_then_sum(x, out, t):
+    #pragma parallel for
+    for i in range(x.shape[0]):
+        s = 0.0
+        #pragma simd
+        for j in range(x.shape[1]):
+            s += x[i, j]
+        #pragma simd
+        for j in range(x.shape[1]):
+            out[i, j] = x[i, j] / s
+        u = 0.0
+        #pragma simd
+        for j in range(x.shape[1]):
+            u += x[i, j]
+        t[i] = u
+
+
+def test_rows_are_not_kept_in_registers_when_arguments_share_memory(gpu):
+    """`out` and `x` the same array: the third loop must see what the second stored."""
+    import torch
+
+    rng = np.random.default_rng(3)
+    x = rng.random((200, 1024), dtype=np.float32) + 0.5
+    sep_out, t = np.zeros_like(x), np.zeros(200, np.float32)
+    normalise_then_sum(x, sep_out, t)
+    np.testing.assert_allclose(t, x.sum(axis=1), rtol=1e-5)
+    y, t = x.copy(), np.zeros(200, np.float32)
+    normalise_then_sum(y, y, t)
+    np.testing.assert_allclose(y, sep_out, rtol=1e-6)
+    np.testing.assert_allclose(t, np.ones(200), rtol=1e-5)
+    yd, td = torch.tensor(x, device="cuda"), torch.zeros(200, device="cuda")
+    normalise_then_sum(yd, yd, td)
+    np.testing.assert_allclose(td.cpu().numpy(), np.ones(200), rtol=1e-5)
