@@ -1192,3 +1192,41 @@ def test_rows_are_not_kept_in_registers_when_arguments_share_memory(gpu):
     yd, td = torch.tensor(x, device="cuda"), torch.zeros(200, device="cuda")
     normalise_then_sum(yd, yd, td)
     np.testing.assert_allclose(td.cpu().numpy(), np.ones(200), rtol=1e-5)
+
+
+@appy.jit
+def weighted_rows(x, w, out):
+    #pragma parallel for
+    for i in range(x.shape[0]):
+        s = 0.0
+        #pragma simd
+        for j in range(x.shape[1]):
+            s += x[i, j] * w[i, j]
+        #pragma simd
+        for j in range(x.shape[1]):
+            out[i, j] = x[i, j] * s - w[i, j]
+
+
+@pytest.mark.parametrize("dtype,n,d", [("float64", 100, 512), ("float64", 7, 16384), ("float64", 1000, 3072),
+                                       ("float32", 20000, 128), ("float32", 2, 32768), ("float32", 64, 12288),
+                                       ("float16", 300, 256), ("float16", 50, 1024)])
+def test_two_rows_kept_in_registers_over_element_types(gpu, dtype, n, d):
+    """Two arrays cached per iteration (x and w), 2, 4 and 8 elements per vector step, teams
+    from two lanes to a whole workgroup."""
+    from appy_amd.backends.hip import codegen as cg
+
+    rng = np.random.default_rng(d + n)
+    x = (rng.standard_normal((n, d)) * 0.25).astype(dtype)
+    w = (rng.standard_normal((n, d)) * 0.25).astype(dtype)
+    out = np.zeros_like(x)
+    weighted_rows(x, w, out)
+    x64, w64 = x.astype(np.float64), w.astype(np.float64)
+    ref = x64 * (x64 * w64).sum(axis=1, keepdims=True) - w64
+    tol = {"float64": 1e-11, "float32": 2e-4, "float16": 3e-2}[dtype]
+    np.testing.assert_allclose(out, ref, rtol=tol, atol=tol)
+    loop = next(v[0] for k, v in cg.code_cache.items()
+                if k[-1] == "weighted_rows" and v[0].analysis.arrays["x"].ty.name == dtype)
+    spec = loop.last_launch.spec
+    assert spec.row_steps == d // (spec.width * spec.vec) > 0, spec.tag()
+    text = loop.kernel_for(spec).src.text
+    assert "__rc0[" in text and "__rc1[" in text
