@@ -80,6 +80,13 @@ REPLAY_CACHE_ENTRIES = 2048
 COLLAPSE_BELOW_ROWS = 8192
 # vector steps of a row that a lane keeps in registers between the simd loops of an iteration
 ROW_CACHE_STEPS = 16
+# rows whose simd loop has bounds read per row (CSR rows) are sorted by trip count before they run,
+# from this many rows on
+BIN_MIN_ROWS = 1 << 15
+# a gathered operand larger than this is walked one stripe at a time by long rows; eight stripes (one per
+# XCD and its 4 MiB L2) of at most STRIPE_BYTES each, or a multiple of eight
+STRIPE_MIN_BYTES = 3 << 20
+STRIPE_BYTES = 2 << 20
 
 
 def device_header() -> str:
@@ -323,6 +330,10 @@ class CompiledLoop:
             if isinstance(n, ast.For):
                 for arg in n.iter.args:
                     steering.update(x.id for x in ast.walk(arg) if isinstance(x, ast.Name))
+        # scalars in subscripts the host checks against the extents (`a[2 * i + off]`): a replay
+        # with another value would skip that check, so the value is part of the call's identity
+        for _name, _dim, text in a.affine_checks:
+            steering.update(x.id for x in ast.walk(ast.parse(text, mode="eval")) if isinstance(x, ast.Name))
         # bounds that ask an array for its length or shape (`range(len(a) // 2)`) are given
         # shape-only stand-ins of the arrays when they are evaluated on the host
         self._bounds_name_arrays = bool(steering & set(a.arrays))
@@ -393,6 +404,8 @@ class CompiledLoop:
                 if k is None:
                     fn = self.options.get("fn_name")
                     sym = f"{fn}_{self.loop_name}" if fn and str(fn).isidentifier() else self.loop_name
+                    # the helper kernels of a loop with binned rows go by names of their own in traces
+                    sym += ("_" + spec.aux if spec.aux else {1: "_parts", 2: "_fold"}[spec.phase] if spec.rows == "list" else "")
                     builder = KernelBuilder(self.analysis, sym, self.module_names, spec)
                     k = Kernel(builder.build(device_header()))
                     self.kernels[spec] = k
@@ -552,6 +565,12 @@ class CompiledLoop:
         if nj:
             n_outer *= nj       # the pairs (i, j) are the rows from here on
         trip, uniform = self._estimate_trip(env, arrays, n_outer)
+        if (self.analysis.ragged is not None and not uniform and not nj and n_outer >= BIN_MIN_ROWS and restrict
+                and v > 1 and self.options.get("hip_bins", True) and not self.options.get("check_bounds")):
+            # rows of very different lengths (CSR): sorted into classes by a pass over their bounds,
+            # every class with the team width that suits it, long rows in column stripes
+            # (arguments that share memory: the pass over the bounds could read what the rows store)
+            return Spec("team", block=256, vec=v, width=64, restrict=restrict, stream_loads=stream, rows="mixed")
         if trip < 2 * v:
             v = 1
         # one vector step per lane for short rows; two rows per wavefront at most
@@ -757,11 +776,12 @@ class CompiledLoop:
             return
         plan.run()
         if key is not None and plan.replayable():
-            if len(self._replays) >= REPLAY_CACHE_ENTRIES:
-                # drop the older half (dicts keep insertion order)
-                for old in list(self._replays)[:REPLAY_CACHE_ENTRIES // 2]:
-                    del self._replays[old]
-            self._replays[key] = plan
+            with self._lock:        # launches may come from several interpreter threads
+                if len(self._replays) >= REPLAY_CACHE_ENTRIES:
+                    # drop the older half (dicts keep insertion order)
+                    for old in list(self._replays)[:REPLAY_CACHE_ENTRIES // 2]:
+                        self._replays.pop(old, None)
+                self._replays[key] = plan
 
     def overwrites(self, name, lo, hi, env, shape) -> bool:
         """True if this launch stores every element of array ``name`` (so that its
@@ -838,6 +858,8 @@ class Launch:
         self.staged_twice = {}   # (address, bytes, strides, dtype) of a staged host array -> (index in temps, uploaded?)
         self.aliases = []        # (name, dptr, bytes, stored) of host arrays that share the copy of another name
         self.keepalive = []
+        self.sequence = None
+        self.bin = None
         try:
             self._stage(vals, arrays)
         except BaseException:
@@ -956,6 +978,15 @@ class Launch:
             reds = len(loop_ir.reductions_of(a.team_split))
             self.scratch_ptr = loop.scratch(device, self.stream, max(1, reds) * self.nsplit * n_outer * 8)
         self.scalar_fields = {}      # by-value scalar -> field of the argument block
+        self.sequence = None         # binned rows: [(kernel, argument block, grid, block)] launched in this order
+        if spec.rows == "mixed":
+            if hi >= (1 << 31):
+                raise OverflowError(f"{loop.loop_name}: rows are listed as 32-bit numbers; the range ends at {hi}")
+            self._stage_binned(vals, arrays, lo, hi, spec)
+            self.args = self.sequence[2][1]
+            self.grid, self.block = self.sequence[2][2], self.sequence[2][3]
+            loop.last_launch = self
+            return
         self.args = self._argument_block(self.kernel, vals, arrays, lo, hi)
         if spec.phase == 1 and spec.kind == "strip":
             strips = -(-n_outer // 64)
@@ -975,6 +1006,75 @@ class Launch:
                                        row_hint=loop.row_hint(n_outer, env, arrays)), 1, 1)
         self.block = (spec.block, 1, 1)
         loop.last_launch = self
+
+    def _stage_binned(self, vals, arrays, lo, hi, spec):
+        """The launches of a loop whose rows are sorted by the trip count of their simd loop first:
+        clear the counters, sort (`bins`), the rows of all classes (`mixed`), and for long rows that
+        gather from a large operand: cut them at the stripes of that operand (`plan`), run the parts
+        (phase 1), fold the partial results and run the rest of the body (phase 2)."""
+        loop, a, env = self.loop, self.loop.analysis, self.env
+        n = hi - lo
+        V = spec.vec
+        thresholds = [V, 8 * V, 32 * V]
+        widthlog = [0, 2, 4, 6]
+        trip, _uniform = loop._estimate_trip(env, arrays, n)
+        base = sum(1 for t in thresholds if trip > t)
+        parts, stripe, cap = 0, 0, 0
+        gather = a.ragged[1]
+        if gather is not None:
+            x = arrays[gather[0]]
+            x_bytes = int(x.shape[0]) * a.arrays[gather[0]].ty.size
+            if x_bytes > STRIPE_MIN_BYTES:
+                parts = min(64, 8 * -(-x_bytes // (8 * STRIPE_BYTES)))
+                stripe = -(-int(x.shape[0]) // parts)
+                thresholds[2] = max(thresholds[2], 16 * parts)       # sixteen elements per part at least
+                # rows longer than the threshold: no more of them than the streamed arrays have room for
+                bound = max([int(arrays[nm].shape[0]) for _code, streamed in loop._simd_loops for nm in streamed
+                             if arrays[nm].ndim == 1] or [0])
+                cap = min(n, bound // thresholds[2] + 1) if bound else n
+        reds = max(1, len(loop_ir.reductions_of(a.team_split)))
+        # one buffer: counters | row lists of the four classes | part boundaries | partial results
+        off_rows = 256
+        off_bnd = off_rows + 4 * 4 * n
+        off_part = (off_bnd + 4 * (parts + 1) * cap + 255) // 256 * 256
+        total = off_part + 8 * reds * parts * cap
+        buf = loop.scratch(self.device, self.stream, total)
+        self.bin = {
+            "counts": buf, "zero": buf + 64, "rows": buf + off_rows, "m": n, "base": base, "threshold": thresholds,
+            "widthlog": widthlog, "skip": cap if parts else 0, "bnd": buf + off_bnd, "cap": cap, "stripe": stripe,
+            "nrows": buf + 4 * 3, "tlo": thresholds[base - 1] if base > 0 else -(1 << 62),
+            "thi": thresholds[base] if base < 3 else (1 << 62),
+        }
+        self.scratch_ptr = buf + off_part
+        self.nsplit = parts
+        common = dict(block=256, vec=V, restrict=spec.restrict, stream_loads=spec.stream_loads)
+        bins = loop.kernel_for(Spec("team", block=1024, vec=1, width=1, restrict=spec.restrict, aux="bins"))
+        seq = []
+        # the counters are cleared by the binning kernel itself, run over an empty range
+        self.bin["zero"] = buf
+        seq.append((bins, self._argument_block(bins, vals, arrays, 0, 0), (1, 1, 1), (1024, 1, 1)))
+        self.bin["zero"] = buf + 64
+        seq.append((bins, self._argument_block(bins, vals, arrays, lo, hi),
+                    (max(1, min(512, -(-n // 4096))), 1, 1), (1024, 1, 1)))
+        waves = -(-(n << widthlog[base]) // 64)
+        seq.append((self.kernel, self._argument_block(self.kernel, vals, arrays, lo, hi),
+                    (max(256, min(16384, -(-waves // 4))), 1, 1), (256, 1, 1)))
+        if parts:
+            ts = 8
+            while ts < parts:
+                ts *= 2
+            self.bin["rows"] = buf + off_rows + 4 * 3 * n         # the list of class 3
+            plan = loop.kernel_for(Spec("team", width=ts, rows="list", parts=parts, aux="plan",
+                                        **{**common, "vec": 1, "stream_loads": False}))
+            first = loop.kernel_for(Spec("team", width=16, phase=1, rows="list", parts=parts, **common))
+            last = loop.kernel_for(Spec("team", width=1, phase=2, rows="list", parts=parts, **common))
+            seq.append((plan, self._argument_block(plan, vals, arrays, lo, hi),
+                        (max(1, min(2048, -(-cap * ts // 256))), 1, 1), (256, 1, 1)))
+            seq.append((first, self._argument_block(first, vals, arrays, lo, hi),
+                        (max(8, min(2048, 8 * -(-cap * 16 // 256))), 1, 1), (256, 1, 1)))
+            seq.append((last, self._argument_block(last, vals, arrays, lo, hi),
+                        (max(1, min(1024, -(-cap // 256))), 1, 1), (256, 1, 1)))
+        self.sequence = seq
 
     def _argument_block(self, kernel, vals, arrays, lo, hi):
         loop = self.loop
@@ -1004,6 +1104,10 @@ class Launch:
                 val = self.scratch_ptr
             elif p.role == "nsplit":
                 val = self.nsplit
+            elif p.role in ("threshold", "widthlog"):
+                val = self.bin[p.role][p.dim]
+            elif p.role in ("rows", "counts", "zero", "nrows", "bnd", "cap", "stripe", "m", "base", "skip", "tlo", "thi"):
+                val = self.bin[p.role]
             elif p.role == "lo":
                 val = lo
             else:
@@ -1058,7 +1162,7 @@ class Launch:
     def replayable(self) -> bool:
         """True if nothing but the kernel launch happens when this call is repeated."""
         return not (self.temps or self.mirrored or self.keepalive_copies or self.oob or self.capture is not None
-                    or self.second is not None)
+                    or self.second is not None or self.sequence is not None)
 
     def _no_capture(self, name, why):
         if self.capture is not None:
@@ -1068,7 +1172,12 @@ class Launch:
         return self.kernel.function(self.device)
 
     def launch_only(self):
-        if self.second is None:
+        if self.sequence is not None:
+            # the kernels share the loop's scratch buffer for this stream: queued as one run
+            with self.loop._lock:
+                for kernel, args, grid, block in self.sequence:
+                    rt.launch(kernel.function(self.device), grid, block, args, self.stream)
+        elif self.second is None:
             rt.launch(self.function(), self.grid, self.block, self.args, self.stream)
         else:
             # both kernels share the loop's scratch buffer for this stream: they are queued as a
@@ -1088,8 +1197,19 @@ class Launch:
                     g.stored_mirrors.append(m)
 
     def time_kernel(self, warmup=3, reps=20) -> float:
-        """Mean milliseconds per launch (HIP events on the launch stream)."""
-        return rt.launch_timed(self.function(), self.grid, self.block, self.args, self.stream, warmup=warmup, reps=reps)
+        """Mean milliseconds per launch (HIP events on the launch stream); for a launch made of
+        several kernels, of the whole run of them."""
+        if self.sequence is None and self.second is None:
+            return rt.launch_timed(self.function(), self.grid, self.block, self.args, self.stream, warmup=warmup, reps=reps)
+        for _ in range(warmup):
+            self.launch_only()
+        e0, e1 = rt.Event(), rt.Event()
+        e0.record(self.stream)
+        for _ in range(reps):
+            self.launch_only()
+        e1.record(self.stream)
+        e1.synchronize()
+        return e0.elapsed_ms(e1) / reps
 
     def _check_report(self):
         if not self.oob:
@@ -1180,7 +1300,8 @@ def _copy(node):
 # ---------------------------------------------------------------------------
 def codegen(loop_source, loop_name, val_map, options):
     key = (loop_source, loop_name, _signature(val_map), options.get("hip_spec") and repr(options.get("hip_spec")),
-           options.get("hip_max_blocks"), bool(options.get("check_bounds")), options.get("fn_name"))
+           options.get("hip_max_blocks"), bool(options.get("check_bounds")), bool(options.get("hip_bins", True)),
+           options.get("fn_name"))
     # `clear_cache=True` regenerates the loop on every call instead of using the cached kernel
     # (reference: appy/backends/metal/codegen.py:23)
     fresh = bool(options.get("clear_cache"))

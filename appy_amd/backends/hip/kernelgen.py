@@ -75,6 +75,14 @@ class Spec:
                                  # simd loops of one iteration read; those rows stay in registers between the loops
     collapse: bool = False       # team only: the parallel loop and the sequential loop that is its whole body
                                  # run as one iteration space (the analysis has shown the inner iterations independent)
+    rows: str = ""               # team only, rows binned by the trip count of their simd loop: 'mixed' = the rows of the
+                                 # base class in their natural order plus the listed rows of the other classes, the
+                                 # team width chosen per wavefront at run time; 'list' = the rows of one list
+    parts: int = 0               # with rows='list' and a phase: the simd loop of a row runs in this many parts whose
+                                 # boundaries a planning kernel has written (column stripes of a gathered operand),
+                                 # one part per workgroup slot, the stripes dealt to the XCDs by workgroup number
+    aux: str = ""                # 'bins' = the kernel that sorts rows into classes, 'plan' = the kernel that finds
+                                 # the part boundaries of listed rows; '' = a kernel that runs the loop body
 
     def __post_init__(self):
         def pow2(n):
@@ -93,9 +101,20 @@ class Spec:
         if self.checked and (self.vec != 1 or self.unroll != 1 or self.extent or self.lds_tile):
             raise ValueError("a bounds-checked kernel takes one element per access (vec = unroll = 1, no row extent, no LDS tile)")
         if self.phase not in (0, 1, 2) or (self.phase and not (
-                self.kind == "strip" or (self.kind == "team" and self.width in (64, self.block)
+                self.kind == "strip" or (self.kind == "team" and (self.width in (64, self.block) or self.rows == "list")
                                          and not self.extent and not self.lds_tile and not self.collapse))):
-            raise ValueError("only strip kernels and teams of a whole wavefront or workgroup run in two phases")
+            raise ValueError("only strip kernels, teams of a whole wavefront or workgroup, and teams over listed rows "
+                             "run in two phases")
+        if self.rows not in ("", "mixed", "list") or self.aux not in ("", "bins", "plan"):
+            raise ValueError(f"unknown row source {self.rows!r} / auxiliary kernel {self.aux!r}")
+        if (self.rows or self.aux) and (self.kind != "team" or self.extent or self.lds_tile or self.collapse
+                                        or self.row_steps or self.checked or self.width > 64):
+            raise ValueError("rows are binned for plain team kernels only (teams inside a wavefront)")
+        if self.parts and (self.rows != "list" or not (self.phase or self.aux == "plan") or self.parts % 8
+                           or not 8 <= self.parts <= 64):
+            raise ValueError("planned parts belong to the two-phase kernels over listed rows (8, 16, ... 64 parts)")
+        if self.aux == "plan" and (self.rows != "list" or not self.parts or self.width < self.parts):
+            raise ValueError("the planning kernel takes listed rows, with one lane per part at least")
         if self.row_steps and (self.kind != "team" or self.phase or self.extent or self.lds_tile or self.vec < 2
                                or not 1 <= self.row_steps <= 16 or self.checked):
             raise ValueError("rows are kept in registers by plain team kernels only, for 1 to 16 vector steps per lane")
@@ -108,7 +127,8 @@ class Spec:
         return (f"{self.kind}_b{self.block}_v{self.vec}_u{self.unroll}_w{self.width}"
                 f"{'_r' if self.restrict else ''}{'_nt' if self.stream_loads else ''}"
                 f"{'_e' + str(self.extent) if self.extent else ''}{'_nts' if self.stream_stores else ''}"
-                f"{'_lds' + str(self.lds_tile) if self.lds_tile else ''}{'' if self.hoist_guarded else '_g'}{'_chk' if self.checked else ''}{'_c2' if self.collapse else ''}{'_p' + str(self.phase) if self.phase else ''}{'_rc' + str(self.row_steps) if self.row_steps else ''}")
+                f"{'_lds' + str(self.lds_tile) if self.lds_tile else ''}{'' if self.hoist_guarded else '_g'}{'_chk' if self.checked else ''}{'_c2' if self.collapse else ''}{'_p' + str(self.phase) if self.phase else ''}{'_rc' + str(self.row_steps) if self.row_steps else ''}"
+                f"{'_' + self.rows if self.rows else ''}{'_s' + str(self.parts) if self.parts else ''}{'_' + self.aux if self.aux else ''}")
 
 
 @dataclass
@@ -425,6 +445,38 @@ class LoopAnalysis:
         if not self._set_up_is_repeatable(body[:at], loops[0]):
             return None
         return loops[0]
+
+    def _find_ragged(self):
+        """``(loop, gather)`` when the rows of a team nest can be sorted by the trip count of
+        their ``simd`` loop before they run (CSR rows): the nest has the two-phase form (scalar
+        set-up, one ``simd`` loop directly in the body, the rest), the bounds of that loop come
+        out of the set-up, and nothing else ties the iterations together.  ``gather`` is
+        ``(X, IDX)`` when the loop reads ``X[IDX[j]]`` with ``j`` its own variable, ``X`` and
+        ``IDX`` one-dimensional and not stored to: long rows can then be walked one stripe of
+        ``X`` at a time."""
+        loop = self.team_split
+        if loop is None or self.outer_reductions or skips_iterations(self.outer.body):
+            return None
+        lo, hi, _ = loop.iter.args
+        if not any(isinstance(n, ast.Name) and (n.id in self.assigned or n.id == self.var)
+                   for b in (lo, hi) for n in ast.walk(b)):
+            return None
+        jv = loop.target.id
+        pairs = set()
+        for n in ast.walk(loop):
+            if not (isinstance(n, ast.Subscript) and isinstance(n.ctx, ast.Load) and isinstance(n.value, ast.Name)):
+                continue
+            x = self.arrays.get(n.value.id)
+            inner = n.slice
+            if (x is None or x.ndim != 1 or x.name in self.stored or not isinstance(inner, ast.Subscript)
+                    or not isinstance(inner.value, ast.Name)):
+                continue
+            idx = self.arrays.get(inner.value.id)
+            if (idx is not None and idx.ndim == 1 and idx.ty.is_int and not idx.ty.is_bool and idx.name not in self.stored
+                    and isinstance(inner.slice, ast.Name) and inner.slice.id == jv):
+                pairs.add((x.name, idx.name))
+        gather = next(iter(pairs)) if len(pairs) == 1 else None
+        return loop, gather
 
     def split_needs_finish(self) -> bool:
         """True if the two-phase form of a team nest needs its second kernel (the loop
@@ -776,6 +828,7 @@ class LoopAnalysis:
                         item = (n.value.id, d, ast.unparse(e))
                         if item not in self.affine_checks:
                             self.affine_checks.append(item)
+        self.ragged = self._find_ragged()
 
 
 def _partial_type(ty: Ty) -> Ty:
@@ -1224,6 +1277,8 @@ class KernelBuilder:
         whole workgroup (rows too long and too few for wavefront teams) goes
         through LDS."""
         W = self.spec.width
+        if self.spec.rows == "mixed":
+            return f"appy::team_reduce_dyn<{_OPS[op]}, {ty.c}>({partial}, __W)"
         if W <= 64:
             return f"appy::team_reduce<{_OPS[op]}, {W}, {ty.c}>({partial})"
         return f"appy::workgroup_reduce_all<{_OPS[op]}, {self.spec.block}, {ty.c}>({partial}, {T.identity_literal(op, ty)})"
@@ -1322,6 +1377,7 @@ class KernelBuilder:
             return self.tiled_spread_loop(st)
         var = st.target.id
         W, V = self.spec.width, self.spec.vec
+        Wc = "__W" if self.spec.rows == "mixed" else str(W)     # the stride of the lanes of a team, in the text
         lo, hi = self._range_args(st)
         self.ex.locals[var] = T.WEAK_INT
         reds = {}
@@ -1362,7 +1418,13 @@ class KernelBuilder:
             self.ind -= 1
             self.w("}")
             return
-        if self.spec.phase == 1:
+        if self.spec.phase == 1 and self.spec.parts:
+            # the part of this workgroup slot, as the planning kernel has cut the row
+            lo_c, hi_c = self.fresh("lo"), self.fresh("hi")
+            self.w(f"const appy::i64 {lo_c} = __bnd[__chunk * __cap + __t];")
+            self.w(f"const appy::i64 {hi_c} = __bnd[(__chunk + 1) * __cap + __t];")
+            lo_v, hi_v = lo_c, hi_c
+        elif self.spec.phase == 1:
             part = self.fresh("part")
             self.w(f"const appy::i64 {part} = ({hi_v} - {lo_v} + __nsplit - 1) / __nsplit;")
             lo_c, hi_c = self.fresh("lo"), self.fresh("hi")
@@ -1402,7 +1464,7 @@ class KernelBuilder:
             q = self.fresh("q")
             self.w(f"const appy::i64 {nv} = ({hi_v} - {lo_v}) / {V};")
             self.w("#pragma unroll 2")
-            self.w(f"for (appy::i64 {q} = __lane; {q} < {nv}; {q} += {W}) {{")
+            self.w(f"for (appy::i64 {q} = __lane; {q} < {nv}; {q} += {Wc}) {{")
             self.ind += 1
             base = self.fresh("j")
             self.w(f"const appy::i64 {base} = {lo_v} + {q} * {V};")
@@ -1413,7 +1475,7 @@ class KernelBuilder:
         else:
             start = f"{lo_v} + __lane"
         if not in_registers:
-            self.w(f"for (appy::i64 {cname(var)} = {start}; {cname(var)} < {hi_v}; {cname(var)} += {W}) {{")
+            self.w(f"for (appy::i64 {cname(var)} = {start}; {cname(var)} < {hi_v}; {cname(var)} += {Wc}) {{")
             self.ind += 1
             self.iteration_body(st.body)
             self.ind -= 1
@@ -1425,8 +1487,9 @@ class KernelBuilder:
                           for b in st.body for n in ast.walk(b)):
             # a team of several wavefronts: what one of them stored is read by the others only after this
             self.w("__syncthreads();")
-        elif 1 < W <= 64 and any(isinstance(n, ast.Subscript) and isinstance(n.value, ast.Name) and n.value.id in self.a.stored
-                                 for b in st.body for n in ast.walk(b)):
+        elif (1 < W <= 64 or self.spec.rows == "mixed") and any(
+                isinstance(n, ast.Subscript) and isinstance(n.value, ast.Name) and n.value.id in self.a.stored
+                for b in st.body for n in ast.walk(b)):
             # lanes of one wavefront: the loop touches an array that the nest stores to, and another
             # lane may touch the same elements in a later loop (slices that overlap, shifted reads)
             self.w("appy::wave_fence();")
@@ -1863,6 +1926,9 @@ class KernelBuilder:
     def _scratch_slot(self, r: int, chunk: str, pty: Ty) -> str:
         """Partial result number ``r`` of part ``chunk`` of this lane's column (8-byte slots)."""
         var = cname(self.a.var)
+        if self.spec.rows == "list":
+            # listed rows: the slot follows the position in the list, `__cap` rows at most
+            return f"*reinterpret_cast<{pty.c}*>(__scratch + (({r} * __nsplit + {chunk}) * __cap + __t))"
         return f"*reinterpret_cast<{pty.c}*>(__scratch + (({r} * __nsplit + {chunk}) * (__hi - __lo) + ({var} - __lo)))"
 
     def strip_spread_loop(self, st: ast.For):
@@ -1911,7 +1977,13 @@ class KernelBuilder:
             self.ind -= 1
             self.w("}")
             return
-        if self.spec.phase == 1:
+        if self.spec.phase == 1 and self.spec.parts:
+            # the part of this workgroup slot, as the planning kernel has cut the row
+            lo_c, hi_c = self.fresh("lo"), self.fresh("hi")
+            self.w(f"const appy::i64 {lo_c} = __bnd[__chunk * __cap + __t];")
+            self.w(f"const appy::i64 {hi_c} = __bnd[(__chunk + 1) * __cap + __t];")
+            lo_v, hi_v = lo_c, hi_c
+        elif self.spec.phase == 1:
             part = self.fresh("part")
             self.w(f"const appy::i64 {part} = ({hi_v} - {lo_v} + __nsplit - 1) / __nsplit;")
             lo_c, hi_c = self.fresh("lo"), self.fresh("hi")
@@ -2011,6 +2083,14 @@ class KernelBuilder:
         var = self.a.var
         self.ex.locals[var] = T.WEAK_INT
         self.lds_plan = self._find_lds_plan()
+        if s.aux or s.rows:
+            if self.a.ragged is None or self.lds_plan is not None:
+                raise Unsupported("the loop nest does not suit kernels over binned rows")
+            if s.aux == "bins":
+                return self._body_bins()
+            if s.rows == "mixed":
+                return self._body_mixed()
+            return self._body_listed()
         self.w(f"const int __lane = threadIdx.x & {W - 1};")
         self.w(f"const appy::i64 __team = threadIdx.x / {W};")
         if self.spec.phase:
@@ -2070,6 +2150,196 @@ class KernelBuilder:
         self.mode = "lane"
         self.ind -= 1
         self.w("}")
+
+    # ---- rows binned by the trip count of their simd loop ----------------------------------------
+    # Classes: 0..3 by rising trip count (thresholds are kernel arguments).  The rows of one class,
+    # the base class, are taken in their natural order; the rows of the others are listed by the
+    # binning kernel: `__rows[c * __m + k]`, `__counts[c]` of them.
+    def _split_iteration(self, idx_code: str, guard=None, upto=None):
+        """One iteration, the scalar set-up first; ``guard`` (a C condition that may use
+        ``__trip``, the trip count of the simd loop) decides whether the rest runs."""
+        a = self.a
+        body = a.outer.body
+        at = next(k for k, st in enumerate(body) if st is a.team_split)
+        self.w("{")
+        self.ind += 1
+        self.w(f"const appy::i64 {cname(a.var)} = {idx_code};")
+        self._declare_locals()
+        self.block(body[:at])
+        if guard is not None:
+            lo, hi = self._range_args(a.team_split)
+            self.w(f"const appy::i64 __trip = ({hi}) - ({lo});")
+            self.w(f"if ({guard}) {{")
+            self.ind += 1
+        self.block(body[at:upto])
+        if guard is not None:
+            self.ind -= 1
+            self.w("}")
+        self.ind -= 1
+        self.w("}")
+
+    def _body_bins(self):
+        """The kernel that sorts rows into classes: one lane per row runs the set-up, the rows of
+        every class but the base class are appended to the list of their class (one reservation
+        per workgroup, chunk and class).  It also clears the counters of the next launch."""
+        RPT = 4
+        B = self.spec.block
+        var = self.a.var
+        self.ex.locals[var] = T.WEAK_INT
+        self.mode = "lane"
+        self.w("__shared__ int __cnt[4];")
+        self.w("__shared__ int __first[4];")
+        self.w("if (blockIdx.x == 0 && threadIdx.x < 8) __zero[threadIdx.x] = 0;")
+        self.w(f"for (appy::i64 __c0 = __lo + (appy::i64)blockIdx.x * {B * RPT}; __c0 < __hi; __c0 += (appy::i64)gridDim.x * {B * RPT}) {{")
+        self.ind += 1
+        self.w("if (threadIdx.x < 4) __cnt[threadIdx.x] = 0;")
+        self.w("__syncthreads();")
+        self.w(f"int __cl[{RPT}], __pos[{RPT}];")
+        self.w("#pragma unroll")
+        self.w(f"for (int __r = 0; __r < {RPT}; ++__r) {{")
+        self.ind += 1
+        self.w(f"const appy::i64 __i = __c0 + (appy::i64)__r * {B} + threadIdx.x;")
+        self.w("__cl[__r] = -1;")
+        self.w("__pos[__r] = 0;")
+        self.w("if (__i < __hi) {")
+        self.ind += 1
+        body = self.a.outer.body
+        at = next(k for k, st in enumerate(body) if st is self.a.team_split)
+        self.w(f"const appy::i64 {cname(var)} = __i;")
+        self._declare_locals()
+        self.block(body[:at])
+        lo, hi = self._range_args(self.a.team_split)
+        self.w(f"const appy::i64 __trip = ({hi}) - ({lo});")
+        self.w("const int __c = __trip <= __t0 ? 0 : __trip <= __t1 ? 1 : __trip <= __t2 ? 2 : 3;")
+        self.w("if (__c != __base) { __cl[__r] = __c; __pos[__r] = atomicAdd(&__cnt[__c], 1); }")
+        self.ind -= 1
+        self.w("}")
+        self.ind -= 1
+        self.w("}")
+        self.w("__syncthreads();")
+        self.w("if (threadIdx.x < 4) __first[threadIdx.x] = __cnt[threadIdx.x] ? atomicAdd(&__counts[threadIdx.x], __cnt[threadIdx.x]) : 0;")
+        self.w("__syncthreads();")
+        self.w("#pragma unroll")
+        self.w(f"for (int __r = 0; __r < {RPT}; ++__r) {{")
+        self.w(f"    if (__cl[__r] >= 0) __rows[(appy::i64)__cl[__r] * __m + __first[__cl[__r]] + __pos[__r]] = "
+               f"(int)(__c0 + (appy::i64)__r * {B} + threadIdx.x);")
+        self.w("}")
+        self.w("__syncthreads();")
+        self.ind -= 1
+        self.w("}")
+
+    def _body_mixed(self):
+        """Rows of all classes in one kernel: the wavefronts walk a row of slots, first the rows of
+        the base class in their natural order (rows of other classes are passed over), then the
+        listed rows class by class; the team width of a wavefront follows the class of its slot."""
+        NWB = self.spec.block // 64
+        var = self.a.var
+        self.ex.locals[var] = T.WEAK_INT
+        self.w("const int __lid = threadIdx.x & 63;")
+        self.w(f"const appy::i64 __wv = (appy::i64)blockIdx.x * {NWB} + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);")
+        self.w(f"const appy::i64 __nwv = (appy::i64)gridDim.x * {NWB};")
+        prev = "0"
+        for c in range(4):
+            skip = "__skip3" if c == 3 else "0"
+            self.w(f"const appy::i64 __l{c} = (appy::i64)__counts[{c}] - {skip};")
+            self.w(f"const appy::i64 __n{c} = (__base == {c}) ? (__hi - __lo) : (__l{c} > 0 ? __l{c} : 0);")
+            self.w(f"const appy::i64 __e{c} = {prev} + (((__n{c} << __wl{c}) + 63) >> 6);")
+            prev = f"__e{c}"
+        self.w("for (appy::i64 __v = __wv; __v < __e3; __v += __nwv) {")
+        self.ind += 1
+        self.w("const int __c = (int)(__v >= __e0) + (int)(__v >= __e1) + (int)(__v >= __e2);")
+        self.w("const int __wl = __c == 0 ? __wl0 : __c == 1 ? __wl1 : __c == 2 ? __wl2 : __wl3;")
+        self.w("const int __W = 1 << __wl;")
+        self.w("const int __lane = __lid & (__W - 1);")
+        self.w("const appy::i64 __vb = __c == 0 ? 0 : __c == 1 ? __e0 : __c == 2 ? __e1 : __e2;")
+        self.w("const appy::i64 __nc = __c == 0 ? __n0 : __c == 1 ? __n1 : __c == 2 ? __n2 : __n3;")
+        self.w("const appy::i64 __t = ((__v - __vb) << (6 - __wl)) + (__lid >> __wl);")
+        self.w("if (__t < __nc) {")
+        self.ind += 1
+        self.w("const appy::i64 __i = (__c == __base) ? (__lo + __t) : "
+               "(appy::i64)__rows[(appy::i64)__c * __m + (__c == 3 ? __skip3 : 0) + __t];")
+        self.mode = "team"
+        self._split_iteration("__i", guard="__c != __base || (__trip > __tlo && __trip <= __thi)")
+        self.mode = "lane"
+        self.ind -= 1
+        self.w("}")
+        self.ind -= 1
+        self.w("}")
+
+    def _body_listed(self):
+        """Kernels over the rows of one list whose simd loop runs in planned parts: the planning
+        kernel, the kernel that runs the parts (part p on the workgroups whose number is p modulo 8:
+        workgroups go to the eight XCDs in turn, so every L2 sees one stripe of the gathered
+        operand), and the finishing kernel."""
+        s = self.spec
+        W, B, S = s.width, s.block, s.parts
+        tpb = B // W
+        var = self.a.var
+        self.ex.locals[var] = T.WEAK_INT
+        self.w(f"const int __lane = threadIdx.x & {W - 1};")
+        self.w(f"const appy::i64 __team = threadIdx.x / {W};")
+        self.w("const appy::i64 __listed = (appy::i64)__nrows[0];")
+        self.w("const appy::i64 __n = __listed < __cap ? __listed : __cap;")
+        if s.aux == "plan":
+            x_name, idx_name = self.a.ragged[1]
+            idx = self.a.arrays[idx_name]
+            idx.loaded = True
+            self.w(f"for (appy::i64 __t = (appy::i64)blockIdx.x * {tpb} + __team; __t < __n; __t += (appy::i64)gridDim.x * {tpb}) {{")
+            self.ind += 1
+            self.mode = "team"
+            self.w("{")
+            self.ind += 1
+            self.w(f"const appy::i64 {cname(var)} = (appy::i64)__rows[__t];")
+            self._declare_locals()
+            body = self.a.outer.body
+            at = next(k for k, st in enumerate(body) if st is self.a.team_split)
+            self.block(body[:at])
+            lo, hi = self._range_args(self.a.team_split)
+            self.w(f"const appy::i64 __rlo = {lo};")
+            self.w(f"const appy::i64 __rhi = ({hi}) > __rlo ? ({hi}) : __rlo;")
+            # lane p < S - 1 looks for the first position whose index reaches stripe p + 1; a running
+            # maximum over the lanes keeps the cuts in order, so that every position lies in exactly
+            # one part whatever the order of the indices (sorted rows are cut at the stripes)
+            self.w("appy::i64 __b = __rhi;")
+            self.w(f"if (__lane < {S - 1}) {{")
+            self.w("    const appy::i64 __target = (appy::i64)(__lane + 1) * __stripe;")
+            self.w("    appy::i64 __a = __rlo, __z = __rhi;")
+            self.w("    while (__a < __z) {")
+            self.w("        const appy::i64 __mid = __a + ((__z - __a) >> 1);")
+            self.w(f"        if ((appy::i64){cname(idx_name)}[__mid] < __target) __a = __mid + 1; else __z = __mid;")
+            self.w("    }")
+            self.w("    __b = __a;")
+            self.w("}")
+            self.w(f"__b = appy::team_running_max<{W}>(__b, __lane);")
+            self.w("if (__lane == 0) __bnd[__t] = (int)__rlo;")
+            self.w(f"if (__lane < {S}) __bnd[(appy::i64)(__lane + 1) * __cap + __t] = (int)(__lane < {S - 1} ? __b : __rhi);")
+            self.ind -= 1
+            self.w("}")
+            self.mode = "lane"
+            self.ind -= 1
+            self.w("}")
+            return
+        self.mode = "team"
+        if s.phase == 1:
+            self.w("const appy::i64 __rank = blockIdx.x >> 3, __nrank = gridDim.x >> 3;")
+            self.w(f"for (appy::i64 __chunk = blockIdx.x & 7; __chunk < {S}; __chunk += 8) {{")
+            self.ind += 1
+            self.w(f"for (appy::i64 __t = __rank * {tpb} + __team; __t < __n; __t += __nrank * {tpb}) {{")
+            self.ind += 1
+            body = self.a.outer.body
+            at = next(k for k, st in enumerate(body) if st is self.a.team_split)
+            self._split_iteration("(appy::i64)__rows[__t]", upto=at + 1)
+            self.ind -= 1
+            self.w("}")
+            self.ind -= 1
+            self.w("}")
+        else:
+            self.w(f"for (appy::i64 __t = (appy::i64)blockIdx.x * {tpb} + __team; __t < __n; __t += (appy::i64)gridDim.x * {tpb}) {{")
+            self.ind += 1
+            self._split_iteration("(appy::i64)__rows[__t]")
+            self.ind -= 1
+            self.w("}")
+        self.mode = "lane"
 
     def tiled_spread_loop(self, st: ast.For):
         """The LDS-staged form of :meth:`spread_loop` for the loop of the plan."""
@@ -2214,6 +2484,33 @@ class KernelBuilder:
         if self.spec.phase:
             params.append(Param("__scratch", "double* __scratch", C.c_void_p, "scratch"))
             params.append(Param("__nsplit", "const appy::i64 __nsplit", C.c_int64, "nsplit"))
+        sp = self.spec
+        if sp.aux == "bins":
+            params.append(Param("__rows", "int* __rows", C.c_void_p, "rows"))
+            params.append(Param("__counts", "int* __counts", C.c_void_p, "counts"))
+            params.append(Param("__zero", "int* __zero", C.c_void_p, "zero"))
+        elif sp.rows == "mixed":
+            params.append(Param("__rows", "const int* __rows", C.c_void_p, "rows"))
+            params.append(Param("__counts", "const int* __counts", C.c_void_p, "counts"))
+        elif sp.rows == "list":
+            params.append(Param("__rows", "const int* __rows", C.c_void_p, "rows"))
+            params.append(Param("__nrows", "const int* __nrows", C.c_void_p, "nrows"))
+            params.append(Param("__bnd", ("int* __bnd" if sp.aux == "plan" else "const int* __bnd"), C.c_void_p, "bnd"))
+            params.append(Param("__cap", "const appy::i64 __cap", C.c_int64, "cap"))
+            if sp.aux == "plan":
+                params.append(Param("__stripe", "const appy::i64 __stripe", C.c_int64, "stripe"))
+        if sp.aux == "bins" or sp.rows == "mixed":
+            params.append(Param("__m", "const appy::i64 __m", C.c_int64, "m"))
+            params.append(Param("__base", "const int __base", C.c_int32, "base"))
+        if sp.aux == "bins":
+            for k in range(3):
+                params.append(Param(f"__t{k}", f"const appy::i64 __t{k}", C.c_int64, "threshold", dim=k))
+        if sp.rows == "mixed":
+            for k in range(4):
+                params.append(Param(f"__wl{k}", f"const int __wl{k}", C.c_int32, "widthlog", dim=k))
+            params.append(Param("__skip3", "const appy::i64 __skip3", C.c_int64, "skip"))
+            params.append(Param("__tlo", "const appy::i64 __tlo", C.c_int64, "tlo"))
+            params.append(Param("__thi", "const appy::i64 __thi", C.c_int64, "thi"))
         params.append(Param("__lo", "const appy::i64 __lo", C.c_int64, "lo"))
         params.append(Param("__hi", "const appy::i64 __hi", C.c_int64, "hi"))
         return params

@@ -232,6 +232,36 @@ __device__ __forceinline__ T team_reduce(T v) {
     return v;
 }
 
+// The same butterfly for a width that is only known at run time (the same for the whole
+// wavefront: rows binned by length are dealt to wavefronts class by class).
+template <typename Op, typename T>
+__device__ __forceinline__ T team_reduce_dyn(T v, int w) {
+    if (w >= 2) v = Op::f(v, dpp_move<0xB1>(v));
+    if (w >= 4) v = Op::f(v, dpp_move<0x4E>(v));
+    if (w >= 8) v = Op::f(v, dpp_move<0x141>(v));
+    if (w >= 16) v = Op::f(v, dpp_move<0x140>(v));
+    if (w >= 32) v = Op::f(v, lane_xor(v, 16));
+    if (w >= 64) v = Op::f(v, lane_xor(v, 32));
+    return v;
+}
+
+// Running maximum over the lanes of a team of W adjacent lanes (lane k gets the maximum of
+// lanes 0..k of its team).  Every lane of the team must be active.
+template <int W>
+__device__ __forceinline__ i64 team_running_max(i64 v, int lane) {
+    static_assert(W >= 1 && W <= 64 && (W & (W - 1)) == 0, "team width is a power of two up to 64");
+#pragma unroll
+    for (int d = 1; d < W; d <<= 1) {
+        const int src = ((int)__lane_id() - d) << 2;
+        const unsigned long long u = (unsigned long long)v;
+        const unsigned lo = (unsigned)__builtin_amdgcn_ds_bpermute(src, (int)(unsigned)(u & 0xffffffffull));
+        const unsigned hi = (unsigned)__builtin_amdgcn_ds_bpermute(src, (int)(unsigned)(u >> 32));
+        const i64 o = (i64)(((unsigned long long)hi << 32) | (unsigned long long)lo);
+        if (lane >= d && o > v) v = o;
+    }
+    return v;
+}
+
 // Between two loops that the lanes of one wavefront share: what any lane stored in the first is
 // visible to every lane in the second, and nothing of the second is started before the first is
 // through.  The hardware runs the lanes in lockstep; this keeps the compiler from moving one

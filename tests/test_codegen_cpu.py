@@ -161,6 +161,19 @@ def test_out_of_range_loop_is_caught_on_the_host():
         f.prepare({"c": a, "a": a, "n": 8})
 
 
+def test_scalars_in_host_checked_subscripts_are_part_of_a_replayed_call_s_identity():
+    """`a[2 * i + off]` is compared with the extent of `a` on the host before a launch.  A repeat
+    of the call that only launches again must not carry another `off` past that check."""
+    a = np.zeros(64, np.float32)
+    b = np.zeros(8, np.float32)
+    f, _ = compiled("#pragma parallel for simd\nfor i in range(n):\n    b[i] = a[2 * i + off] * f", a=a, b=b, n=8, off=0, f=2.0)
+    assert [(nm, d, t) for nm, d, t in f.analysis.affine_checks] == [("a", 0, "2 * i + off")]
+    names = [f.arg_names[i] for i in f._value_only]
+    assert "off" not in names and "n" not in names and names == ["f"]
+    with pytest.raises(IndexError):
+        f.prepare({"a": a, "b": b, "n": 8, "off": 60, "f": 2.0})
+
+
 def test_lds_staging_is_an_option_and_refuses_unsafe_loops():
     g, _ = selfcheck_loop("gemv")
     k = body_of(g.kernel_for(Spec("team", block=256, vec=4, width=32, lds_tile=2048)).src.text)

@@ -387,6 +387,38 @@ def test_prange_only_programs_vectorise_their_inner_loops(gpu):
     assert kinds == {"hl_gemv": "team", "hl_spmv": "team", "hl_spmm": "team", "hl_mat_add": "team", "hl_colsum": "flat"}
 
 
+def test_replayed_call_with_an_out_of_range_subscript_offset_is_refused_on_the_host(gpu):
+    """The offset of an affine subscript is checked on the host for every value it takes: the
+    second call, which would otherwise only repeat the launch, raises before anything runs."""
+    import torch
+
+    from appy_amd.backends.hip import codegen as cg
+
+    @appy.jit
+    def strided_pick(a, b, off):
+        #pragma parallel for simd
+        for i in range(b.shape[0]):
+            b[i] = a[2 * i + off]
+
+    a = torch.arange(64, dtype=torch.float32, device="cuda")
+    b = torch.zeros(8, dtype=torch.float32, device="cuda")
+    strided_pick(a, b, 1)
+    assert torch.equal(b, a[1:17:2])
+    loop = [v[0] for kk, v in cg.code_cache.items() if kk[-1] == "strided_pick"][-1]
+    first = loop.last_launch
+    strided_pick(a, b, 1)
+    assert loop.last_launch is first                          # an exact repeat is replayed
+    strided_pick(a, b, 3)                                     # another offset: staged (and checked) again
+    assert loop.last_launch is not first and torch.equal(b, a[3:19:2])
+    before = b.clone()
+    with pytest.raises(IndexError):
+        strided_pick(a, b, 60)                                # 2 * 7 + 60 = 74 is past the end of `a`
+    with pytest.raises(IndexError):
+        strided_pick(a, b, -1)
+    torch.cuda.synchronize()
+    assert torch.equal(b, before)                             # nothing was launched
+
+
 def test_repeated_calls_on_gpu_tensors_replay_the_staged_launch(gpu):
     """A call with the same tensors, scalars and stream as before repeats only the
     launch; anything that differs goes through staging again."""
