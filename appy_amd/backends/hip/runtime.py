@@ -12,7 +12,7 @@ import threading
 _LIB_NAME = "libappy_hip.so"
 _PKG_ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 
 class Props(C.Structure):
@@ -80,6 +80,8 @@ SIGNATURES = {
     "appy_hip_memset_async": (C.c_int, [_vp, C.c_int, C.c_size_t, _vp]),
     "appy_hip_launch": (C.c_int, [_vp, _u32, _u32, _u32, _u32, _u32, _u32, _u32, _vp, _vp, C.c_size_t]),
     "appy_hip_sync": (C.c_int, [_vp]),
+    "appy_hip_launch_static_scratch": (
+        C.c_int, [_vp, _u32, _u32, _u32, _u32, _u32, _u32, _u32, _vp, _vp, C.c_size_t, C.c_size_t, C.c_size_t]),
     "appy_hip_rtc_version": (C.c_int, [C.POINTER(C.c_int)]),
     "appy_hip_stream_create": (C.c_int, [C.POINTER(_vp)]),
     "appy_hip_stream_destroy": (C.c_int, [_vp]),
@@ -283,6 +285,24 @@ def launch(func, grid, block, args_struct, stream: int = 0, dynamic_lds: int = 0
         lib().appy_hip_launch(
             func, gx, gy, gz, bx, by, bz, int(dynamic_lds), _vp(stream),
             C.byref(args_struct), C.sizeof(args_struct),
+        )
+    )
+
+
+STATIC_SCRATCH_BYTES = 8 << 20
+
+
+def launch_static_scratch(func, grid, block, args_struct, scratch_field: str, scratch_bytes: int, stream: int = 0,
+                          dynamic_lds: int = 0) -> None:
+    """Launch with the pointer field ``scratch_field`` of the argument block replaced by the
+    library's static scratch buffer of the current device; allocates nothing."""
+    gx, gy, gz = grid
+    bx, by, bz = block
+    offset = getattr(type(args_struct), scratch_field).offset
+    check(
+        lib().appy_hip_launch_static_scratch(
+            func, gx, gy, gz, bx, by, bz, int(dynamic_lds), _vp(stream),
+            C.byref(args_struct), C.sizeof(args_struct), offset, int(scratch_bytes),
         )
     )
 

@@ -1,10 +1,11 @@
 // libappy_hip.so - device runtime behind the APPy HIP code generator.
 //
-// Host-only translation unit: hiprtc compilation, code-object loading, a pooled
-// device allocator, stream-ordered copies, kernel launch and HIP-event timing,
-// exported through the C ABI declared in include/appy_hip.h.  The generated
-// kernels themselves are produced at run time by the Python code generator and
-// compiled here through hiprtc for gfx950.
+// hiprtc compilation, code-object loading, a pooled device allocator, stream-ordered
+// copies, kernel launch and HIP-event timing, exported through the C ABI declared in
+// include/appy_hip.h.  The generated kernels themselves are produced at run time by
+// the Python code generator and compiled here through hiprtc for gfx950; the only
+// device-side object of this file is the static scratch buffer of
+// appy_hip_launch_static_scratch.
 #include "appy_hip.h"
 
 #include <hip/hip_runtime.h>
@@ -21,6 +22,12 @@
 #include <thread>
 #include <unordered_map>
 #include <vector>
+
+// Scratch memory for launches that may not allocate (appy_hip_launch_static_scratch): part of
+// the library's code object, so every GPU the library runs on holds a copy of its own until the
+// process ends.  Host code never uses this name as an address: the address on a device comes
+// from hipGetSymbolAddress (static_scratch_of below).
+static __device__ __align__(256) unsigned char scratch[APPY_HIP_STATIC_SCRATCH_BYTES];
 
 namespace {
 
@@ -307,6 +314,30 @@ hipError_t staged_copy(void* dev, void* host, size_t n, bool to_device, hipStrea
     return hipSuccess;
 }
 
+// Address of the static scratch buffer on each device, looked up once per device with that
+// device current.
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+hipError_t static_scratch_of(int device, void** out) {
+    if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> g(g_scratch_mu);
+    if (!g_scratch_ptr[device]) {
+        int current = -1;
+        hipError_t e = hipGetDevice(&current);
+        if (e != hipSuccess) return e;
+        if (current != device) return hipErrorInvalidDevice;    // the caller makes the device current first
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        if (!p) return hipErrorInvalidSymbol;
+        g_scratch_ptr[device] = p;
+    }
+    *out = g_scratch_ptr[device];
+    return hipSuccess;
+}
+
 bool staging_enabled() {
     static const bool on = [] {
         const char* s = std::getenv("APPY_HIP_NO_STAGING");
@@ -342,6 +373,9 @@ int appy_hip_device_count(int* count_out) {
 int appy_hip_init(int device) {
     HIP_TRY(hipSetDevice(device));
     HIP_TRY(hipFree(nullptr));  // forces creation of the primary context
+    // the device's copy of the static scratch buffer (appy_hip_launch_static_scratch)
+    void* p = nullptr;
+    HIP_TRY(static_scratch_of(device, &p));
     return 0;
 }
 
@@ -669,6 +703,35 @@ int appy_hip_launch(void* func,
 
 int appy_hip_sync(void* stream) {
     HIP_TRY(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+    return 0;
+}
+
+int appy_hip_launch_static_scratch(void* func,
+                                   uint32_t grid_x, uint32_t grid_y, uint32_t grid_z,
+                                   uint32_t block_x, uint32_t block_y, uint32_t block_z,
+                                   uint32_t dynamic_lds_bytes, void* stream,
+                                   const void* args, size_t args_bytes,
+                                   size_t scratch_arg_offset, size_t scratch_bytes) {
+    constexpr size_t kMaxArgs = 4096;
+    if (!func) return fail_arg("func is NULL");
+    if (!args || args_bytes == 0) return fail_arg("args is NULL or empty");
+    if (args_bytes > kMaxArgs) return fail_arg("argument block larger than 4096 bytes");
+    if (scratch_arg_offset % alignof(void*) || scratch_arg_offset + sizeof(void*) > args_bytes)
+        return fail_arg("scratch_arg_offset does not name a pointer inside the argument block");
+    if (scratch_bytes > APPY_HIP_STATIC_SCRATCH_BYTES)
+        return fail_arg("scratch_bytes exceeds APPY_HIP_STATIC_SCRATCH_BYTES (the static scratch buffer holds 8 MiB)");
+    if (!launch_shape_ok(grid_x, grid_y, grid_z, block_x, block_y, block_z))
+        return fail_arg("grid/block shape out of range");
+    int device = 0;
+    HIP_TRY(hipGetDevice(&device));
+    void* dev_scratch = nullptr;
+    HIP_TRY(static_scratch_of(device, &dev_scratch));
+    alignas(16) char buf[kMaxArgs];                 // no heap: the argument block is copied on the stack
+    std::memcpy(buf, args, args_bytes);
+    std::memcpy(buf + scratch_arg_offset, &dev_scratch, sizeof(void*));
+    HIP_TRY(launch_packed(static_cast<hipFunction_t>(func), grid_x, grid_y, grid_z,
+                          block_x, block_y, block_z, dynamic_lds_bytes,
+                          static_cast<hipStream_t>(stream), buf, args_bytes));
     return 0;
 }
 

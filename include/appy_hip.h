@@ -24,9 +24,9 @@
 extern "C" {
 #endif
 
-/* 2: page-locked host memory, streams and graphs, appy_hip_rtc_version (additions only:
- * every entry point of version 1 is unchanged). */
-#define APPY_HIP_ABI_VERSION 2
+/* 2: page-locked host memory, streams and graphs, appy_hip_rtc_version; 3: appy_hip_launch_static_scratch
+ * (additions only: every entry point of the earlier versions is unchanged). */
+#define APPY_HIP_ABI_VERSION 3
 
 typedef struct appy_hip_props {
     char     name[128];        /* marketing name */
@@ -132,6 +132,26 @@ int appy_hip_launch(void* func,
                     uint32_t dynamic_lds_bytes, void* stream,
                     const void* args, size_t args_bytes);
 int appy_hip_sync(void* stream);               /* hipStreamSynchronize */
+
+/* appy_hip_launch for a kernel that takes a scratch buffer among its arguments (the partial results
+ * of a loop that runs as two kernels), without any allocation: the library keeps one buffer of
+ * APPY_HIP_STATIC_SCRATCH_BYTES per GPU inside its own code object, and writes that buffer's address
+ * over the 8 bytes at `scratch_arg_offset` of (its copy of) the argument block before the launch.
+ * `scratch_bytes` is what the kernel will use of it: more than APPY_HIP_STATIC_SCRATCH_BYTES is refused
+ * (invalid value), as is an argument block of more than 4096 bytes.
+ * Nothing in the reference corresponds to this.  It is for callers that cannot call hipMalloc where
+ * they launch: code under stream capture, serving loops with a fixed memory budget, harnesses that
+ * forbid allocation.  Neither device nor host memory is allocated or freed by the call.
+ * Every call on a GPU shares that GPU's buffer, which keeps what the last kernel left in it: kernels
+ * must write what they read (the two-phase kernels generated here do), and two launches that use it
+ * may not overlap on one GPU (same stream, or otherwise ordered by the caller). */
+#define APPY_HIP_STATIC_SCRATCH_BYTES (8u << 20)
+int appy_hip_launch_static_scratch(void* func,
+                                   uint32_t grid_x, uint32_t grid_y, uint32_t grid_z,
+                                   uint32_t block_x, uint32_t block_y, uint32_t block_z,
+                                   uint32_t dynamic_lds_bytes, void* stream,
+                                   const void* args, size_t args_bytes,
+                                   size_t scratch_arg_offset, size_t scratch_bytes);
 
 /* ---- streams and graphs -----------------------------------------------------
  * A loop nest that launches many short kernels (a time-stepping host loop
