@@ -41,6 +41,20 @@ def test_abi_version():
     assert f"#define APPY_HIP_ABI_VERSION {rt.ABI_VERSION}" in text
 
 
+def test_a_library_built_from_other_sources_is_rebuilt(monkeypatch):
+    """The build leaves a digest of the library's sources and flags next to the binary; the tests,
+    the smoke run and the benchmark rebuild when it does not match the tree."""
+    import __graft_entry__ as entry
+
+    assert entry.library_is_current()
+    monkeypatch.setattr(entry, "_sources_digest", lambda: "0" * 64)
+    assert not entry.library_is_current()
+    calls = []
+    monkeypatch.setattr(entry, "build", lambda: calls.append(1))
+    entry.ensure_built()
+    assert calls == [1]
+
+
 def test_compile_produces_a_gfx950_code_object():
     src = 'extern "C" __global__ void k(float* a, long long n) { long long i = blockIdx.x * 64ll + threadIdx.x; if (i < n) a[i] += 1.0f; }'
     code = rt.compile_to_code_object(src, "k.hip")
