@@ -1,0 +1,47 @@
+// kernel for spmv_kernel_loop_1_plan: team_b256_v1_u1_w8_r_list_s8_plan
+extern "C" __global__ void __launch_bounds__(256)
+_spmv_kernel_loop_1_plan(
+    const int* __restrict__ A_indptr,
+    const float* __restrict__ A_data,
+    const float* __restrict__ x,
+    const int* __restrict__ A_indices,
+    float* __restrict__ y,
+    const int* __rows,
+    const int* __nrows,
+    int* __bnd,
+    const appy::i64 __cap,
+    const appy::i64 __stripe,
+    const appy::i64 __lo,
+    const appy::i64 __hi)
+{
+    const int __lane = threadIdx.x & 7;
+    const appy::i64 __team = threadIdx.x / 8;
+    const appy::i64 __listed = (appy::i64)__nrows[0];
+    const appy::i64 __n = __listed < __cap ? __listed : __cap;
+    for (appy::i64 __t = (appy::i64)blockIdx.x * 32 + __team; __t < __n; __t += (appy::i64)gridDim.x * 32) {
+        {
+            const appy::i64 i = (appy::i64)__rows[__t];
+            int start = 0;
+            int end = 0;
+            double s = 0;
+            start = A_indptr[i];
+            end = A_indptr[(i + 1LL)];
+            s = 0.0;
+            const appy::i64 __rlo = ((long long)(start));
+            const appy::i64 __rhi = (((long long)(end))) > __rlo ? (((long long)(end))) : __rlo;
+            appy::i64 __b = __rhi;
+            if (__lane < 7) {
+                const appy::i64 __target = (appy::i64)(__lane + 1) * __stripe;
+                appy::i64 __a = __rlo, __z = __rhi;
+                while (__a < __z) {
+                    const appy::i64 __mid = __a + ((__z - __a) >> 1);
+                    if ((appy::i64)A_indices[__mid] < __target) __a = __mid + 1; else __z = __mid;
+                }
+                __b = __a;
+            }
+            __b = appy::team_running_max<8>(__b, __lane);
+            if (__lane == 0) __bnd[__t] = (int)__rlo;
+            if (__lane < 8) __bnd[(appy::i64)(__lane + 1) * __cap + __t] = (int)(__lane < 7 ? __b : __rhi);
+        }
+    }
+}

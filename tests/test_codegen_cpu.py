@@ -117,6 +117,39 @@ def selfcheck_loop(name):
     raise AssertionError(name)
 
 
+def test_csr_rows_are_sorted_by_length_from_32768_rows_on():
+    """Loops whose simd loop has bounds read per row take the binned shape when there are many
+    rows; the analysis names the gathered operand whose stripes long rows are cut at."""
+    f, _ = selfcheck_loop("spmv")
+    assert f.analysis.ragged is not None and f.analysis.ragged[1] == ("x", "A_indices")
+    arrays = {"A_data": np.zeros(16 * 40_000, np.float32)}
+    sp = f.choose_spec(40_000, {}, arrays)
+    assert sp.rows == "mixed" and sp.vec == 4
+    assert f.choose_spec(30_000, {}, arrays).rows == ""                          # too few rows to be worth a pass
+    assert f.choose_spec(40_000, {}, arrays, restrict=False).rows == ""          # arguments that share memory
+    g, _ = selfcheck_loop("gemv")
+    assert g.analysis.ragged is None and g.choose_spec(1 << 20, {"A_shape_1": 64}, {}).rows == ""    # rows of equal length
+    m, _ = selfcheck_loop("spmm")
+    assert m.analysis.ragged is None                                             # its ragged loop is sequential
+    # the kernels of the binned launch
+    bins = body_of(f.kernel_for(Spec("team", block=1024, vec=1, width=1, aux="bins")).src.text)
+    assert "__trip <= __t0 ? 0 : __trip <= __t1 ? 1 : __trip <= __t2 ? 2 : 3" in bins and "__zero[threadIdx.x] = 0" in bins
+    assert "x[" not in bins.split("{", 1)[1]                                     # only the set-up of a row runs here
+    mixed = body_of(f.kernel_for(Spec("team", block=256, vec=4, width=64, stream_loads=True, rows="mixed")).src.text)
+    assert "team_reduce_dyn<appy::OpAdd, float>" in mixed and "+= __W" in mixed
+    assert "__c != __base || (__trip > __tlo && __trip <= __thi)" in mixed
+    plan = body_of(f.kernel_for(Spec("team", block=256, vec=1, width=8, rows="list", parts=8, aux="plan")).src.text)
+    assert "A_indices[__mid] < __target" in plan and "team_running_max<8>" in plan
+    parts = body_of(f.kernel_for(Spec("team", block=256, vec=4, width=16, phase=1, rows="list", parts=8)).src.text)
+    assert "__chunk = blockIdx.x & 7" in parts and "__bnd[(__chunk + 1) * __cap + __t]" in parts
+    fold = body_of(f.kernel_for(Spec("team", block=256, vec=4, width=1, phase=2, rows="list", parts=8)).src.text)
+    assert "__c < __nsplit" in fold and "y[i] = s" in fold
+    with pytest.raises(ValueError):
+        Spec("team", width=16, phase=1, rows="list", parts=12)                   # parts go to the eight XCDs in turn
+    with pytest.raises(ValueError):
+        Spec("flat", rows="mixed")
+
+
 def test_spmm_row_lives_in_registers():
     loop, _ = selfcheck_loop("spmm")
     spec = Spec("team", block=256, vec=4, width=32, extent=128)

@@ -14,24 +14,33 @@ from appy_amd.backends.hip.kernelgen import Spec
 
 HERE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "kernels")
 
-# loop (function name) -> the launch shape the bench workloads use
+# snapshot name -> (loop (function name), the launch shape the bench workloads use)
 CASES = {
-    "vec_add": Spec("flat", block=256, vec=4, unroll=2),
-    "copy": Spec("flat", block=256, vec=4, unroll=1, stream_loads=True, stream_stores=True),
-    "vector_sum": Spec("flat", block=256, vec=4, unroll=2, stream_loads=True),
-    "masked_sum": Spec("flat", block=256, vec=4, unroll=2, stream_loads=True),
-    "gemv": Spec("team", block=256, vec=4, width=32, stream_loads=True),
-    "gemv_columns": Spec("strip", block=1024, vec=1, unroll=8, stream_loads=True),
-    "spmv": Spec("team", block=256, vec=4, width=4, stream_loads=True),
-    "spmm": Spec("team", block=256, vec=4, width=32, extent=128),
+    "vec_add": ("vec_add", Spec("flat", block=256, vec=4, unroll=2)),
+    "vec_add_streaming": ("vec_add", Spec("flat", block=1024, vec=4, unroll=1, stream_loads=True, stream_stores=True)),
+    "copy": ("copy", Spec("flat", block=512, vec=4, unroll=1, stream_loads=True, stream_stores=True)),
+    "vector_sum": ("vector_sum", Spec("flat", block=512, vec=4, unroll=2, stream_loads=True)),
+    "masked_sum": ("masked_sum", Spec("flat", block=512, vec=4, unroll=4, stream_loads=True)),
+    "gemv": ("gemv", Spec("team", block=256, vec=4, width=32, stream_loads=True)),
+    "gemv_columns": ("gemv_columns", Spec("strip", block=1024, vec=1, unroll=8, stream_loads=True)),
+    # CSR rows below the size from which rows are sorted by length: one team width for all rows
+    "spmv": ("spmv", Spec("team", block=256, vec=4, width=4, stream_loads=True)),
+    # the five kernels of a launch with rows sorted by length (config 4)
+    "spmv_bins": ("spmv", Spec("team", block=1024, vec=1, width=1, aux="bins")),
+    "spmv_rows_of_all_classes": ("spmv", Spec("team", block=256, vec=4, width=64, stream_loads=True, rows="mixed")),
+    "spmv_plan": ("spmv", Spec("team", block=256, vec=1, width=8, rows="list", parts=8, aux="plan")),
+    "spmv_parts": ("spmv", Spec("team", block=256, vec=4, width=16, stream_loads=True, phase=1, rows="list", parts=8)),
+    "spmv_fold": ("spmv", Spec("team", block=256, vec=4, width=1, stream_loads=True, phase=2, rows="list", parts=8)),
+    "spmm": ("spmm", Spec("team", block=256, vec=4, width=32, extent=128)),
 }
 
 
 def kernel_text(name):
     selfcheck.compile_all_patterns()
-    loops = [loop for key, (loop, _) in cg.code_cache.items() if key[-1] == name]
+    fn, spec = CASES[name]
+    loops = [loop for key, (loop, _) in cg.code_cache.items() if key[-1] == fn]
     assert loops, name
-    text = loops[-1].kernel_for(CASES[name]).src.text
+    text = loops[-1].kernel_for(spec).src.text
     return text[text.index("// kernel for"):]
 
 
