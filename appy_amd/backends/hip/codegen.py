@@ -476,15 +476,16 @@ class CompiledLoop:
                 best = max(best, 64.0)
         return best, uniform
 
-    def choose_spec(self, n_outer, env, arrays, restrict=True) -> Spec:
-        spec = self._choose_spec(n_outer, env, arrays, restrict)
+    def choose_spec(self, n_outer, env, arrays, restrict=True, listable=True) -> Spec:
+        """``listable``: the iterations can be named by 32-bit numbers (rows sorted by length are)."""
+        spec = self._choose_spec(n_outer, env, arrays, restrict, listable)
         if self.options.get("check_bounds"):
             # one element per access, every access through the checking path
             spec = dataclasses.replace(spec, vec=1, unroll=1, extent=0, lds_tile=0, stream_loads=False,
                                        stream_stores=False, checked=True)
         return spec
 
-    def _choose_spec(self, n_outer, env, arrays, restrict=True) -> Spec:
+    def _choose_spec(self, n_outer, env, arrays, restrict=True, listable=True) -> Spec:
         forced = self.options.get("hip_spec")
         d = self.default_spec
         if isinstance(forced, dict):
@@ -568,7 +569,7 @@ class CompiledLoop:
             n_outer *= nj       # the pairs (i, j) are the rows from here on
         trip, uniform = self._estimate_trip(env, arrays, n_outer)
         if (self.analysis.ragged is not None and not uniform and not nj and n_outer >= BIN_MIN_ROWS and restrict
-                and v > 1 and self.options.get("hip_bins", True) and not self.options.get("check_bounds")):
+                and listable and v > 1 and self.options.get("hip_bins", True) and not self.options.get("check_bounds")):
             # rows of very different lengths (CSR): sorted into classes by a pass over their bounds,
             # every class with the team width that suits it, long rows in column stripes
             # (arguments that share memory: the pass over the bounds could read what the rows store)
@@ -958,7 +959,7 @@ class Launch:
 
         # -- kernel variant, argument block, grid
         n_outer = hi - lo
-        spec = loop.choose_spec(n_outer, env, arrays, restrict=restrict)
+        spec = loop.choose_spec(n_outer, env, arrays, restrict=restrict, listable=hi < (1 << 31))
         if spec.kind == "flat" and spec.hoist_guarded and a.guarded_checks:
             # loads the program guards with a condition may only be issued early when
             # they cannot leave their array anywhere in the range
@@ -982,8 +983,6 @@ class Launch:
         self.scalar_fields = {}      # by-value scalar -> field of the argument block
         self.sequence = None         # binned rows: [(kernel, argument block, grid, block)] launched in this order
         if spec.rows == "mixed":
-            if hi >= (1 << 31):
-                raise OverflowError(f"{loop.loop_name}: rows are listed as 32-bit numbers; the range ends at {hi}")
             self._stage_binned(vals, arrays, lo, hi, spec)
             self.args = self.sequence[2][1]
             self.grid, self.block = self.sequence[2][2], self.sequence[2][3]
@@ -1036,13 +1035,15 @@ class Launch:
                 cap = min(n, bound // thresholds[2] + 1) if bound else n
         reds = max(1, len(loop_ir.reductions_of(a.team_split)))
         # one buffer: counters | row lists of the four classes | part boundaries | partial results
-        off_rows = 256
+        # header: 8 counters, 64 part loads (8 bytes each), and a second such block that the binning kernel
+        # clears instead when it is not run to clear the first
+        off_rows = 2048
         off_bnd = off_rows + 4 * 4 * n
         off_part = (off_bnd + 4 * (parts + 1) * cap + 255) // 256 * 256
         total = off_part + 8 * reds * parts * cap
         buf = loop.scratch(self.device, self.stream, total)
         self.bin = {
-            "counts": buf, "zero": buf + 64, "rows": buf + off_rows, "m": n, "base": base, "threshold": thresholds,
+            "counts": buf, "load": buf + 32, "zero": buf + 1024, "rows": buf + off_rows, "m": n, "base": base, "threshold": thresholds,
             "widthlog": widthlog, "skip": cap if parts else 0, "bnd": buf + off_bnd, "cap": cap, "stripe": stripe,
             "nrows": buf + 4 * 3, "tlo": thresholds[base - 1] if base > 0 else -(1 << 62),
             "thi": thresholds[base] if base < 3 else (1 << 62),
@@ -1055,7 +1056,7 @@ class Launch:
         # the counters are cleared by the binning kernel itself, run over an empty range
         self.bin["zero"] = buf
         seq.append((bins, self._argument_block(bins, vals, arrays, 0, 0), (1, 1, 1), (1024, 1, 1)))
-        self.bin["zero"] = buf + 64
+        self.bin["zero"] = buf + 1024
         seq.append((bins, self._argument_block(bins, vals, arrays, lo, hi),
                     (max(1, min(512, -(-n // 4096))), 1, 1), (1024, 1, 1)))
         # a wavefront for every slot of the base class: the other classes follow in further passes of the grid
@@ -1110,7 +1111,7 @@ class Launch:
                 val = self.nsplit
             elif p.role in ("threshold", "widthlog"):
                 val = self.bin[p.role][p.dim]
-            elif p.role in ("rows", "counts", "zero", "nrows", "bnd", "cap", "stripe", "m", "base", "skip", "tlo", "thi"):
+            elif p.role in ("rows", "counts", "zero", "nrows", "bnd", "cap", "stripe", "m", "base", "skip", "tlo", "thi", "load"):
                 val = self.bin[p.role]
             elif p.role == "lo":
                 val = lo

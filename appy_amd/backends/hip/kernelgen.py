@@ -1419,10 +1419,10 @@ class KernelBuilder:
             self.w("}")
             return
         if self.spec.phase == 1 and self.spec.parts:
-            # the part of this workgroup slot, as the planning kernel has cut the row
+            # the part of this workgroup slot, as the planning kernel has cut the row (relative to its start)
             lo_c, hi_c = self.fresh("lo"), self.fresh("hi")
-            self.w(f"const appy::i64 {lo_c} = __bnd[__chunk * __cap + __t];")
-            self.w(f"const appy::i64 {hi_c} = __bnd[(__chunk + 1) * __cap + __t];")
+            self.w(f"const appy::i64 {lo_c} = {lo_v} + __bnd[__chunk * __cap + __t];")
+            self.w(f"const appy::i64 {hi_c} = {lo_v} + __bnd[(__chunk + 1) * __cap + __t];")
             lo_v, hi_v = lo_c, hi_c
         elif self.spec.phase == 1:
             part = self.fresh("part")
@@ -1978,7 +1978,7 @@ class KernelBuilder:
             self.w("}")
             return
         if self.spec.phase == 1 and self.spec.parts:
-            # the part of this workgroup slot, as the planning kernel has cut the row
+            # the part of this workgroup slot, as the planning kernel has cut the row (relative to its start)
             lo_c, hi_c = self.fresh("lo"), self.fresh("hi")
             self.w(f"const appy::i64 {lo_c} = __bnd[__chunk * __cap + __t];")
             self.w(f"const appy::i64 {hi_c} = __bnd[(__chunk + 1) * __cap + __t];")
@@ -2189,7 +2189,7 @@ class KernelBuilder:
         self.mode = "lane"
         self.w("__shared__ int __cnt[4];")
         self.w("__shared__ int __first[4];")
-        self.w("if (blockIdx.x == 0 && threadIdx.x < 8) __zero[threadIdx.x] = 0;")
+        self.w("if (blockIdx.x == 0 && threadIdx.x < 136) __zero[threadIdx.x] = 0;     // 8 counters, 64 part loads of 8 bytes")
         self.w(f"for (appy::i64 __c0 = __lo + (appy::i64)blockIdx.x * {B * RPT}; __c0 < __hi; __c0 += (appy::i64)gridDim.x * {B * RPT}) {{")
         self.ind += 1
         self.w("if (threadIdx.x < 4) __cnt[threadIdx.x] = 0;")
@@ -2284,6 +2284,11 @@ class KernelBuilder:
             x_name, idx_name = self.a.ragged[1]
             idx = self.a.arrays[idx_name]
             idx.loaded = True
+            # elements per part over all rows: the kernel that runs the parts looks at these before it
+            # ties parts to XCDs (columns that crowd into few stripes would leave most XCDs idle)
+            self.w(f"__shared__ unsigned long long __work[{S}];")
+            self.w(f"if (threadIdx.x < {S}) __work[threadIdx.x] = 0;")
+            self.w("__syncthreads();")
             self.w(f"for (appy::i64 __t = (appy::i64)blockIdx.x * {tpb} + __team; __t < __n; __t += (appy::i64)gridDim.x * {tpb}) {{")
             self.ind += 1
             self.mode = "team"
@@ -2311,26 +2316,47 @@ class KernelBuilder:
             self.w("    __b = __a;")
             self.w("}")
             self.w(f"__b = appy::team_running_max<{W}>(__b, __lane);")
-            self.w("if (__lane == 0) __bnd[__t] = (int)__rlo;")
-            self.w(f"if (__lane < {S}) __bnd[(appy::i64)(__lane + 1) * __cap + __t] = (int)(__lane < {S - 1} ? __b : __rhi);")
+            # (cuts are kept relative to the start of the row: 32 bits are enough whatever the array size)
+            self.w("if (__lane == 0) __bnd[__t] = 0;")
+            self.w(f"const appy::i64 __cut = (__lane < {S - 1} ? __b : __rhi) - __rlo;      // where part __lane ends")
+            self.w(f"if (__lane < {S}) __bnd[(appy::i64)(__lane + 1) * __cap + __t] = (int)__cut;")
+            self.w(f"const appy::i64 __before = appy::team_lane_below<{W}>(__cut, __lane);")
+            self.w(f"if (__lane < {S} && __cut > (__lane ? __before : 0)) "
+                   f"atomicAdd(&__work[__lane], (unsigned long long)(__cut - (__lane ? __before : 0)));")
             self.ind -= 1
             self.w("}")
             self.mode = "lane"
             self.ind -= 1
             self.w("}")
+            self.w("__syncthreads();")
+            self.w(f"if (threadIdx.x < {S} && __work[threadIdx.x]) atomicAdd(&__load[threadIdx.x], __work[threadIdx.x]);")
             return
         self.mode = "team"
         if s.phase == 1:
-            self.w("const appy::i64 __rank = blockIdx.x >> 3, __nrank = gridDim.x >> 3;")
-            self.w(f"for (appy::i64 __chunk = blockIdx.x & 7; __chunk < {S}; __chunk += 8) {{")
+            # Part p of every row runs on the workgroups whose number is p modulo 8, i.e. on one XCD, whose L2
+            # then holds stripe p of the gathered operand and nothing else of it.  That ties the work of an XCD
+            # to the elements that fall into its stripes: when one XCD would get more than 1.5 times its share
+            # (columns crowded into few stripes), the parts are dealt to all workgroups alike instead, stripe
+            # after stripe.
+            self.w("unsigned long long __tot = 0, __most = 0;")
+            self.w("for (int __x = 0; __x < 8; ++__x) {")
+            self.w("    unsigned long long __sum = 0;")
+            self.w(f"    for (int __p = __x; __p < {S}; __p += 8) __sum += __load[__p];")
+            self.w("    __tot += __sum;")
+            self.w("    __most = __sum > __most ? __sum : __most;")
+            self.w("}")
+            self.w("const bool __even = __most * 16 <= __tot * 3;")
+            self.w(f"const appy::i64 __items = __n * (__even ? {S // 8} : {S});")
+            self.w(f"const appy::i64 __q0 = (__even ? (appy::i64)(blockIdx.x >> 3) : (appy::i64)blockIdx.x) * {tpb} + __team;")
+            self.w(f"const appy::i64 __dq = (__even ? (appy::i64)(gridDim.x >> 3) : (appy::i64)gridDim.x) * {tpb};")
+            self.w("for (appy::i64 __q = __q0; __q < __items; __q += __dq) {")
             self.ind += 1
-            self.w(f"for (appy::i64 __t = __rank * {tpb} + __team; __t < __n; __t += __nrank * {tpb}) {{")
-            self.ind += 1
+            self.w("const appy::i64 __pass = __q / __n;")
+            self.w("const appy::i64 __t = __q - __pass * __n;")
+            self.w("const appy::i64 __chunk = __even ? (appy::i64)(blockIdx.x & 7) + 8 * __pass : __pass;")
             body = self.a.outer.body
             at = next(k for k, st in enumerate(body) if st is self.a.team_split)
             self._split_iteration("(appy::i64)__rows[__t]", upto=at + 1)
-            self.ind -= 1
-            self.w("}")
             self.ind -= 1
             self.w("}")
         else:
@@ -2499,6 +2525,9 @@ class KernelBuilder:
             params.append(Param("__cap", "const appy::i64 __cap", C.c_int64, "cap"))
             if sp.aux == "plan":
                 params.append(Param("__stripe", "const appy::i64 __stripe", C.c_int64, "stripe"))
+                params.append(Param("__load", "unsigned long long* __load", C.c_void_p, "load"))
+            elif sp.phase == 1:
+                params.append(Param("__load", "const unsigned long long* __load", C.c_void_p, "load"))
         if sp.aux == "bins" or sp.rows == "mixed":
             params.append(Param("__m", "const appy::i64 __m", C.c_int64, "m"))
             params.append(Param("__base", "const int __base", C.c_int32, "base"))

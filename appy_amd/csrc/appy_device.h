@@ -262,6 +262,17 @@ __device__ __forceinline__ i64 team_running_max(i64 v, int lane) {
     return v;
 }
 
+// The value of the lane below in a team of W adjacent lanes (lane 0 of a team gets an unspecified value).
+template <int W>
+__device__ __forceinline__ i64 team_lane_below(i64 v, int lane) {
+    const int src = ((int)__lane_id() - 1) << 2;
+    const unsigned long long u = (unsigned long long)v;
+    const unsigned lo = (unsigned)__builtin_amdgcn_ds_bpermute(src, (int)(unsigned)(u & 0xffffffffull));
+    const unsigned hi = (unsigned)__builtin_amdgcn_ds_bpermute(src, (int)(unsigned)(u >> 32));
+    (void)lane;
+    return (i64)(((unsigned long long)hi << 32) | (unsigned long long)lo);
+}
+
 // Between two loops that the lanes of one wavefront share: what any lane stored in the first is
 // visible to every lane in the second, and nothing of the second is started before the first is
 // through.  The hardware runs the lanes in lockstep; this keeps the compiler from moving one

@@ -19,7 +19,7 @@ _spmv_kernel_loop_1_bins(
 {
     __shared__ int __cnt[4];
     __shared__ int __first[4];
-    if (blockIdx.x == 0 && threadIdx.x < 8) __zero[threadIdx.x] = 0;
+    if (blockIdx.x == 0 && threadIdx.x < 136) __zero[threadIdx.x] = 0;     // 8 counters, 64 part loads of 8 bytes
     for (appy::i64 __c0 = __lo + (appy::i64)blockIdx.x * 4096; __c0 < __hi; __c0 += (appy::i64)gridDim.x * 4096) {
         if (threadIdx.x < 4) __cnt[threadIdx.x] = 0;
         __syncthreads();

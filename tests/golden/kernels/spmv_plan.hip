@@ -11,6 +11,7 @@ _spmv_kernel_loop_1_plan(
     int* __bnd,
     const appy::i64 __cap,
     const appy::i64 __stripe,
+    unsigned long long* __load,
     const appy::i64 __lo,
     const appy::i64 __hi)
 {
@@ -18,6 +19,9 @@ _spmv_kernel_loop_1_plan(
     const appy::i64 __team = threadIdx.x / 8;
     const appy::i64 __listed = (appy::i64)__nrows[0];
     const appy::i64 __n = __listed < __cap ? __listed : __cap;
+    __shared__ unsigned long long __work[8];
+    if (threadIdx.x < 8) __work[threadIdx.x] = 0;
+    __syncthreads();
     for (appy::i64 __t = (appy::i64)blockIdx.x * 32 + __team; __t < __n; __t += (appy::i64)gridDim.x * 32) {
         {
             const appy::i64 i = (appy::i64)__rows[__t];
@@ -40,8 +44,13 @@ _spmv_kernel_loop_1_plan(
                 __b = __a;
             }
             __b = appy::team_running_max<8>(__b, __lane);
-            if (__lane == 0) __bnd[__t] = (int)__rlo;
-            if (__lane < 8) __bnd[(appy::i64)(__lane + 1) * __cap + __t] = (int)(__lane < 7 ? __b : __rhi);
+            if (__lane == 0) __bnd[__t] = 0;
+            const appy::i64 __cut = (__lane < 7 ? __b : __rhi) - __rlo;      // where part __lane ends
+            if (__lane < 8) __bnd[(appy::i64)(__lane + 1) * __cap + __t] = (int)__cut;
+            const appy::i64 __before = appy::team_lane_below<8>(__cut, __lane);
+            if (__lane < 8 && __cut > (__lane ? __before : 0)) atomicAdd(&__work[__lane], (unsigned long long)(__cut - (__lane ? __before : 0)));
         }
     }
+    __syncthreads();
+    if (threadIdx.x < 8 && __work[threadIdx.x]) atomicAdd(&__load[threadIdx.x], __work[threadIdx.x]);
 }

@@ -125,6 +125,26 @@ def test_spmv_columns_in_any_order_and_int64_indices(k):
     assert ok, worst
 
 
+def test_spmv_columns_crowded_into_one_stripe(k):
+    """Every long row has its columns in the first eighth of the vector: the parts of the other seven
+    stripes are empty, and the parts are dealt to all workgroups instead of one XCD per stripe."""
+    rng = np.random.default_rng(31)
+    m, n = 40_000, 1 << 21
+    lengths = np.clip(rng.zipf(1.4, m), 1, 3000).astype(np.int64)
+    data, indptr, indices = wl.csr_matrix(lengths, n // 8, rng)          # columns below n / 8 only
+    x = rng.standard_normal(n, dtype=np.float32)
+    ref, budget = vo.spmv_csr(data, indptr, indices, x, (m, n))
+    y = k.spmv(data, indptr, indices, x, m, n)
+    assert _loop("spmv").last_launch.nsplit == 8
+    ok, worst = vo.within_budget(y, ref, budget, TOL)
+    assert ok, worst
+    # and columns in the last two stripes only
+    indices2 = (indices.astype(np.int64) * 2 + (n - n // 4)).astype(np.int32)
+    ref, budget = vo.spmv_csr(data, indptr, indices2, x, (m, n))
+    ok, worst = vo.within_budget(k.spmv(data, indptr, indices2, x, m, n), ref, budget, TOL)
+    assert ok, worst
+
+
 def test_more_long_rows_than_the_streamed_arrays_account_for(k):
     """Row pointers that overlap (not a CSR matrix, but a legal loop): more rows of the longest class
     than nnz / threshold.  The rows beyond the room set aside for parts run whole."""
