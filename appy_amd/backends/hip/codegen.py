@@ -321,6 +321,7 @@ class CompiledLoop:
             name: (None if node is None else compile(ast.Expression(body=ast.fix_missing_locations(_copy(node))), "<n>", "eval"))
             for name, node in a.overwritten.items()}
         self._scratch = {}  # (device, stream) -> (device pointer, bytes): partial results of two-phase launches
+        self._hints = {}    # device -> (address, ctypes view) of page-locked words the binned kernels report to
         self._scratch_retired = []
         self._replays = {}  # call identity -> Launch that can simply be launched again
         # scalars that no host-side decision looks at (range of the loop, inner trip counts,
@@ -664,6 +665,21 @@ class CompiledLoop:
                 self._scratch[key] = have
             return have[0]
 
+    def hint(self, device: int):
+        """Five page-locked 64-bit words per device that the kernel over binned rows writes (a flag, then
+        the number of rows of each class it found) and the host reads when it stages the next launch.
+        What is read may be old or half updated: it shapes a launch, it never decides what is computed."""
+        with self._lock:
+            have = self._hints.get(device)
+            if have is None:
+                addr = rt.host_alloc(64)
+                view = (C.c_int64 * 8).from_address(addr)
+                for k in range(8):
+                    view[k] = 0
+                have = (addr, view)
+                self._hints[device] = have
+            return have
+
     def release(self):
         """Give back the device memory this loop holds (scratch buffers of two-phase launches),
         once the launches that use it have finished."""
@@ -677,6 +693,10 @@ class CompiledLoop:
                     rt.sync(key[1])
             for _key, ptr in held:
                 rt.free(ptr)
+            with self._lock:
+                hints, self._hints = self._hints, {}
+            for addr, _view in hints.values():
+                rt.host_free(addr)
         except Exception:           # the runtime may be shutting down
             pass
 
@@ -1020,6 +1040,13 @@ class Launch:
         widthlog = [0, 2, 4, 6]
         trip, _uniform = loop._estimate_trip(env, arrays, n)
         base = sum(1 for t in thresholds if trip > t)
+        # what the last launch of this loop that has got that far found in its classes (a hint: it may
+        # describe other arrays).  The class with most rows is the one to take in natural order; without
+        # long rows last time, this launch sets nothing up for parts (long rows, if there are some after
+        # all, then run whole).
+        hint_addr, hint = loop.hint(self.device)
+        seen = [int(hint[k]) for k in range(5)] if self.loop.options.get("hip_hints", True) else [0] * 5
+        known = seen[0] == 1 and sum(seen[1:]) == n and min(seen[1:]) >= 0
         parts, stripe, cap = 0, 0, 0
         gather = a.ragged[1]
         if gather is not None:
@@ -1033,19 +1060,26 @@ class Launch:
                 bound = max([int(arrays[nm].shape[0]) for _code, streamed in loop._simd_loops for nm in streamed
                              if arrays[nm].ndim == 1] or [0])
                 cap = min(n, bound // thresholds[2] + 1) if bound else n
+        if known:
+            # (the thresholds follow from element sizes and the size of the gathered operand, so the classes
+            #  of the hint are the classes of this launch whenever the hint is about these arrays)
+            base = max(range(4), key=lambda c: seen[c + 1])
+            if seen[4] == 0:
+                parts, stripe, cap = 0, 0, 0
         reds = max(1, len(loop_ir.reductions_of(a.team_split)))
-        # one buffer: counters | row lists of the four classes | part boundaries | partial results
+        # one buffer: counters | row lists of the four classes | part boundaries | row starts | partial results
         # header: 8 counters, 64 part loads (8 bytes each), and a second such block that the binning kernel
         # clears instead when it is not run to clear the first
         off_rows = 2048
         off_bnd = off_rows + 4 * 4 * n
-        off_part = (off_bnd + 4 * (parts + 1) * cap + 255) // 256 * 256
+        off_start = (off_bnd + 4 * (parts + 1) * cap + 255) // 256 * 256        # where each listed row starts (8 bytes)
+        off_part = (off_start + 8 * cap + 255) // 256 * 256
         total = off_part + 8 * reds * parts * cap
         buf = loop.scratch(self.device, self.stream, total)
         self.bin = {
             "counts": buf, "load": buf + 32, "zero": buf + 1024, "rows": buf + off_rows, "m": n, "base": base, "threshold": thresholds,
-            "widthlog": widthlog, "skip": cap if parts else 0, "bnd": buf + off_bnd, "cap": cap, "stripe": stripe,
-            "nrows": buf + 4 * 3, "tlo": thresholds[base - 1] if base > 0 else -(1 << 62),
+            "widthlog": widthlog, "skip": cap if parts else 0, "bnd": buf + off_bnd, "rowstart": buf + off_start, "cap": cap, "stripe": stripe,
+            "nrows": buf + 4 * 3, "hint": hint_addr, "tlo": thresholds[base - 1] if base > 0 else -(1 << 62),
             "thi": thresholds[base] if base < 3 else (1 << 62),
         }
         self.scratch_ptr = buf + off_part
@@ -1111,7 +1145,7 @@ class Launch:
                 val = self.nsplit
             elif p.role in ("threshold", "widthlog"):
                 val = self.bin[p.role][p.dim]
-            elif p.role in ("rows", "counts", "zero", "nrows", "bnd", "cap", "stripe", "m", "base", "skip", "tlo", "thi", "load"):
+            elif p.role in ("rows", "counts", "zero", "nrows", "bnd", "cap", "stripe", "m", "base", "skip", "tlo", "thi", "load", "hint", "rowstart"):
                 val = self.bin[p.role]
             elif p.role == "lo":
                 val = lo

@@ -1421,8 +1421,9 @@ class KernelBuilder:
         if self.spec.phase == 1 and self.spec.parts:
             # the part of this workgroup slot, as the planning kernel has cut the row (relative to its start)
             lo_c, hi_c = self.fresh("lo"), self.fresh("hi")
-            self.w(f"const appy::i64 {lo_c} = {lo_v} + __bnd[__chunk * __cap + __t];")
-            self.w(f"const appy::i64 {hi_c} = {lo_v} + __bnd[(__chunk + 1) * __cap + __t];")
+            self.w("const appy::i64 __first = __start[__t];     // (from the plan: no need to wait for the set-up's loads)")
+            self.w(f"const appy::i64 {lo_c} = __first + __bnd[__chunk * __cap + __t];")
+            self.w(f"const appy::i64 {hi_c} = __first + __bnd[(__chunk + 1) * __cap + __t];")
             lo_v, hi_v = lo_c, hi_c
         elif self.spec.phase == 1:
             part = self.fresh("part")
@@ -2245,6 +2246,15 @@ class KernelBuilder:
             self.w(f"const appy::i64 __n{c} = (__base == {c}) ? (__hi - __lo) : (__l{c} > 0 ? __l{c} : 0);")
             self.w(f"const appy::i64 __e{c} = {prev} + (((__n{c} << __wl{c}) + 63) >> 6);")
             prev = f"__e{c}"
+        # what the classes held this time, left where the host can see it when it stages the next launch
+        # (a hint for shaping that launch: which class to take in natural order, whether long rows exist)
+        self.w("if (blockIdx.x == 0 && threadIdx.x == 0) {")
+        self.w("    const appy::i64 __others = (__base == 0 ? 0 : (appy::i64)__counts[0]) + (__base == 1 ? 0 : (appy::i64)__counts[1]) "
+               "+ (__base == 2 ? 0 : (appy::i64)__counts[2]) + (__base == 3 ? 0 : (appy::i64)__counts[3]);")
+        for c in range(4):
+            self.w(f"    __hint[{c + 1}] = (__base == {c}) ? (__hi - __lo) - __others : (appy::i64)__counts[{c}];")
+        self.w("    __hint[0] = 1;")
+        self.w("}")
         self.w("for (appy::i64 __v = __wv; __v < __e3; __v += __nwv) {")
         self.ind += 1
         self.w("const int __c = (int)(__v >= __e0) + (int)(__v >= __e1) + (int)(__v >= __e2);")
@@ -2289,6 +2299,7 @@ class KernelBuilder:
             self.w(f"__shared__ unsigned long long __work[{S}];")
             self.w(f"if (threadIdx.x < {S}) __work[threadIdx.x] = 0;")
             self.w("__syncthreads();")
+            self.w("unsigned long long __mine = 0;      // elements in the part of this lane, over the rows of its team")
             self.w(f"for (appy::i64 __t = (appy::i64)blockIdx.x * {tpb} + __team; __t < __n; __t += (appy::i64)gridDim.x * {tpb}) {{")
             self.ind += 1
             self.mode = "team"
@@ -2317,17 +2328,17 @@ class KernelBuilder:
             self.w("}")
             self.w(f"__b = appy::team_running_max<{W}>(__b, __lane);")
             # (cuts are kept relative to the start of the row: 32 bits are enough whatever the array size)
-            self.w("if (__lane == 0) __bnd[__t] = 0;")
+            self.w("if (__lane == 0) { __bnd[__t] = 0; __start[__t] = __rlo; }")
             self.w(f"const appy::i64 __cut = (__lane < {S - 1} ? __b : __rhi) - __rlo;      // where part __lane ends")
             self.w(f"if (__lane < {S}) __bnd[(appy::i64)(__lane + 1) * __cap + __t] = (int)__cut;")
             self.w(f"const appy::i64 __before = appy::team_lane_below<{W}>(__cut, __lane);")
-            self.w(f"if (__lane < {S} && __cut > (__lane ? __before : 0)) "
-                   f"atomicAdd(&__work[__lane], (unsigned long long)(__cut - (__lane ? __before : 0)));")
+            self.w(f"if (__lane < {S} && __cut > (__lane ? __before : 0)) __mine += (unsigned long long)(__cut - (__lane ? __before : 0));")
             self.ind -= 1
             self.w("}")
             self.mode = "lane"
             self.ind -= 1
             self.w("}")
+            self.w(f"if (__lane < {S} && __mine) atomicAdd(&__work[__lane], __mine);")
             self.w("__syncthreads();")
             self.w(f"if (threadIdx.x < {S} && __work[threadIdx.x]) atomicAdd(&__load[threadIdx.x], __work[threadIdx.x]);")
             return
@@ -2346,17 +2357,18 @@ class KernelBuilder:
             self.w("    __most = __sum > __most ? __sum : __most;")
             self.w("}")
             self.w("const bool __even = __most * 16 <= __tot * 3;")
-            self.w(f"const appy::i64 __items = __n * (__even ? {S // 8} : {S});")
-            self.w(f"const appy::i64 __q0 = (__even ? (appy::i64)(blockIdx.x >> 3) : (appy::i64)blockIdx.x) * {tpb} + __team;")
-            self.w(f"const appy::i64 __dq = (__even ? (appy::i64)(gridDim.x >> 3) : (appy::i64)gridDim.x) * {tpb};")
-            self.w("for (appy::i64 __q = __q0; __q < __items; __q += __dq) {")
+            self.w(f"const appy::i64 __t0 = (__even ? (appy::i64)(blockIdx.x >> 3) : (appy::i64)blockIdx.x) * {tpb} + __team;")
+            self.w(f"const appy::i64 __dt = (__even ? (appy::i64)(gridDim.x >> 3) : (appy::i64)gridDim.x) * {tpb};")
+            self.w(f"for (appy::i64 __pass = 0; __pass < (__even ? {S // 8} : {S}); ++__pass) {{")
             self.ind += 1
-            self.w("const appy::i64 __pass = __q / __n;")
-            self.w("const appy::i64 __t = __q - __pass * __n;")
             self.w("const appy::i64 __chunk = __even ? (appy::i64)(blockIdx.x & 7) + 8 * __pass : __pass;")
+            self.w("for (appy::i64 __t = __t0; __t < __n; __t += __dt) {")
+            self.ind += 1
             body = self.a.outer.body
             at = next(k for k, st in enumerate(body) if st is self.a.team_split)
             self._split_iteration("(appy::i64)__rows[__t]", upto=at + 1)
+            self.ind -= 1
+            self.w("}")
             self.ind -= 1
             self.w("}")
         else:
@@ -2523,6 +2535,9 @@ class KernelBuilder:
             params.append(Param("__nrows", "const int* __nrows", C.c_void_p, "nrows"))
             params.append(Param("__bnd", ("int* __bnd" if sp.aux == "plan" else "const int* __bnd"), C.c_void_p, "bnd"))
             params.append(Param("__cap", "const appy::i64 __cap", C.c_int64, "cap"))
+            if sp.aux == "plan" or sp.phase == 1:
+                params.append(Param("__start", ("appy::i64* __start" if sp.aux == "plan" else "const appy::i64* __start"),
+                                    C.c_void_p, "rowstart"))
             if sp.aux == "plan":
                 params.append(Param("__stripe", "const appy::i64 __stripe", C.c_int64, "stripe"))
                 params.append(Param("__load", "unsigned long long* __load", C.c_void_p, "load"))
@@ -2538,6 +2553,7 @@ class KernelBuilder:
             for k in range(4):
                 params.append(Param(f"__wl{k}", f"const int __wl{k}", C.c_int32, "widthlog", dim=k))
             params.append(Param("__skip3", "const appy::i64 __skip3", C.c_int64, "skip"))
+            params.append(Param("__hint", "long long* __hint", C.c_void_p, "hint"))
             params.append(Param("__tlo", "const appy::i64 __tlo", C.c_int64, "tlo"))
             params.append(Param("__thi", "const appy::i64 __thi", C.c_int64, "thi"))
         params.append(Param("__lo", "const appy::i64 __lo", C.c_int64, "lo"))

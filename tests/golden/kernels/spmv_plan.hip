@@ -10,6 +10,7 @@ _spmv_kernel_loop_1_plan(
     const int* __nrows,
     int* __bnd,
     const appy::i64 __cap,
+    appy::i64* __start,
     const appy::i64 __stripe,
     unsigned long long* __load,
     const appy::i64 __lo,
@@ -22,6 +23,7 @@ _spmv_kernel_loop_1_plan(
     __shared__ unsigned long long __work[8];
     if (threadIdx.x < 8) __work[threadIdx.x] = 0;
     __syncthreads();
+    unsigned long long __mine = 0;      // elements in the part of this lane, over the rows of its team
     for (appy::i64 __t = (appy::i64)blockIdx.x * 32 + __team; __t < __n; __t += (appy::i64)gridDim.x * 32) {
         {
             const appy::i64 i = (appy::i64)__rows[__t];
@@ -44,13 +46,14 @@ _spmv_kernel_loop_1_plan(
                 __b = __a;
             }
             __b = appy::team_running_max<8>(__b, __lane);
-            if (__lane == 0) __bnd[__t] = 0;
+            if (__lane == 0) { __bnd[__t] = 0; __start[__t] = __rlo; }
             const appy::i64 __cut = (__lane < 7 ? __b : __rhi) - __rlo;      // where part __lane ends
             if (__lane < 8) __bnd[(appy::i64)(__lane + 1) * __cap + __t] = (int)__cut;
             const appy::i64 __before = appy::team_lane_below<8>(__cut, __lane);
-            if (__lane < 8 && __cut > (__lane ? __before : 0)) atomicAdd(&__work[__lane], (unsigned long long)(__cut - (__lane ? __before : 0)));
+            if (__lane < 8 && __cut > (__lane ? __before : 0)) __mine += (unsigned long long)(__cut - (__lane ? __before : 0));
         }
     }
+    if (__lane < 8 && __mine) atomicAdd(&__work[__lane], __mine);
     __syncthreads();
     if (threadIdx.x < 8 && __work[threadIdx.x]) atomicAdd(&__load[threadIdx.x], __work[threadIdx.x]);
 }

@@ -15,6 +15,7 @@ _spmv_kernel_loop_1(
     const int __wl2,
     const int __wl3,
     const appy::i64 __skip3,
+    long long* __hint,
     const appy::i64 __tlo,
     const appy::i64 __thi,
     const appy::i64 __lo,
@@ -35,6 +36,14 @@ _spmv_kernel_loop_1(
     const appy::i64 __l3 = (appy::i64)__counts[3] - __skip3;
     const appy::i64 __n3 = (__base == 3) ? (__hi - __lo) : (__l3 > 0 ? __l3 : 0);
     const appy::i64 __e3 = __e2 + (((__n3 << __wl3) + 63) >> 6);
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        const appy::i64 __others = (__base == 0 ? 0 : (appy::i64)__counts[0]) + (__base == 1 ? 0 : (appy::i64)__counts[1]) + (__base == 2 ? 0 : (appy::i64)__counts[2]) + (__base == 3 ? 0 : (appy::i64)__counts[3]);
+        __hint[1] = (__base == 0) ? (__hi - __lo) - __others : (appy::i64)__counts[0];
+        __hint[2] = (__base == 1) ? (__hi - __lo) - __others : (appy::i64)__counts[1];
+        __hint[3] = (__base == 2) ? (__hi - __lo) - __others : (appy::i64)__counts[2];
+        __hint[4] = (__base == 3) ? (__hi - __lo) - __others : (appy::i64)__counts[3];
+        __hint[0] = 1;
+    }
     for (appy::i64 __v = __wv; __v < __e3; __v += __nwv) {
         const int __c = (int)(__v >= __e0) + (int)(__v >= __e1) + (int)(__v >= __e2);
         const int __wl = __c == 0 ? __wl0 : __c == 1 ? __wl1 : __c == 2 ? __wl2 : __wl3;

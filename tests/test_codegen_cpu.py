@@ -141,7 +141,7 @@ def test_csr_rows_are_sorted_by_length_from_32768_rows_on():
     plan = body_of(f.kernel_for(Spec("team", block=256, vec=1, width=8, rows="list", parts=8, aux="plan")).src.text)
     assert "A_indices[__mid] < __target" in plan and "team_running_max<8>" in plan and "atomicAdd(&__load[threadIdx.x]" in plan
     parts = body_of(f.kernel_for(Spec("team", block=256, vec=4, width=16, phase=1, rows="list", parts=8)).src.text)
-    assert "(blockIdx.x & 7) + 8 * __pass" in parts and "__bnd[(__chunk + 1) * __cap + __t]" in parts
+    assert "(appy::i64)(blockIdx.x & 7) + 8 * __pass : __pass" in parts and "__bnd[(__chunk + 1) * __cap + __t]" in parts
     assert "__most * 16 <= __tot * 3" in parts                  # parts tied to XCDs only while their loads are even
     fold = body_of(f.kernel_for(Spec("team", block=256, vec=4, width=1, phase=2, rows="list", parts=8)).src.text)
     assert "__c < __nsplit" in fold and "y[i] = s" in fold

@@ -30,9 +30,20 @@ def plain(gpu):
     return selfcheck.kernels(hip_bins=False)
 
 
-def _loop(name, bins=True):
-    hits = [v[0] for kk, v in cg.code_cache.items() if kk[-1] == name and bool(v[0].options.get("hip_bins", True)) == bins]
+def _loop(name, bins=True, index_type="int32"):
+    """The compiled loop of function ``name`` (for `spmv`: the one for row pointers of ``index_type``)."""
+    hits = [v[0] for kk, v in cg.code_cache.items() if kk[-1] == name and bool(v[0].options.get("hip_bins", True)) == bins
+            and (name != "spmv" or v[0].analysis.arrays["A_indptr"].ty.name == index_type)]
     return hits[-1]
+
+
+def _forget(name="spmv"):
+    """Drop what earlier launches of the loop have reported about their rows (the hint that shapes
+    the next launch), so that a test sees the launch of a loop that knows nothing yet."""
+    for kk, v in cg.code_cache.items():
+        if kk[-1] == name:
+            for _addr, view in v[0]._hints.values():
+                view[0] = 0
 
 
 def _powerlaw(m, n, clip, seed, exponent=1.5):
@@ -47,6 +58,7 @@ def _powerlaw(m, n, clip, seed, exponent=1.5):
 def test_spmv_powerlaw_rows_are_binned_and_striped(k, plain, m, n, clip):
     data, indptr, indices, x, lengths = _powerlaw(m, n, clip, seed=m)
     ref, budget = vo.spmv_csr(data, indptr, indices, x, (m, n))
+    _forget()
     y = k.spmv(data, indptr, indices, x, m, n)
     launch = _loop("spmv").last_launch
     assert launch.spec.rows == "mixed" and launch.sequence is not None
@@ -68,9 +80,15 @@ def test_spmv_uniform_rows_stay_in_their_natural_order(k, plain):
     m = 50_000
     data, indptr, indices, x = wl.spmv_uniform(m, 1 << 20, 16)
     ref, budget = vo.spmv_csr(data, indptr, indices, x, (m, 1 << 20))
+    _forget()
     y = k.spmv(data, indptr, indices, x, m, 1 << 20)
     launch = _loop("spmv").last_launch
     assert launch.spec.rows == "mixed" and launch.bin["base"] == 1      # 16 per row: the class of teams of four
+    assert len(launch.sequence) == 6                                    # nothing known yet: set up for long rows too
+    # the launch has reported what its classes held: the next one sets nothing up for long rows
+    y2 = k.spmv(data, indptr, indices, x, m, 1 << 20)
+    again = _loop("spmv").last_launch
+    assert len(again.sequence) == 3 and again.bin["base"] == 1 and np.array_equal(y, y2)
     assert vo.within_budget(y, ref, budget, TOL)[0]
     assert np.array_equal(y, plain.spmv(data, indptr, indices, x, m, 1 << 20))
 
@@ -125,6 +143,33 @@ def test_spmv_columns_in_any_order_and_int64_indices(k):
     assert ok, worst
 
 
+def test_the_hint_of_an_earlier_launch_shapes_the_next_one_and_never_its_results(k):
+    """The kernel over the binned rows reports the sizes of its classes in page-locked memory.  The next
+    launch takes the most populous class in natural order and leaves out the kernels for long rows when
+    there were none; a matrix that has long rows after all is still computed correctly (its long rows
+    then run whole), and the launch after that cuts them into parts again."""
+    m, n = 40_000, 1 << 20
+    short = wl.spmv_uniform(m, n, 3)                        # every row in the class of single lanes
+    data, indptr, indices, x, lengths = _powerlaw(m, n, 4096, seed=77)
+    _forget()
+    y = k.spmv(*short, m, n)
+    first = _loop("spmv").last_launch
+    assert first.bin["base"] == 0 and len(first.sequence) == 6
+    ref, budget = vo.spmv_csr(*short, (m, n))
+    assert vo.within_budget(y, ref, budget, TOL)[0]
+    ref, budget = vo.spmv_csr(data, indptr, indices, x, (m, n))
+    y1 = k.spmv(data, indptr, indices, x, m, n)             # shaped by the hint of the short rows
+    second = _loop("spmv").last_launch
+    assert len(second.sequence) == 3 and second.bin["skip"] == 0
+    ok, worst = vo.within_budget(y1, ref, budget, TOL)
+    assert ok, worst
+    y2 = k.spmv(data, indptr, indices, x, m, n)             # now it is known to have long rows
+    third = _loop("spmv").last_launch
+    assert len(third.sequence) == 6 and third.bin["base"] == int(np.argmax(np.bincount(np.digitize(lengths, [4, 32, 128], right=True), minlength=4)))
+    ok, worst = vo.within_budget(y2, ref, budget, TOL)
+    assert ok, worst
+
+
 def test_spmv_columns_crowded_into_one_stripe(k):
     """Every long row has its columns in the first eighth of the vector: the parts of the other seven
     stripes are empty, and the parts are dealt to all workgroups instead of one XCD per stripe."""
@@ -134,6 +179,7 @@ def test_spmv_columns_crowded_into_one_stripe(k):
     data, indptr, indices = wl.csr_matrix(lengths, n // 8, rng)          # columns below n / 8 only
     x = rng.standard_normal(n, dtype=np.float32)
     ref, budget = vo.spmv_csr(data, indptr, indices, x, (m, n))
+    _forget()
     y = k.spmv(data, indptr, indices, x, m, n)
     assert _loop("spmv").last_launch.nsplit == 8
     ok, worst = vo.within_budget(y, ref, budget, TOL)
@@ -171,6 +217,7 @@ def test_more_long_rows_than_the_streamed_arrays_account_for(k):
     y = np.empty(m, dtype=np.float32)
     windows(data, start, length, indices, x, y, m)
     launch = _loop("windows").last_launch
+    assert len(launch.sequence) == 6
     assert launch.sequence is not None and launch.bin["cap"] < int((length > launch.bin["threshold"][2]).sum())
     terms = data.astype(np.float64) * x.astype(np.float64)[indices]
     cs = np.concatenate([[0.0], np.cumsum(terms)])
