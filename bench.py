@@ -48,14 +48,14 @@ def load_profile_traffic(path=TRAFFIC_PROFILE):
     for ln in lines:
         parts = ln.split()
         if parts[:1] == ["calibration"]:
-            kv = dict(p.split("=", 1) for p in parts[1:])
+            kv = dict(p.split("=", 1) for p in parts[1:] if "=" in p)
             fs, ws = float(kv["fetch_scale"]), float(kv["write_scale"])
     if fs is None:
         return out
     for ln in lines:
         parts = ln.split()
         if parts[:1] == ["traffic"] and len(parts) >= 5:
-            kv = dict(p.split("=", 1) for p in parts[2:])
+            kv = dict(p.split("=", 1) for p in parts[2:] if "=" in p)
             out[parts[1]] = (kv["spec"], int((float(kv["fetch_kib"]) * fs + float(kv["write_kib"]) * ws) * 1024))
     return out
 
