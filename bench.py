@@ -10,8 +10,12 @@ over K steps between device synchronisations.  ``roofline`` gives the same
 kernel's algorithmic bytes per launch divided by its mean launch duration
 measured with HIP events on the launch stream, against the 8 TB/s HBM peak.
 ``kernels`` lists the same figures for the other generated kernels
-(vec_add, masked_sum, GEMV, CSR SpMV uniform and power-law, CSR SpMM), each
-checked against the float64 oracle on the identical inputs in the same run.
+(vec_add at 2^24 and 2^27, masked_sum, GEMV, CSR SpMV uniform and power-law, CSR SpMM), each
+checked against the float64 oracle on the identical inputs in the same run; a launch
+that is a sequence of kernels (CSR rows sorted by length) is timed as a whole.
+``roofline`` also says which kernel of configs 1-4 is furthest from the roofline and
+which of their bars are met.  HBM traffic per launch comes from the committed
+summary of the rocprofv3 counter runs of this program (``profiles/``).
 ``cpu_baseline`` times the oracle (NumPy, one core) on the host.
 """
 from __future__ import annotations
