@@ -534,7 +534,9 @@ class CompiledLoop:
                 # pure streaming beyond the memory-side cache: one tile per workgroup, loads and stores
                 # non-temporal (copy: 0.82 of peak against 0.67), in large workgroups (c = a + b over 2^27
                 # floats: 0.82 of peak with 1024 lanes, 0.78 with 256; copy does best with 512: 0.815 / 0.81)
-                block = 1024 if len(self._indexed_arrays()) >= 3 else 512
+                # (a store-only loop, c[i] = v over 2^28 floats: 0.85 of peak with 256 lanes, 0.79 / 0.78 with 512 / 1024)
+                streams = len(self._indexed_arrays())
+                block = 1024 if streams >= 3 else (512 if streams == 2 else 256)
                 return Spec("flat", block=block, vec=d.vec, unroll=1, restrict=restrict,
                             stream_loads=True, stream_stores=True)
             if stream and self.analysis.outer_reductions:
