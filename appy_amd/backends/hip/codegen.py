@@ -87,6 +87,8 @@ BIN_MIN_ROWS = 1 << 15
 # XCD and its 4 MiB L2) of at most STRIPE_BYTES each, or a multiple of eight
 STRIPE_MIN_BYTES = 3 << 20
 STRIPE_BYTES = 2 << 20
+GROUP_MAX_STRIPE_LOG = 19          # elements grouped by stripe: stripes of 2^19 elements of 4 bytes (half an L2) at most, 8 or 16 of them
+GROUP_MIN_TRIP = 4                 # ... for rows of this many elements on average, at least
 
 
 def device_header() -> str:
@@ -321,6 +323,7 @@ class CompiledLoop:
             name: (None if node is None else compile(ast.Expression(body=ast.fix_missing_locations(_copy(node))), "<n>", "eval"))
             for name, node in a.overwritten.items()}
         self._scratch = {}  # (device, stream) -> (device pointer, bytes): partial results of two-phase launches
+        self._group_off = False     # a kernel of the grouped form could not be generated for this loop
         self._hints = {}    # device -> (address, ctypes view) of page-locked words the binned kernels report to
         self._scratch_retired = []
         self._replays = {}  # call identity -> Launch that can simply be launched again
@@ -1004,6 +1007,9 @@ class Launch:
             self.scratch_ptr = loop.scratch(device, self.stream, max(1, reds) * self.nsplit * n_outer * 8)
         self.scalar_fields = {}      # by-value scalar -> field of the argument block
         self.sequence = None         # binned rows: [(kernel, argument block, grid, block)] launched in this order
+        if spec.rows == "mixed" and self._stage_grouped(vals, arrays, lo, hi, spec):
+            loop.last_launch = self
+            return
         if spec.rows == "mixed":
             self._stage_binned(vals, arrays, lo, hi, spec)
             self.args = self.sequence[2][1]
@@ -1117,6 +1123,72 @@ class Launch:
                         (max(1, min(1024, -(-cap // 256))), 1, 1), (256, 1, 1)))
         self.sequence = seq
 
+    def _stage_grouped(self, vals, arrays, lo, hi, spec) -> bool:
+        """The launches of a loop of short rows whose simd loop sums terms that gather from an operand
+        larger than an L2: group the elements of every 256 rows by the stripe of the operand they read
+        (`group`), run the groups, stripe s on XCD s mod 8, sums per row and stripe to the scratch buffer
+        (`cells`), add the sums of a row and run the rest of the body (phase 2).  The grouping kernel
+        checks that the rows' ranges follow one another (as those of a CSR matrix do); where they do
+        not, it raises a flag, the kernels after it return at once, and the loop runs row by row.
+        False (nothing staged) when the launch does not qualify."""
+        loop, a, env = self.loop, self.loop.analysis, self.env
+        n = hi - lo
+        g = a.grouping
+        if g is None or loop._group_off or not loop.options.get("hip_group", True) or not loop.options.get("hip_hints", True):
+            return False
+        V = spec.vec
+        _addr, hint = loop.hint(self.device)
+        seen = [int(hint[k]) for k in range(5)]
+        # the last launch has sorted these rows and found none in the class of the longest
+        if not (seen[0] == 1 and sum(seen[1:]) == n and min(seen[1:]) >= 0 and seen[4] == 0):
+            return False
+        x = arrays[g["x"]]
+        nx = int(x.shape[0])
+        if nx * 4 <= STRIPE_MIN_BYTES or nx > (16 << GROUP_MAX_STRIPE_LOG):
+            return False
+        parts = 8 if nx <= (8 << GROUP_MAX_STRIPE_LOG) else 16
+        shift = max(1, (-(-nx // parts) - 1).bit_length())
+        entries = min(int(arrays[nm].shape[0]) for nm in (g["idx"], g["carried"]) if nm)
+        trip, _uniform = loop._estimate_trip(env, arrays, n)
+        if entries >= (1 << 31) or trip < GROUP_MIN_TRIP:
+            return False
+        R = 256
+        nblk = -(-n // R)
+        common = dict(block=256, restrict=spec.restrict)
+        try:
+            group = loop.kernel_for(Spec("team", vec=1, width=64, parts=parts, aux="group", **common))
+            cells = loop.kernel_for(Spec("team", vec=1, width=64, parts=parts, aux="cells", guard=1, **common))
+            fold = loop.kernel_for(Spec("team", vec=V, width=1, phase=2, guard=1, **common))
+            plain = loop._choose_spec(n, env, arrays, restrict=spec.restrict, listable=False)
+            if plain.kind != "team" or plain.phase or plain.rows:
+                raise Unsupported("no plain team kernel to fall back to")
+            rest = loop.kernel_for(dataclasses.replace(plain, guard=2))
+        except Unsupported:
+            loop._group_off = True
+            return False
+        # one buffer: header (the flag) | where the cells start | the grouped elements | sums per row and stripe
+        off_desc = 2048
+        off_ent = (off_desc + 4 * (parts + 1) * nblk + 255) // 256 * 256
+        off_part = (off_ent + 8 * entries + 255) // 256 * 256
+        buf = loop.scratch(self.device, self.stream, off_part + 4 * parts * n)
+        hint_addr, _ = loop.hint(self.device)
+        self.bin = {"flag": buf + 1984, "desc": buf + off_desc, "ent": buf + off_ent, "shiftc": shift, "entries": entries,
+                    "rowmax": 32 * V, "hint": hint_addr}
+        self.scratch_ptr = buf + off_part
+        self.nsplit = parts
+        seq = [(None, (buf + 1984, 8), None, None)]         # the flag starts at zero
+        seq.append((group, self._argument_block(group, vals, arrays, lo, hi), (max(1, min(1 << 20, -(-nblk // 4))), 1, 1), (256, 1, 1)))
+        seq.append((cells, self._argument_block(cells, vals, arrays, lo, hi), (8 * max(1, min(8192, -(-nblk // 4))), 1, 1), (256, 1, 1)))
+        seq.append((fold, self._argument_block(fold, vals, arrays, lo, hi), (max(1, min(4096, -(-n // 256))), 1, 1), (256, 1, 1)))
+        # (the kernel that runs the loop row by row when the input was refused: few workgroups that loop - it returns at
+        #  once otherwise, and 65536 workgroups take 15 us to do that, 1024 take 3)
+        seq.append((rest, self._argument_block(rest, vals, arrays, lo, hi),
+                    (min(1024, loop.grid_for(plain, n, kernel=rest, row_hint=loop.row_hint(n, env, arrays))), 1, 1), (plain.block, 1, 1)))
+        self.sequence = seq
+        self.kernel, self.spec = cells, cells.src.spec
+        self.args, self.grid, self.block = seq[2][1], seq[2][2], seq[2][3]
+        return True
+
     def _argument_block(self, kernel, vals, arrays, lo, hi):
         loop = self.loop
         st = kernel.ArgStruct()
@@ -1147,7 +1219,8 @@ class Launch:
                 val = self.nsplit
             elif p.role in ("threshold", "widthlog"):
                 val = self.bin[p.role][p.dim]
-            elif p.role in ("rows", "counts", "zero", "nrows", "bnd", "cap", "stripe", "m", "base", "skip", "tlo", "thi", "load", "hint", "rowstart"):
+            elif p.role in ("rows", "counts", "zero", "nrows", "bnd", "cap", "stripe", "m", "base", "skip", "tlo", "thi", "load", "hint", "rowstart",
+                            "flag", "desc", "ent", "shiftc", "entries", "rowmax"):
                 val = self.bin[p.role]
             elif p.role == "lo":
                 val = lo
@@ -1217,7 +1290,10 @@ class Launch:
             # the kernels share the loop's scratch buffer for this stream: queued as one run
             with self.loop._lock:
                 for kernel, args, grid, block in self.sequence:
-                    rt.launch(kernel.function(self.device), grid, block, args, self.stream)
+                    if kernel is None:
+                        rt.memset_async(args[0], 0, args[1], self.stream)
+                    else:
+                        rt.launch(kernel.function(self.device), grid, block, args, self.stream)
         elif self.second is None:
             rt.launch(self.function(), self.grid, self.block, self.args, self.stream)
         else:
@@ -1342,7 +1418,7 @@ def _copy(node):
 def codegen(loop_source, loop_name, val_map, options):
     key = (loop_source, loop_name, _signature(val_map), options.get("hip_spec") and repr(options.get("hip_spec")),
            options.get("hip_max_blocks"), bool(options.get("check_bounds")), bool(options.get("hip_bins", True)),
-           options.get("fn_name"))
+           bool(options.get("hip_group", True)), options.get("fn_name"))
     # `clear_cache=True` regenerates the loop on every call instead of using the cached kernel
     # (reference: appy/backends/metal/codegen.py:23)
     fresh = bool(options.get("clear_cache"))

@@ -82,7 +82,13 @@ class Spec:
                                  # boundaries a planning kernel has written (column stripes of a gathered operand),
                                  # one part per workgroup slot, the stripes dealt to the XCDs by workgroup number
     aux: str = ""                # 'bins' = the kernel that sorts rows into classes, 'plan' = the kernel that finds
-                                 # the part boundaries of listed rows; '' = a kernel that runs the loop body
+                                 # the part boundaries of listed rows; 'group' = the kernel that groups the elements
+                                 # of every block of rows by the stripe of the gathered operand they read, 'cells' =
+                                 # the kernel that runs those groups (`parts` stripes, dealt to the XCDs by workgroup
+                                 # number); '' = a kernel that runs the loop body
+    guard: int = 0               # 1 = the kernel returns at once when the grouping kernel of this launch has refused
+                                 # its input (row ranges that do not follow one another: a flag in device memory),
+                                 # 2 = when it has not
 
     def __post_init__(self):
         def pow2(n):
@@ -101,18 +107,24 @@ class Spec:
         if self.checked and (self.vec != 1 or self.unroll != 1 or self.extent or self.lds_tile):
             raise ValueError("a bounds-checked kernel takes one element per access (vec = unroll = 1, no row extent, no LDS tile)")
         if self.phase not in (0, 1, 2) or (self.phase and not (
-                self.kind == "strip" or (self.kind == "team" and (self.width in (64, self.block) or self.rows == "list")
+                self.kind == "strip" or (self.kind == "team" and (self.width in (64, self.block) or self.rows == "list"
+                                                                 or (self.phase == 2 and self.guard == 1))
                                          and not self.extent and not self.lds_tile and not self.collapse))):
             raise ValueError("only strip kernels, teams of a whole wavefront or workgroup, and teams over listed rows "
                              "run in two phases")
-        if self.rows not in ("", "mixed", "list") or self.aux not in ("", "bins", "plan"):
+        if self.rows not in ("", "mixed", "list") or self.aux not in ("", "bins", "plan", "group", "cells"):
             raise ValueError(f"unknown row source {self.rows!r} / auxiliary kernel {self.aux!r}")
         if (self.rows or self.aux) and (self.kind != "team" or self.extent or self.lds_tile or self.collapse
                                         or self.row_steps or self.checked or self.width > 64):
             raise ValueError("rows are binned for plain team kernels only (teams inside a wavefront)")
-        if self.parts and (self.rows != "list" or not (self.phase or self.aux == "plan") or self.parts % 8
-                           or not 8 <= self.parts <= 64):
+        if self.aux in ("group", "cells"):
+            if self.rows or self.phase or self.parts not in (8, 16) or self.width != 64 or self.block != 256:
+                raise ValueError("elements are grouped by 8 or 16 stripes, one wavefront per block of rows, four per workgroup")
+        elif self.parts and (self.rows != "list" or not (self.phase or self.aux == "plan") or self.parts % 8
+                             or not 8 <= self.parts <= 64):
             raise ValueError("planned parts belong to the two-phase kernels over listed rows (8, 16, ... 64 parts)")
+        if self.guard not in (0, 1, 2) or (self.guard and self.kind != "team"):
+            raise ValueError("only team kernels wait on the verdict of a grouping kernel (guard 1 or 2)")
         if self.aux == "plan" and (self.rows != "list" or not self.parts or self.width < self.parts):
             raise ValueError("the planning kernel takes listed rows, with one lane per part at least")
         if self.row_steps and (self.kind != "team" or self.phase or self.extent or self.lds_tile or self.vec < 2
@@ -128,7 +140,8 @@ class Spec:
                 f"{'_r' if self.restrict else ''}{'_nt' if self.stream_loads else ''}"
                 f"{'_e' + str(self.extent) if self.extent else ''}{'_nts' if self.stream_stores else ''}"
                 f"{'_lds' + str(self.lds_tile) if self.lds_tile else ''}{'' if self.hoist_guarded else '_g'}{'_chk' if self.checked else ''}{'_c2' if self.collapse else ''}{'_p' + str(self.phase) if self.phase else ''}{'_rc' + str(self.row_steps) if self.row_steps else ''}"
-                f"{'_' + self.rows if self.rows else ''}{'_s' + str(self.parts) if self.parts else ''}{'_' + self.aux if self.aux else ''}")
+                f"{'_' + self.rows if self.rows else ''}{'_s' + str(self.parts) if self.parts else ''}{'_' + self.aux if self.aux else ''}"
+                f"{'_if' + str(self.guard) if self.guard else ''}")
 
 
 @dataclass
@@ -477,6 +490,61 @@ class LoopAnalysis:
                 pairs.add((x.name, idx.name))
         gather = next(iter(pairs)) if len(pairs) == 1 else None
         return loop, gather
+
+    def _find_grouping(self):
+        """``{"x", "idx", "carried", "stmt", "name"}`` when the ``simd`` loop of a ragged nest is nothing
+        but ``s += f(A[j], X[IDX[j]])``: one sum into a scalar whose terms read the gathered operand
+        ``X`` through ``IDX``, at most one other array ``A`` (``carried``) at the loop's own position, and
+        values that do not change from row to row.  The terms of such a loop can be computed in any
+        grouping - by column stripe of ``X`` instead of by row - and added to their rows afterwards.
+        ``X``, ``IDX`` and ``A`` have 4-byte elements (``IDX`` signed)."""
+        if self.ragged is None or self.ragged[1] is None:
+            return None
+        loop = self.team_split
+        x_name, idx_name = self.ragged[1]
+        reds = loop_ir.reductions_of(loop)
+        if len(reds) != 1 or len(loop.body) != 1:
+            return None
+        (name, op), = reds.items()
+        st = loop.body[0]
+        if not (op == "+" and isinstance(st, ast.Assign) and getattr(st, "reduce", None) == "+"
+                and isinstance(st.targets[0], ast.Name) and st.targets[0].id == name):
+            return None
+        x, idx = self.arrays[x_name], self.arrays[idx_name]
+        if x.ty.size != 4 or x.ty.is_bool or idx.ty.name != "int32":
+            return None
+        jv = loop.target.id
+        term = loop_ir.reduction_operand(st)
+        gather = f"{x_name}[{idx_name}[{jv}]]"
+        carried = set()
+        covered = set()          # subscript nodes that are (part of) an accepted load
+
+        def accept(n):
+            for m in ast.walk(n):
+                covered.add(id(m))
+
+        for n in ast.walk(term):
+            if id(n) in covered:
+                continue
+            if isinstance(n, ast.Subscript):
+                text = ast.unparse(n)
+                if text == gather:
+                    accept(n)
+                    continue
+                arr = self.arrays.get(n.value.id) if isinstance(n.value, ast.Name) else None
+                if (arr is None or arr.ndim != 1 or arr.name in self.stored or arr.ty.size != 4 or arr.ty.is_bool
+                        or not (isinstance(n.slice, ast.Name) and n.slice.id == jv) or arr.name == idx_name):
+                    return None
+                carried.add(arr.name)
+                accept(n)
+            elif isinstance(n, ast.Name) and isinstance(n.ctx, ast.Load):
+                if n.id == jv or n.id == self.var or n.id in self.assigned or n.id in self.arrays:
+                    return None
+            elif isinstance(n, (ast.Lambda, ast.NamedExpr, ast.ListComp, ast.Starred)):
+                return None
+        if len(carried) > 1 or gather not in ast.unparse(term):
+            return None
+        return {"x": x_name, "idx": idx_name, "carried": next(iter(carried), None), "stmt": st, "name": name}
 
     def split_needs_finish(self) -> bool:
         """True if the two-phase form of a team nest needs its second kernel (the loop
@@ -829,6 +897,7 @@ class LoopAnalysis:
                         if item not in self.affine_checks:
                             self.affine_checks.append(item)
         self.ragged = self._find_ragged()
+        self.grouping = self._find_grouping()
 
 
 def _partial_type(ty: Ty) -> Ty:
@@ -1930,6 +1999,9 @@ class KernelBuilder:
         if self.spec.rows == "list":
             # listed rows: the slot follows the position in the list, `__cap` rows at most
             return f"*reinterpret_cast<{pty.c}*>(__scratch + (({r} * __nsplit + {chunk}) * __cap + __t))"
+        if self.spec.guard == 1 and pty.size == 4:
+            # sums of grouped elements: 4-byte slots
+            return f"reinterpret_cast<{pty.c}*>(__scratch)[({r} * __nsplit + {chunk}) * (__hi - __lo) + ({var} - __lo)]"
         return f"*reinterpret_cast<{pty.c}*>(__scratch + (({r} * __nsplit + {chunk}) * (__hi - __lo) + ({var} - __lo)))"
 
     def strip_spread_loop(self, st: ast.For):
@@ -2084,9 +2156,16 @@ class KernelBuilder:
         var = self.a.var
         self.ex.locals[var] = T.WEAK_INT
         self.lds_plan = self._find_lds_plan()
+        if s.guard:
+            # the grouping kernel of this launch raises the flag when it refuses its input
+            self.w(f"if ((__flag[0] != 0) == {'true' if s.guard == 1 else 'false'}) return;")
         if s.aux or s.rows:
             if self.a.ragged is None or self.lds_plan is not None:
                 raise Unsupported("the loop nest does not suit kernels over binned rows")
+            if s.aux in ("group", "cells"):
+                if self.a.grouping is None:
+                    raise Unsupported("the simd loop is not a sum of terms that gather from one operand")
+                return self._body_group() if s.aux == "group" else self._body_cells()
             if s.aux == "bins":
                 return self._body_bins()
             if s.rows == "mixed":
@@ -2379,6 +2458,274 @@ class KernelBuilder:
             self.w("}")
         self.mode = "lane"
 
+    # ---- elements grouped by the stripe of the gathered operand they read -------------------------------
+    # Blocks of 256 rows, one wavefront each.  The grouping kernel writes the elements of a block - the
+    # 32 bits of the carried operand, the row within the block (8 bits) and the position within the stripe
+    # (24 bits) - over the block's own range of positions, stripe after stripe, and where every stripe
+    # starts (`__desc`, `parts + 1` numbers per block).  A cell is one stripe of one block.
+    GROUP_ROWS = 256
+
+    def _group_setup_types(self):
+        """Walks the set-up of an iteration and the term of the sum into a buffer that is thrown away:
+        the types of the locals settle as they do in the kernels that run the loop row by row.
+        Returns (code of the term with `__cv` / `__cx` for the two loads, its type, partial type)."""
+        a, g = self.a, self.a.grouping
+        body = a.outer.body
+        at = next(k for k, st in enumerate(body) if st is a.team_split)
+        kept, self.lines = self.lines, []
+        saved_mode, self.mode = self.mode, "lane"
+        self.ex.locals[a.team_split.target.id] = T.WEAK_INT
+        self.block(body[:at])
+        name = g["name"]
+        ty = self.ex.locals.get(name)
+        if ty is None:
+            raise NameError(f"reduction variable `{name}` has no value before the loop")
+        jv = a.team_split.target.id
+        x, idx = a.arrays[g["x"]], a.arrays[g["idx"]]
+        saved = dict(self.ex.load_subst)
+        self.ex.load_subst[f"{g['x']}[{g['idx']}[{jv}]]"] = ("__cx", x.ty)
+        if g["carried"]:
+            self.ex.load_subst[f"{g['carried']}[{jv}]"] = ("__cv", a.arrays[g["carried"]].ty)
+        oc, ot = self.ex.emit(loop_ir.reduction_operand(g["stmt"]))
+        self.ex.load_subst = saved
+        pty = _partial_type(ty)
+        self.set_local(name, T.promote(ty, ot))
+        self.lines, self.mode = kept, saved_mode
+        return oc, ot, pty
+
+    def _body_group(self):
+        a, g, S, R = self.a, self.a.grouping, self.spec.parts, self.GROUP_ROWS
+        var = a.var
+        self.ex.locals[var] = T.WEAK_INT
+        self.mode = "lane"
+        idx_c = cname(g["idx"])
+        a.arrays[g["idx"]].loaded = True
+        car_c = f"reinterpret_cast<const int*>({cname(g['carried'])})" if g["carried"] else None
+        body = a.outer.body
+        at = next(k for k, st in enumerate(body) if st is a.team_split)
+        U = 4       # vectors of four elements per lane and step
+        w = self.w
+        w("const int __lid = threadIdx.x & 63;")
+        w("const int __wvl = threadIdx.x >> 6;")
+        w(f"__shared__ int __lp_all[4][{R + 1}];      // where the rows of the block start; the last entry: where it ends")
+        w(f"__shared__ int __hq_all[4][{R}];          // where they end")
+        w("int* __lp = __lp_all[__wvl];")
+        w("int* __hq = __hq_all[__wvl];")
+        w(f"const appy::i64 __nblk = (__hi - __lo + {R - 1}) / {R};")
+        w("const int __cmask = (1 << __shiftc) - 1;")
+        w("const unsigned long long __below = (1ull << __lid) - 1ull;")
+        w("for (appy::i64 __b = (appy::i64)blockIdx.x * 4 + __wvl; __b < __nblk; __b += (appy::i64)gridDim.x * 4) {")
+        self.ind += 1
+        w(f"const appy::i64 __r0 = __lo + __b * {R};")
+        w(f"const int __nr = (int)((__hi - __r0) < {R} ? (__hi - __r0) : {R});")
+        w("appy::wave_fence();       // the block before this one has been read out of __lp")
+        w("bool __good = true, __long = false;")
+        w("#pragma unroll")
+        w(f"for (int __k = 0; __k < {R // 64 + 1}; ++__k) {{      // and the first row of the next block, if there is one")
+        self.ind += 1
+        w("const int __r = __k * 64 + __lid;")
+        w(f"if (__r <= __nr && __r0 + __r < __hi && (__k < {R // 64} || __lid == 0)) {{")
+        self.ind += 1
+        w(f"const appy::i64 {cname(var)} = __r0 + __r;")
+        self._declare_locals()
+        self.block(body[:at])
+        lo, hi = self._range_args(a.team_split)
+        w(f"const appy::i64 __rlo = {lo};")
+        w(f"const appy::i64 __rhi = {hi};")
+        w("if (__rlo < 0 || __rhi < __rlo || __rhi > __len) __good = false;")
+        w("__lp[__r] = (int)__rlo;")
+        w("if (__r < __nr) { __hq[__r] = (int)__rhi; __long = __long || (__rhi - __rlo > __rowmax); }")
+        self.ind -= 1
+        w("}")
+        self.ind -= 1
+        w("}")
+        w("appy::wave_fence();")
+        w("// every row ends where the next one starts; the block ends no later than the next one starts")
+        w("#pragma unroll")
+        w(f"for (int __k = 0; __k < {R // 64}; ++__k) {{")
+        w("    const int __r = __k * 64 + __lid;")
+        w("    if (__r < __nr - 1) __good = __good && __lp[__r + 1] == __hq[__r];")
+        w("    else if (__r == __nr - 1 && __r0 + __nr < __hi) __good = __good && __lp[__nr] >= __hq[__r];")
+        w("}")
+        w("__good = __ballot(!__good) == 0ull;")
+        w("if (__ballot(__long) != 0ull && __lid == 0) __hint[0] = 2;      // rows too long for this treatment: the next launch sorts them")
+        w("const int __first = __good ? __lp[0] : 0, __end = __good ? __hq[__nr - 1] : 0;")
+        w("appy::wave_fence();")
+        w("#pragma unroll")
+        w(f"for (int __k = 0; __k < {R // 64 + 1}; ++__k) {{")
+        w("    const int __r = __k * 64 + __lid;")
+        w(f"    if (__r >= __nr && __r <= {R} && (__k < {R // 64} || __lid == 0)) __lp[__r] = __end;")
+        w("}")
+        w("appy::wave_fence();")
+        w("if (!__good) {")
+        w("    // refused: the launch runs the loop row by row instead; the cells of this block stay empty")
+        w("    if (__lid == 0) __flag[0] = 1;")
+        w(f"    if (__lid <= {S}) __desc[__b * {S + 1} + __lid] = 0;")
+        w("    continue;")
+        w("}")
+        def load_indices(k, j0, kk):
+            w(f"{{ const int __j = {j0} + {kk} * 256 + __lid * 4;")
+            w(f"if (__j + 4 <= __end) __c[{k}] = appy::vload<int, 4>({idx_c} + __j);")
+            w("else {")
+            w("#pragma unroll")
+            w(f"    for (int __q = 0; __q < 4; ++__q) __c[{k}][__q] = __j + __q < __end ? {idx_c}[__j + __q] : -1;")
+            w("} }")
+
+        def load_carried(k, j0, kk):
+            if car_c:
+                w(f"{{ const int __j = {j0} + {kk} * 256 + __lid * 4;")
+                w(f"if (__j + 4 <= __end) __v[{k}] = appy::vload<int, 4>({car_c} + __j);")
+                w("else {")
+                w("#pragma unroll")
+                w(f"    for (int __q = 0; __q < 4; ++__q) __v[{k}][__q] = __j + __q < __end ? {car_c}[__j + __q] : 0;")
+                w("} }")
+            else:
+                w(f"__v[{k}] = 0;")
+
+        def count(k):
+            w("#pragma unroll")
+            w("for (int __q = 0; __q < 4; ++__q)")
+            w("#pragma unroll")
+            w(f"    for (int __s = 0; __s < {S}; ++__s) __cnt[__s] += __popcll(__ballot((__c[{k}][__q] >> __shiftc) == __s));")
+
+        def starts():
+            w("__at[0] = __first;")
+            w("#pragma unroll")
+            w(f"for (int __s = 0; __s < {S}; ++__s) __at[__s + 1] = __at[__s] + __cnt[__s];")
+            w("#pragma unroll")
+            w(f"for (int __s = 0; __s <= {S}; ++__s) if (__lid == __s) __desc[__b * {S + 1} + __s] = __at[__s];")
+
+        def place(kc, kv, j0, kk):
+            w(f"const int __j = {j0} + {kk} * 256 + __lid * 4;")
+            w(f"int __row = 0, __past = {R};       // the last row that starts at or before __j")
+            w("#pragma unroll")
+            w(f"for (int __it = 0; __it < {R.bit_length() - 1}; ++__it) {{")
+            w("    const int __mid = (__row + __past) >> 1;")
+            w("    if (__lp[__mid] <= __j) __row = __mid; else __past = __mid;")
+            w("}")
+            w("#pragma unroll")
+            w("for (int __q = 0; __q < 4; ++__q) {")
+            self.ind += 1
+            w(f"const int __cq = __c[{kc}][__q];")
+            w("const int __sq = __cq >> __shiftc;          // negative past the end (and for negative indices: such elements are dropped)")
+            w("if (__j + __q < __end) while (__lp[__row + 1] <= __j + __q) ++__row;")
+            w("int __pos = 0;")
+            w("#pragma unroll")
+            w(f"for (int __s = 0; __s < {S}; ++__s) {{")
+            w("    const unsigned long long __m = __ballot(__sq == __s);")
+            w("    if (__sq == __s) __pos = __at[__s] + __popcll(__m & __below);")
+            w("    __at[__s] += __popcll(__m);")
+            w("}")
+            w(f"if (__sq >= 0 && __sq < {S})")
+            w("    __ent[__pos] = (long long)(((unsigned long long)(((unsigned)__row << 24) | (unsigned)(__cq & __cmask)) << 32) "
+              f"| (unsigned long long)(unsigned)__v[{kv}][__q]);")
+            self.ind -= 1
+            w("}")
+
+        def unrolled(n, fn):
+            w("#pragma unroll")
+            w(f"for (int __k = 0; __k < {n}; ++__k) {{")
+            self.ind += 1
+            fn()
+            self.ind -= 1
+            w("}")
+
+        w(f"int __cnt[{S}], __at[{S + 1}];")
+        w("#pragma unroll")
+        w(f"for (int __s = 0; __s < {S}; ++__s) __cnt[__s] = 0;")
+        # (indices of a whole block kept in registers between the two passes - 64 registers, half the wavefronts per
+        #  SIMD - made this kernel slower: 455 us against 306 for 2^26 elements)
+        w(f"for (int __j0 = __first; __j0 < __end; __j0 += {256 * U}) {{")
+        self.ind += 1
+        w(f"appy::vec<int, 4>::type __c[{U}];")
+        unrolled(U, lambda: load_indices("__k", "__j0", "__k"))
+        unrolled(U, lambda: count("__k"))
+        self.ind -= 1
+        w("}")
+        starts()
+        w(f"for (int __j0 = __first; __j0 < __end; __j0 += {256 * U}) {{")
+        self.ind += 1
+        w(f"appy::vec<int, 4>::type __c[{U}], __v[{U}];")
+        unrolled(U, lambda: (load_indices("__k", "__j0", "__k"), load_carried("__k", "__j0", "__k")))
+        unrolled(U, lambda: place("__k", "__k", "__j0", "__k"))
+        self.ind -= 1
+        w("}")
+        self.ind -= 1
+        w("}")
+
+    def _body_cells(self):
+        a, g, S, R = self.a, self.a.grouping, self.spec.parts, self.GROUP_ROWS
+        self.ex.locals[a.var] = T.WEAK_INT
+        self.mode = "lane"
+        term, tty, pty = self._group_setup_types()
+        if pty.name not in ("float32", "int32", "uint32") and not self.dirty:
+            raise Unsupported(f"sums of {pty.name} are not accumulated in LDS")
+        x = a.arrays[g["x"]]
+        x.loaded = True
+        U = 8
+        w = self.w
+        w("const int __lid = threadIdx.x & 63;")
+        w("const int __wvl = threadIdx.x >> 6;")
+        w(f"__shared__ {pty.c} __acc_all[4][{R}];        // the sums of the rows of a cell, one cell per wavefront")
+        w(f"{pty.c}* __acc = __acc_all[__wvl];")
+        w(f"const appy::i64 __nblk = (__hi - __lo + {R - 1}) / {R};")
+        w("// workgroup g serves the stripes g mod 8, g mod 8 + 8, ...: workgroups go to the eight XCDs in turn, so every L2")
+        w("// holds one stripe of the gathered operand at a time")
+        w("const appy::i64 __w0 = (appy::i64)(blockIdx.x >> 3) * 4 + __wvl, __nw = (appy::i64)(gridDim.x >> 3) * 4;")
+        w(f"for (int __pass = 0; __pass < {S // 8}; ++__pass) {{")
+        self.ind += 1
+        w("const int __s = (int)(blockIdx.x & 7) + 8 * __pass;")
+        w("const appy::i64 __x0 = (appy::i64)__s << __shiftc;")
+        w("for (appy::i64 __b = __w0; __b < __nblk; __b += __nw) {")
+        self.ind += 1
+        w(f"const int __clo = __desc[__b * {S + 1} + __s], __chi = __desc[__b * {S + 1} + __s + 1];")
+        w("#pragma unroll")
+        w(f"for (int __k = 0; __k < {R // 64}; ++__k) __acc[__k * 64 + __lid] = 0;")
+        w("appy::wave_fence();")
+        w(f"for (int __j0 = __clo; __j0 < __chi; __j0 += {64 * U}) {{")
+        self.ind += 1
+        w(f"long long __e[{U}];")
+        w(f"{x.elem_c} __xv[{U}];")
+        w("#pragma unroll")
+        w(f"for (int __k = 0; __k < {U}; ++__k) {{")
+        w("    const int __j = __j0 + __k * 64 + __lid;")
+        w("    __e[__k] = __j < __chi ? __builtin_nontemporal_load(__ent + __j) : 0ll;")
+        w("}")
+        w("#pragma unroll")
+        w(f"for (int __k = 0; __k < {U}; ++__k) {{")
+        w("    const int __j = __j0 + __k * 64 + __lid;")
+        w(f"    __xv[__k] = {cname(g['x'])}[__j < __chi ? __x0 + (appy::i64)((unsigned)((unsigned long long)__e[__k] >> 32) & 0xffffffu) : 0];")
+        w("}")
+        w("#pragma unroll")
+        w(f"for (int __k = 0; __k < {U}; ++__k) {{")
+        self.ind += 1
+        w("const int __j = __j0 + __k * 64 + __lid;")
+        w("if (__j < __chi) {")
+        self.ind += 1
+        if g["carried"]:
+            cty = a.arrays[g["carried"]].ty
+            bits = "(int)(unsigned)(unsigned long long)__e[__k]"
+            w(f"const {cty.c} __cv = {'__int_as_float(' + bits + ')' if cty.is_float else '(' + cty.c + ')' + bits};")
+        w(f"const {x.elem_c} __cx = __xv[__k];")
+        w(f"atomicAdd(&__acc[(unsigned)((unsigned long long)__e[__k] >> 56)], {cast(term, tty, pty)});")
+        self.ind -= 1
+        w("}")
+        self.ind -= 1
+        w("}")
+        self.ind -= 1
+        w("}")
+        w("appy::wave_fence();")
+        w("#pragma unroll")
+        w(f"for (int __k = 0; __k < {R // 64}; ++__k) {{")
+        w(f"    const appy::i64 __row = __b * {R} + __k * 64 + __lid;")
+        w(f"    if (__row < __hi - __lo) reinterpret_cast<{pty.c}*>(__scratch)[(appy::i64)__s * (__hi - __lo) + __row] = __acc[__k * 64 + __lid];")
+        w("}")
+        w("appy::wave_fence();")
+        self.ind -= 1
+        w("}")
+        self.ind -= 1
+        w("}")
+
     def tiled_spread_loop(self, st: ast.For):
         """The LDS-staged form of :meth:`spread_loop` for the loop of the plan."""
         var = st.target.id
@@ -2543,6 +2890,18 @@ class KernelBuilder:
                 params.append(Param("__load", "unsigned long long* __load", C.c_void_p, "load"))
             elif sp.phase == 1:
                 params.append(Param("__load", "const unsigned long long* __load", C.c_void_p, "load"))
+        if sp.aux in ("group", "cells"):
+            params.append(Param("__ent", ("long long* __ent" if sp.aux == "group" else "const long long* __ent"), C.c_void_p, "ent"))
+            params.append(Param("__desc", ("int* __desc" if sp.aux == "group" else "const int* __desc"), C.c_void_p, "desc"))
+            params.append(Param("__shiftc", "const int __shiftc", C.c_int32, "shiftc"))
+        if sp.aux == "group":
+            params.append(Param("__len", "const appy::i64 __len", C.c_int64, "entries"))
+            params.append(Param("__rowmax", "const appy::i64 __rowmax", C.c_int64, "rowmax"))
+            params.append(Param("__hint", "long long* __hint", C.c_void_p, "hint"))
+        if sp.aux == "cells":
+            params.append(Param("__scratch", "double* __scratch", C.c_void_p, "scratch"))
+        if sp.aux == "group" or sp.guard:
+            params.append(Param("__flag", ("long long* __flag" if sp.aux == "group" else "const long long* __flag"), C.c_void_p, "flag"))
         if sp.aux == "bins" or sp.rows == "mixed":
             params.append(Param("__m", "const appy::i64 __m", C.c_int64, "m"))
             params.append(Param("__base", "const int __base", C.c_int32, "base"))

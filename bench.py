@@ -404,7 +404,7 @@ def main():
         nbytes = 8 * nnz + 4 * (m + 1) + 4 * ncol + 4 * m
         results[name] = run.measure(loop, vals, nbytes, K, W)
         seq = loop.last_launch.sequence
-        results[name].update({"kernels_per_launch": len(seq) if seq else 1,
+        results[name].update({"kernels_per_launch": sum(1 for step in seq if step[0] is not None) if seq else 1,
                               "nnz": int(nnz), "rows": m, "mean_row": float(nnz) / m, "max_row": int(lens.max().item()),
                               "giga_nnz_per_s": nnz / results[name]["kernel_ms"] / 1e6})
         if "gather" in results:
