@@ -409,7 +409,8 @@ class CompiledLoop:
                     fn = self.options.get("fn_name")
                     sym = f"{fn}_{self.loop_name}" if fn and str(fn).isidentifier() else self.loop_name
                     # the helper kernels of a loop with binned rows go by names of their own in traces
-                    sym += ("_" + spec.aux if spec.aux else {1: "_parts", 2: "_fold"}[spec.phase] if spec.rows == "list" else "")
+                    sym += ("_" + spec.aux if spec.aux else {1: "_parts", 2: "_fold"}[spec.phase] if spec.rows == "list" else
+                            {1: "_sums", 2: "_rowwise"}[spec.guard] if spec.guard else "")
                     builder = KernelBuilder(self.analysis, sym, self.module_names, spec)
                     k = Kernel(builder.build(device_header()))
                     self.kernels[spec] = k
@@ -653,6 +654,25 @@ class CompiledLoop:
         parts = min(DEFAULT_CUS // max(1, strips), max(1, trip // (4 * nw)), 1024)
         return max(1, parts)
 
+    def grouped_shape(self, n_outer, env, arrays):
+        """``(stripes, log2 of the elements per stripe, positions to group)`` for a launch that groups the
+        elements of its rows by the stripe of the gathered operand they read, or None when the loop or
+        these arrays do not qualify: the operand is larger than an L2 can keep next to the streams and
+        no larger than 16 stripes of half an L2, the rows hold a few elements at least."""
+        g = self.analysis.grouping
+        if g is None or self._group_off or not self.options.get("hip_group", True) or not self.options.get("hip_hints", True):
+            return None
+        nx = int(arrays[g["x"]].shape[0])
+        if nx * 4 <= STRIPE_MIN_BYTES or nx > (16 << GROUP_MAX_STRIPE_LOG):
+            return None
+        parts = 8 if nx <= (8 << GROUP_MAX_STRIPE_LOG) else 16
+        shift = max(1, (-(-nx // parts) - 1).bit_length())
+        entries = min(int(arrays[nm].shape[0]) for nm in (g["idx"], g["carried"]) if nm)
+        trip, _uniform = self._estimate_trip(env, arrays, n_outer)
+        if entries >= (1 << 31) or trip < GROUP_MIN_TRIP:
+            return None
+        return parts, shift, entries
+
     def scratch(self, device: int, stream: int, nbytes: int) -> int:
         """Device memory for partial results of two-phase launches of this loop: one buffer per
         device and stream, kept for the life of the loop (launches on one stream follow one
@@ -874,8 +894,12 @@ class CompiledLoop:
 class Launch:
     """One staged launch: device pointers, argument block, grid."""
 
+    serial = 0      # launches staged so far in this process (a diagnostic: which of two loops ran last)
+
     def __init__(self, loop: CompiledLoop, vals, arrays, env, lo, hi):
         self.loop = loop
+        Launch.serial += 1
+        self.serial = Launch.serial
         a = loop.analysis
         self.lo, self.hi = lo, hi
         self.env = env
@@ -1134,7 +1158,7 @@ class Launch:
         loop, a, env = self.loop, self.loop.analysis, self.env
         n = hi - lo
         g = a.grouping
-        if g is None or loop._group_off or not loop.options.get("hip_group", True) or not loop.options.get("hip_hints", True):
+        if g is None:
             return False
         V = spec.vec
         _addr, hint = loop.hint(self.device)
@@ -1142,16 +1166,10 @@ class Launch:
         # the last launch has sorted these rows and found none in the class of the longest
         if not (seen[0] == 1 and sum(seen[1:]) == n and min(seen[1:]) >= 0 and seen[4] == 0):
             return False
-        x = arrays[g["x"]]
-        nx = int(x.shape[0])
-        if nx * 4 <= STRIPE_MIN_BYTES or nx > (16 << GROUP_MAX_STRIPE_LOG):
+        shape = loop.grouped_shape(n, env, arrays)
+        if shape is None:
             return False
-        parts = 8 if nx <= (8 << GROUP_MAX_STRIPE_LOG) else 16
-        shift = max(1, (-(-nx // parts) - 1).bit_length())
-        entries = min(int(arrays[nm].shape[0]) for nm in (g["idx"], g["carried"]) if nm)
-        trip, _uniform = loop._estimate_trip(env, arrays, n)
-        if entries >= (1 << 31) or trip < GROUP_MIN_TRIP:
-            return False
+        parts, shift, entries = shape
         R = 256
         nblk = -(-n // R)
         common = dict(block=256, restrict=spec.restrict)

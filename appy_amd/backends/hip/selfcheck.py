@@ -172,4 +172,22 @@ def compile_all_patterns() -> int:
             for w in (1, 4, 16, 64):
                 loop.kernel_for(Spec("team", block=256, vec=loop.default_spec.vec, width=w)).code
                 count += 1
+        v = loop.default_spec.vec
+        more = []
+        if loop.analysis.ragged is not None and v > 1:
+            # rows sorted by the length of their simd loop; long rows in planned parts
+            more += [Spec("team", block=1024, vec=1, width=1, aux="bins"), Spec("team", block=256, vec=v, width=64, rows="mixed")]
+            if loop.analysis.ragged[1] is not None:
+                more += [Spec("team", block=256, vec=1, width=8, rows="list", parts=8, aux="plan"),
+                         Spec("team", block=256, vec=v, width=16, phase=1, rows="list", parts=8),
+                         Spec("team", block=256, vec=v, width=1, phase=2, rows="list", parts=8)]
+            if loop.analysis.grouping is not None:
+                # elements grouped by the stripe of the gathered operand
+                more += [Spec("team", block=256, vec=1, width=64, parts=8, aux="group"),
+                         Spec("team", block=256, vec=1, width=64, parts=16, aux="cells", guard=1),
+                         Spec("team", block=256, vec=v, width=1, phase=2, guard=1),
+                         Spec("team", block=256, vec=v, width=4, guard=2)]
+        for spec in more:
+            loop.kernel_for(spec).code
+            count += 1
     return count

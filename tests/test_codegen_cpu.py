@@ -151,6 +151,50 @@ def test_csr_rows_are_sorted_by_length_from_32768_rows_on():
         Spec("flat", rows="mixed")
 
 
+def test_sums_of_gathered_terms_can_be_grouped_by_the_stripe_they_read():
+    """`s += A[j] * x[idx[j]]` and its relatives qualify; terms that read a value of their row, a
+    second gathered operand, or operands that are not four bytes wide do not."""
+    f, _ = selfcheck_loop("spmv")
+    g = f.analysis.grouping
+    assert g is not None and (g["x"], g["idx"], g["carried"], g["name"]) == ("x", "A_indices", "A_data", "s")
+    i32, f32 = np.zeros(9, np.int32), np.zeros(16, np.float32)
+
+    def csr(term, init="0.0", pre="", **more):
+        src = ("#pragma parallel for\nfor i in range(m):\n" + pre + f"    s = {init}\n    #pragma simd\n"
+               f"    for j in range(p[i], p[i + 1]):\n        s += {term}\n    y[i] = s")
+        vals = dict(p=i32, c=np.zeros(16, np.int32), v=f32, x=f32, y=np.zeros(8, np.float32), m=8)
+        vals.update(more)
+        return compiled(src, **vals)[0].analysis
+
+    assert csr("x[c[j]]").grouping["carried"] is None
+    assert csr("alpha * (v[j] * x[c[j]])", alpha=0.5).grouping["carried"] == "v"
+    assert csr("x[c[j]] * x[c[j]]").grouping is not None                     # the same load twice
+    assert csr("f * v[j] * x[c[j]]", pre="    f = y[i]\n").grouping is None  # a value of the row
+    assert csr("v[j] * x[c[j]] * j").grouping is None                         # the position itself
+    assert csr("v[j] * w[j] * x[c[j]]", w=f32).grouping is None               # two operands to carry
+    assert csr("v[j] * x[c[j]] + z[c[j]]", z=f32).grouping is None            # two gathered operands
+    assert csr("v[j] * x[c[j]]", x=np.zeros(16, np.float64)).grouping is None
+    assert csr("v[j] * x[c[j]]", c=np.zeros(16, np.int64)).grouping is None
+    # the kernels
+    group = body_of(f.kernel_for(Spec("team", block=256, vec=1, width=64, parts=8, aux="group")).src.text)
+    assert "__lp[__r + 1] == __hq[__r]" in group and "__flag[0] = 1" in group and "__hint[0] = 2" in group
+    assert "x[" not in group.split("{", 1)[1]                                 # the gathered operand is not read here
+    cells = body_of(f.kernel_for(Spec("team", block=256, vec=1, width=64, parts=16, aux="cells", guard=1)).src.text)
+    assert "if ((__flag[0] != 0) == true) return;" in cells and "for (int __pass = 0; __pass < 2; ++__pass)" in cells
+    assert "atomicAdd(&__acc[" in cells and "(__cv * __cx)" in cells and "A_indptr[" not in cells.split("{", 1)[1]
+    sums = body_of(f.kernel_for(Spec("team", block=256, vec=4, width=1, phase=2, guard=1)).src.text)
+    assert "reinterpret_cast<float*>(__scratch)[(0 * __nsplit + __c) * (__hi - __lo) + (i - __lo)]" in sums and "y[i] = s" in sums
+    rest = body_of(f.kernel_for(Spec("team", block=256, vec=4, width=4, guard=2)).src.text)
+    assert "if ((__flag[0] != 0) == false) return;" in rest
+    with pytest.raises(ValueError):
+        Spec("team", block=256, width=64, parts=24, aux="group")
+    with pytest.raises(ValueError):
+        Spec("flat", guard=1)
+    # sums of float64 are not taken: the loop keeps its rows sorted by length
+    d = csr("v[j] * x[c[j]]", v=np.zeros(16, np.float64))
+    assert d.grouping is None
+
+
 def test_spmm_row_lives_in_registers():
     loop, _ = selfcheck_loop("spmm")
     spec = Spec("team", block=256, vec=4, width=32, extent=128)

@@ -30,11 +30,19 @@ def plain(gpu):
     return selfcheck.kernels(hip_bins=False)
 
 
-def _loop(name, bins=True, index_type="int32"):
+@pytest.fixture(scope="module")
+def sorted_only(gpu):
+    """Rows sorted by length, but never the grouped form that short rows take from their second launch on."""
+    return selfcheck.kernels(hip_group=False)
+
+
+def _loop(name, bins=True, index_type="int32", group=True):
     """The compiled loop of function ``name`` (for `spmv`: the one for row pointers of ``index_type``)."""
     hits = [v[0] for kk, v in cg.code_cache.items() if kk[-1] == name and bool(v[0].options.get("hip_bins", True)) == bins
-            and (name != "spmv" or v[0].analysis.arrays["A_indptr"].ty.name == index_type)]
-    return hits[-1]
+            and bool(v[0].options.get("hip_group", True)) == group
+            and (name != "spmv" or ("A_indptr" in v[0].analysis.arrays and v[0].analysis.arrays["A_indptr"].ty.name == index_type
+                                   and v[0].analysis.arrays["x"].ty.name == "float32"))]
+    return max(hits, key=lambda lp: lp.last_launch.serial if getattr(lp, "last_launch", None) is not None else -1)
 
 
 def _forget(name="spmv"):
@@ -76,18 +84,19 @@ def test_spmv_powerlaw_rows_are_binned_and_striped(k, plain, m, n, clip):
     assert np.array_equal(y[short], y0[short])
 
 
-def test_spmv_uniform_rows_stay_in_their_natural_order(k, plain):
+def test_spmv_uniform_rows_stay_in_their_natural_order(sorted_only, plain):
+    k = sorted_only
     m = 50_000
     data, indptr, indices, x = wl.spmv_uniform(m, 1 << 20, 16)
     ref, budget = vo.spmv_csr(data, indptr, indices, x, (m, 1 << 20))
     _forget()
     y = k.spmv(data, indptr, indices, x, m, 1 << 20)
-    launch = _loop("spmv").last_launch
+    launch = _loop("spmv", group=False).last_launch
     assert launch.spec.rows == "mixed" and launch.bin["base"] == 1      # 16 per row: the class of teams of four
     assert len(launch.sequence) == 6                                    # nothing known yet: set up for long rows too
     # the launch has reported what its classes held: the next one sets nothing up for long rows
     y2 = k.spmv(data, indptr, indices, x, m, 1 << 20)
-    again = _loop("spmv").last_launch
+    again = _loop("spmv", group=False).last_launch
     assert len(again.sequence) == 3 and again.bin["base"] == 1 and np.array_equal(y, y2)
     assert vo.within_budget(y, ref, budget, TOL)[0]
     assert np.array_equal(y, plain.spmv(data, indptr, indices, x, m, 1 << 20))
@@ -143,28 +152,29 @@ def test_spmv_columns_in_any_order_and_int64_indices(k):
     assert ok, worst
 
 
-def test_the_hint_of_an_earlier_launch_shapes_the_next_one_and_never_its_results(k):
+def test_the_hint_of_an_earlier_launch_shapes_the_next_one_and_never_its_results(sorted_only):
     """The kernel over the binned rows reports the sizes of its classes in page-locked memory.  The next
     launch takes the most populous class in natural order and leaves out the kernels for long rows when
     there were none; a matrix that has long rows after all is still computed correctly (its long rows
     then run whole), and the launch after that cuts them into parts again."""
+    k = sorted_only
     m, n = 40_000, 1 << 20
     short = wl.spmv_uniform(m, n, 3)                        # every row in the class of single lanes
     data, indptr, indices, x, lengths = _powerlaw(m, n, 4096, seed=77)
     _forget()
     y = k.spmv(*short, m, n)
-    first = _loop("spmv").last_launch
+    first = _loop("spmv", group=False).last_launch
     assert first.bin["base"] == 0 and len(first.sequence) == 6
     ref, budget = vo.spmv_csr(*short, (m, n))
     assert vo.within_budget(y, ref, budget, TOL)[0]
     ref, budget = vo.spmv_csr(data, indptr, indices, x, (m, n))
     y1 = k.spmv(data, indptr, indices, x, m, n)             # shaped by the hint of the short rows
-    second = _loop("spmv").last_launch
+    second = _loop("spmv", group=False).last_launch
     assert len(second.sequence) == 3 and second.bin["skip"] == 0
     ok, worst = vo.within_budget(y1, ref, budget, TOL)
     assert ok, worst
     y2 = k.spmv(data, indptr, indices, x, m, n)             # now it is known to have long rows
-    third = _loop("spmv").last_launch
+    third = _loop("spmv", group=False).last_launch
     assert len(third.sequence) == 6 and third.bin["base"] == int(np.argmax(np.bincount(np.digitize(lengths, [4, 32, 128], right=True), minlength=4)))
     ok, worst = vo.within_budget(y2, ref, budget, TOL)
     assert ok, worst

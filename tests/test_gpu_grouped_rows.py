@@ -1,0 +1,296 @@
+"""Loops over short rows that sum terms gathered from an operand larger than an L2 (CSR SpMV with
+a few to a hundred elements per row): from their second launch on, the elements of every 256 rows
+are grouped by the stripe of the operand they read, the groups run with one stripe per XCD, and the
+sums of a row are added up afterwards.  Every result is compared with the float64 oracle to the bar
+of the parity tests (``|out - oracle| <= 1e-5 * sum(|terms|)`` per output).
+
+Pattern: the CSR loop of the reference's examples/03-spmv.py:5-16 and
+tests/integration/triton/tutorial/test_spmv.py:10-30."""
+import numpy as np
+import pytest
+
+import appy_amd as appy
+from appy_amd.backends.hip import codegen as cg
+from appy_amd.backends.hip import selfcheck
+from oracle import vectorised as vo
+from oracle import workloads as wl
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-5
+
+
+@pytest.fixture(scope="module")
+def k(gpu):
+    return selfcheck.kernels()
+
+
+def _loop(name, index_type="int32"):
+    hits = [v[0] for kk, v in cg.code_cache.items() if kk[-1] == name and v[0].options.get("hip_bins", True)
+            and v[0].options.get("hip_group", True) and getattr(v[0], "last_launch", None) is not None
+            and (name != "spmv" or ("A_indptr" in v[0].analysis.arrays and v[0].analysis.arrays["A_indptr"].ty.name == index_type
+                                   and v[0].analysis.arrays["x"].ty.name == "float32"))]
+    return max(hits, key=lambda lp: lp.last_launch.serial if getattr(lp, "last_launch", None) is not None else -1)
+
+
+def _forget(name="spmv"):
+    for kk, v in cg.code_cache.items():
+        if kk[-1] == name:
+            for _addr, view in v[0]._hints.values():
+                view[0] = 0
+
+
+def _grouped(launch):
+    return launch.sequence is not None and launch.spec.aux == "cells"
+
+
+def _matrix(lengths, n, seed):
+    rng = np.random.default_rng(seed)
+    data, indptr, indices = wl.csr_matrix(np.asarray(lengths, dtype=np.int64), n, rng)
+    x = rng.standard_normal(n, dtype=np.float32)
+    return data, indptr, indices, x
+
+
+@pytest.mark.parametrize("m,n,lengths", [
+    (50_000, 1 << 20, "16"),                 # the uniform matrix of the benchmark, scaled down
+    (40_003, (1 << 22) - 12345, "1..31"),    # a ragged last block, a last stripe that is not full
+    (70_000, 3 << 20, "0,10,20"),            # empty rows; stripes that are not a power of two of the operand
+    (33_000, 7 << 20, "8"),                  # sixteen stripes, two per XCD
+    (36_000, 1 << 21, "1..127"),             # rows of the three classes that qualify
+])
+def test_short_rows_are_grouped_from_the_second_launch_on(k, m, n, lengths):
+    rng = np.random.default_rng(m)
+    if lengths == "0,10,20":
+        ln = rng.integers(0, 3, m) * 10
+    elif ".." in lengths:
+        a, b = lengths.split("..")
+        ln = rng.integers(int(a), int(b) + 1, m)
+    else:
+        ln = np.full(m, int(lengths))
+    data, indptr, indices, x = _matrix(ln, n, seed=m + 1)
+    ref, budget = vo.spmv_csr(data, indptr, indices, x, (m, n))
+    _forget()
+    y0 = k.spmv(data, indptr, indices, x, m, n)
+    first = _loop("spmv").last_launch
+    assert first.spec.rows == "mixed"                       # nothing known about the rows yet: sorted by length
+    ok, worst = vo.within_budget(y0, ref, budget, TOL)
+    assert ok, worst
+    y1 = k.spmv(data, indptr, indices, x, m, n)
+    second = _loop("spmv").last_launch
+    assert _grouped(second) and second.nsplit == (16 if n > (8 << 19) else 8)
+    assert [step[0].src.spec.aux if step[0] else "clear" for step in second.sequence] == ["clear", "group", "cells", "", ""]
+    ok, worst = vo.within_budget(y1, ref, budget, TOL)
+    assert ok, worst
+    assert np.all(y1[ln == 0] == 0.0)
+    # the same launch again gives the same bits: the order of the additions does not depend on timing
+    assert np.array_equal(y1, k.spmv(data, indptr, indices, x, m, n))
+
+
+def test_a_matrix_with_long_rows_goes_back_to_rows_sorted_by_length(k):
+    """The grouped form is chosen from what the last launch reported.  When the rows it then meets are
+    longer than that, the result is still right, and the launch after it sorts the rows again."""
+    m, n = 40_000, 1 << 20
+    short = _matrix(np.full(m, 12), n, seed=1)
+    rng = np.random.default_rng(2)
+    ln = np.clip(rng.zipf(1.5, m), 1, 4096)
+    long_ = _matrix(ln, n, seed=3)
+    _forget()
+    k.spmv(*short, m, n)
+    k.spmv(*short, m, n)
+    assert _grouped(_loop("spmv").last_launch)
+    ref, budget = vo.spmv_csr(*long_, (m, n))
+    y = k.spmv(*long_, m, n)
+    assert _grouped(_loop("spmv").last_launch)              # shaped by the report on the short rows
+    ok, worst = vo.within_budget(y, ref, budget, TOL)
+    assert ok, worst
+    y = k.spmv(*long_, m, n)
+    assert _loop("spmv").last_launch.spec.rows == "mixed"   # the grouping kernel has seen the long rows
+    ok, worst = vo.within_budget(y, ref, budget, TOL)
+    assert ok, worst
+    y = k.spmv(*long_, m, n)
+    assert _loop("spmv").last_launch.spec.rows == "mixed" and len(_loop("spmv").last_launch.sequence) == 6
+
+
+def test_row_ranges_that_do_not_follow_one_another_run_row_by_row(gpu):
+    """`range(start[i], end[i])` need not describe a CSR matrix.  Ranges out of order, ranges that overlap
+    and ranges with gaps are legal loops; the grouping kernel refuses them and the launch runs the loop
+    as written - once: the statement after the loop updates `y` in place."""
+    rng = np.random.default_rng(4)
+    m, n, per = 40_000, 1 << 20, 16
+    data, indptr, indices, x = _matrix(np.full(m, per), n, seed=5)
+
+    @appy.jit
+    def windows(data, start, end, indices, x, y, beta, m):
+        #pragma parallel for
+        for i in range(m):
+            s = 0.0
+            #pragma simd
+            for j in range(start[i], end[i]):
+                s += data[j] * x[indices[j]]
+            y[i] = beta * y[i] + s
+
+    def run(start, end, expect_grouped=True):
+        y = np.ones(m, dtype=np.float32)
+        windows(data, start, end, indices, x, y, 0.5, m)
+        assert _grouped(_loop("windows").last_launch) == expect_grouped
+        terms = data.astype(np.float64) * x.astype(np.float64)[indices]
+        cs = np.concatenate([[0.0], np.cumsum(terms)])
+        ca = np.concatenate([[0.0], np.cumsum(np.abs(terms))])
+        ln = np.maximum(end.astype(np.int64) - start, 0)
+        ref = 0.5 + cs[start + ln] - cs[start]
+        budget = 0.5 + ca[start + ln] - ca[start]
+        assert np.all(np.abs(y - ref) <= TOL * budget + 1e-9 * ca[-1]), np.max(np.abs(y - ref))
+
+    start, end = indptr[:-1].copy(), indptr[1:].copy()
+    _forget("windows")
+    run(start, end, expect_grouped=False)       # first launch: rows sorted by length
+    run(start, end)                             # a CSR matrix in two arrays: grouped
+    # two rows swapped: ranges out of order
+    s2, e2 = start.copy(), end.copy()
+    s2[[1000, 1001]] = s2[[1001, 1000]]
+    e2[[1000, 1001]] = e2[[1001, 1000]]
+    run(s2, e2)
+    # a range that reaches into its neighbour's, a range that ends before its own start, a gap
+    s3, e3 = start.copy(), end.copy()
+    e3[5] += 7
+    e3[20_000] = s3[20_000] - 3
+    s3[30_000] += 2
+    run(s3, e3)
+    # a range that ends beyond the arrays' extent would be refused as well; within it, the last row may stop short
+    e4 = end.copy()
+    e4[-1] -= 5
+    run(start, e4)
+
+
+def test_terms_with_a_scalar_factor_integer_values_and_no_second_operand(gpu):
+    rng = np.random.default_rng(6)
+    m, n = 40_000, 1 << 20
+    ln = rng.integers(4, 24, m)
+    data, indptr, indices, x = _matrix(ln, n, seed=7)
+    nnz = len(indices)
+    w = rng.integers(-5, 6, nnz).astype(np.int32)
+    xi = rng.integers(-100, 100, n).astype(np.int32)
+
+    @appy.jit
+    def scaled(data, indptr, indices, x, y, alpha, m):
+        #pragma parallel for
+        for i in range(m):
+            s = 0.0
+            #pragma simd
+            for j in range(indptr[i], indptr[i + 1]):
+                s += alpha * (data[j] * x[indices[j]])
+            y[i] = s
+
+    @appy.jit
+    def weighted_counts(w, indptr, indices, x, y, m):
+        #pragma parallel for
+        for i in range(m):
+            s = 0
+            #pragma simd
+            for j in range(indptr[i], indptr[i + 1]):
+                s += w[j] * x[indices[j]]
+            y[i] = s
+
+    @appy.jit
+    def gathered(indptr, indices, x, y, m):
+        #pragma parallel for
+        for i in range(m):
+            s = 0.0
+            #pragma simd
+            for j in range(indptr[i], indptr[i + 1]):
+                s += x[indices[j]]
+            y[i] = s
+
+    rows = np.repeat(np.arange(m), ln)
+    x64 = x.astype(np.float64)
+    cases = (
+        ("scaled", lambda y: scaled(data, indptr, indices, x, y, 0.25, m), 0.25 * data * x64[indices], np.float32),
+        ("weighted_counts", lambda y: weighted_counts(w, indptr, indices, xi, y, m), (w.astype(np.int64) * xi[indices]).astype(np.float64), np.int32),
+        ("gathered", lambda y: gathered(indptr, indices, x, y, m), x64[indices], np.float32),
+    )
+    for name, call, terms, dtype in cases:
+        ref = np.bincount(rows, weights=terms, minlength=m)
+        budget = np.bincount(rows, weights=np.abs(terms), minlength=m)
+        _forget(name)
+        for launch_no in range(2):
+            y = np.zeros(m, dtype=dtype)
+            call(y)
+            assert _grouped(_loop(name).last_launch) == (launch_no == 1), name
+            if dtype is np.int32:
+                assert np.array_equal(y, ref.astype(np.int64)), name
+            else:
+                assert np.all(np.abs(y - ref) <= TOL * budget), name
+
+
+def test_loops_that_do_not_qualify_keep_their_rows_sorted(k):
+    """Terms that read a value of their row, sums of float64, operands that fit an L2, and the option."""
+    rng = np.random.default_rng(8)
+    m, n = 40_000, 1 << 20
+    data, indptr, indices, x = _matrix(np.full(m, 10), n, seed=9)
+    scale = rng.standard_normal(m).astype(np.float32)
+
+    @appy.jit
+    def row_scaled(data, indptr, indices, x, scale, y, m):
+        #pragma parallel for
+        for i in range(m):
+            f = scale[i]
+            s = 0.0
+            #pragma simd
+            for j in range(indptr[i], indptr[i + 1]):
+                s += f * data[j] * x[indices[j]]
+            y[i] = s
+
+    y = np.empty(m, dtype=np.float32)
+    for _ in range(2):
+        row_scaled(data, indptr, indices, x, scale, y, m)
+        launch = _loop("row_scaled").last_launch
+        assert launch.spec.rows == "mixed" and launch.loop.analysis.grouping is None
+    ref, budget = vo.spmv_csr(data, indptr, indices, x, (m, n))
+    assert np.all(np.abs(y - scale * ref) <= TOL * np.abs(scale) * budget)
+    # float64 sums
+    x64 = x.astype(np.float64)
+    for _ in range(2):
+        y64 = k.spmv(data.astype(np.float64), indptr, indices, x64, m, n)
+        assert not _grouped([v[0] for kk, v in cg.code_cache.items() if kk[-1] == "spmv"
+                             and "A_indptr" in v[0].analysis.arrays and v[0].analysis.arrays["x"].ty.name == "float64"][-1].last_launch)
+    assert np.all(np.abs(y64 - ref) <= 1e-12 * budget)
+    # an operand of 2 MiB stays in every L2 anyway
+    small = _matrix(np.full(m, 10), 1 << 19, seed=10)
+    _forget()
+    for _ in range(2):
+        k.spmv(*small, m, 1 << 19)
+        assert _loop("spmv").last_launch.spec.rows == "mixed"
+    # hip_group=False
+    off = selfcheck.kernels(hip_group=False)
+    for _ in range(2):
+        y = off.spmv(data, indptr, indices, x, m, n)
+    last = [v[0] for kk, v in cg.code_cache.items() if kk[-1] == "spmv" and not v[0].options.get("hip_group", True)
+            and "A_indptr" in v[0].analysis.arrays and v[0].analysis.arrays["x"].ty.name == "float32"
+            and v[0].analysis.arrays["A_indptr"].ty.name == "int32"][-1].last_launch
+    assert last.spec.rows == "mixed"
+    assert vo.within_budget(y, ref, budget, TOL)[0]
+
+
+def test_grouped_launches_on_gpu_tensors_follow_changes_of_the_matrix(gpu):
+    """Nothing about the matrix is kept between launches: the same tensors with other contents give the
+    other matrix's product."""
+    import torch
+
+    k = selfcheck.kernels()
+    m, n = 60_000, 1 << 20
+    a = _matrix(np.full(m, 16), n, seed=11)
+    b = _matrix(np.full(m, 16), n, seed=13)
+    d = [torch.from_numpy(v).cuda() for v in a]
+    _forget()
+    for _ in range(2):
+        y = k.spmv(*d, m, n)
+    assert _grouped(_loop("spmv").last_launch)
+    ref, budget = vo.spmv_csr(*a, (m, n))
+    assert vo.within_budget(y.cpu().numpy(), ref, budget, TOL)[0]
+    for t, v in zip(d, b):
+        t.copy_(torch.from_numpy(v))
+    y = k.spmv(*d, m, n)
+    assert _grouped(_loop("spmv").last_launch)
+    ref, budget = vo.spmv_csr(*b, (m, n))
+    ok, worst = vo.within_budget(y.cpu().numpy(), ref, budget, TOL)
+    assert ok, worst
