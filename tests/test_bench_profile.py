@@ -90,5 +90,7 @@ def test_traffic_figures_are_plausible():
     # streams: traffic equals the algorithmic bytes to a percent; gathers: several times more
     for name in ("vector_sum", "masked_sum", "copy", "gemv", "vec_add_2p27"):
         assert traffic[name][1] <= 1.01 * alg[name], name
-    assert traffic["spmv_uniform"][1] > 10 * alg["spmv_uniform"] and traffic["spmv_powerlaw"][1] < 4 * alg["spmv_powerlaw"]
+    assert traffic["gather"][1] > 10 * alg["gather"] and traffic["spmv_powerlaw"][1] < 4 * alg["spmv_powerlaw"]
+    # rows of 16 elements grouped by column stripe: the elements are written and read once more, the gathers hit in the L2s
+    assert 3 * alg["spmv_uniform"] < traffic["spmv_uniform"][1] < 5 * alg["spmv_uniform"]
     assert np.isfinite(float(traffic["spmm"][1]))
