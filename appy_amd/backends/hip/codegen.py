@@ -692,7 +692,8 @@ class CompiledLoop:
 
     def hint(self, device: int):
         """Five page-locked 64-bit words per device that the kernel over binned rows writes (a flag, then
-        the number of rows of each class it found) and the host reads when it stages the next launch.
+        the number of rows of each class it found; the kernel that groups the elements of short rows sets
+        the flag to 2 when it meets rows too long for it) and the host reads when it stages the next launch.
         What is read may be old or half updated: it shapes a launch, it never decides what is computed."""
         with self._lock:
             have = self._hints.get(device)
@@ -1158,7 +1159,9 @@ class Launch:
         loop, a, env = self.loop, self.loop.analysis, self.env
         n = hi - lo
         g = a.grouping
-        if g is None:
+        if g is None or self.capture is not None:
+            # (a launch recorded into a graph keeps its rows sorted by length: this form clears its flag with a
+            #  memory-set node, and those are kept out of graphs)
             return False
         V = spec.vec
         _addr, hint = loop.hint(self.device)

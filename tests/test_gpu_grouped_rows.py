@@ -294,3 +294,43 @@ def test_grouped_launches_on_gpu_tensors_follow_changes_of_the_matrix(gpu):
     ref, budget = vo.spmv_csr(*b, (m, n))
     ok, worst = vo.within_budget(y.cpu().numpy(), ref, budget, TOL)
     assert ok, worst
+
+
+def test_launches_recorded_into_a_graph_keep_their_rows_sorted(gpu):
+    """The grouped form clears a flag with a memory-set node; recorded launches use the kernels over sorted
+    rows instead, and every replay follows the contents of the tensors."""
+    import torch
+
+    k = selfcheck.kernels()
+    m, n = 50_000, 1 << 20
+    a = _matrix(np.full(m, 16), n, seed=21)
+    d = [torch.from_numpy(v).cuda() for v in a]
+    y = torch.zeros(m, device="cuda", dtype=torch.float32)
+
+    @appy.jit
+    def spmv_into(A_data, A_indptr, A_indices, x, y, M):
+        #pragma parallel for
+        for i in range(M):
+            s = 0.0
+            #pragma simd
+            for j in range(A_indptr[i], A_indptr[i + 1]):
+                s += A_data[j] * x[A_indices[j]]
+            y[i] = s
+
+    _forget("spmv_into")
+    for _ in range(2):
+        spmv_into(*d, y, m)
+    assert _grouped(_loop("spmv_into").last_launch)
+    with appy.graph() as g:
+        spmv_into(*d, y, m)
+    assert _loop("spmv_into").last_launch.spec.rows == "mixed"
+    for replay in range(3):
+        d[0].mul_(1.5)
+        y.zero_()
+        spmv_into(*d, torch.empty_like(y), m)             # eager (grouped) launches between the replays
+        g.launch()
+        g.synchronize()
+        ref, budget = vo.spmv_csr(d[0].cpu().numpy(), a[1], a[2], a[3], (m, n))
+        ok, worst = vo.within_budget(y.cpu().numpy(), ref, budget, TOL)
+        assert ok, (replay, worst)
+    g.close()
