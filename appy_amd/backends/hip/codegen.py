@@ -1088,7 +1088,7 @@ class Launch:
             if x_bytes > STRIPE_MIN_BYTES:
                 parts = min(64, 8 * -(-x_bytes // (8 * STRIPE_BYTES)))
                 stripe = -(-int(x.shape[0]) // parts)
-                thresholds[2] = max(thresholds[2], 16 * parts)       # sixteen elements per part at least
+                thresholds[2] = max(thresholds[2], 32 * parts)       # 32 elements per part at least
                 # rows longer than the threshold: no more of them than the streamed arrays have room for
                 bound = max([int(arrays[nm].shape[0]) for _code, streamed in loop._simd_loops for nm in streamed
                              if arrays[nm].ndim == 1] or [0])
@@ -1166,9 +1166,10 @@ class Launch:
         V = spec.vec
         _addr, hint = loop.hint(self.device)
         seen = [int(hint[k]) for k in range(5)]
-        # the last launch has sorted these rows and found none in the class of the longest
-        if not (seen[0] == 1 and sum(seen[1:]) == n and min(seen[1:]) >= 0 and seen[4] == 0):
+        # the last launch has sorted these rows: with rows in the class of the longest, those run in planned parts
+        if not (seen[0] == 1 and sum(seen[1:]) == n and min(seen[1:]) >= 0):
             return False
+        long_rows = seen[4] > 0
         shape = loop.grouped_shape(n, env, arrays)
         if shape is None:
             return False
@@ -1176,38 +1177,75 @@ class Launch:
         R = 256
         nblk = -(-n // R)
         common = dict(block=256, restrict=spec.restrict)
+        # rows beyond this many elements are cut at the stripes of the gathered operand, the others have their elements
+        # grouped (power-law matrix: 3.14 ms with 128, 3.05 with 256, 3.02 with 512, 3.09 with 1024)
+        cut = max(32 * V, 64 * parts)
         try:
-            group = loop.kernel_for(Spec("team", vec=1, width=64, parts=parts, aux="group", **common))
+            group = loop.kernel_for(Spec("team", vec=1, width=64, parts=parts, aux="group", skip_long=long_rows, **common))
             cells = loop.kernel_for(Spec("team", vec=1, width=64, parts=parts, aux="cells", guard=1, **common))
-            fold = loop.kernel_for(Spec("team", vec=V, width=1, phase=2, guard=1, **common))
+            sums = loop.kernel_for(Spec("team", vec=V, width=1, phase=2, guard=1, skip_long=long_rows, **common))
             plain = loop._choose_spec(n, env, arrays, restrict=spec.restrict, listable=False)
             if plain.kind != "team" or plain.phase or plain.rows:
                 raise Unsupported("no plain team kernel to fall back to")
             rest = loop.kernel_for(dataclasses.replace(plain, guard=2))
+            if long_rows:
+                ts = 8
+                while ts < parts:
+                    ts *= 2
+                listed = dict(common, rows="list", parts=parts, guard=1)
+                bins = loop.kernel_for(Spec("team", block=1024, vec=1, width=1, restrict=spec.restrict, aux="bins"))
+                plan = loop.kernel_for(Spec("team", vec=1, width=ts, aux="plan", **listed))
+                first = loop.kernel_for(Spec("team", vec=V, width=16, phase=1, stream_loads=spec.stream_loads, **listed))
+                last = loop.kernel_for(Spec("team", vec=V, width=1, phase=2, stream_loads=spec.stream_loads, **listed))
         except Unsupported:
             loop._group_off = True
             return False
-        # one buffer: header (the flag) | where the cells start | the grouped elements | sums per row and stripe
-        off_desc = 2048
+        reds = max(1, len(loop_ir.reductions_of(a.team_split)))
+        cap = 0
+        if long_rows:
+            bound = max([int(arrays[nm].shape[0]) for _code, streamed in loop._simd_loops for nm in streamed
+                         if arrays[nm].ndim == 1] or [0])
+            cap = min(n, bound // cut + 1) if bound else n
+        # one buffer: header (counters of the sorting kernel, the flag) | lists of rows by class | cuts of the long rows |
+        # their starts | their partial results | where the cells start | the grouped elements | sums per row and stripe
+        off_rows = 2048
+        off_bnd = off_rows + (4 * 4 * n if long_rows else 0)
+        off_start = (off_bnd + 4 * (parts + 1) * cap + 255) // 256 * 256
+        off_long = (off_start + 8 * cap + 255) // 256 * 256
+        off_desc = (off_long + 8 * reds * parts * cap + 255) // 256 * 256
         off_ent = (off_desc + 4 * (parts + 1) * nblk + 255) // 256 * 256
         off_part = (off_ent + 8 * entries + 255) // 256 * 256
         buf = loop.scratch(self.device, self.stream, off_part + 4 * parts * n)
         hint_addr, _ = loop.hint(self.device)
+        base = max(range(3), key=lambda c: seen[c + 1])
         self.bin = {"flag": buf + 1984, "desc": buf + off_desc, "ent": buf + off_ent, "shiftc": shift, "entries": entries,
-                    "rowmax": 32 * V, "hint": hint_addr}
+                    "rowmax": cut if long_rows else 32 * V, "hint": hint_addr,
+                    "counts": buf, "load": buf + 32, "zero": buf + 1024, "rows": buf + off_rows, "m": n, "base": base,
+                    "threshold": [V, 8 * V, cut], "bnd": buf + off_bnd, "rowstart": buf + off_start, "cap": cap,
+                    "stripe": -(-int(arrays[g["x"]].shape[0]) // parts), "nrows": buf + 4 * 3}
         self.scratch_ptr = buf + off_part
         self.nsplit = parts
-        seq = [(None, (buf + 1984, 8), None, None)]         # the flag starts at zero
+        # the flag starts at zero, and with it the counters of the sorting kernel
+        seq = [(None, ((buf, 2048) if long_rows else (buf + 1984, 8)), None, None)]
+        if long_rows:
+            seq.append((bins, self._argument_block(bins, vals, arrays, lo, hi), (max(1, min(512, -(-n // 4096))), 1, 1), (1024, 1, 1)))
         seq.append((group, self._argument_block(group, vals, arrays, lo, hi), (max(1, min(1 << 20, -(-nblk // 4))), 1, 1), (256, 1, 1)))
         seq.append((cells, self._argument_block(cells, vals, arrays, lo, hi), (8 * max(1, min(8192, -(-nblk // 4))), 1, 1), (256, 1, 1)))
-        seq.append((fold, self._argument_block(fold, vals, arrays, lo, hi), (max(1, min(4096, -(-n // 256))), 1, 1), (256, 1, 1)))
+        args_of_cells = seq[-1]
+        seq.append((sums, self._argument_block(sums, vals, arrays, lo, hi), (max(1, min(4096, -(-n // 256))), 1, 1), (256, 1, 1)))
+        if long_rows:
+            self.bin["rows"] = buf + off_rows + 4 * 3 * n         # the list of the longest class
+            self.scratch_ptr = buf + off_long
+            seq.append((plan, self._argument_block(plan, vals, arrays, lo, hi), (max(1, min(2048, -(-cap * ts // 256))), 1, 1), (256, 1, 1)))
+            seq.append((first, self._argument_block(first, vals, arrays, lo, hi), (max(8, min(2048, 8 * -(-cap * 16 // 256))), 1, 1), (256, 1, 1)))
+            seq.append((last, self._argument_block(last, vals, arrays, lo, hi), (max(1, min(1024, -(-cap // 256))), 1, 1), (256, 1, 1)))
         # (the kernel that runs the loop row by row when the input was refused: few workgroups that loop - it returns at
         #  once otherwise, and 65536 workgroups take 15 us to do that, 1024 take 3)
         seq.append((rest, self._argument_block(rest, vals, arrays, lo, hi),
                     (min(1024, loop.grid_for(plain, n, kernel=rest, row_hint=loop.row_hint(n, env, arrays))), 1, 1), (plain.block, 1, 1)))
         self.sequence = seq
         self.kernel, self.spec = cells, cells.src.spec
-        self.args, self.grid, self.block = seq[2][1], seq[2][2], seq[2][3]
+        self.args, self.grid, self.block = args_of_cells[1], args_of_cells[2], args_of_cells[3]
         return True
 
     def _argument_block(self, kernel, vals, arrays, lo, hi):

@@ -86,6 +86,8 @@ class Spec:
                                  # of every block of rows by the stripe of the gathered operand they read, 'cells' =
                                  # the kernel that runs those groups (`parts` stripes, dealt to the XCDs by workgroup
                                  # number); '' = a kernel that runs the loop body
+    skip_long: bool = False      # with 'group' and the kernel that adds the sums of its cells: rows whose simd loop is longer
+                                 # than a limit given at the launch are passed over (they run in planned parts)
     guard: int = 0               # 1 = the kernel returns at once when the grouping kernel of this launch has refused
                                  # its input (row ranges that do not follow one another: a flag in device memory),
                                  # 2 = when it has not
@@ -123,6 +125,8 @@ class Spec:
         elif self.parts and (self.rows != "list" or not (self.phase or self.aux == "plan") or self.parts % 8
                              or not 8 <= self.parts <= 64):
             raise ValueError("planned parts belong to the two-phase kernels over listed rows (8, 16, ... 64 parts)")
+        if self.skip_long and not (self.aux == "group" or (self.phase == 2 and self.guard == 1 and not self.rows)):
+            raise ValueError("only the grouping kernel and the kernel that adds the sums of its cells pass over long rows")
         if self.guard not in (0, 1, 2) or (self.guard and self.kind != "team"):
             raise ValueError("only team kernels wait on the verdict of a grouping kernel (guard 1 or 2)")
         if self.aux == "plan" and (self.rows != "list" or not self.parts or self.width < self.parts):
@@ -141,7 +145,7 @@ class Spec:
                 f"{'_e' + str(self.extent) if self.extent else ''}{'_nts' if self.stream_stores else ''}"
                 f"{'_lds' + str(self.lds_tile) if self.lds_tile else ''}{'' if self.hoist_guarded else '_g'}{'_chk' if self.checked else ''}{'_c2' if self.collapse else ''}{'_p' + str(self.phase) if self.phase else ''}{'_rc' + str(self.row_steps) if self.row_steps else ''}"
                 f"{'_' + self.rows if self.rows else ''}{'_s' + str(self.parts) if self.parts else ''}{'_' + self.aux if self.aux else ''}"
-                f"{'_if' + str(self.guard) if self.guard else ''}")
+                f"{'_sl' if self.skip_long else ''}{'_if' + str(self.guard) if self.guard else ''}")
 
 
 @dataclass
@@ -2188,7 +2192,11 @@ class KernelBuilder:
             else:
                 self.w(f"for (appy::i64 __i = __lo + blockIdx.x * {tpb}LL + __team; __i < __hi; __i += gridDim.x * {tpb}LL) {{")
                 self.ind += 1
-                self._iteration("__i")
+                if s.skip_long:
+                    # rows beyond the limit have run in planned parts, their statements after the loop with them
+                    self._split_iteration("__i", guard="__trip <= __rowmax")
+                else:
+                    self._iteration("__i")
             self.mode = "lane"
             self.ind -= 1
             self.w("}")
@@ -2508,7 +2516,7 @@ class KernelBuilder:
         w("const int __lid = threadIdx.x & 63;")
         w("const int __wvl = threadIdx.x >> 6;")
         w(f"__shared__ int __lp_all[4][{R + 1}];      // where the rows of the block start; the last entry: where it ends")
-        w(f"__shared__ int __hq_all[4][{R}];          // where they end")
+        w(f"__shared__ int __hq_all[4][{R + 1}];      // where they end")
         w("int* __lp = __lp_all[__wvl];")
         w("int* __hq = __hq_all[__wvl];")
         w(f"const appy::i64 __nblk = (__hi - __lo + {R - 1}) / {R};")
@@ -2548,7 +2556,8 @@ class KernelBuilder:
         w("    else if (__r == __nr - 1 && __r0 + __nr < __hi) __good = __good && __lp[__nr] >= __hq[__r];")
         w("}")
         w("__good = __ballot(!__good) == 0ull;")
-        w("if (__ballot(__long) != 0ull && __lid == 0) __hint[0] = 2;      // rows too long for this treatment: the next launch sorts them")
+        if not self.spec.skip_long:
+            w("if (__ballot(__long) != 0ull && __lid == 0) __hint[0] = 2;      // rows too long for this treatment: the next launch sorts them")
         w("const int __first = __good ? __lp[0] : 0, __end = __good ? __hq[__nr - 1] : 0;")
         w("appy::wave_fence();")
         w("#pragma unroll")
@@ -2563,6 +2572,60 @@ class KernelBuilder:
         w(f"    if (__lid <= {S}) __desc[__b * {S + 1} + __lid] = 0;")
         w("    continue;")
         w("}")
+        skip = self.spec.skip_long
+
+        def find_row(table, at):
+            w(f"int __row = 0, __past = {R};       // the last row that starts at or before {at}")
+            w("#pragma unroll")
+            w(f"for (int __it = 0; __it < {R.bit_length() - 1}; ++__it) {{")
+            w("    const int __mid = (__row + __past) >> 1;")
+            w(f"    if ({table}[__mid] <= {at}) __row = __mid; else __past = __mid;")
+            w("}")
+
+        def count(k):
+            w("#pragma unroll")
+            w("for (int __q = 0; __q < 4; ++__q)")
+            w("#pragma unroll")
+            w(f"    for (int __s = 0; __s < {S}; ++__s) __cnt[__s] += __popcll(__ballot((__c[{k}][__q] >> __shiftc) == __s));")
+
+        def starts():
+            w("__at[0] = __first;")
+            w("#pragma unroll")
+            w(f"for (int __s = 0; __s < {S}; ++__s) __at[__s + 1] = __at[__s] + __cnt[__s];")
+            w("#pragma unroll")
+            w(f"for (int __s = 0; __s <= {S}; ++__s) if (__lid == __s) __desc[__b * {S + 1} + __s] = __at[__s];")
+
+        def place_one(kc, kv):
+            w(f"const int __cq = __c[{kc}][__q];")
+            w("const int __sq = __cq >> __shiftc;          // negative past the end (and for negative indices: such elements are dropped)")
+            w("int __pos = 0;")
+            w("#pragma unroll")
+            w(f"for (int __s = 0; __s < {S}; ++__s) {{")
+            w("    const unsigned long long __m = __ballot(__sq == __s);")
+            w("    if (__sq == __s) __pos = __at[__s] + __popcll(__m & __below);")
+            w("    __at[__s] += __popcll(__m);")
+            w("}")
+            w(f"if (__sq >= 0 && __sq < {S})")
+            w("    __ent[__pos] = (long long)(((unsigned long long)(((unsigned)__row << 24) | (unsigned)(__cq & __cmask)) << 32) "
+              f"| (unsigned long long)(unsigned)__v[{kv}][__q]);")
+
+        def unrolled(n, fn):
+            w("#pragma unroll")
+            w(f"for (int __k = 0; __k < {n}; ++__k) {{")
+            self.ind += 1
+            fn()
+            self.ind -= 1
+            w("}")
+
+        w(f"int __cnt[{S}], __at[{S + 1}];")
+        w("#pragma unroll")
+        w(f"for (int __s = 0; __s < {S}; ++__s) __cnt[__s] = 0;")
+        if skip:
+            self._group_walk_kept(idx_c, car_c, U, find_row, count, starts, place_one, unrolled)
+            self.ind -= 1
+            w("}")
+            return
+
         def load_indices(k, j0, kk):
             w(f"{{ const int __j = {j0} + {kk} * 256 + __lid * 4;")
             w(f"if (__j + 4 <= __end) __c[{k}] = appy::vload<int, 4>({idx_c} + __j);")
@@ -2582,57 +2645,17 @@ class KernelBuilder:
             else:
                 w(f"__v[{k}] = 0;")
 
-        def count(k):
-            w("#pragma unroll")
-            w("for (int __q = 0; __q < 4; ++__q)")
-            w("#pragma unroll")
-            w(f"    for (int __s = 0; __s < {S}; ++__s) __cnt[__s] += __popcll(__ballot((__c[{k}][__q] >> __shiftc) == __s));")
-
-        def starts():
-            w("__at[0] = __first;")
-            w("#pragma unroll")
-            w(f"for (int __s = 0; __s < {S}; ++__s) __at[__s + 1] = __at[__s] + __cnt[__s];")
-            w("#pragma unroll")
-            w(f"for (int __s = 0; __s <= {S}; ++__s) if (__lid == __s) __desc[__b * {S + 1} + __s] = __at[__s];")
-
         def place(kc, kv, j0, kk):
             w(f"const int __j = {j0} + {kk} * 256 + __lid * 4;")
-            w(f"int __row = 0, __past = {R};       // the last row that starts at or before __j")
-            w("#pragma unroll")
-            w(f"for (int __it = 0; __it < {R.bit_length() - 1}; ++__it) {{")
-            w("    const int __mid = (__row + __past) >> 1;")
-            w("    if (__lp[__mid] <= __j) __row = __mid; else __past = __mid;")
-            w("}")
+            find_row("__lp", "__j")
             w("#pragma unroll")
             w("for (int __q = 0; __q < 4; ++__q) {")
             self.ind += 1
-            w(f"const int __cq = __c[{kc}][__q];")
-            w("const int __sq = __cq >> __shiftc;          // negative past the end (and for negative indices: such elements are dropped)")
             w("if (__j + __q < __end) while (__lp[__row + 1] <= __j + __q) ++__row;")
-            w("int __pos = 0;")
-            w("#pragma unroll")
-            w(f"for (int __s = 0; __s < {S}; ++__s) {{")
-            w("    const unsigned long long __m = __ballot(__sq == __s);")
-            w("    if (__sq == __s) __pos = __at[__s] + __popcll(__m & __below);")
-            w("    __at[__s] += __popcll(__m);")
-            w("}")
-            w(f"if (__sq >= 0 && __sq < {S})")
-            w("    __ent[__pos] = (long long)(((unsigned long long)(((unsigned)__row << 24) | (unsigned)(__cq & __cmask)) << 32) "
-              f"| (unsigned long long)(unsigned)__v[{kv}][__q]);")
+            place_one(kc, kv)
             self.ind -= 1
             w("}")
 
-        def unrolled(n, fn):
-            w("#pragma unroll")
-            w(f"for (int __k = 0; __k < {n}; ++__k) {{")
-            self.ind += 1
-            fn()
-            self.ind -= 1
-            w("}")
-
-        w(f"int __cnt[{S}], __at[{S + 1}];")
-        w("#pragma unroll")
-        w(f"for (int __s = 0; __s < {S}; ++__s) __cnt[__s] = 0;")
         # (indices of a whole block kept in registers between the two passes - 64 registers, half the wavefronts per
         #  SIMD - made this kernel slower: 455 us against 306 for 2^26 elements)
         w(f"for (int __j0 = __first; __j0 < __end; __j0 += {256 * U}) {{")
@@ -2650,6 +2673,97 @@ class KernelBuilder:
         unrolled(U, lambda: place("__k", "__k", "__j0", "__k"))
         self.ind -= 1
         w("}")
+        self.ind -= 1
+        w("}")
+
+    def _group_walk_kept(self, idx_c, car_c, U, find_row, count, starts, place_one, unrolled):
+        """The two passes of the grouping kernel over the elements of the rows that are kept (rows
+        beyond `__rowmax` elements run in planned parts): the lanes walk the kept elements of the block
+        as one sequence; `__kp[r]` is where row r starts in it."""
+        R = self.GROUP_ROWS
+        w = self.w
+        w("// where every row starts among the elements that are kept (rows beyond the limit hold none): lane l sums rows 4l .. 4l + 3")
+        w("int* __kp = __hq;")
+        w("int __kt[4], __mine = 0;")
+        w("#pragma unroll")
+        w("for (int __i = 0; __i < 4; ++__i) {")
+        w("    const int __r = 4 * __lid + __i;")
+        w("    const int __n = __r < __nr ? __hq[__r] - __lp[__r] : 0;")
+        w("    __kt[__i] = __n > __rowmax ? 0 : __n;")
+        w("    __mine += __kt[__i];")
+        w("}")
+        w("int __incl = __mine;")
+        w("#pragma unroll")
+        w("for (int __d = 1; __d < 64; __d <<= 1) {")
+        w("    const int __o = __shfl_up(__incl, __d, 64);")
+        w("    if (__lid >= __d) __incl += __o;")
+        w("}")
+        w("appy::wave_fence();       // the ends of the rows have been read: their table now holds the starts among the kept")
+        w("__kp[4 * __lid] = __incl - __mine;")
+        w("__kp[4 * __lid + 1] = __incl - __mine + __kt[0];")
+        w("__kp[4 * __lid + 2] = __incl - __mine + __kt[0] + __kt[1];")
+        w("__kp[4 * __lid + 3] = __incl - __mine + __kt[0] + __kt[1] + __kt[2];")
+        w(f"if (__lid == 63) __kp[{R}] = __incl;")
+        w("appy::wave_fence();")
+        w(f"const int __kept = __kp[{R}];")
+
+        def positions(k):
+            """Row and array positions of the four kept elements __t .. __t + 3 of this lane."""
+            w(f"const int __t = __t0 + {k} * 256 + __lid * 4;")
+            find_row("__kp", "__t")
+            w("int __jq[4];")
+            w("#pragma unroll")
+            w("for (int __q = 0; __q < 4; ++__q) {")
+            w("    if (__t + __q < __kept) while (__kp[__row + 1] <= __t + __q) ++__row;")
+            w("    __jq[__q] = __lp[__row] + (__t + __q - __kp[__row]);")
+            w("}")
+            w("const bool __run = __t + 4 <= __kept && __jq[3] == __jq[0] + 3;       // four elements in a row of the arrays")
+
+        def load(k, both):
+            w("{")
+            self.ind += 1
+            positions(k)
+            w(f"if (__run) __c[{k}] = appy::vload<int, 4>({idx_c} + __jq[0]);")
+            w("else {")
+            w("#pragma unroll")
+            w(f"    for (int __q = 0; __q < 4; ++__q) __c[{k}][__q] = __t + __q < __kept ? {idx_c}[__jq[__q]] : -1;")
+            w("}")
+            if both:
+                if car_c:
+                    w(f"if (__run) __v[{k}] = appy::vload<int, 4>({car_c} + __jq[0]);")
+                    w("else {")
+                    w("#pragma unroll")
+                    w(f"    for (int __q = 0; __q < 4; ++__q) __v[{k}][__q] = __t + __q < __kept ? {car_c}[__jq[__q]] : 0;")
+                    w("}")
+                else:
+                    w(f"__v[{k}] = 0;")
+            self.ind -= 1
+            w("}")
+
+        def place(k):
+            w(f"const int __t = __t0 + {k} * 256 + __lid * 4;")
+            find_row("__kp", "__t")
+            w("#pragma unroll")
+            w("for (int __q = 0; __q < 4; ++__q) {")
+            self.ind += 1
+            w("if (__t + __q < __kept) while (__kp[__row + 1] <= __t + __q) ++__row;")
+            place_one(k, k)
+            self.ind -= 1
+            w("}")
+
+        w(f"for (int __t0 = 0; __t0 < __kept; __t0 += {256 * U}) {{")
+        self.ind += 1
+        w(f"appy::vec<int, 4>::type __c[{U}];")
+        unrolled(U, lambda: load("__k", False))
+        unrolled(U, lambda: count("__k"))
+        self.ind -= 1
+        w("}")
+        starts()
+        w(f"for (int __t0 = 0; __t0 < __kept; __t0 += {256 * U}) {{")
+        self.ind += 1
+        w(f"appy::vec<int, 4>::type __c[{U}], __v[{U}];")
+        unrolled(U, lambda: load("__k", True))
+        unrolled(U, lambda: place("__k"))
         self.ind -= 1
         w("}")
 
@@ -2898,6 +3012,8 @@ class KernelBuilder:
             params.append(Param("__len", "const appy::i64 __len", C.c_int64, "entries"))
             params.append(Param("__rowmax", "const appy::i64 __rowmax", C.c_int64, "rowmax"))
             params.append(Param("__hint", "long long* __hint", C.c_void_p, "hint"))
+        if sp.skip_long and sp.aux != "group":
+            params.append(Param("__rowmax", "const appy::i64 __rowmax", C.c_int64, "rowmax"))
         if sp.aux == "cells":
             params.append(Param("__scratch", "double* __scratch", C.c_void_p, "scratch"))
         if sp.aux == "group" or sp.guard:

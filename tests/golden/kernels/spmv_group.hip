@@ -19,7 +19,7 @@ _spmv_kernel_loop_1_group(
     const int __lid = threadIdx.x & 63;
     const int __wvl = threadIdx.x >> 6;
     __shared__ int __lp_all[4][257];      // where the rows of the block start; the last entry: where it ends
-    __shared__ int __hq_all[4][256];          // where they end
+    __shared__ int __hq_all[4][257];      // where they end
     int* __lp = __lp_all[__wvl];
     int* __hq = __hq_all[__wvl];
     const appy::i64 __nblk = (__hi - __lo + 255) / 256;
@@ -127,9 +127,9 @@ _spmv_kernel_loop_1_group(
                 }
                 #pragma unroll
                 for (int __q = 0; __q < 4; ++__q) {
+                    if (__j + __q < __end) while (__lp[__row + 1] <= __j + __q) ++__row;
                     const int __cq = __c[__k][__q];
                     const int __sq = __cq >> __shiftc;          // negative past the end (and for negative indices: such elements are dropped)
-                    if (__j + __q < __end) while (__lp[__row + 1] <= __j + __q) ++__row;
                     int __pos = 0;
                     #pragma unroll
                     for (int __s = 0; __s < 8; ++__s) {

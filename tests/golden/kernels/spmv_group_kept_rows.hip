@@ -1,0 +1,198 @@
+// kernel for spmv_kernel_loop_1_group: team_b256_v1_u1_w64_r_s8_group_sl
+extern "C" __global__ void __launch_bounds__(256)
+_spmv_kernel_loop_1_group(
+    const int* __restrict__ A_indptr,
+    const float* __restrict__ A_data,
+    const float* __restrict__ x,
+    const int* __restrict__ A_indices,
+    float* __restrict__ y,
+    long long* __ent,
+    int* __desc,
+    const int __shiftc,
+    const appy::i64 __len,
+    const appy::i64 __rowmax,
+    long long* __hint,
+    long long* __flag,
+    const appy::i64 __lo,
+    const appy::i64 __hi)
+{
+    const int __lid = threadIdx.x & 63;
+    const int __wvl = threadIdx.x >> 6;
+    __shared__ int __lp_all[4][257];      // where the rows of the block start; the last entry: where it ends
+    __shared__ int __hq_all[4][257];      // where they end
+    int* __lp = __lp_all[__wvl];
+    int* __hq = __hq_all[__wvl];
+    const appy::i64 __nblk = (__hi - __lo + 255) / 256;
+    const int __cmask = (1 << __shiftc) - 1;
+    const unsigned long long __below = (1ull << __lid) - 1ull;
+    for (appy::i64 __b = (appy::i64)blockIdx.x * 4 + __wvl; __b < __nblk; __b += (appy::i64)gridDim.x * 4) {
+        const appy::i64 __r0 = __lo + __b * 256;
+        const int __nr = (int)((__hi - __r0) < 256 ? (__hi - __r0) : 256);
+        appy::wave_fence();       // the block before this one has been read out of __lp
+        bool __good = true, __long = false;
+        #pragma unroll
+        for (int __k = 0; __k < 5; ++__k) {      // and the first row of the next block, if there is one
+            const int __r = __k * 64 + __lid;
+            if (__r <= __nr && __r0 + __r < __hi && (__k < 4 || __lid == 0)) {
+                const appy::i64 i = __r0 + __r;
+                int start = 0;
+                int end = 0;
+                double s = 0;
+                start = A_indptr[i];
+                end = A_indptr[(i + 1LL)];
+                s = 0.0;
+                const appy::i64 __rlo = ((long long)(start));
+                const appy::i64 __rhi = ((long long)(end));
+                if (__rlo < 0 || __rhi < __rlo || __rhi > __len) __good = false;
+                __lp[__r] = (int)__rlo;
+                if (__r < __nr) { __hq[__r] = (int)__rhi; __long = __long || (__rhi - __rlo > __rowmax); }
+            }
+        }
+        appy::wave_fence();
+        // every row ends where the next one starts; the block ends no later than the next one starts
+        #pragma unroll
+        for (int __k = 0; __k < 4; ++__k) {
+            const int __r = __k * 64 + __lid;
+            if (__r < __nr - 1) __good = __good && __lp[__r + 1] == __hq[__r];
+            else if (__r == __nr - 1 && __r0 + __nr < __hi) __good = __good && __lp[__nr] >= __hq[__r];
+        }
+        __good = __ballot(!__good) == 0ull;
+        const int __first = __good ? __lp[0] : 0, __end = __good ? __hq[__nr - 1] : 0;
+        appy::wave_fence();
+        #pragma unroll
+        for (int __k = 0; __k < 5; ++__k) {
+            const int __r = __k * 64 + __lid;
+            if (__r >= __nr && __r <= 256 && (__k < 4 || __lid == 0)) __lp[__r] = __end;
+        }
+        appy::wave_fence();
+        if (!__good) {
+            // refused: the launch runs the loop row by row instead; the cells of this block stay empty
+            if (__lid == 0) __flag[0] = 1;
+            if (__lid <= 8) __desc[__b * 9 + __lid] = 0;
+            continue;
+        }
+        int __cnt[8], __at[9];
+        #pragma unroll
+        for (int __s = 0; __s < 8; ++__s) __cnt[__s] = 0;
+        // where every row starts among the elements that are kept (rows beyond the limit hold none): lane l sums rows 4l .. 4l + 3
+        int* __kp = __hq;
+        int __kt[4], __mine = 0;
+        #pragma unroll
+        for (int __i = 0; __i < 4; ++__i) {
+            const int __r = 4 * __lid + __i;
+            const int __n = __r < __nr ? __hq[__r] - __lp[__r] : 0;
+            __kt[__i] = __n > __rowmax ? 0 : __n;
+            __mine += __kt[__i];
+        }
+        int __incl = __mine;
+        #pragma unroll
+        for (int __d = 1; __d < 64; __d <<= 1) {
+            const int __o = __shfl_up(__incl, __d, 64);
+            if (__lid >= __d) __incl += __o;
+        }
+        appy::wave_fence();       // the ends of the rows have been read: their table now holds the starts among the kept
+        __kp[4 * __lid] = __incl - __mine;
+        __kp[4 * __lid + 1] = __incl - __mine + __kt[0];
+        __kp[4 * __lid + 2] = __incl - __mine + __kt[0] + __kt[1];
+        __kp[4 * __lid + 3] = __incl - __mine + __kt[0] + __kt[1] + __kt[2];
+        if (__lid == 63) __kp[256] = __incl;
+        appy::wave_fence();
+        const int __kept = __kp[256];
+        for (int __t0 = 0; __t0 < __kept; __t0 += 1024) {
+            appy::vec<int, 4>::type __c[4];
+            #pragma unroll
+            for (int __k = 0; __k < 4; ++__k) {
+                {
+                    const int __t = __t0 + __k * 256 + __lid * 4;
+                    int __row = 0, __past = 256;       // the last row that starts at or before __t
+                    #pragma unroll
+                    for (int __it = 0; __it < 8; ++__it) {
+                        const int __mid = (__row + __past) >> 1;
+                        if (__kp[__mid] <= __t) __row = __mid; else __past = __mid;
+                    }
+                    int __jq[4];
+                    #pragma unroll
+                    for (int __q = 0; __q < 4; ++__q) {
+                        if (__t + __q < __kept) while (__kp[__row + 1] <= __t + __q) ++__row;
+                        __jq[__q] = __lp[__row] + (__t + __q - __kp[__row]);
+                    }
+                    const bool __run = __t + 4 <= __kept && __jq[3] == __jq[0] + 3;       // four elements in a row of the arrays
+                    if (__run) __c[__k] = appy::vload<int, 4>(A_indices + __jq[0]);
+                    else {
+                    #pragma unroll
+                        for (int __q = 0; __q < 4; ++__q) __c[__k][__q] = __t + __q < __kept ? A_indices[__jq[__q]] : -1;
+                    }
+                }
+            }
+            #pragma unroll
+            for (int __k = 0; __k < 4; ++__k) {
+                #pragma unroll
+                for (int __q = 0; __q < 4; ++__q)
+                #pragma unroll
+                    for (int __s = 0; __s < 8; ++__s) __cnt[__s] += __popcll(__ballot((__c[__k][__q] >> __shiftc) == __s));
+            }
+        }
+        __at[0] = __first;
+        #pragma unroll
+        for (int __s = 0; __s < 8; ++__s) __at[__s + 1] = __at[__s] + __cnt[__s];
+        #pragma unroll
+        for (int __s = 0; __s <= 8; ++__s) if (__lid == __s) __desc[__b * 9 + __s] = __at[__s];
+        for (int __t0 = 0; __t0 < __kept; __t0 += 1024) {
+            appy::vec<int, 4>::type __c[4], __v[4];
+            #pragma unroll
+            for (int __k = 0; __k < 4; ++__k) {
+                {
+                    const int __t = __t0 + __k * 256 + __lid * 4;
+                    int __row = 0, __past = 256;       // the last row that starts at or before __t
+                    #pragma unroll
+                    for (int __it = 0; __it < 8; ++__it) {
+                        const int __mid = (__row + __past) >> 1;
+                        if (__kp[__mid] <= __t) __row = __mid; else __past = __mid;
+                    }
+                    int __jq[4];
+                    #pragma unroll
+                    for (int __q = 0; __q < 4; ++__q) {
+                        if (__t + __q < __kept) while (__kp[__row + 1] <= __t + __q) ++__row;
+                        __jq[__q] = __lp[__row] + (__t + __q - __kp[__row]);
+                    }
+                    const bool __run = __t + 4 <= __kept && __jq[3] == __jq[0] + 3;       // four elements in a row of the arrays
+                    if (__run) __c[__k] = appy::vload<int, 4>(A_indices + __jq[0]);
+                    else {
+                    #pragma unroll
+                        for (int __q = 0; __q < 4; ++__q) __c[__k][__q] = __t + __q < __kept ? A_indices[__jq[__q]] : -1;
+                    }
+                    if (__run) __v[__k] = appy::vload<int, 4>(reinterpret_cast<const int*>(A_data) + __jq[0]);
+                    else {
+                    #pragma unroll
+                        for (int __q = 0; __q < 4; ++__q) __v[__k][__q] = __t + __q < __kept ? reinterpret_cast<const int*>(A_data)[__jq[__q]] : 0;
+                    }
+                }
+            }
+            #pragma unroll
+            for (int __k = 0; __k < 4; ++__k) {
+                const int __t = __t0 + __k * 256 + __lid * 4;
+                int __row = 0, __past = 256;       // the last row that starts at or before __t
+                #pragma unroll
+                for (int __it = 0; __it < 8; ++__it) {
+                    const int __mid = (__row + __past) >> 1;
+                    if (__kp[__mid] <= __t) __row = __mid; else __past = __mid;
+                }
+                #pragma unroll
+                for (int __q = 0; __q < 4; ++__q) {
+                    if (__t + __q < __kept) while (__kp[__row + 1] <= __t + __q) ++__row;
+                    const int __cq = __c[__k][__q];
+                    const int __sq = __cq >> __shiftc;          // negative past the end (and for negative indices: such elements are dropped)
+                    int __pos = 0;
+                    #pragma unroll
+                    for (int __s = 0; __s < 8; ++__s) {
+                        const unsigned long long __m = __ballot(__sq == __s);
+                        if (__sq == __s) __pos = __at[__s] + __popcll(__m & __below);
+                        __at[__s] += __popcll(__m);
+                    }
+                    if (__sq >= 0 && __sq < 8)
+                        __ent[__pos] = (long long)(((unsigned long long)(((unsigned)__row << 24) | (unsigned)(__cq & __cmask)) << 32) | (unsigned long long)(unsigned)__v[__k][__q]);
+                }
+            }
+        }
+    }
+}

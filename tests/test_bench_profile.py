@@ -63,8 +63,8 @@ def test_profile_was_measured_with_the_shape_the_bench_launches(workload):
     env = dict(env, __appy_mid=n_outer // 2)
     arrays = {k: v for k, v in arrays.items() if k in loop.analysis.arrays}
     spec = loop.choose_spec(n_outer, env, arrays)
-    if workload == "spmv_uniform":
-        # rows of 16 elements: from the second launch on (the bench times those) the elements are grouped by stripe
+    if workload.startswith("spmv_"):
+        # from the second launch on (the bench times those) the elements of rows up to 512 elements are grouped by stripe
         assert spec.rows == "mixed"
         stripes, _shift, _entries = loop.grouped_shape(n_outer, env, arrays)
         spec = cg.Spec("team", block=256, vec=1, width=64, parts=stripes, aux="cells", guard=1)

@@ -44,6 +44,17 @@ def _grouped(launch):
     return launch.sequence is not None and launch.spec.aux == "cells"
 
 
+@appy.jit
+def windows(data, start, end, indices, x, y, beta, m):
+    #pragma parallel for
+    for i in range(m):
+        s = 0.0
+        #pragma simd
+        for j in range(start[i], end[i]):
+            s += data[j] * x[indices[j]]
+        y[i] = beta * y[i] + s
+
+
 def _matrix(lengths, n, seed):
     rng = np.random.default_rng(seed)
     data, indptr, indices = wl.csr_matrix(np.asarray(lengths, dtype=np.int64), n, rng)
@@ -86,9 +97,10 @@ def test_short_rows_are_grouped_from_the_second_launch_on(k, m, n, lengths):
     assert np.array_equal(y1, k.spmv(data, indptr, indices, x, m, n))
 
 
-def test_a_matrix_with_long_rows_goes_back_to_rows_sorted_by_length(k):
-    """The grouped form is chosen from what the last launch reported.  When the rows it then meets are
-    longer than that, the result is still right, and the launch after it sorts the rows again."""
+def test_matrices_with_long_rows_group_their_short_rows_and_cut_the_long_ones(k):
+    """The form of a launch follows what the last launch reported.  Rows longer than it was told of are
+    still summed correctly (and reported); once the rows have been sorted again, the elements of the short
+    rows are grouped and the long rows run in parts cut at the stripes, in one launch."""
     m, n = 40_000, 1 << 20
     short = _matrix(np.full(m, 12), n, seed=1)
     rng = np.random.default_rng(2)
@@ -97,18 +109,57 @@ def test_a_matrix_with_long_rows_goes_back_to_rows_sorted_by_length(k):
     _forget()
     k.spmv(*short, m, n)
     k.spmv(*short, m, n)
-    assert _grouped(_loop("spmv").last_launch)
+    launch = _loop("spmv").last_launch
+    assert _grouped(launch) and len(launch.sequence) == 5
     ref, budget = vo.spmv_csr(*long_, (m, n))
     y = k.spmv(*long_, m, n)
-    assert _grouped(_loop("spmv").last_launch)              # shaped by the report on the short rows
+    launch = _loop("spmv").last_launch
+    assert _grouped(launch) and len(launch.sequence) == 5   # shaped by the report on the short rows
     ok, worst = vo.within_budget(y, ref, budget, TOL)
     assert ok, worst
     y = k.spmv(*long_, m, n)
     assert _loop("spmv").last_launch.spec.rows == "mixed"   # the grouping kernel has seen the long rows
     ok, worst = vo.within_budget(y, ref, budget, TOL)
     assert ok, worst
-    y = k.spmv(*long_, m, n)
-    assert _loop("spmv").last_launch.spec.rows == "mixed" and len(_loop("spmv").last_launch.sequence) == 6
+    for _ in range(2):
+        y = k.spmv(*long_, m, n)
+        launch = _loop("spmv").last_launch
+        assert _grouped(launch)
+        names = [step[0].src.name.rsplit("_", 1)[-1] if step[0] else "clear" for step in launch.sequence]
+        assert names == ["clear", "bins", "group", "cells", "sums", "plan", "parts", "fold", "rowwise"], names
+        cut = launch.bin["rowmax"]
+        assert cut == 512 and (ln > cut).sum() > 100 and (ln <= cut).sum() > 100
+        ok, worst = vo.within_budget(y, ref, budget, TOL)
+        assert ok, worst
+    # and back: a matrix of short rows after one with long rows (the lists of long rows are empty)
+    ref, budget = vo.spmv_csr(*short, (m, n))
+    y = k.spmv(*short, m, n)
+    assert len(_loop("spmv").last_launch.sequence) == 9
+    ok, worst = vo.within_budget(y, ref, budget, TOL)
+    assert ok, worst
+
+
+def test_rows_of_every_length_around_the_cut(k):
+    """Row lengths on both sides of the limit between grouped and cut rows, empty rows, blocks made of
+    long rows only, and a last block that is not full."""
+    rng = np.random.default_rng(14)
+    m, n = 36_001, 1 << 21
+    pool = np.array([0, 1, 3, 4, 5, 31, 128, 129, 511, 512, 513, 700, 2000, 4096], dtype=np.int64)
+    ln = pool[rng.integers(0, len(pool), m)]
+    ln[1024:1024 + 512] = 3000              # two whole blocks of long rows
+    ln[4096:4096 + 256] = 0                 # an empty block
+    data, indptr, indices, x = _matrix(ln, n, seed=15)
+    ref, budget = vo.spmv_csr(data, indptr, indices, x, (m, n))
+    _forget()
+    tags = []
+    for _ in range(3):
+        y = k.spmv(data, indptr, indices, x, m, n)
+        launch = _loop("spmv").last_launch
+        tags.append(len(launch.sequence) if _grouped(launch) else 0)
+        ok, worst = vo.within_budget(y, ref, budget, TOL)
+        assert ok, worst
+        assert np.all(y[ln == 0] == 0.0)
+    assert tags == [0, 9, 9]
 
 
 def test_row_ranges_that_do_not_follow_one_another_run_row_by_row(gpu):
@@ -118,16 +169,6 @@ def test_row_ranges_that_do_not_follow_one_another_run_row_by_row(gpu):
     rng = np.random.default_rng(4)
     m, n, per = 40_000, 1 << 20, 16
     data, indptr, indices, x = _matrix(np.full(m, per), n, seed=5)
-
-    @appy.jit
-    def windows(data, start, end, indices, x, y, beta, m):
-        #pragma parallel for
-        for i in range(m):
-            s = 0.0
-            #pragma simd
-            for j in range(start[i], end[i]):
-                s += data[j] * x[indices[j]]
-            y[i] = beta * y[i] + s
 
     def run(start, end, expect_grouped=True):
         y = np.ones(m, dtype=np.float32)
@@ -160,6 +201,39 @@ def test_row_ranges_that_do_not_follow_one_another_run_row_by_row(gpu):
     e4 = end.copy()
     e4[-1] -= 5
     run(start, e4)
+
+
+def test_refused_ranges_in_a_launch_that_also_cuts_long_rows(gpu):
+    """Long and short rows, and ranges out of order: nothing of the launch but the row-by-row kernel may
+    touch `y`, which the statement after the loop updates in place."""
+    m, n = 40_000, 1 << 20
+    rng = np.random.default_rng(16)
+    ln = np.where(rng.random(m) < 0.02, rng.integers(600, 3000, m), rng.integers(1, 40, m))
+    data, indptr, indices, x = _matrix(ln, n, seed=17)
+    start, end = indptr[:-1].copy(), indptr[1:].copy()
+    terms = data.astype(np.float64) * x.astype(np.float64)[indices]
+    cs = np.concatenate([[0.0], np.cumsum(terms)])
+    ca = np.concatenate([[0.0], np.cumsum(np.abs(terms))])
+
+    def run(start, end, steps):
+        y = np.ones(m, dtype=np.float32)
+        windows(data, start, end, indices, x, y, 0.5, m)
+        launch = _loop("windows").last_launch
+        assert (len(launch.sequence) if _grouped(launch) else 0) == steps
+        lens = np.maximum(end.astype(np.int64) - start, 0)
+        ref = 0.5 + cs[start + lens] - cs[start]
+        budget = 0.5 + ca[start + lens] - ca[start]
+        assert np.all(np.abs(y - ref) <= TOL * budget + 1e-9 * ca[-1]), np.max(np.abs(y - ref))
+
+    _forget("windows")
+    run(start, end, 0)
+    run(start, end, 9)
+    long_row = int(np.flatnonzero(ln > 600)[5])
+    s2, e2 = start.copy(), end.copy()
+    s2[[long_row, 7]] = s2[[7, long_row]]
+    e2[[long_row, 7]] = e2[[7, long_row]]
+    run(s2, e2, 9)
+    run(start, end, 9)
 
 
 def test_terms_with_a_scalar_factor_integer_values_and_no_second_operand(gpu):
