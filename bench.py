@@ -400,9 +400,18 @@ def main():
         del h_data, h_ptr, h_idx, h_x
         lens = (indptr_d[1:] - indptr_d[:-1])
         parity[name] = {"worst_err_over_bound": worst, "ok": ok}
+        # the form of a launch follows what the launch before it reported about the rows (sorted by length first, then
+        # with the elements of the shorter rows grouped by column stripe): two more untimed calls reach the form a caller
+        # sees from then on, and the result of the timed launches is checked as well
+        for _ in range(2):
+            y_d = k.spmv(data_d, indptr_d, indices_d, x_d, m, ncol)
+            torch.cuda.synchronize()
         vals = {"A_data": data_d, "A_indptr": indptr_d, "A_indices": indices_d, "x": x_d, "y": y_d, "M": m}
         nbytes = 8 * nnz + 4 * (m + 1) + 4 * ncol + 4 * m
         results[name] = run.measure(loop, vals, nbytes, K, W)
+        ok2, worst2 = vo.within_budget(y_d.cpu().numpy(), ref, budget)
+        parity[name] = {"worst_err_over_bound": max(worst, worst2), "ok": bool(ok and ok2)}
+        del ref, budget
         seq = loop.last_launch.sequence
         results[name].update({"kernels_per_launch": sum(1 for step in seq if step[0] is not None) if seq else 1,
                               "nnz": int(nnz), "rows": m, "mean_row": float(nnz) / m, "max_row": int(lens.max().item()),
