@@ -669,7 +669,8 @@ class CompiledLoop:
         shift = max(1, (-(-nx // parts) - 1).bit_length())
         entries = min(int(arrays[nm].shape[0]) for nm in (g["idx"], g["carried"]) if nm)
         trip, _uniform = self._estimate_trip(env, arrays, n_outer)
-        if entries >= (1 << 31) or trip < GROUP_MIN_TRIP:
+        # (positions are 32-bit in the grouping kernel, and its loops step past the end by up to 1024)
+        if entries >= (1 << 31) - (1 << 16) or trip < GROUP_MIN_TRIP:
             return None
         return parts, shift, entries
 
