@@ -1156,7 +1156,9 @@ class Launch:
         (`cells`), add the sums of a row and run the rest of the body (phase 2).  The grouping kernel
         checks that the rows' ranges follow one another (as those of a CSR matrix do); where they do
         not, it raises a flag, the kernels after it return at once, and the loop runs row by row.
-        False (nothing staged) when the launch does not qualify."""
+        When the last launch has reported rows in the class of the longest, the same launch lists those
+        rows (`bins`), leaves them out of the groups and runs them in parts cut at the stripes (`plan`,
+        `parts`, `fold`).  False (nothing staged) when the launch does not qualify."""
         loop, a, env = self.loop, self.loop.analysis, self.env
         n = hi - lo
         g = a.grouping

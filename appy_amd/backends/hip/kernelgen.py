@@ -2502,6 +2502,11 @@ class KernelBuilder:
         return oc, ot, pty
 
     def _body_group(self):
+        """The grouping kernel.  Per block: the set-up of its rows (and of the first row of the next
+        block) gives the rows' ranges, which must follow one another - otherwise the block is refused
+        and the flag raised; a first pass over the elements counts them per stripe, a second pass
+        writes each element to its place.  The rank of an element within its stripe comes from
+        ballots taken in a fixed order, so the layout does not depend on timing."""
         a, g, S, R = self.a, self.a.grouping, self.spec.parts, self.GROUP_ROWS
         var = a.var
         self.ex.locals[var] = T.WEAK_INT
@@ -2768,6 +2773,9 @@ class KernelBuilder:
         w("}")
 
     def _body_cells(self):
+        """The kernel that runs the cells: the term of the sum is evaluated per grouped element (the carried
+        operand from the element, the gathered operand from its stripe) and added to the element's row
+        in LDS; the sums of a cell's rows go to the scratch table of 4-byte slots per row and stripe."""
         a, g, S, R = self.a, self.a.grouping, self.spec.parts, self.GROUP_ROWS
         self.ex.locals[a.var] = T.WEAK_INT
         self.mode = "lane"
