@@ -1222,7 +1222,8 @@ class Launch:
         hint_addr, _ = loop.hint(self.device)
         base = max(range(3), key=lambda c: seen[c + 1])
         self.bin = {"flag": buf + 1984, "desc": buf + off_desc, "ent": buf + off_ent, "shiftc": shift, "entries": entries,
-                    "rowmax": cut if long_rows else 32 * V, "hint": hint_addr,
+                    # (without long rows: the limit beyond which the launch that sorts the rows would have reported some)
+                    "rowmax": cut if long_rows else max(32 * V, 32 * parts), "hint": hint_addr,
                     "counts": buf, "load": buf + 32, "zero": buf + 1024, "rows": buf + off_rows, "m": n, "base": base,
                     "threshold": [V, 8 * V, cut], "bnd": buf + off_bnd, "rowstart": buf + off_start, "cap": cap,
                     "stripe": -(-int(arrays[g["x"]].shape[0]) // parts), "nrows": buf + 4 * 3}

@@ -162,6 +162,54 @@ def test_rows_of_every_length_around_the_cut(k):
     assert tags == [0, 9, 9]
 
 
+@pytest.mark.parametrize("with_long_rows", [False, True])
+def test_blocks_whose_elements_end_on_step_boundaries(k, with_long_rows):
+    """The grouping kernel walks a block's elements 1024 at a time, four per lane: blocks with exactly one or
+    two steps' worth of elements, one more, one fewer, long rows first, last and in between (their elements
+    are passed over, so four consecutive kept elements need not be consecutive in the arrays), single rows."""
+    rng = np.random.default_rng(30 + with_long_rows)
+    R = 256
+    L = 1000 if with_long_rows else 100          # a row beyond the cut / a long row that is still grouped
+    blocks = []
+
+    def block(lengths):
+        b = np.zeros(R, dtype=np.int64)
+        b[:len(lengths)] = lengths
+        blocks.append(b)
+
+    block([4] * 256)                               # 1024
+    block([4] * 255 + [3])                         # 1023
+    block([4] * 255 + [5])                         # 1025
+    block([8] * 256)                               # 2048
+    block([L] + [4] * 255)                         # long row first
+    block([4] * 255 + [L])                         # long row last
+    block([L if r % 2 else 3 for r in range(256)])  # every other row long
+    block([])                                      # nothing
+    block([512 if with_long_rows else 256])        # one row, exactly at the cut / at the end of the third class
+    block([513] if with_long_rows else [128])      # one row just beyond it
+    block([1] * 256)                               # one element per row
+    block([0, 0, 7, 0, L, 0, 2, 1, 0, 0, 3] * 23)  # gaps of empty rows around long ones
+    block([L] * 256 if with_long_rows else [96] * 256)
+    for _ in range(3):
+        block(rng.integers(0, 9, 256))
+    ln = np.concatenate([blocks[i] for i in rng.permutation(len(blocks) * 9) % len(blocks)])
+    ln = np.concatenate([ln, rng.integers(1, 6, 77)])          # a last block that is not full
+    m, n = len(ln), 1 << 20
+    assert m >= cg.BIN_MIN_ROWS
+    data, indptr, indices, x = _matrix(ln, n, seed=32)
+    ref, budget = vo.spmv_csr(data, indptr, indices, x, (m, n))
+    _forget()
+    forms = []
+    for _ in range(3):
+        y = k.spmv(data, indptr, indices, x, m, n)
+        launch = _loop("spmv").last_launch
+        forms.append(len(launch.sequence) if _grouped(launch) else 0)
+        ok, worst = vo.within_budget(y, ref, budget, TOL)
+        assert ok, (forms, worst)
+        assert np.all(y[ln == 0] == 0.0)
+    assert forms == ([0, 9, 9] if with_long_rows else [0, 5, 5])
+
+
 def test_row_ranges_that_do_not_follow_one_another_run_row_by_row(gpu):
     """`range(start[i], end[i])` need not describe a CSR matrix.  Ranges out of order, ranges that overlap
     and ranges with gaps are legal loops; the grouping kernel refuses them and the launch runs the loop
