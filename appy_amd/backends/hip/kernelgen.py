@@ -2403,10 +2403,28 @@ class KernelBuilder:
             # lane p < S - 1 looks for the first position whose index reaches stripe p + 1; a running
             # maximum over the lanes keeps the cuts in order, so that every position lies in exactly
             # one part whatever the order of the indices (sorted rows are cut at the stripes)
+            # (the search starts where the cut would lie if the indices were spread evenly and widens its steps from
+            #  there - two or three cache lines of indices per cut instead of one per level of a bisection of the whole
+            #  row; 0.14 ms of a 3 ms launch were these lines)
             self.w("appy::i64 __b = __rhi;")
-            self.w(f"if (__lane < {S - 1}) {{")
+            self.w(f"if (__lane < {S - 1} && __rhi > __rlo) {{")
             self.w("    const appy::i64 __target = (appy::i64)(__lane + 1) * __stripe;")
-            self.w("    appy::i64 __a = __rlo, __z = __rhi;")
+            self.w("    appy::i64 __a = __rlo, __z = __rhi;       // the cut lies in [__a, __z]: indices before __a are below the target")
+            self.w(f"    const appy::i64 __guess = __rlo + ((__rhi - __rlo) * (__lane + 1)) / {S};")
+            self.w("    appy::i64 __step = 16;")
+            self.w(f"    if ((appy::i64){cname(idx_name)}[__guess] < __target) {{")
+            self.w("        __a = __guess + 1;")
+            self.w("        while (__a < __z) {")
+            self.w("            const appy::i64 __p = (__a + __step - 1) < (__z - 1) ? (__a + __step - 1) : (__z - 1);")
+            self.w(f"            if ((appy::i64){cname(idx_name)}[__p] < __target) {{ __a = __p + 1; __step *= 4; }} else {{ __z = __p; break; }}")
+            self.w("        }")
+            self.w("    } else {")
+            self.w("        __z = __guess;")
+            self.w("        while (__a < __z) {")
+            self.w("            const appy::i64 __p = (__z - __step) > __a ? (__z - __step) : __a;")
+            self.w(f"            if ((appy::i64){cname(idx_name)}[__p] < __target) {{ __a = __p + 1; break; }} else {{ __z = __p; __step *= 4; }}")
+            self.w("        }")
+            self.w("    }")
             self.w("    while (__a < __z) {")
             self.w("        const appy::i64 __mid = __a + ((__z - __a) >> 1);")
             self.w(f"        if ((appy::i64){cname(idx_name)}[__mid] < __target) __a = __mid + 1; else __z = __mid;")

@@ -36,9 +36,24 @@ _spmv_kernel_loop_1_plan(
             const appy::i64 __rlo = ((long long)(start));
             const appy::i64 __rhi = (((long long)(end))) > __rlo ? (((long long)(end))) : __rlo;
             appy::i64 __b = __rhi;
-            if (__lane < 7) {
+            if (__lane < 7 && __rhi > __rlo) {
                 const appy::i64 __target = (appy::i64)(__lane + 1) * __stripe;
-                appy::i64 __a = __rlo, __z = __rhi;
+                appy::i64 __a = __rlo, __z = __rhi;       // the cut lies in [__a, __z]: indices before __a are below the target
+                const appy::i64 __guess = __rlo + ((__rhi - __rlo) * (__lane + 1)) / 8;
+                appy::i64 __step = 16;
+                if ((appy::i64)A_indices[__guess] < __target) {
+                    __a = __guess + 1;
+                    while (__a < __z) {
+                        const appy::i64 __p = (__a + __step - 1) < (__z - 1) ? (__a + __step - 1) : (__z - 1);
+                        if ((appy::i64)A_indices[__p] < __target) { __a = __p + 1; __step *= 4; } else { __z = __p; break; }
+                    }
+                } else {
+                    __z = __guess;
+                    while (__a < __z) {
+                        const appy::i64 __p = (__z - __step) > __a ? (__z - __step) : __a;
+                        if ((appy::i64)A_indices[__p] < __target) { __a = __p + 1; break; } else { __z = __p; __step *= 4; }
+                    }
+                }
                 while (__a < __z) {
                     const appy::i64 __mid = __a + ((__z - __a) >> 1);
                     if ((appy::i64)A_indices[__mid] < __target) __a = __mid + 1; else __z = __mid;
