@@ -1177,15 +1177,17 @@ class Launch:
         if shape is None:
             return False
         parts, shift, entries = shape
-        R = 256
+        # rows per block (blocks of 512 rows where the kept rows hold 7 elements on average - the power-law matrix with
+        # mean 16 - were measured slower: 0.780 ms against 0.745; there are half as many wavefronts to group them)
+        R = int(loop.options.get("hip_group_rows") or 256)
         nblk = -(-n // R)
         common = dict(block=256, restrict=spec.restrict)
         # rows beyond this many elements are cut at the stripes of the gathered operand, the others have their elements
         # grouped (power-law matrix: 3.14 ms with 128, 3.05 with 256, 3.02 with 512, 3.09 with 1024)
         cut = max(32 * V, 64 * parts)
         try:
-            group = loop.kernel_for(Spec("team", vec=1, width=64, parts=parts, aux="group", skip_long=long_rows, **common))
-            cells = loop.kernel_for(Spec("team", vec=1, width=64, parts=parts, aux="cells", guard=1, **common))
+            group = loop.kernel_for(Spec("team", vec=1, width=64, parts=parts, aux="group", block_rows=R, skip_long=long_rows, **common))
+            cells = loop.kernel_for(Spec("team", vec=1, width=64, parts=parts, aux="cells", block_rows=R, guard=1, **common))
             sums = loop.kernel_for(Spec("team", vec=V, width=1, phase=2, guard=1, skip_long=long_rows, **common))
             plain = loop._choose_spec(n, env, arrays, restrict=spec.restrict, listable=False)
             if plain.kind != "team" or plain.phase or plain.rows:
@@ -1481,7 +1483,7 @@ def _copy(node):
 def codegen(loop_source, loop_name, val_map, options):
     key = (loop_source, loop_name, _signature(val_map), options.get("hip_spec") and repr(options.get("hip_spec")),
            options.get("hip_max_blocks"), bool(options.get("check_bounds")), bool(options.get("hip_bins", True)),
-           bool(options.get("hip_group", True)), options.get("fn_name"))
+           bool(options.get("hip_group", True)), options.get("hip_group_rows"), options.get("fn_name"))
     # `clear_cache=True` regenerates the loop on every call instead of using the cached kernel
     # (reference: appy/backends/metal/codegen.py:23)
     fresh = bool(options.get("clear_cache"))

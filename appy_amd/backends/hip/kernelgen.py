@@ -86,6 +86,8 @@ class Spec:
                                  # of every block of rows by the stripe of the gathered operand they read, 'cells' =
                                  # the kernel that runs those groups (`parts` stripes, dealt to the XCDs by workgroup
                                  # number); '' = a kernel that runs the loop body
+    block_rows: int = 0          # with 'group' and 'cells': rows per block (256, 512 or 1024; more where rows are short,
+                                 # so that a cell still holds a few hundred elements)
     skip_long: bool = False      # with 'group' and the kernel that adds the sums of its cells: rows whose simd loop is longer
                                  # than a limit given at the launch are passed over (they run in planned parts)
     guard: int = 0               # 1 = the kernel returns at once when the grouping kernel of this launch has refused
@@ -120,8 +122,12 @@ class Spec:
                                         or self.row_steps or self.checked or self.width > 64):
             raise ValueError("rows are binned for plain team kernels only (teams inside a wavefront)")
         if self.aux in ("group", "cells"):
-            if self.rows or self.phase or self.parts not in (8, 16) or self.width != 64 or self.block != 256:
-                raise ValueError("elements are grouped by 8 or 16 stripes, one wavefront per block of rows, four per workgroup")
+            if (self.rows or self.phase or self.parts not in (8, 16) or self.width != 64 or self.block != 256
+                    or self.block_rows not in (256, 512, 1024)):
+                raise ValueError("elements are grouped by 8 or 16 stripes, one wavefront per block of 256, 512 or 1024 rows, "
+                                 "four per workgroup")
+        elif self.block_rows:
+            raise ValueError("only the kernels over grouped elements work on blocks of rows")
         elif self.parts and (self.rows != "list" or not (self.phase or self.aux == "plan") or self.parts % 8
                              or not 8 <= self.parts <= 64):
             raise ValueError("planned parts belong to the two-phase kernels over listed rows (8, 16, ... 64 parts)")
@@ -145,7 +151,7 @@ class Spec:
                 f"{'_e' + str(self.extent) if self.extent else ''}{'_nts' if self.stream_stores else ''}"
                 f"{'_lds' + str(self.lds_tile) if self.lds_tile else ''}{'' if self.hoist_guarded else '_g'}{'_chk' if self.checked else ''}{'_c2' if self.collapse else ''}{'_p' + str(self.phase) if self.phase else ''}{'_rc' + str(self.row_steps) if self.row_steps else ''}"
                 f"{'_' + self.rows if self.rows else ''}{'_s' + str(self.parts) if self.parts else ''}{'_' + self.aux if self.aux else ''}"
-                f"{'_sl' if self.skip_long else ''}{'_if' + str(self.guard) if self.guard else ''}")
+                f"{'_R' + str(self.block_rows) if self.block_rows else ''}{'_sl' if self.skip_long else ''}{'_if' + str(self.guard) if self.guard else ''}")
 
 
 @dataclass
@@ -2485,11 +2491,13 @@ class KernelBuilder:
         self.mode = "lane"
 
     # ---- elements grouped by the stripe of the gathered operand they read -------------------------------
-    # Blocks of 256 rows, one wavefront each.  The grouping kernel writes the elements of a block - the
-    # 32 bits of the carried operand, the row within the block (8 bits) and the position within the stripe
-    # (24 bits) - over the block's own range of positions, stripe after stripe, and where every stripe
+    # Blocks of `Spec.block_rows` rows, one wavefront each.  The grouping kernel writes the elements of a block -
+    # the 32 bits of the carried operand, the row within the block (10 bits) and the position within the stripe
+    # (22 bits) - over the block's own range of positions, stripe after stripe, and where every stripe
     # starts (`__desc`, `parts + 1` numbers per block).  A cell is one stripe of one block.
-    GROUP_ROWS = 256
+    @property
+    def GROUP_ROWS(self):
+        return self.spec.block_rows
 
     def _group_setup_types(self):
         """Walks the set-up of an iteration and the term of the sum into a buffer that is thrown away:
@@ -2542,6 +2550,16 @@ class KernelBuilder:
         w(f"__shared__ int __hq_all[4][{R + 1}];      // where they end")
         w("int* __lp = __lp_all[__wvl];")
         w("int* __hq = __hq_all[__wvl];")
+        if self.spec.skip_long:
+            # the sorting kernel of this launch has counted the rows of its classes: they go where the host reads them
+            # when it stages the next launch (as the kernel over rows of all classes does)
+            w("if (blockIdx.x == 0 && threadIdx.x == 0) {")
+            w("    const appy::i64 __others = (__base == 0 ? 0 : (appy::i64)__counts[0]) + (__base == 1 ? 0 : (appy::i64)__counts[1]) "
+              "+ (__base == 2 ? 0 : (appy::i64)__counts[2]) + (__base == 3 ? 0 : (appy::i64)__counts[3]);")
+            for c in range(4):
+                w(f"    __hint[{c + 1}] = (__base == {c}) ? (__hi - __lo) - __others : (appy::i64)__counts[{c}];")
+            w("    __hint[0] = 1;")
+            w("}")
         w(f"const appy::i64 __nblk = (__hi - __lo + {R - 1}) / {R};")
         w("const int __cmask = (1 << __shiftc) - 1;")
         w("const unsigned long long __below = (1ull << __lid) - 1ull;")
@@ -2629,7 +2647,7 @@ class KernelBuilder:
             w("    __at[__s] += __popcll(__m);")
             w("}")
             w(f"if (__sq >= 0 && __sq < {S})")
-            w("    __ent[__pos] = (long long)(((unsigned long long)(((unsigned)__row << 24) | (unsigned)(__cq & __cmask)) << 32) "
+            w("    __ent[__pos] = (long long)(((unsigned long long)(((unsigned)__row << 22) | (unsigned)(__cq & __cmask)) << 32) "
               f"| (unsigned long long)(unsigned)__v[{kv}][__q]);")
 
         def unrolled(n, fn):
@@ -2705,12 +2723,13 @@ class KernelBuilder:
         as one sequence; `__kp[r]` is where row r starts in it."""
         R = self.GROUP_ROWS
         w = self.w
-        w("// where every row starts among the elements that are kept (rows beyond the limit hold none): lane l sums rows 4l .. 4l + 3")
+        P = R // 64
+        w(f"// where every row starts among the elements that are kept (rows beyond the limit hold none): lane l sums rows {P}l .. {P}l + {P - 1}")
         w("int* __kp = __hq;")
-        w("int __kt[4], __mine = 0;")
+        w(f"int __kt[{P}], __mine = 0;")
         w("#pragma unroll")
-        w("for (int __i = 0; __i < 4; ++__i) {")
-        w("    const int __r = 4 * __lid + __i;")
+        w(f"for (int __i = 0; __i < {P}; ++__i) {{")
+        w(f"    const int __r = {P} * __lid + __i;")
         w("    const int __n = __r < __nr ? __hq[__r] - __lp[__r] : 0;")
         w("    __kt[__i] = __n > __rowmax ? 0 : __n;")
         w("    __mine += __kt[__i];")
@@ -2722,10 +2741,11 @@ class KernelBuilder:
         w("    if (__lid >= __d) __incl += __o;")
         w("}")
         w("appy::wave_fence();       // the ends of the rows have been read: their table now holds the starts among the kept")
-        w("__kp[4 * __lid] = __incl - __mine;")
-        w("__kp[4 * __lid + 1] = __incl - __mine + __kt[0];")
-        w("__kp[4 * __lid + 2] = __incl - __mine + __kt[0] + __kt[1];")
-        w("__kp[4 * __lid + 3] = __incl - __mine + __kt[0] + __kt[1] + __kt[2];")
+        w("{")
+        w("    int __run = __incl - __mine;")
+        w("#pragma unroll")
+        w(f"    for (int __i = 0; __i < {P}; ++__i) {{ __kp[{P} * __lid + __i] = __run; __run += __kt[__i]; }}")
+        w("}")
         w(f"if (__lid == 63) __kp[{R}] = __incl;")
         w("appy::wave_fence();")
         w(f"const int __kept = __kp[{R}];")
@@ -2834,7 +2854,7 @@ class KernelBuilder:
         w("#pragma unroll")
         w(f"for (int __k = 0; __k < {U}; ++__k) {{")
         w("    const int __j = __j0 + __k * 64 + __lid;")
-        w(f"    __xv[__k] = {cname(g['x'])}[__j < __chi ? __x0 + (appy::i64)((unsigned)((unsigned long long)__e[__k] >> 32) & 0xffffffu) : 0];")
+        w(f"    __xv[__k] = {cname(g['x'])}[__j < __chi ? __x0 + (appy::i64)((unsigned)((unsigned long long)__e[__k] >> 32) & 0x3fffffu) : 0];")
         w("}")
         w("#pragma unroll")
         w(f"for (int __k = 0; __k < {U}; ++__k) {{")
@@ -2847,7 +2867,7 @@ class KernelBuilder:
             bits = "(int)(unsigned)(unsigned long long)__e[__k]"
             w(f"const {cty.c} __cv = {'__int_as_float(' + bits + ')' if cty.is_float else '(' + cty.c + ')' + bits};")
         w(f"const {x.elem_c} __cx = __xv[__k];")
-        w(f"atomicAdd(&__acc[(unsigned)((unsigned long long)__e[__k] >> 56)], {cast(term, tty, pty)});")
+        w(f"atomicAdd(&__acc[(unsigned)((unsigned long long)__e[__k] >> 54)], {cast(term, tty, pty)});")
         self.ind -= 1
         w("}")
         self.ind -= 1
@@ -3034,6 +3054,9 @@ class KernelBuilder:
             params.append(Param("__ent", ("long long* __ent" if sp.aux == "group" else "const long long* __ent"), C.c_void_p, "ent"))
             params.append(Param("__desc", ("int* __desc" if sp.aux == "group" else "const int* __desc"), C.c_void_p, "desc"))
             params.append(Param("__shiftc", "const int __shiftc", C.c_int32, "shiftc"))
+        if sp.aux == "group" and sp.skip_long:
+            params.append(Param("__counts", "const int* __counts", C.c_void_p, "counts"))
+            params.append(Param("__base", "const int __base", C.c_int32, "base"))
         if sp.aux == "group":
             params.append(Param("__len", "const appy::i64 __len", C.c_int64, "entries"))
             params.append(Param("__rowmax", "const appy::i64 __rowmax", C.c_int64, "rowmax"))

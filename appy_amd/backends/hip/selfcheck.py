@@ -183,11 +183,12 @@ def compile_all_patterns() -> int:
                          Spec("team", block=256, vec=v, width=1, phase=2, rows="list", parts=8)]
             if loop.analysis.grouping is not None:
                 # elements grouped by the stripe of the gathered operand
-                more += [Spec("team", block=256, vec=1, width=64, parts=8, aux="group"),
-                         Spec("team", block=256, vec=1, width=64, parts=8, aux="group", skip_long=True),
+                more += [Spec("team", block=256, vec=1, width=64, parts=8, aux="group", block_rows=256),
+                         Spec("team", block=256, vec=1, width=64, parts=8, aux="group", block_rows=512, skip_long=True),
+                         Spec("team", block=256, vec=1, width=64, parts=8, aux="cells", block_rows=1024, guard=1),
                          Spec("team", block=256, vec=v, width=1, phase=2, guard=1, skip_long=True),
                          Spec("team", block=256, vec=v, width=16, phase=1, rows="list", parts=8, guard=1),
-                         Spec("team", block=256, vec=1, width=64, parts=16, aux="cells", guard=1),
+                         Spec("team", block=256, vec=1, width=64, parts=16, aux="cells", block_rows=256, guard=1),
                          Spec("team", block=256, vec=v, width=1, phase=2, guard=1),
                          Spec("team", block=256, vec=v, width=4, guard=2)]
         for spec in more:

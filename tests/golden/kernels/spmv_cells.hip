@@ -1,4 +1,4 @@
-// kernel for spmv_kernel_loop_1_cells: team_b256_v1_u1_w64_r_s8_cells_if1
+// kernel for spmv_kernel_loop_1_cells: team_b256_v1_u1_w64_r_s8_cells_R256_if1
 extern "C" __global__ void __launch_bounds__(256)
 _spmv_kernel_loop_1_cells(
     const int* __restrict__ A_indptr,
@@ -42,7 +42,7 @@ _spmv_kernel_loop_1_cells(
                 #pragma unroll
                 for (int __k = 0; __k < 8; ++__k) {
                     const int __j = __j0 + __k * 64 + __lid;
-                    __xv[__k] = x[__j < __chi ? __x0 + (appy::i64)((unsigned)((unsigned long long)__e[__k] >> 32) & 0xffffffu) : 0];
+                    __xv[__k] = x[__j < __chi ? __x0 + (appy::i64)((unsigned)((unsigned long long)__e[__k] >> 32) & 0x3fffffu) : 0];
                 }
                 #pragma unroll
                 for (int __k = 0; __k < 8; ++__k) {
@@ -50,7 +50,7 @@ _spmv_kernel_loop_1_cells(
                     if (__j < __chi) {
                         const float __cv = __int_as_float((int)(unsigned)(unsigned long long)__e[__k]);
                         const float __cx = __xv[__k];
-                        atomicAdd(&__acc[(unsigned)((unsigned long long)__e[__k] >> 56)], (__cv * __cx));
+                        atomicAdd(&__acc[(unsigned)((unsigned long long)__e[__k] >> 54)], (__cv * __cx));
                     }
                 }
             }

@@ -1,4 +1,4 @@
-// kernel for spmv_kernel_loop_1_group: team_b256_v1_u1_w64_r_s8_group
+// kernel for spmv_kernel_loop_1_group: team_b256_v1_u1_w64_r_s8_group_R256
 extern "C" __global__ void __launch_bounds__(256)
 _spmv_kernel_loop_1_group(
     const int* __restrict__ A_indptr,
@@ -138,7 +138,7 @@ _spmv_kernel_loop_1_group(
                         __at[__s] += __popcll(__m);
                     }
                     if (__sq >= 0 && __sq < 8)
-                        __ent[__pos] = (long long)(((unsigned long long)(((unsigned)__row << 24) | (unsigned)(__cq & __cmask)) << 32) | (unsigned long long)(unsigned)__v[__k][__q]);
+                        __ent[__pos] = (long long)(((unsigned long long)(((unsigned)__row << 22) | (unsigned)(__cq & __cmask)) << 32) | (unsigned long long)(unsigned)__v[__k][__q]);
                 }
             }
         }

@@ -1,4 +1,4 @@
-// kernel for spmv_kernel_loop_1_group: team_b256_v1_u1_w64_r_s8_group_sl
+// kernel for spmv_kernel_loop_1_group: team_b256_v1_u1_w64_r_s8_group_R256_sl
 extern "C" __global__ void __launch_bounds__(256)
 _spmv_kernel_loop_1_group(
     const int* __restrict__ A_indptr,
@@ -9,6 +9,8 @@ _spmv_kernel_loop_1_group(
     long long* __ent,
     int* __desc,
     const int __shiftc,
+    const int* __counts,
+    const int __base,
     const appy::i64 __len,
     const appy::i64 __rowmax,
     long long* __hint,
@@ -22,6 +24,14 @@ _spmv_kernel_loop_1_group(
     __shared__ int __hq_all[4][257];      // where they end
     int* __lp = __lp_all[__wvl];
     int* __hq = __hq_all[__wvl];
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        const appy::i64 __others = (__base == 0 ? 0 : (appy::i64)__counts[0]) + (__base == 1 ? 0 : (appy::i64)__counts[1]) + (__base == 2 ? 0 : (appy::i64)__counts[2]) + (__base == 3 ? 0 : (appy::i64)__counts[3]);
+        __hint[1] = (__base == 0) ? (__hi - __lo) - __others : (appy::i64)__counts[0];
+        __hint[2] = (__base == 1) ? (__hi - __lo) - __others : (appy::i64)__counts[1];
+        __hint[3] = (__base == 2) ? (__hi - __lo) - __others : (appy::i64)__counts[2];
+        __hint[4] = (__base == 3) ? (__hi - __lo) - __others : (appy::i64)__counts[3];
+        __hint[0] = 1;
+    }
     const appy::i64 __nblk = (__hi - __lo + 255) / 256;
     const int __cmask = (1 << __shiftc) - 1;
     const unsigned long long __below = (1ull << __lid) - 1ull;
@@ -91,10 +101,11 @@ _spmv_kernel_loop_1_group(
             if (__lid >= __d) __incl += __o;
         }
         appy::wave_fence();       // the ends of the rows have been read: their table now holds the starts among the kept
-        __kp[4 * __lid] = __incl - __mine;
-        __kp[4 * __lid + 1] = __incl - __mine + __kt[0];
-        __kp[4 * __lid + 2] = __incl - __mine + __kt[0] + __kt[1];
-        __kp[4 * __lid + 3] = __incl - __mine + __kt[0] + __kt[1] + __kt[2];
+        {
+            int __run = __incl - __mine;
+        #pragma unroll
+            for (int __i = 0; __i < 4; ++__i) { __kp[4 * __lid + __i] = __run; __run += __kt[__i]; }
+        }
         if (__lid == 63) __kp[256] = __incl;
         appy::wave_fence();
         const int __kept = __kp[256];
@@ -190,7 +201,7 @@ _spmv_kernel_loop_1_group(
                         __at[__s] += __popcll(__m);
                     }
                     if (__sq >= 0 && __sq < 8)
-                        __ent[__pos] = (long long)(((unsigned long long)(((unsigned)__row << 24) | (unsigned)(__cq & __cmask)) << 32) | (unsigned long long)(unsigned)__v[__k][__q]);
+                        __ent[__pos] = (long long)(((unsigned long long)(((unsigned)__row << 22) | (unsigned)(__cq & __cmask)) << 32) | (unsigned long long)(unsigned)__v[__k][__q]);
                 }
             }
         }

@@ -67,7 +67,7 @@ def test_profile_was_measured_with_the_shape_the_bench_launches(workload):
         # from the second launch on (the bench times those) the elements of rows up to 512 elements are grouped by stripe
         assert spec.rows == "mixed"
         stripes, _shift, _entries = loop.grouped_shape(n_outer, env, arrays)
-        spec = cg.Spec("team", block=256, vec=1, width=64, parts=stripes, aux="cells", guard=1)
+        spec = cg.Spec("team", block=256, vec=1, width=64, parts=stripes, aux="cells", guard=1, block_rows=256)
     tag, nbytes = traffic[workload]
     assert tag == spec.tag(), f"{workload}: the counter summary was measured with {tag}, the launch picks {spec.tag()} now"
 

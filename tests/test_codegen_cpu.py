@@ -176,17 +176,17 @@ def test_sums_of_gathered_terms_can_be_grouped_by_the_stripe_they_read():
     assert csr("v[j] * x[c[j]]", x=np.zeros(16, np.float64)).grouping is None
     assert csr("v[j] * x[c[j]]", c=np.zeros(16, np.int64)).grouping is None
     # the kernels
-    group = body_of(f.kernel_for(Spec("team", block=256, vec=1, width=64, parts=8, aux="group")).src.text)
+    group = body_of(f.kernel_for(Spec("team", block=256, vec=1, width=64, parts=8, aux="group", block_rows=256)).src.text)
     assert "__lp[__r + 1] == __hq[__r]" in group and "__flag[0] = 1" in group and "__hint[0] = 2" in group
     assert "x[" not in group.split("{", 1)[1]                                 # the gathered operand is not read here
-    cells = body_of(f.kernel_for(Spec("team", block=256, vec=1, width=64, parts=16, aux="cells", guard=1)).src.text)
+    cells = body_of(f.kernel_for(Spec("team", block=256, vec=1, width=64, parts=16, aux="cells", block_rows=256, guard=1)).src.text)
     assert "if ((__flag[0] != 0) == true) return;" in cells and "for (int __pass = 0; __pass < 2; ++__pass)" in cells
     assert "atomicAdd(&__acc[" in cells and "(__cv * __cx)" in cells and "A_indptr[" not in cells.split("{", 1)[1]
     sums = body_of(f.kernel_for(Spec("team", block=256, vec=4, width=1, phase=2, guard=1)).src.text)
     assert "reinterpret_cast<float*>(__scratch)[(0 * __nsplit + __c) * (__hi - __lo) + (i - __lo)]" in sums and "y[i] = s" in sums
     # with long rows in the matrix: the grouping kernel walks the elements of the other rows only, the sums are not
     # added for long rows, and the kernels that cut the long rows wait on the same flag
-    kept = body_of(f.kernel_for(Spec("team", block=256, vec=1, width=64, parts=8, aux="group", skip_long=True)).src.text)
+    kept = body_of(f.kernel_for(Spec("team", block=256, vec=1, width=64, parts=8, aux="group", block_rows=256, skip_long=True)).src.text)
     assert "__kt[__i] = __n > __rowmax ? 0 : __n;" in kept and "__kp[__row + 1] <= __t + __q" in kept and "__hint[0] = 2" not in kept
     sums_kept = body_of(f.kernel_for(Spec("team", block=256, vec=4, width=1, phase=2, guard=1, skip_long=True)).src.text)
     assert "if (__trip <= __rowmax) {" in sums_kept
@@ -197,7 +197,7 @@ def test_sums_of_gathered_terms_can_be_grouped_by_the_stripe_they_read():
     rest = body_of(f.kernel_for(Spec("team", block=256, vec=4, width=4, guard=2)).src.text)
     assert "if ((__flag[0] != 0) == false) return;" in rest
     with pytest.raises(ValueError):
-        Spec("team", block=256, width=64, parts=24, aux="group")
+        Spec("team", block=256, width=64, parts=24, aux="group", block_rows=256)
     with pytest.raises(ValueError):
         Spec("flat", guard=1)
     # sums of float64 are not taken: the loop keeps its rows sorted by length

@@ -32,9 +32,9 @@ CASES = {
     "spmv_parts": ("spmv", Spec("team", block=256, vec=4, width=16, stream_loads=True, phase=1, rows="list", parts=8)),
     "spmv_fold": ("spmv", Spec("team", block=256, vec=4, width=1, stream_loads=True, phase=2, rows="list", parts=8)),
     # the kernels of a launch that groups the elements of short rows by column stripe (config 4, uniform rows)
-    "spmv_group": ("spmv", Spec("team", block=256, vec=1, width=64, parts=8, aux="group")),
-    "spmv_group_kept_rows": ("spmv", Spec("team", block=256, vec=1, width=64, parts=8, aux="group", skip_long=True)),
-    "spmv_cells": ("spmv", Spec("team", block=256, vec=1, width=64, parts=8, aux="cells", guard=1)),
+    "spmv_group": ("spmv", Spec("team", block=256, vec=1, width=64, parts=8, aux="group", block_rows=256)),
+    "spmv_group_kept_rows": ("spmv", Spec("team", block=256, vec=1, width=64, parts=8, aux="group", block_rows=256, skip_long=True)),
+    "spmv_cells": ("spmv", Spec("team", block=256, vec=1, width=64, parts=8, aux="cells", block_rows=256, guard=1)),
     "spmv_sums_of_cells": ("spmv", Spec("team", block=256, vec=4, width=1, phase=2, guard=1)),
     "spmm": ("spmm", Spec("team", block=256, vec=4, width=32, extent=128)),
 }

@@ -418,6 +418,29 @@ def test_grouped_launches_on_gpu_tensors_follow_changes_of_the_matrix(gpu):
     assert ok, worst
 
 
+@pytest.mark.parametrize("rows_per_block", [512, 1024])
+def test_larger_blocks_of_rows(gpu, rows_per_block):
+    """`hip_group_rows` sets the rows per block of the grouped form (256 unless told otherwise)."""
+    kk = selfcheck.kernels(hip_group_rows=rows_per_block)
+    rng = np.random.default_rng(40)
+    m, n = 40_000 + rows_per_block // 2 + 3, 1 << 20
+    ln = np.where(rng.random(m) < 0.01, rng.integers(600, 3000, m), rng.integers(0, 12, m))
+    data, indptr, indices, x = _matrix(ln, n, seed=41)
+    ref, budget = vo.spmv_csr(data, indptr, indices, x, (m, n))
+    for launch_no in range(3):
+        y = kk.spmv(data, indptr, indices, x, m, n)
+        ok, worst = vo.within_budget(y, ref, budget, TOL)
+        assert ok, (launch_no, worst)
+    launch = max((v[0] for key, v in cg.code_cache.items() if key[-1] == "spmv" and v[0].options.get("hip_group_rows") == rows_per_block
+                  and getattr(v[0], "last_launch", None) is not None), key=lambda lp: lp.last_launch.serial).last_launch
+    assert _grouped(launch) and launch.spec.block_rows == rows_per_block and len(launch.sequence) == 9
+    short = _matrix(np.full(m, 9), n, seed=42)
+    ref, budget = vo.spmv_csr(*short, (m, n))
+    for _ in range(3):
+        y = kk.spmv(*short, m, n)
+        assert vo.within_budget(y, ref, budget, TOL)[0]
+
+
 def test_launches_recorded_into_a_graph_keep_their_rows_sorted(gpu):
     """The grouped form clears a flag with a memory-set node; recorded launches use the kernels over sorted
     rows instead, and every replay follows the contents of the tensors."""
