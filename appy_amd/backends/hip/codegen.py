@@ -89,6 +89,24 @@ STRIPE_MIN_BYTES = 3 << 20
 STRIPE_BYTES = 2 << 20
 GROUP_MAX_STRIPE_LOG = 19          # elements grouped by stripe: stripes of 2^19 elements of 4 bytes (half an L2) at most, 8 or 16 of them
 GROUP_MIN_TRIP = 4                 # ... for rows of this many elements on average, at least
+# row plans (the order of the elements of a CSR-like sum, worked out once and kept between launches)
+PLAN_ROW_BITS = 15                 # rows per block: what fits a workgroup's LDS as 4-byte sums
+PLAN_GROUPS = 8                    # column ranges of the gathered operand, one per XCD
+PLANS_PER_LOOP = 2                 # plans a loop keeps (least recently used goes first)
+
+
+def scratch_limit(device: int) -> int:
+    """Most bytes of device memory one loop may hold for its own purposes (scratch buffers of launches made of
+    several kernels, row plans): `APPY_HIP_SCRATCH_MAX_BYTES`, or a quarter of the device's memory."""
+    env = os.environ.get("APPY_HIP_SCRATCH_MAX_BYTES")
+    if env:
+        return int(env)
+    if device not in _hbm_bytes:
+        _hbm_bytes[device] = int(rt.device_props(device)["hbm_bytes"])
+    return _hbm_bytes[device] // 4
+
+
+_hbm_bytes = {}
 
 
 def device_header() -> str:
@@ -260,6 +278,77 @@ def _pow2ceil(x: float) -> int:
     return n
 
 
+
+class RowPlan:
+    """The elements of one set of arrays in the order `xcells` kernels walk them, in device memory
+    that this object owns.  It describes the arrays as they were when it was built: it is used only
+    while every array it read is still the same object with the same version counter (tensors count
+    the in-place operations PyTorch performs on them), and it is dropped when a launch of this
+    package stores into memory one of those arrays occupies."""
+
+    def __init__(self, device, key, refs, ranges):
+        self.device = device
+        self.key = key
+        self.refs = refs            # weak references to the tensors the plan was built from
+        self.ranges = ranges        # (address, bytes) of those tensors
+        self.buffers = []           # device allocations of the plan
+        self.nbytes = 0
+        self.valid = False
+        self.bin = {}               # arguments of the kernels that run the plan
+        self.ncell = 0
+        self.tile = 0
+        self.split = 1              # workgroups per cell
+        self.inspector_ms = None
+
+    def alloc(self, nbytes):
+        ptr = rt.malloc(max(256, nbytes))
+        self.buffers.append(ptr)
+        self.nbytes += nbytes
+        return ptr
+
+    def alive(self, tensors) -> bool:
+        return self.valid and all(r() is t for r, t in zip(self.refs, tensors))
+
+    def release(self):
+        self.valid = False
+        bufs, self.buffers = self.buffers, []
+        for ptr in bufs:
+            try:
+                rt.free(ptr)
+            except Exception:       # the runtime may be shutting down
+                pass
+        with _plans_lock:
+            if self in _live_plans:
+                _live_plans.remove(self)
+
+
+_live_plans = []        # every valid plan of the process: launches that store into their arrays drop them
+_plans_lock = threading.Lock()
+
+
+def drop_plans_overlapping(extents):
+    """``extents``: (name, address, bytes, stored) of a launch's arrays.  Plans built from memory that
+    the launch stores into are no longer true."""
+    if not _live_plans:
+        return
+    stored = [(p, n) for _name, p, n, st in extents if st]
+    if not stored:
+        return
+    with _plans_lock:
+        hit = [plan for plan in _live_plans
+               if any(p < q + m and q < p + n for p, n in stored for q, m in plan.ranges)]
+    for plan in hit:
+        plan.valid = False      # its memory goes back once the launches that use it have drained (CompiledLoop.release / next build)
+        with _plans_lock:
+            if plan in _live_plans:
+                _live_plans.remove(plan)
+
+
+def release_all_plans():
+    for _f, _src in list(code_cache.values()):
+        _f.release_plans()
+
+
 class CompiledLoop:
     """Callable launcher of one annotated loop for one argument signature."""
 
@@ -327,6 +416,11 @@ class CompiledLoop:
         self._hints = {}    # device -> (address, ctypes view) of page-locked words the binned kernels report to
         self._scratch_retired = []
         self._replays = {}  # call identity -> Launch that can simply be launched again
+        self._plans = []    # row plans of this loop, most recently used last
+        self._plan_seen = {}        # identity of the arrays of a launch that could use a plan -> launches seen with it
+        self._plan_off = False      # a kernel of the planned form could not be generated for this loop
+        self._plan_refused = set()  # identities whose arrays the inspector has refused
+        self.last_plan = None
         # scalars that no host-side decision looks at (range of the loop, inner trip counts,
         # row extents): a replayed launch may carry new values of these
         steering = set()
@@ -708,8 +802,9 @@ class CompiledLoop:
             return have
 
     def release(self):
-        """Give back the device memory this loop holds (scratch buffers of two-phase launches),
+        """Give back the device memory this loop holds (scratch buffers of two-phase launches, row plans),
         once the launches that use it have finished."""
+        self.release_plans()
         with self._lock:
             held, self._scratch, self._scratch_retired = (
                 [(k, p) for k, (p, _n) in self._scratch.items()] + [(None, p) for p in self._scratch_retired], {}, [])
@@ -726,6 +821,64 @@ class CompiledLoop:
                 rt.host_free(addr)
         except Exception:           # the runtime may be shutting down
             pass
+
+    def release_plans(self):
+        """Give back the memory of this loop's row plans, once the launches that use them have finished."""
+        with self._lock:
+            plans, self._plans = self._plans, []
+            self._plan_seen.clear()
+        for plan in plans:
+            try:
+                _ensure_device(plan.device)
+                rt.sync(0)
+                for stream in {st for (dev, st) in self._scratch if dev == plan.device}:
+                    rt.sync(stream)
+            except Exception:
+                pass
+            plan.release()
+
+    def plan_arrays(self):
+        """Names of the arrays a row plan is built from: what the set-up of a row reads, the index array
+        and the array whose elements travel with the indices."""
+        a = self.analysis
+        g = a.grouping
+        body = a.outer.body
+        at = next(k for k, st in enumerate(body) if st is a.team_split)
+        names = []
+        for st in body[:at]:
+            for n in ast.walk(st):
+                if isinstance(n, ast.Name) and n.id in a.arrays and n.id not in names:
+                    names.append(n.id)
+        for b in a.team_split.iter.args[:2]:
+            for n in ast.walk(b):
+                if isinstance(n, ast.Name) and n.id in a.arrays and n.id not in names:
+                    names.append(n.id)
+        for nm in (g["idx"], g["carried"]):
+            if nm and nm not in names:
+                names.append(nm)
+        return names
+
+    def plan_shape(self, n_outer, env, arrays):
+        """The shape of a row plan for these arrays (runtime.RowPlanShape), or None when they do not
+        qualify: the conditions of the grouped form (an operand too large for an L2, rows of a few
+        elements), and keys and packed words of 32 bits."""
+        base = self.grouped_shape(n_outer, env, arrays)
+        if base is None or self._plan_off:
+            return None
+        g = self.analysis.grouping
+        nx = int(arrays[g["x"]].shape[0])
+        entries = base[2]
+        width = -(-(-(-nx // PLAN_GROUPS)) // 32) * 32
+        col_bits = max(5, (width - 1).bit_length())
+        if col_bits > 20:
+            return None
+        lines = PLAN_GROUPS * (width >> 5)
+        line_bits = max(1, (lines - 1).bit_length())
+        blocks = -(-n_outer // (1 << PLAN_ROW_BITS))
+        if (blocks << line_bits) > (1 << 31) or entries >= (1 << 31):
+            return None
+        return rt.RowPlanShape(entries=entries, row_blocks=blocks, groups=PLAN_GROUPS, group_width=width,
+                               col_bits=col_bits, tile=6144 if col_bits <= 19 else 4096, line_bits=line_bits)
 
     def collapse_count(self, n_outer, env) -> int:
         """Trip count of the sequential loop that may be collapsed into the parallel loop,
@@ -914,6 +1067,7 @@ class Launch:
         self.keepalive = []
         self.sequence = None
         self.bin = None
+        self.plan = None         # the row plan this launch runs, if any
         try:
             self._stage(vals, arrays)
         except BaseException:
@@ -1007,6 +1161,7 @@ class Launch:
         for _m, dptr, host, stored, name in self.mirrored:
             extents.append((name, dptr, host.nbytes, stored))
         restrict = not _overlaps(extents)
+        drop_plans_overlapping(extents)
 
         # -- kernel variant, argument block, grid
         n_outer = hi - lo
@@ -1033,6 +1188,9 @@ class Launch:
             self.scratch_ptr = loop.scratch(device, self.stream, max(1, reds) * self.nsplit * n_outer * 8)
         self.scalar_fields = {}      # by-value scalar -> field of the argument block
         self.sequence = None         # binned rows: [(kernel, argument block, grid, block)] launched in this order
+        if spec.rows == "mixed" and self._stage_planned(vals, arrays, lo, hi, spec):
+            loop.last_launch = self
+            return
         if spec.rows == "mixed" and self._stage_grouped(vals, arrays, lo, hi, spec):
             loop.last_launch = self
             return
@@ -1254,6 +1412,182 @@ class Launch:
         self.args, self.grid, self.block = args_of_cells[1], args_of_cells[2], args_of_cells[3]
         return True
 
+    def _plan_identity(self, arrays, lo, hi, vals):
+        """``(key, tensors)`` naming the contents a row plan of this launch would describe, or None when
+        they cannot be named: every array the plan reads must be a tensor on the GPU (its version counter
+        tells of in-place changes)."""
+        loop = self.loop
+        names = loop.plan_arrays()
+        tensors, key = [], [self.device, lo, hi, int(arrays[loop.analysis.grouping["x"]].shape[0])]
+        for nm in names:
+            t = arrays[nm]
+            if isinstance(t, np.ndarray) or not getattr(t, "is_cuda", False) or not hasattr(t, "_version"):
+                return None
+            tensors.append(t)
+            key.append((nm, t.data_ptr(), tuple(t.shape), tuple(t.stride()), t._version))
+        for nm in loop.arg_names:
+            if nm in loop.analysis.scalars:
+                v = vals[nm]
+                key.append((nm, v.item() if isinstance(v, np.generic) else v))
+        return tuple(key), tensors
+
+    def _stage_planned(self, vals, arrays, lo, hi, spec) -> bool:
+        """The launches of a loop whose elements have been ordered by an earlier launch with the same arrays
+        (a row plan): the kernel that runs the plan, then the kernel that adds the sums of a row's eight
+        column ranges and runs the rest of the body.  A plan is built the second time a set of arrays is
+        seen unchanged (`hip_reuse="now"`: the first time); the first time the launch takes the forms that
+        keep nothing.  False (nothing staged) when the launch does not qualify or has no plan yet."""
+        loop, a, env = self.loop, self.loop.analysis, self.env
+        reuse = loop.options.get("hip_reuse", True)
+        if a.grouping is None or not reuse or loop._plan_off:
+            return False
+        n = hi - lo
+        ident = self._plan_identity(arrays, lo, hi, vals)
+        if ident is None:
+            return False
+        key, tensors = ident
+        plan = None
+        if any(not pl.valid for pl in loop._plans):
+            # plans that a store into their arrays has made untrue: their memory goes back once the launches
+            # that were queued with them have finished
+            with loop._lock:
+                dead = [pl for pl in loop._plans if not pl.valid]
+                loop._plans = [pl for pl in loop._plans if pl.valid]
+            rt.sync(self.stream)
+            rt.sync(0)
+            for pl in dead:
+                pl.release()
+        with loop._lock:
+            for cand in loop._plans:
+                if cand.key == key and cand.alive(tensors):
+                    plan = cand
+                    loop._plans.remove(cand)
+                    loop._plans.append(cand)
+                    break
+        if plan is None:
+            if key in loop._plan_refused or self.capture is not None:
+                return False
+            shape = loop.plan_shape(n, env, arrays)
+            if shape is None:
+                return False
+            with loop._lock:
+                seen = loop._plan_seen.get(key, 0) + 1
+                if len(loop._plan_seen) > 64:
+                    loop._plan_seen.clear()
+                loop._plan_seen[key] = seen
+            if seen < (1 if reuse == "now" else 2):
+                return False
+            plan = self._build_plan(key, tensors, shape, vals, arrays, lo, hi, spec)
+            if plan is None:
+                return False
+        V = spec.vec
+        try:
+            cells = loop.kernel_for(Spec("team", block=1024, vec=1, width=1024, unroll=plan.tile // 1024, parts=PLAN_GROUPS,
+                                         aux="xcells", restrict=spec.restrict))
+            sums = loop.kernel_for(Spec("team", block=256, vec=V, width=1, phase=2, guard=1, restrict=spec.restrict))
+        except Unsupported:
+            loop._plan_off = True
+            return False
+        self.bin = dict(plan.bin)
+        split = plan.split
+        self.bin["split"] = split
+        self.scratch_ptr = loop.scratch(self.device, self.stream, 4 * PLAN_GROUPS * split * n)
+        self.nsplit = PLAN_GROUPS * split
+        self.plan = plan
+        seq = [(cells, self._argument_block(cells, vals, arrays, lo, hi), (plan.ncell * split, 1, 1), (1024, 1, 1)),
+               (sums, self._argument_block(sums, vals, arrays, lo, hi), (max(1, min(4096, -(-n // 256))), 1, 1), (256, 1, 1))]
+        self.sequence = seq
+        self.kernel, self.spec = cells, cells.src.spec
+        self.args, self.grid, self.block = seq[0][1], seq[0][2], seq[0][3]
+        return True
+
+    def _build_plan(self, key, tensors, shape, vals, arrays, lo, hi, spec):
+        """Runs the inspector for these arrays: the generated kernel writes one (key, value) pair per element, the
+        library sorts the pairs and lays out cells, tiles and slots.  Waits for the device once, to learn whether
+        the arrays were accepted (row ranges that follow one another, indices inside the operand)."""
+        loop = self.loop
+        n = hi - lo
+        try:
+            rkeys = loop.kernel_for(Spec("team", block=256, vec=1, width=64, aux="rkeys", block_rows=256, restrict=spec.restrict))
+        except Unsupported:
+            loop._plan_off = True
+            return None
+        lib = rt.lib()
+        temp_bytes, max_tiles, words = C.c_size_t(0), C.c_size_t(0), C.c_size_t(0)
+        rt.check(lib.appy_hip_rowplan_sizes(C.byref(shape), C.byref(temp_bytes), C.byref(max_tiles), C.byref(words)))
+        entries = int(shape.entries)
+        ncell = int(shape.row_blocks) * int(shape.groups)
+        limit = scratch_limit(self.device)
+        slack = 4 * int(shape.tile)      # the kernel that runs the plan reads whole tiles, a few beyond the end of a cell
+        kept = 8 * (entries + slack) + 4 * (words.value + slack) + 8 * (ncell + 1) + 256
+        if kept + 16 * entries + temp_bytes.value > limit:
+            return None
+        # older plans of this loop make room first (their launches have been queued before this one on their streams)
+        with loop._lock:
+            old = [pl for pl in loop._plans if not pl.valid] + [pl for pl in loop._plans if pl.valid][:-(PLANS_PER_LOOP - 1) or None]
+            loop._plans = [pl for pl in loop._plans if pl not in old]
+        if old:
+            rt.sync(self.stream)
+            for pl in old:
+                rt.sync(0)
+                pl.release()
+        import weakref
+
+        plan = RowPlan(self.device, key, [weakref.ref(t) for t in tensors],
+                       [(t.data_ptr(), t.numel() * t.element_size()) for t in tensors])
+        temps = []
+        t0 = t1 = None
+        try:
+            elements = plan.alloc(8 * (entries + slack))
+            cstart = plan.alloc(4 * (ncell + 1))
+            tbase = plan.alloc(4 * (ncell + 1))
+            rstream = plan.alloc(4 * (words.value + slack))
+            flag = plan.alloc(256)
+            for nb in (4 * entries, 8 * entries, 4 * entries, temp_bytes.value):
+                temps.append(rt.malloc(max(256, nb)))
+            keys, pairs, keys_sorted, temp = temps
+            t0, t1 = rt.Event(), rt.Event()
+            t0.record(self.stream)
+            rt.memset_async(keys, 0xFF, 4 * entries, self.stream)
+            rt.memset_async(flag, 0, 256, self.stream)
+            self.bin = {"keys": keys, "vals": pairs, "entries": entries, "nx": int(arrays[loop.analysis.grouping["x"]].shape[0]),
+                        "lbits": int(shape.line_bits), "flag": flag}
+            args = self._argument_block(rkeys, vals, arrays, lo, hi)
+            nblk = -(-n // 256)
+            rt.launch(rkeys.function(self.device), (max(1, min(1 << 20, -(-nblk // 4))), 1, 1), (256, 1, 1), args, self.stream)
+            rt.check(lib.appy_hip_rowplan_build(C.byref(shape), keys, pairs, keys_sorted, elements, temp, temp_bytes.value,
+                                                cstart, tbase, rstream, self.stream))
+            t1.record(self.stream)
+            word = C.c_int64(0)
+            rt.memcpy_d2h(C.addressof(word), flag, 8, self.stream)      # waits for the stream
+            plan.inspector_ms = t0.elapsed_ms(t1)
+        except BaseException:
+            plan.release()
+            raise
+        finally:
+            for ptr in temps:
+                rt.free(ptr)
+        if word.value:
+            plan.release()
+            loop._plan_refused.add(key)
+            return None
+        plan.bin = {"ent": elements, "cstart": cstart, "tbase": tbase, "rstream": rstream, "ncell": ncell,
+                    "gwidth": int(shape.group_width), "colbits": int(shape.col_bits), "flag": flag,
+                    "nx": int(arrays[loop.analysis.grouping["x"]].shape[0])}
+        plan.ncell = ncell
+        plan.tile = int(shape.tile)
+        # few cells (a matrix of few blocks of rows): several workgroups share a cell, each with a run of its tiles,
+        # until there are some four workgroups per compute unit or a workgroup is down to two tiles
+        forced = loop.options.get("hip_plan_split")
+        plan.split = int(forced) if forced else max(1, min(-(-4 * DEFAULT_CUS // ncell), entries // (2 * plan.tile * ncell), 32))
+        plan.valid = True
+        with loop._lock:
+            loop._plans.append(plan)
+        with _plans_lock:
+            _live_plans.append(plan)
+        loop.last_plan = plan
+        return plan
+
     def _argument_block(self, kernel, vals, arrays, lo, hi):
         loop = self.loop
         st = kernel.ArgStruct()
@@ -1285,7 +1619,8 @@ class Launch:
             elif p.role in ("threshold", "widthlog"):
                 val = self.bin[p.role][p.dim]
             elif p.role in ("rows", "counts", "zero", "nrows", "bnd", "cap", "stripe", "m", "base", "skip", "tlo", "thi", "load", "hint", "rowstart",
-                            "flag", "desc", "ent", "shiftc", "entries", "rowmax"):
+                            "flag", "desc", "ent", "shiftc", "entries", "rowmax", "keys", "vals", "nx", "lbits", "cstart", "tbase",
+                            "rstream", "ncell", "gwidth", "colbits", "split"):
                 val = self.bin[p.role]
             elif p.role == "lo":
                 val = lo
@@ -1483,7 +1818,8 @@ def _copy(node):
 def codegen(loop_source, loop_name, val_map, options):
     key = (loop_source, loop_name, _signature(val_map), options.get("hip_spec") and repr(options.get("hip_spec")),
            options.get("hip_max_blocks"), bool(options.get("check_bounds")), bool(options.get("hip_bins", True)),
-           bool(options.get("hip_group", True)), options.get("hip_group_rows"), options.get("fn_name"))
+           bool(options.get("hip_group", True)), options.get("hip_group_rows"), bool(options.get("hip_hints", True)),
+           options.get("hip_reuse", True), options.get("hip_plan_split"), options.get("fn_name"))
     # `clear_cache=True` regenerates the loop on every call instead of using the cached kernel
     # (reference: appy/backends/metal/codegen.py:23)
     fresh = bool(options.get("clear_cache"))

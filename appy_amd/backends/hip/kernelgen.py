@@ -90,6 +90,9 @@ class Spec:
                                  # so that a cell still holds a few hundred elements)
     skip_long: bool = False      # with 'group' and the kernel that adds the sums of its cells: rows whose simd loop is longer
                                  # than a limit given at the launch are passed over (they run in planned parts)
+                                 # 'rkeys' = the kernel that turns the elements of `block_rows` rows per wavefront into the
+                                 # (key, value) pairs a row plan is built from, 'xcells' = the kernel that runs a row plan
+                                 # (`parts` column ranges, `unroll` x 1024 elements per tile)
     guard: int = 0               # 1 = the kernel returns at once when the grouping kernel of this launch has refused
                                  # its input (row ranges that do not follow one another: a flag in device memory),
                                  # 2 = when it has not
@@ -116,12 +119,18 @@ class Spec:
                                          and not self.extent and not self.lds_tile and not self.collapse))):
             raise ValueError("only strip kernels, teams of a whole wavefront or workgroup, and teams over listed rows "
                              "run in two phases")
-        if self.rows not in ("", "mixed", "list") or self.aux not in ("", "bins", "plan", "group", "cells"):
+        if self.rows not in ("", "mixed", "list") or self.aux not in ("", "bins", "plan", "group", "cells", "rkeys", "xcells"):
             raise ValueError(f"unknown row source {self.rows!r} / auxiliary kernel {self.aux!r}")
         if (self.rows or self.aux) and (self.kind != "team" or self.extent or self.lds_tile or self.collapse
-                                        or self.row_steps or self.checked or self.width > 64):
+                                        or self.row_steps or self.checked or (self.width > 64 and self.aux != "xcells")):
             raise ValueError("rows are binned for plain team kernels only (teams inside a wavefront)")
-        if self.aux in ("group", "cells"):
+        if self.aux == "rkeys":
+            if self.rows or self.phase or self.parts or self.width != 64 or self.block != 256 or self.block_rows != 256:
+                raise ValueError("the kernel that writes the pairs of a row plan takes blocks of 256 rows, one per wavefront")
+        elif self.aux == "xcells":
+            if self.rows or self.phase or self.parts != 8 or self.block != 1024 or self.unroll not in (4, 6) or self.block_rows:
+                raise ValueError("a row plan runs in workgroups of 1024 lanes, 8 column ranges, tiles of 4096 or 6144 elements")
+        elif self.aux in ("group", "cells"):
             if (self.rows or self.phase or self.parts not in (8, 16) or self.width != 64 or self.block != 256
                     or self.block_rows not in (256, 512, 1024)):
                 raise ValueError("elements are grouped by 8 or 16 stripes, one wavefront per block of 256, 512 or 1024 rows, "
@@ -2172,10 +2181,11 @@ class KernelBuilder:
         if s.aux or s.rows:
             if self.a.ragged is None or self.lds_plan is not None:
                 raise Unsupported("the loop nest does not suit kernels over binned rows")
-            if s.aux in ("group", "cells"):
+            if s.aux in ("group", "cells", "rkeys", "xcells"):
                 if self.a.grouping is None:
                     raise Unsupported("the simd loop is not a sum of terms that gather from one operand")
-                return self._body_group() if s.aux == "group" else self._body_cells()
+                return {"group": self._body_group, "cells": self._body_cells, "rkeys": self._body_rkeys,
+                        "xcells": self._body_xcells}[s.aux]()
             if s.aux == "bins":
                 return self._body_bins()
             if s.rows == "mixed":
@@ -2886,6 +2896,323 @@ class KernelBuilder:
         self.ind -= 1
         w("}")
 
+    # ---- row plans: the elements of a sum over a gathered operand, ordered once and kept ----------------
+    # A plan orders the elements by cell (a block of 32768 rows x one of eight column ranges of the gathered
+    # operand) and, within a cell, by the 128-byte line of the operand they read.  `rkeys` writes one (key,
+    # value) pair per element, the library sorts them and works out, tile by tile, where each product goes so
+    # that the tile's products lie sorted by row (include/appy_hip.h, "row plans"); `xcells` runs the result.
+    PLAN_ROW_BITS = 15
+
+    def _body_rkeys(self):
+        """The kernel that writes the pairs.  Per block of 256 rows (one wavefront): the set-up of its rows
+        gives the rows' ranges, which must follow one another as those of a CSR matrix do and hold indices
+        inside the gathered operand - otherwise the flag is raised and no plan comes of it; then every element
+        goes to its own position of the two arrays: the key (block of 32768 rows, line of the operand) and the
+        value (bits of the carried operand, row within the block, column within the line)."""
+        a, g, R = self.a, self.a.grouping, self.GROUP_ROWS
+        var = a.var
+        self.ex.locals[var] = T.WEAK_INT
+        self.mode = "lane"
+        idx_c = cname(g["idx"])
+        a.arrays[g["idx"]].loaded = True
+        car_c = f"reinterpret_cast<const int*>({cname(g['carried'])})" if g["carried"] else None
+        body = a.outer.body
+        at = next(k for k, st in enumerate(body) if st is a.team_split)
+        U = 4
+        w = self.w
+        RB = self.PLAN_ROW_BITS
+        w("const int __lid = threadIdx.x & 63;")
+        w("const int __wvl = threadIdx.x >> 6;")
+        w(f"__shared__ int __lp_all[4][{R + 1}];      // where the rows of the block start; the last entry: where it ends")
+        w(f"__shared__ int __hq_all[4][{R + 1}];      // where they end")
+        w("int* __lp = __lp_all[__wvl];")
+        w("int* __hq = __hq_all[__wvl];")
+        w(f"const appy::i64 __nblk = (__hi - __lo + {R - 1}) / {R};")
+        w("for (appy::i64 __b = (appy::i64)blockIdx.x * 4 + __wvl; __b < __nblk; __b += (appy::i64)gridDim.x * 4) {")
+        self.ind += 1
+        w(f"const appy::i64 __r0 = __lo + __b * {R};")
+        w(f"const int __nr = (int)((__hi - __r0) < {R} ? (__hi - __r0) : {R});")
+        w("appy::wave_fence();       // the block before this one has been read out of __lp")
+        w("bool __good = true;")
+        w("#pragma unroll")
+        w(f"for (int __k = 0; __k < {R // 64 + 1}; ++__k) {{      // and the first row of the next block, if there is one")
+        self.ind += 1
+        w("const int __r = __k * 64 + __lid;")
+        w(f"if (__r <= __nr && __r0 + __r < __hi && (__k < {R // 64} || __lid == 0)) {{")
+        self.ind += 1
+        w(f"const appy::i64 {cname(var)} = __r0 + __r;")
+        self._declare_locals()
+        self.block(body[:at])
+        lo, hi = self._range_args(a.team_split)
+        w(f"const appy::i64 __rlo = {lo};")
+        w(f"const appy::i64 __rhi = {hi};")
+        w("if (__rlo < 0 || __rhi < __rlo || __rhi > __len) __good = false;")
+        w("__lp[__r] = (int)__rlo;")
+        w("if (__r < __nr) __hq[__r] = (int)__rhi;")
+        self.ind -= 1
+        w("}")
+        self.ind -= 1
+        w("}")
+        w("appy::wave_fence();")
+        w("// every row ends where the next one starts; the block ends no later than the next one starts")
+        w("#pragma unroll")
+        w(f"for (int __k = 0; __k < {R // 64}; ++__k) {{")
+        w("    const int __r = __k * 64 + __lid;")
+        w("    if (__r < __nr - 1) __good = __good && __lp[__r + 1] == __hq[__r];")
+        w("    else if (__r == __nr - 1 && __r0 + __nr < __hi) __good = __good && __lp[__nr] >= __hq[__r];")
+        w("}")
+        w("__good = __ballot(!__good) == 0ull;")
+        w("const int __first = __good ? __lp[0] : 0, __end = __good ? __hq[__nr - 1] : 0;")
+        w("appy::wave_fence();")
+        w("#pragma unroll")
+        w(f"for (int __k = 0; __k < {R // 64 + 1}; ++__k) {{")
+        w("    const int __r = __k * 64 + __lid;")
+        w(f"    if (__r >= __nr && __r <= {R} && (__k < {R // 64} || __lid == 0)) __lp[__r] = __end;")
+        w("}")
+        w("appy::wave_fence();")
+        w("if (!__good) {")
+        w("    if (__lid == 0) __flag[0] = 1;")
+        w("    continue;")
+        w("}")
+        w(f"const unsigned __rel0 = (unsigned)(__b * {R});       // first row of the block, counted from the start of the range")
+        w("bool __inside = true;")
+        w(f"for (int __j0 = __first; __j0 < __end; __j0 += {256 * U}) {{")
+        self.ind += 1
+        w("#pragma unroll")
+        w(f"for (int __k = 0; __k < {U}; ++__k) {{")
+        self.ind += 1
+        w("const int __j = __j0 + __k * 256 + __lid * 4;")
+        w("if (__j >= __end) continue;")
+        w("appy::vec<int, 4>::type __c, __v;")
+        w(f"if (__j + 4 <= __end) __c = appy::vload<int, 4>({idx_c} + __j);")
+        w("else {")
+        w("#pragma unroll")
+        w(f"    for (int __q = 0; __q < 4; ++__q) __c[__q] = __j + __q < __end ? {idx_c}[__j + __q] : 0;")
+        w("}")
+        if car_c:
+            w(f"if (__j + 4 <= __end) __v = appy::vload<int, 4>({car_c} + __j);")
+            w("else {")
+            w("#pragma unroll")
+            w(f"    for (int __q = 0; __q < 4; ++__q) __v[__q] = __j + __q < __end ? {car_c}[__j + __q] : 0;")
+            w("}")
+        else:
+            w("__v = 0;")
+        w(f"int __row = 0, __past = {R};       // the last row that starts at or before __j")
+        w("#pragma unroll")
+        w(f"for (int __it = 0; __it < {R.bit_length() - 1}; ++__it) {{")
+        w("    const int __mid = (__row + __past) >> 1;")
+        w("    if (__lp[__mid] <= __j) __row = __mid; else __past = __mid;")
+        w("}")
+        w("#pragma unroll")
+        w("for (int __q = 0; __q < 4; ++__q) {")
+        w("    if (__j + __q >= __end) break;")
+        w("    while (__lp[__row + 1] <= __j + __q) ++__row;")
+        w("    const int __cq = __c[__q];")
+        w("    if (__cq < 0 || __cq >= __nx) { __inside = false; continue; }")
+        w("    const unsigned __rel = __rel0 + (unsigned)__row;")
+        w(f"    __keys[__j + __q] = ((__rel >> {RB}) << __lbits) | ((unsigned)__cq >> 5);")
+        w(f"    __vals[__j + __q] = (unsigned long long)(unsigned)__v[__q] | ((unsigned long long)((__rel & {(1 << RB) - 1}u) "
+          f"| (((unsigned)__cq & 31u) << {RB})) << 32);")
+        w("}")
+        self.ind -= 1
+        w("}")
+        self.ind -= 1
+        w("}")
+        w("if (__ballot(!__inside) != 0ull && __lid == 0) __flag[0] = 1;      // an index outside the gathered operand: no plan")
+        self.ind -= 1
+        w("}")
+
+    def _body_xcells(self):
+        """The kernel that runs a row plan: one workgroup of 1024 lanes per cell, the cells of column range
+        g on the workgroups g mod 8 (one XCD and its L2 per range).  Tile by tile: the lanes gather the
+        operand in the order of the plan (adjacent lanes read the same lines), put the value of each term into
+        its slot in LDS, and after a barrier add the slots to the sums of the cell's rows, which are in LDS
+        too - first the rows with one slot, a lane per row, then the rows with a run of slots, a lane per run,
+        in slot order.  A row is touched by one lane per tile and tiles are separated by barriers: the sums do
+        not depend on timing.  The sums of a cell go to the scratch table of 4-byte slots per row and range.
+
+        A wavefront instruction takes four cycles on a SIMD and only four wavefronts share one, so the loop is
+        written for few instructions: every load is a per-tile base held in scalar registers plus a lane
+        offset that never changes, nothing is loaded under a branch (the plan's arrays end in spare room, and
+        what is read beyond a cell is masked where it would matter), and headers are scalars."""
+        a, g = self.a, self.a.grouping
+        U = self.spec.unroll
+        TILE = 1024 * U
+        H = U // 2
+        SEG = TILE // 2 + 4          # words of the row stream from one tile of a cell to the next
+        RB = self.PLAN_ROW_BITS
+        ROWS = 1 << RB
+        self.ex.locals[a.var] = T.WEAK_INT
+        self.mode = "lane"
+        term, tty, pty = self._group_setup_types()
+        if pty.name not in ("float32", "int32", "uint32") and not self.dirty:
+            raise Unsupported(f"sums of {pty.name} are not accumulated in LDS")
+        x = a.arrays[g["x"]]
+        x.loaded = True
+        xc = cname(g["x"])
+        w = self.w
+        P = pty.c
+
+        def value(e, xv):
+            """Code of the term for element word `e` and gathered value `xv`."""
+            pre = ""
+            if g["carried"]:
+                cty = a.arrays[g["carried"]].ty
+                bits = f"(int)(unsigned)({e})"
+                pre = f"const {cty.c} __cv = {'__int_as_float(' + bits + ')' if cty.is_float else '(' + cty.c + ')' + bits}; "
+            return f"{{ {pre}const {x.elem_c} __cx = {xv}; __val = {cast(term, tty, pty)}; }}"
+
+        w("const unsigned __tid = threadIdx.x;")
+        w(f"__shared__ {P} __sum[{ROWS}];        // the sums of the rows of the cell")
+        w(f"__shared__ __attribute__((aligned(8))) {P} __prod[{TILE}];       // the terms of a tile, sorted by row")
+        w("const appy::i64 __n = __hi - __lo;")
+        w("const unsigned __cmask = (1u << __colbits) - 1u;")
+        w("const unsigned __xlast = (unsigned)(__nx - 1);")
+        w("const char* __xb = reinterpret_cast<const char*>(" + xc + ");")
+        w("// a cell may be shared by __split workgroups, each with a run of its tiles and a slot of its own for the sums")
+        w("for (appy::i64 __vc = blockIdx.x; __vc < __ncell * __split; __vc += gridDim.x) {")
+        self.ind += 1
+        w("const int __g = (int)(__vc & 7);")
+        w("const appy::i64 __b = (__vc >> 3) / __split;")
+        w("const int __part = (int)((__vc >> 3) % __split);")
+        w("const appy::i64 __cell = __b * 8 + __g;")
+        w("const appy::i64 __ce = __cstart[__cell + 1];")
+        w("const int __nta = (int)(__tbase[__cell + 1] - __tbase[__cell]);")
+        w("const int __tlo = (int)((appy::i64)__part * __nta / __split), __nt = (int)((appy::i64)(__part + 1) * __nta / __split) - __tlo;")
+        w(f"const appy::i64 __cs = (appy::i64)__cstart[__cell] + (appy::i64)__tlo * {TILE};")
+        w("const unsigned __x0 = (unsigned)(__g * __gwidth);")
+        w("// tile t of this workgroup: elements at __eb + t * TILE, row stream at __sb + t * SEG")
+        w("const char* __eb = reinterpret_cast<const char*>(__ent + __cs);")
+        w("const char* __sb = reinterpret_cast<const char*>(__rstream + ((__cs >> 1) + 4 * ((appy::i64)__tbase[__cell] + __tlo)));")
+        w("#pragma unroll")
+        w(f"for (int __k = 0; __k < {ROWS // 1024}; ++__k) __sum[__k * 1024 + __tid] = 0;")
+        w(f"unsigned long long __e0[{U}], __e1[{U}], __e2[{U}];")
+        w(f"{x.elem_c} __xv[{U}], __x1[{U}];")
+        w(f"unsigned __r0[{H}], __r1[{H}];")
+        w("unsigned __da0, __db0, __da1, __db1;")
+        w("unsigned __h0, __h1, __h2;")
+
+        def load_tile(dst, hdr, t):
+            w(f"{{ const char* __p = __eb + (appy::i64)({t}) * {TILE * 8};")
+            w("#pragma unroll")
+            w(f"  for (int __u = 0; __u < {U}; ++__u)")
+            w(f"      {dst}[__u] = __builtin_nontemporal_load(reinterpret_cast<const unsigned long long*>(__p + (unsigned)((__u * 1024 + __tid) * 8)));")
+            w(f"  {hdr} = __builtin_amdgcn_readfirstlane(*reinterpret_cast<const unsigned*>(__sb + (appy::i64)({t}) * {SEG * 4})); }}")
+
+        def load_rows(dst, da, db, hdr, t):
+            """Row numbers of the slots this lane adds up, and the first run of slots it may have to walk."""
+            w(f"{{ const char* __p = __sb + (appy::i64)({t}) * {SEG * 4};")
+            w("#pragma unroll")
+            w(f"  for (int __u = 0; __u < {H}; ++__u)")
+            w(f"      {dst}[__u] = __builtin_nontemporal_load(reinterpret_cast<const unsigned*>(__p + (unsigned)((1 + __u * 1024 + __tid) * 4)));")
+            w(f"  const char* __q = __p + (appy::i64)(1 + ((({hdr} & 0xffffu) + 1) >> 1)) * 4;")
+            w(f"  {da} = *reinterpret_cast<const unsigned*>(__q + (unsigned)(__tid * 4));")
+            w(f"  {db} = *reinterpret_cast<const unsigned*>(__q + (unsigned)(__tid * 4 + 4)); }}")
+
+        def gather(dst, src):
+            w("#pragma unroll")
+            w(f"for (int __u = 0; __u < {U}; ++__u) {{")
+            w(f"    unsigned __c = __x0 + ((unsigned)({src}[__u] >> 32) & __cmask);")
+            w("    __c = __c < __xlast ? __c : __xlast;        // (what was read beyond the cell may hold anything)")
+            w(f"    {dst}[__u] = *reinterpret_cast<const {x.elem_c}*>(__xb + (unsigned)(__c << 2));")
+            w("}")
+
+        def add_run(d, d1):
+            w(f"{{ const int __row = (int)({d} & {ROWS - 1}u), __from = (int)({d} >> {RB}), __to = (int)({d1} >> {RB});")
+            w(f"  {P} __acc = __sum[__row];")
+            w("  for (int __k = __from; __k < __to; __k += 4) {")
+            w(f"      const {P} __p0 = __prod[__k], __p1 = __k + 1 < __to ? __prod[__k + 1] : 0, "
+              "__p2 = __k + 2 < __to ? __prod[__k + 2] : 0, __p3 = __k + 3 < __to ? __prod[__k + 3] : 0;")
+            w("      __acc += __p0;")
+            w("      if (__k + 1 < __to) __acc += __p1;")
+            w("      if (__k + 2 < __to) __acc += __p2;")
+            w("      if (__k + 3 < __to) __acc += __p3;")
+            w("  }")
+            w("  __sum[__row] = __acc; }")
+
+        load_tile("__e0", "__h0", "0")
+        load_tile("__e1", "__h1", "1")
+        load_rows("__r0", "__da0", "__db0", "__h0", "0")
+        gather("__xv", "__e0")
+        w("__syncthreads();")
+        w("for (int __t = 0; __t < __nt; ++__t) {")
+        self.ind += 1
+        w(f"const appy::i64 __left = __ce - (__cs + (appy::i64)__t * {TILE});")
+        w(f"const unsigned __cnt = (unsigned)(__left < {TILE} ? __left : {TILE});")
+        w("const unsigned __ns = __h0 & 0xffffu, __nm = __h0 >> 16;")
+        w(f"if (__cnt == {TILE}u) {{")
+        w("#pragma unroll")
+        w(f"    for (int __u = 0; __u < {U}; ++__u) {{")
+        w(f"        {P} __val;")
+        w("        " + value("__e0[__u]", "__xv[__u]"))
+        w("        __prod[(unsigned)(__e0[__u] >> 32) >> __colbits] = __val;")
+        w("    }")
+        w("} else {")
+        w("#pragma unroll")
+        w(f"    for (int __u = 0; __u < {U}; ++__u) {{")
+        w(f"        {P} __val;")
+        w("        " + value("__e0[__u]", "__xv[__u]"))
+        w("        if (__u * 1024 + __tid < __cnt) __prod[(unsigned)(__e0[__u] >> 32) >> __colbits] = __val;")
+        w("    }")
+        w("}")
+        w("// the elements of the tile after the next, the row numbers and the gathers of the next one travel while this one is added up")
+        load_tile("__e2", "__h2", "__t + 2")
+        load_rows("__r1", "__da1", "__db1", "__h1", "__t + 1")
+        gather("__x1", "__e1")
+        w("__syncthreads();")
+        w("{")
+        w(f"    {P} __sa[{H}], __sb_[{H}];")
+        w(f"    appy::vec<{P}, 2>::type __pp[{H}];")
+        w("#pragma unroll")
+        w(f"    for (int __u = 0; __u < {H}; ++__u) {{")
+        w(f"        __pp[__u] = *reinterpret_cast<const appy::vec<{P}, 2>::type*>(&__prod[2 * (__u * 1024 + __tid)]);")
+        w("        __sa[__u] = __sum[__r0[__u] & 0x7fffu]; __sb_[__u] = __sum[(__r0[__u] >> 16) & 0x7fffu];")
+        w("    }")
+        w("#pragma unroll")
+        w(f"    for (int __u = 0; __u < {H}; ++__u) {{")
+        w("        const unsigned __s = 2 * (__u * 1024 + __tid);")
+        w("        if (__s < __ns) __sum[__r0[__u] & 0x7fffu] = __sa[__u] + __pp[__u][0];")
+        w("        if (__s + 1 < __ns) __sum[(__r0[__u] >> 16) & 0x7fffu] = __sb_[__u] + __pp[__u][1];")
+        w("    }")
+        w("}")
+        w("if (__nm > 0) {")
+        self.ind += 1
+        w("if (__tid < __nm) {")
+        self.ind += 1
+        add_run("__da0", "__db0")
+        self.ind -= 1
+        w("}")
+        w("if (__nm > 1024) {")
+        w(f"    const unsigned* __runs = reinterpret_cast<const unsigned*>(__sb + (appy::i64)__t * {SEG * 4}) + 1 + ((__ns + 1) >> 1);")
+        w("    for (unsigned __m = __tid + 1024; __m < __nm; __m += 1024) {")
+        w("        const unsigned __d = __runs[__m], __d1 = __runs[__m + 1];")
+        self.ind += 2
+        add_run("__d", "__d1")
+        self.ind -= 2
+        w("    }")
+        w("}")
+        self.ind -= 1
+        w("}")
+        w("__syncthreads();")
+        w("#pragma unroll")
+        w(f"for (int __u = 0; __u < {U}; ++__u) {{ __e0[__u] = __e1[__u]; __e1[__u] = __e2[__u]; __xv[__u] = __x1[__u]; }}")
+        w("#pragma unroll")
+        w(f"for (int __u = 0; __u < {H}; ++__u) __r0[__u] = __r1[__u];")
+        w("__h0 = __h1; __h1 = __h2; __da0 = __da1; __db0 = __db1;")
+        self.ind -= 1
+        w("}")
+        w(f"{P}* __out = reinterpret_cast<{P}*>(__scratch) + ((appy::i64)__part * 8 + __g) * __n + __b * {ROWS};")
+        w(f"if ((__b + 1) * {ROWS} <= __n) {{")
+        w("#pragma unroll")
+        w(f"    for (int __k = 0; __k < {ROWS // 1024}; ++__k) __out[__k * 1024 + __tid] = __sum[__k * 1024 + __tid];")
+        w("} else {")
+        w(f"    for (int __k = 0; __k < {ROWS // 1024}; ++__k)")
+        w(f"        if (__b * {ROWS} + __k * 1024 + __tid < __n) __out[__k * 1024 + __tid] = __sum[__k * 1024 + __tid];")
+        w("}")
+        w("__syncthreads();")
+        self.ind -= 1
+        w("}")
+
     def tiled_spread_loop(self, st: ast.For):
         """The LDS-staged form of :meth:`spread_loop` for the loop of the plan."""
         var = st.target.id
@@ -3054,6 +3381,24 @@ class KernelBuilder:
             params.append(Param("__ent", ("long long* __ent" if sp.aux == "group" else "const long long* __ent"), C.c_void_p, "ent"))
             params.append(Param("__desc", ("int* __desc" if sp.aux == "group" else "const int* __desc"), C.c_void_p, "desc"))
             params.append(Param("__shiftc", "const int __shiftc", C.c_int32, "shiftc"))
+        if sp.aux == "rkeys":
+            params.append(Param("__keys", "unsigned* __keys", C.c_void_p, "keys"))
+            params.append(Param("__vals", "unsigned long long* __vals", C.c_void_p, "vals"))
+            params.append(Param("__len", "const appy::i64 __len", C.c_int64, "entries"))
+            params.append(Param("__nx", "const appy::i64 __nx", C.c_int64, "nx"))
+            params.append(Param("__lbits", "const int __lbits", C.c_int32, "lbits"))
+            params.append(Param("__flag", "long long* __flag", C.c_void_p, "flag"))
+        if sp.aux == "xcells":
+            params.append(Param("__ent", "const unsigned long long* __ent", C.c_void_p, "ent"))
+            params.append(Param("__cstart", "const unsigned* __cstart", C.c_void_p, "cstart"))
+            params.append(Param("__tbase", "const unsigned* __tbase", C.c_void_p, "tbase"))
+            params.append(Param("__rstream", "const unsigned* __rstream", C.c_void_p, "rstream"))
+            params.append(Param("__ncell", "const appy::i64 __ncell", C.c_int64, "ncell"))
+            params.append(Param("__split", "const appy::i64 __split", C.c_int64, "split"))
+            params.append(Param("__gwidth", "const appy::i64 __gwidth", C.c_int64, "gwidth"))
+            params.append(Param("__colbits", "const int __colbits", C.c_int32, "colbits"))
+            params.append(Param("__nx", "const appy::i64 __nx", C.c_int64, "nx"))
+            params.append(Param("__scratch", "double* __scratch", C.c_void_p, "scratch"))
         if sp.aux == "group" and sp.skip_long:
             params.append(Param("__counts", "const int* __counts", C.c_void_p, "counts"))
             params.append(Param("__base", "const int __base", C.c_int32, "base"))

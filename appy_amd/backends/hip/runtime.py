@@ -12,7 +12,7 @@ import threading
 _LIB_NAME = "libappy_hip.so"
 _PKG_ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 
 class Props(C.Structure):
@@ -37,6 +37,18 @@ class FuncInfo(C.Structure):
         ("static_lds_bytes", C.c_int32),
         ("scratch_bytes", C.c_int32),
         ("max_threads_per_block", C.c_int32),
+    ]
+
+
+class RowPlanShape(C.Structure):
+    _fields_ = [
+        ("entries", C.c_uint64),
+        ("row_blocks", C.c_uint32),
+        ("groups", C.c_uint32),
+        ("group_width", C.c_uint32),
+        ("col_bits", C.c_uint32),
+        ("tile", C.c_uint32),
+        ("line_bits", C.c_uint32),
     ]
 
 
@@ -83,6 +95,8 @@ SIGNATURES = {
     "appy_hip_launch_static_scratch": (
         C.c_int, [_vp, _u32, _u32, _u32, _u32, _u32, _u32, _u32, _vp, _vp, C.c_size_t, C.c_size_t, C.c_size_t]),
     "appy_hip_rtc_version": (C.c_int, [C.POINTER(C.c_int)]),
+    "appy_hip_rowplan_sizes": (C.c_int, [C.POINTER(RowPlanShape), C.POINTER(C.c_size_t), C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]),
+    "appy_hip_rowplan_build": (C.c_int, [C.POINTER(RowPlanShape), _vp, _vp, _vp, _vp, _vp, C.c_size_t, _vp, _vp, _vp, _vp]),
     "appy_hip_stream_create": (C.c_int, [C.POINTER(_vp)]),
     "appy_hip_stream_destroy": (C.c_int, [_vp]),
     "appy_hip_graph_begin": (C.c_int, [_vp]),

@@ -190,7 +190,12 @@ def compile_all_patterns() -> int:
                          Spec("team", block=256, vec=v, width=16, phase=1, rows="list", parts=8, guard=1),
                          Spec("team", block=256, vec=1, width=64, parts=16, aux="cells", block_rows=256, guard=1),
                          Spec("team", block=256, vec=v, width=1, phase=2, guard=1),
-                         Spec("team", block=256, vec=v, width=4, guard=2)]
+                         Spec("team", block=256, vec=v, width=4, guard=2),
+                         # the order of the elements worked out once and kept: the kernel that writes the pairs to
+                         # sort, the kernel that runs the plan
+                         Spec("team", block=256, vec=1, width=64, aux="rkeys", block_rows=256),
+                         Spec("team", block=1024, vec=1, width=1024, unroll=6, parts=8, aux="xcells"),
+                         Spec("team", block=1024, vec=1, width=1024, unroll=4, parts=8, aux="xcells")]
         for spec in more:
             loop.kernel_for(spec).code
             count += 1

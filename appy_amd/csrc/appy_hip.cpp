@@ -51,6 +51,14 @@ int fail_arg(const char* what) {
     return static_cast<int>(hipErrorInvalidValue);
 }
 
+}  // namespace
+
+// error reporting for the other source files of the library (not exported)
+__attribute__((visibility("hidden"))) int appy_hip_internal_fail(hipError_t e, const char* what) { return fail_hip(e, what); }
+__attribute__((visibility("hidden"))) int appy_hip_internal_fail_arg(const char* what) { return fail_arg(what); }
+
+namespace {
+
 #define HIP_TRY(expr)                                   \
     do {                                                \
         hipError_t e__ = (expr);                        \

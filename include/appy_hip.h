@@ -24,9 +24,10 @@
 extern "C" {
 #endif
 
-/* 2: page-locked host memory, streams and graphs, appy_hip_rtc_version; 3: appy_hip_launch_static_scratch
+/* 2: page-locked host memory, streams and graphs, appy_hip_rtc_version; 3: appy_hip_launch_static_scratch;
+ * 4: row plans (appy_hip_rowplan_*), appy_hip_device_topology
  * (additions only: every entry point of the earlier versions is unchanged). */
-#define APPY_HIP_ABI_VERSION 3
+#define APPY_HIP_ABI_VERSION 4
 
 typedef struct appy_hip_props {
     char     name[128];        /* marketing name */
@@ -152,6 +153,45 @@ int appy_hip_launch_static_scratch(void* func,
                                    uint32_t dynamic_lds_bytes, void* stream,
                                    const void* args, size_t args_bytes,
                                    size_t scratch_arg_offset, size_t scratch_bytes);
+
+/* ---- row plans ------------------------------------------------------------
+ * The reference runs the CSR loop of examples/03-spmv.py:5-16
+ * (tests/integration/triton/tutorial/test_spmv.py:10-21) one row per program, every launch from the raw
+ * arrays.  When the same arrays come back launch after launch, the order in which the elements of
+ * `s += f(A[j], X[IDX[j]])` are walked can be worked out once ("inspector") and kept: a row plan.  A
+ * generated kernel turns every position j of the streamed arrays into
+ *     key  = (block of 2^APPY_HIP_ROWPLAN_ROW_BITS rows) << line_bits | (IDX[j] >> 5)   (0xFFFFFFFF: no element here)
+ *     val  = bits of A[j] | (row within the block) << 32 | (IDX[j] & 31) << (32 + APPY_HIP_ROWPLAN_ROW_BITS)
+ * and appy_hip_rowplan_build orders them, on `stream`, without waiting for it and without allocating:
+ *   keys_sorted / elements   the pairs sorted by key (stable); `elements` is then rewritten in place to
+ *                            bits of A[j] | (column within its group | slot << col_bits) << 32
+ *   cell_start[cells + 1]    cell c = block c / groups, column range c % groups (`group_width` columns each):
+ *                            elements [cell_start[c], cell_start[c + 1]); cell_start[cells] = all elements
+ *   tile_base[cells + 1]     number of tiles (of `tile` elements, the last of a cell shorter) before cell c
+ *   row_stream               per tile, at word (first element >> 1) + 4 * (tile number): one word
+ *                            singles | runs << 16; the rows of the slots [0, singles) as 16-bit numbers
+ *                            (rows that occur once in the tile); then runs + 1 words row | first slot <<
+ *                            APPY_HIP_ROWPLAN_ROW_BITS of the rows that occur several times, whose elements
+ *                            hold consecutive slots from `singles` on (the last word: the end)
+ * Within a tile no row appears in two slots of the singles or in two runs, so a kernel may add the slots
+ * to per-row sums with plain loads and stores.  appy_hip_rowplan_sizes gives the bytes of `sort_temp`, the
+ * most tiles there can be and the words of `row_stream`.  Shapes that do not fit a 32-bit key or packed
+ * word are refused (invalid value). */
+#define APPY_HIP_ROWPLAN_ROW_BITS 15
+typedef struct appy_hip_rowplan_shape {
+    uint64_t entries;       /* positions of the streamed arrays (pairs to sort), < 2^31 */
+    uint32_t row_blocks;    /* blocks of 2^APPY_HIP_ROWPLAN_ROW_BITS rows */
+    uint32_t groups;        /* column ranges of X (8: one per XCD) */
+    uint32_t group_width;   /* columns per range, a multiple of 32 */
+    uint32_t col_bits;      /* bits of the column within its range in a packed word */
+    uint32_t tile;          /* elements per tile: 4096 or 6144 */
+    uint32_t line_bits;     /* bits of IDX[j] >> 5 in a key */
+} appy_hip_rowplan_shape;
+int appy_hip_rowplan_sizes(const appy_hip_rowplan_shape* shape, size_t* sort_temp_bytes_out, size_t* max_tiles_out,
+                           size_t* stream_words_out);
+int appy_hip_rowplan_build(const appy_hip_rowplan_shape* shape, const uint32_t* keys, const uint64_t* vals,
+                           uint32_t* keys_sorted, uint64_t* elements, void* sort_temp, size_t sort_temp_bytes,
+                           uint32_t* cell_start, uint32_t* tile_base, uint32_t* row_stream, void* stream);
 
 /* ---- streams and graphs -----------------------------------------------------
  * A loop nest that launches many short kernels (a time-stepping host loop
