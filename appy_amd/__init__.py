@@ -52,6 +52,19 @@ def _reduction_result(buffer, start):
     return value
 
 
+def release():
+    """Give back the device memory the compiled loops hold between launches - scratch buffers of launches made of
+    several kernels, row plans (the kept order of the elements of CSR-like loops) - and what the pooled
+    allocator has cached.  Waits for the launches that use that memory.  The loops stay compiled; the next
+    launch of a loop allocates again what it needs."""
+    from .backends.hip import codegen as _cg
+    from .backends.hip import runtime as _rt
+
+    for _f, _src in list(_cg.code_cache.values()):
+        _f.release()
+    _rt.check(_rt.lib().appy_hip_pool_trim())
+
+
 def set_default_options(options):
     for key, val in _DEFAULT_OPTIONS:
         options.setdefault(key, val)

@@ -298,6 +298,7 @@ class RowPlan:
         self.ncell = 0
         self.tile = 0
         self.split = 1              # workgroups per cell
+        self.owner = None           # the loop the plan belongs to
         self.inspector_ms = None
 
     def alloc(self, nbytes):
@@ -339,6 +340,8 @@ def drop_plans_overlapping(extents):
                if any(p < q + m and q < p + n for p, n in stored for q, m in plan.ranges)]
     for plan in hit:
         plan.valid = False      # its memory goes back once the launches that use it have drained (CompiledLoop.release / next build)
+        if plan.owner is not None:
+            plan.owner._plan_seen.clear()       # the arrays have changed: they count as new
         with _plans_lock:
             if plan in _live_plans:
                 _live_plans.remove(plan)
@@ -414,6 +417,7 @@ class CompiledLoop:
         self._scratch = {}  # (device, stream) -> (device pointer, bytes): partial results of two-phase launches
         self._group_off = False     # a kernel of the grouped form could not be generated for this loop
         self._hints = {}    # device -> (address, ctypes view) of page-locked words the binned kernels report to
+        self._hint_key = {} # device -> which arrays the launch that reports next was about
         self._scratch_retired = []
         self._replays = {}  # call identity -> Launch that can simply be launched again
         self._plans = []    # row plans of this loop, most recently used last
@@ -754,7 +758,7 @@ class CompiledLoop:
         these arrays do not qualify: the operand is larger than an L2 can keep next to the streams and
         no larger than 16 stripes of half an L2, the rows hold a few elements at least."""
         g = self.analysis.grouping
-        if g is None or self._group_off or not self.options.get("hip_group", True) or not self.options.get("hip_hints", True):
+        if g is None or self._group_off or not self.options.get("hip_group", True):
             return None
         nx = int(arrays[g["x"]].shape[0])
         if nx * 4 <= STRIPE_MIN_BYTES or nx > (16 << GROUP_MAX_STRIPE_LOG):
@@ -768,22 +772,42 @@ class CompiledLoop:
             return None
         return parts, shift, entries
 
-    def scratch(self, device: int, stream: int, nbytes: int) -> int:
+    def scratch(self, device: int, stream: int, nbytes: int):
         """Device memory for partial results of two-phase launches of this loop: one buffer per
-        device and stream, kept for the life of the loop (launches on one stream follow one
-        another, so they may share it; it only ever grows)."""
+        device and stream, kept until `release` (launches on one stream follow one another, so they
+        may share it; it only ever grows).  None when the loop would hold more than `scratch_limit`
+        allows: the caller then takes a form that needs less."""
         key = (device, stream)
         with self._lock:
             have = self._scratch.get(key)
-            if have is None or have[1] < nbytes:
-                if have is not None:
-                    # launches in flight (or recorded in a graph) may still name the smaller buffer:
-                    # it is kept, not freed; doubling bounds what is kept to less than the final size
-                    self._scratch_retired.append(have[0])
-                    nbytes = max(nbytes, 2 * have[1])
-                have = (rt.malloc(nbytes), nbytes)
-                self._scratch[key] = have
-            return have[0]
+            if have is not None and have[1] >= nbytes:
+                return have[0]
+            if nbytes > scratch_limit(device):
+                return None
+            if have is not None:
+                # launches in flight (or recorded in a graph) may still name the smaller buffer: it goes back
+                # once its stream has drained (at the next growth or at `release`); doubling bounds what
+                # is held meanwhile
+                nbytes = min(max(nbytes, 2 * have[1]), max(nbytes, scratch_limit(device)))
+                retired, self._scratch_retired = self._scratch_retired, [(have[0], stream)]
+            else:
+                retired = []
+            have = (rt.malloc(nbytes), nbytes)
+            self._scratch[key] = have
+        if retired and graphs.current() is None:
+            for ptr, st in retired:
+                rt.sync(st)
+                rt.free(ptr)
+        elif retired:
+            with self._lock:
+                self._scratch_retired = retired + self._scratch_retired
+        return have[0]
+
+    def scratch_bytes(self, device: int) -> int:
+        """Device memory this loop holds on `device` between launches (scratch buffers and row plans)."""
+        with self._lock:
+            return (sum(n for (dev, _st), (_p, n) in self._scratch.items() if dev == device)
+                    + sum(pl.nbytes for pl in self._plans if pl.device == device and pl.buffers))
 
     def hint(self, device: int):
         """Five page-locked 64-bit words per device that the kernel over binned rows writes (a flag, then
@@ -807,12 +831,12 @@ class CompiledLoop:
         self.release_plans()
         with self._lock:
             held, self._scratch, self._scratch_retired = (
-                [(k, p) for k, (p, _n) in self._scratch.items()] + [(None, p) for p in self._scratch_retired], {}, [])
+                [(k, p) for k, (p, _n) in self._scratch.items()] + [((None, st), p) for p, st in self._scratch_retired], {}, [])
         try:
             for key, _ptr in held:
-                if key is not None:
+                if key[0] is not None:
                     _ensure_device(key[0])
-                    rt.sync(key[1])
+                rt.sync(key[1])
             for _key, ptr in held:
                 rt.free(ptr)
             with self._lock:
@@ -1186,20 +1210,20 @@ class Launch:
             self.nsplit = loop.team_parts(spec, n_outer, env, arrays)
             reds = len(loop_ir.reductions_of(a.team_split))
             self.scratch_ptr = loop.scratch(device, self.stream, max(1, reds) * self.nsplit * n_outer * 8)
+        if spec.phase == 1 and self.scratch_ptr is None:
+            # more scratch memory than the loop may hold: one kernel, one workgroup per strip or row
+            spec = dataclasses.replace(spec, phase=0)
+            self.kernel, self.spec, self.nsplit, self.scratch_ptr = loop.kernel_for(spec), spec, 1, 0
         self.scalar_fields = {}      # by-value scalar -> field of the argument block
         self.sequence = None         # binned rows: [(kernel, argument block, grid, block)] launched in this order
-        if spec.rows == "mixed" and self._stage_planned(vals, arrays, lo, hi, spec):
-            loop.last_launch = self
-            return
-        if spec.rows == "mixed" and self._stage_grouped(vals, arrays, lo, hi, spec):
-            loop.last_launch = self
-            return
         if spec.rows == "mixed":
-            self._stage_binned(vals, arrays, lo, hi, spec)
-            self.args = self.sequence[2][1]
-            self.grid, self.block = self.sequence[2][2], self.sequence[2][3]
-            loop.last_launch = self
-            return
+            if (self._stage_planned(vals, arrays, lo, hi, spec) or self._stage_grouped(vals, arrays, lo, hi, spec)
+                    or self._stage_binned(vals, arrays, lo, hi, spec)):
+                loop.last_launch = self
+                return
+            # not even the lists of rows fit what the loop may hold: one team width for all rows
+            spec = loop.choose_spec(n_outer, env, arrays, restrict=restrict, listable=False)
+            self.kernel, self.spec = loop.kernel_for(spec), spec
         self.args = self._argument_block(self.kernel, vals, arrays, lo, hi)
         if spec.phase == 1 and spec.kind == "strip":
             strips = -(-n_outer // 64)
@@ -1232,13 +1256,15 @@ class Launch:
         widthlog = [0, 2, 4, 6]
         trip, _uniform = loop._estimate_trip(env, arrays, n)
         base = sum(1 for t in thresholds if trip > t)
-        # what the last launch of this loop that has got that far found in its classes (a hint: it may
-        # describe other arrays).  The class with most rows is the one to take in natural order; without
+        # what the last launch of this loop found in its classes, if it was about the same arrays (a hint: their
+        # contents may have changed).  The class with most rows is the one to take in natural order; without
         # long rows last time, this launch sets nothing up for parts (long rows, if there are some after
-        # all, then run whole).
+        # all, then run whole).  Neither changes the order in which the terms of a row are added.
         hint_addr, hint = loop.hint(self.device)
         seen = [int(hint[k]) for k in range(5)] if self.loop.options.get("hip_hints", True) else [0] * 5
-        known = seen[0] == 1 and sum(seen[1:]) == n and min(seen[1:]) >= 0
+        ident = self._hint_identity(arrays, lo, hi) if a.grouping is not None else (lo, hi)
+        known = loop._hint_key.get(self.device) == ident and seen[0] == 1 and sum(seen[1:]) == n and min(seen[1:]) >= 0
+        loop._hint_key[self.device] = ident
         parts, stripe, cap = 0, 0, 0
         gather = a.ragged[1]
         if gather is not None:
@@ -1268,6 +1294,8 @@ class Launch:
         off_part = (off_start + 8 * cap + 255) // 256 * 256
         total = off_part + 8 * reds * parts * cap
         buf = loop.scratch(self.device, self.stream, total)
+        if buf is None:
+            return False
         self.bin = {
             "counts": buf, "load": buf + 32, "zero": buf + 1024, "rows": buf + off_rows, "m": n, "base": base, "threshold": thresholds,
             "widthlog": widthlog, "skip": cap if parts else 0, "bnd": buf + off_bnd, "rowstart": buf + off_start, "cap": cap, "stripe": stripe,
@@ -1306,6 +1334,8 @@ class Launch:
             seq.append((last, self._argument_block(last, vals, arrays, lo, hi),
                         (max(1, min(1024, -(-cap // 256))), 1, 1), (256, 1, 1)))
         self.sequence = seq
+        self.args, self.grid, self.block = seq[2][1], seq[2][2], seq[2][3]
+        return True
 
     def _stage_grouped(self, vals, arrays, lo, hi, spec) -> bool:
         """The launches of a loop of short rows whose simd loop sums terms that gather from an operand
@@ -1325,12 +1355,16 @@ class Launch:
             #  memory-set node, and those are kept out of graphs)
             return False
         V = spec.vec
+        # The form of the launch follows from what the host knows of these arrays (their sizes).  What the last
+        # launch of the loop reported about the lengths of the rows only prunes it: when that launch was about
+        # these same arrays and found no row beyond the limit, the kernels for such rows - which would run
+        # empty - are left out.  Both forms add the terms of a row in the same order.
         _addr, hint = loop.hint(self.device)
         seen = [int(hint[k]) for k in range(5)]
-        # the last launch has sorted these rows: with rows in the class of the longest, those run in planned parts
-        if not (seen[0] == 1 and sum(seen[1:]) == n and min(seen[1:]) >= 0):
-            return False
-        long_rows = seen[4] > 0
+        ident = self._hint_identity(arrays, lo, hi)
+        trusted = (loop.options.get("hip_hints", True) and loop._hint_key.get(self.device) == ident
+                   and seen[0] == 1 and sum(seen[1:]) == n and min(seen[1:]) >= 0)
+        long_rows = not trusted or seen[4] > 0
         shape = loop.grouped_shape(n, env, arrays)
         if shape is None:
             return False
@@ -1379,11 +1413,19 @@ class Launch:
         off_ent = (off_desc + 4 * (parts + 1) * nblk + 255) // 256 * 256
         off_part = (off_ent + 8 * entries + 255) // 256 * 256
         buf = loop.scratch(self.device, self.stream, off_part + 4 * parts * n)
+        if buf is None:
+            return False
         hint_addr, _ = loop.hint(self.device)
-        base = max(range(3), key=lambda c: seen[c + 1])
+        if trusted:
+            base = max(range(3), key=lambda c: seen[c + 1])
+        else:
+            trip, _uniform = loop._estimate_trip(env, arrays, n)
+            base = sum(1 for t in (V, 8 * V) if trip > t)
+        loop._hint_key[self.device] = ident
         self.bin = {"flag": buf + 1984, "desc": buf + off_desc, "ent": buf + off_ent, "shiftc": shift, "entries": entries,
-                    # (without long rows: the limit beyond which the launch that sorts the rows would have reported some)
-                    "rowmax": cut if long_rows else max(32 * V, 32 * parts), "hint": hint_addr,
+                    # (one limit in every form: rows beyond it are cut at the stripes when the launch has kernels for
+                    #  them, and reported by the grouping kernel when it has not)
+                    "rowmax": cut, "hint": hint_addr,
                     "counts": buf, "load": buf + 32, "zero": buf + 1024, "rows": buf + off_rows, "m": n, "base": base,
                     "threshold": [V, 8 * V, cut], "bnd": buf + off_bnd, "rowstart": buf + off_start, "cap": cap,
                     "stripe": -(-int(arrays[g["x"]].shape[0]) // parts), "nrows": buf + 4 * 3}
@@ -1411,6 +1453,15 @@ class Launch:
         self.kernel, self.spec = cells, cells.src.spec
         self.args, self.grid, self.block = args_of_cells[1], args_of_cells[2], args_of_cells[3]
         return True
+
+    def _hint_identity(self, arrays, lo, hi):
+        """Names the arrays the lengths of the rows come from (address and shape, not contents): what a launch
+        reports about the rows is only believed by a launch over the same arrays."""
+        out = [lo, hi]
+        for nm in self.loop.plan_arrays():
+            v = arrays[nm]
+            out.append((nm, v.ctypes.data if isinstance(v, np.ndarray) else v.data_ptr(), tuple(v.shape)))
+        return tuple(out)
 
     def _plan_identity(self, arrays, lo, hi, vals):
         """``(key, tensors)`` naming the contents a row plan of this launch would describe, or None when
@@ -1492,6 +1543,8 @@ class Launch:
         split = plan.split
         self.bin["split"] = split
         self.scratch_ptr = loop.scratch(self.device, self.stream, 4 * PLAN_GROUPS * split * n)
+        if self.scratch_ptr is None:
+            return False
         self.nsplit = PLAN_GROUPS * split
         self.plan = plan
         seq = [(cells, self._argument_block(cells, vals, arrays, lo, hi), (plan.ncell * split, 1, 1), (1024, 1, 1)),
@@ -1581,6 +1634,7 @@ class Launch:
         forced = loop.options.get("hip_plan_split")
         plan.split = int(forced) if forced else max(1, min(-(-4 * DEFAULT_CUS // ncell), entries // (2 * plan.tile * ncell), 32))
         plan.valid = True
+        plan.owner = loop
         with loop._lock:
             loop._plans.append(plan)
         with _plans_lock:
