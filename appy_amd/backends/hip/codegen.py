@@ -784,23 +784,22 @@ class CompiledLoop:
                 return have[0]
             if nbytes > scratch_limit(device):
                 return None
+            retired = []
             if have is not None:
-                # launches in flight (or recorded in a graph) may still name the smaller buffer: it goes back
-                # once its stream has drained (at the next growth or at `release`); doubling bounds what
-                # is held meanwhile
+                # launches in flight may still name the smaller buffer: it goes back once its stream has drained
+                # (at the next growth or at `release`); a buffer that launches recorded into a graph name stays
+                # until `release`.  Doubling bounds what is held meanwhile.
                 nbytes = min(max(nbytes, 2 * have[1]), max(nbytes, scratch_limit(device)))
-                retired, self._scratch_retired = self._scratch_retired, [(have[0], stream)]
-            else:
-                retired = []
+                recorded = graphs.current() is not None
+                self._scratch_retired.append((have[0], stream, recorded))
+                if not recorded:
+                    retired = [r for r in self._scratch_retired if not r[2]]
+                    self._scratch_retired = [r for r in self._scratch_retired if r[2]]
             have = (rt.malloc(nbytes), nbytes)
             self._scratch[key] = have
-        if retired and graphs.current() is None:
-            for ptr, st in retired:
-                rt.sync(st)
-                rt.free(ptr)
-        elif retired:
-            with self._lock:
-                self._scratch_retired = retired + self._scratch_retired
+        for ptr, st, _recorded in retired:
+            rt.sync(st)
+            rt.free(ptr)
         return have[0]
 
     def scratch_bytes(self, device: int) -> int:
@@ -831,12 +830,11 @@ class CompiledLoop:
         self.release_plans()
         with self._lock:
             held, self._scratch, self._scratch_retired = (
-                [(k, p) for k, (p, _n) in self._scratch.items()] + [((None, st), p) for p, st in self._scratch_retired], {}, [])
+                [(k, p) for k, (p, _n) in self._scratch.items()] + [((None, st), p) for p, st, _rec in self._scratch_retired], {}, [])
         try:
-            for key, _ptr in held:
-                if key[0] is not None:
-                    _ensure_device(key[0])
-                rt.sync(key[1])
+            for dev in {key[0] for key, _ptr in held if key[0] is not None} or ({0} if held else set()):
+                _ensure_device(dev)
+                rt.device_sync()        # (streams named by the keys may have been destroyed since)
             for _key, ptr in held:
                 rt.free(ptr)
             with self._lock:
@@ -854,9 +852,7 @@ class CompiledLoop:
         for plan in plans:
             try:
                 _ensure_device(plan.device)
-                rt.sync(0)
-                for stream in {st for (dev, st) in self._scratch if dev == plan.device}:
-                    rt.sync(stream)
+                rt.device_sync()        # (the streams the plan was used on may no longer exist)
             except Exception:
                 pass
             plan.release()
@@ -1490,7 +1486,9 @@ class Launch:
         keep nothing.  False (nothing staged) when the launch does not qualify or has no plan yet."""
         loop, a, env = self.loop, self.loop.analysis, self.env
         reuse = loop.options.get("hip_reuse", True)
-        if a.grouping is None or not reuse or loop._plan_off:
+        if a.grouping is None or not reuse or loop._plan_off or self.capture is not None:
+            # (a launch recorded into a graph is replayed without being staged again: it must read the arrays
+            #  themselves every time, not an order worked out from what they held when it was recorded)
             return False
         n = hi - lo
         ident = self._plan_identity(arrays, lo, hi, vals)
@@ -1504,8 +1502,7 @@ class Launch:
             with loop._lock:
                 dead = [pl for pl in loop._plans if not pl.valid]
                 loop._plans = [pl for pl in loop._plans if pl.valid]
-            rt.sync(self.stream)
-            rt.sync(0)
+            rt.device_sync()
             for pl in dead:
                 pl.release()
         with loop._lock:
@@ -1516,7 +1513,7 @@ class Launch:
                     loop._plans.append(cand)
                     break
         if plan is None:
-            if key in loop._plan_refused or self.capture is not None:
+            if key in loop._plan_refused:
                 return False
             shape = loop.plan_shape(n, env, arrays)
             if shape is None:
@@ -1580,9 +1577,8 @@ class Launch:
             old = [pl for pl in loop._plans if not pl.valid] + [pl for pl in loop._plans if pl.valid][:-(PLANS_PER_LOOP - 1) or None]
             loop._plans = [pl for pl in loop._plans if pl not in old]
         if old:
-            rt.sync(self.stream)
+            rt.device_sync()
             for pl in old:
-                rt.sync(0)
                 pl.release()
         import weakref
 

@@ -92,6 +92,7 @@ SIGNATURES = {
     "appy_hip_memset_async": (C.c_int, [_vp, C.c_int, C.c_size_t, _vp]),
     "appy_hip_launch": (C.c_int, [_vp, _u32, _u32, _u32, _u32, _u32, _u32, _u32, _vp, _vp, C.c_size_t]),
     "appy_hip_sync": (C.c_int, [_vp]),
+    "appy_hip_device_sync": (C.c_int, []),
     "appy_hip_launch_static_scratch": (
         C.c_int, [_vp, _u32, _u32, _u32, _u32, _u32, _u32, _u32, _vp, _vp, C.c_size_t, C.c_size_t, C.c_size_t]),
     "appy_hip_rtc_version": (C.c_int, [C.POINTER(C.c_int)]),
@@ -338,6 +339,11 @@ def launch_timed(func, grid, block, args_struct, stream: int = 0, dynamic_lds: i
 
 def sync(stream: int = 0) -> None:
     check(lib().appy_hip_sync(_vp(stream)))
+
+
+def device_sync() -> None:
+    """Wait for every stream of the current device."""
+    check(lib().appy_hip_device_sync())
 
 
 def stream_create() -> int:

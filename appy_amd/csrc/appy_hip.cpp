@@ -714,6 +714,11 @@ int appy_hip_sync(void* stream) {
     return 0;
 }
 
+int appy_hip_device_sync(void) {
+    HIP_TRY(hipDeviceSynchronize());
+    return 0;
+}
+
 int appy_hip_launch_static_scratch(void* func,
                                    uint32_t grid_x, uint32_t grid_y, uint32_t grid_z,
                                    uint32_t block_x, uint32_t block_y, uint32_t block_z,

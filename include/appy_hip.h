@@ -25,7 +25,7 @@ extern "C" {
 #endif
 
 /* 2: page-locked host memory, streams and graphs, appy_hip_rtc_version; 3: appy_hip_launch_static_scratch;
- * 4: row plans (appy_hip_rowplan_*), appy_hip_device_topology
+ * 4: row plans (appy_hip_rowplan_*), appy_hip_device_sync
  * (additions only: every entry point of the earlier versions is unchanged). */
 #define APPY_HIP_ABI_VERSION 4
 
@@ -133,6 +133,9 @@ int appy_hip_launch(void* func,
                     uint32_t dynamic_lds_bytes, void* stream,
                     const void* args, size_t args_bytes);
 int appy_hip_sync(void* stream);               /* hipStreamSynchronize */
+/* Wait for everything queued on the current device, on every stream (hipDeviceSynchronize): what a caller
+ * does before it gives back memory that launches on streams it no longer knows may still use. */
+int appy_hip_device_sync(void);
 
 /* appy_hip_launch for a kernel that takes a scratch buffer among its arguments (the partial results
  * of a loop that runs as two kernels), without any allocation: the library keeps one buffer of

@@ -32,7 +32,7 @@ def plain(gpu):
 
 @pytest.fixture(scope="module")
 def sorted_only(gpu):
-    """Rows sorted by length, but never the grouped form that short rows take from their second launch on."""
+    """Rows sorted by length, but never the form that groups the elements of short rows by stripe."""
     return selfcheck.kernels(hip_group=False)
 
 
@@ -63,12 +63,13 @@ def _powerlaw(m, n, clip, seed, exponent=1.5):
 
 
 @pytest.mark.parametrize("m,n,clip", [(40_000, 1 << 20, 4096), (33_000, 5_000_000, 3000), (100_000, 1 << 19, 700)])
-def test_spmv_powerlaw_rows_are_binned_and_striped(k, plain, m, n, clip):
+def test_spmv_powerlaw_rows_are_binned_and_striped(sorted_only, plain, m, n, clip):
+    k = sorted_only
     data, indptr, indices, x, lengths = _powerlaw(m, n, clip, seed=m)
     ref, budget = vo.spmv_csr(data, indptr, indices, x, (m, n))
     _forget()
     y = k.spmv(data, indptr, indices, x, m, n)
-    launch = _loop("spmv").last_launch
+    launch = _loop("spmv", group=False).last_launch
     assert launch.spec.rows == "mixed" and launch.sequence is not None
     striped = 4 * n > cg.STRIPE_MIN_BYTES
     assert len(launch.sequence) == (6 if striped else 3)
@@ -154,9 +155,9 @@ def test_spmv_columns_in_any_order_and_int64_indices(k):
 
 def test_the_hint_of_an_earlier_launch_shapes_the_next_one_and_never_its_results(sorted_only):
     """The kernel over the binned rows reports the sizes of its classes in page-locked memory.  The next
-    launch takes the most populous class in natural order and leaves out the kernels for long rows when
-    there were none; a matrix that has long rows after all is still computed correctly (its long rows
-    then run whole), and the launch after that cuts them into parts again."""
+    launch over the same arrays takes the most populous class in natural order and leaves out the kernels
+    for long rows when there were none; a launch over other arrays believes nothing of it.  The bits of the
+    result are the same either way."""
     k = sorted_only
     m, n = 40_000, 1 << 20
     short = wl.spmv_uniform(m, n, 3)                        # every row in the class of single lanes
@@ -167,17 +168,19 @@ def test_the_hint_of_an_earlier_launch_shapes_the_next_one_and_never_its_results
     assert first.bin["base"] == 0 and len(first.sequence) == 6
     ref, budget = vo.spmv_csr(*short, (m, n))
     assert vo.within_budget(y, ref, budget, TOL)[0]
+    y_again = k.spmv(*short, m, n)
+    again = _loop("spmv", group=False).last_launch
+    assert len(again.sequence) == 3 and again.bin["skip"] == 0 and np.array_equal(y, y_again)
     ref, budget = vo.spmv_csr(data, indptr, indices, x, (m, n))
-    y1 = k.spmv(data, indptr, indices, x, m, n)             # shaped by the hint of the short rows
+    y1 = k.spmv(data, indptr, indices, x, m, n)             # other arrays: set up for long rows whatever was reported
     second = _loop("spmv", group=False).last_launch
-    assert len(second.sequence) == 3 and second.bin["skip"] == 0
+    assert len(second.sequence) == 6
     ok, worst = vo.within_budget(y1, ref, budget, TOL)
     assert ok, worst
-    y2 = k.spmv(data, indptr, indices, x, m, n)             # now it is known to have long rows
+    y2 = k.spmv(data, indptr, indices, x, m, n)             # now it is known which class holds most rows
     third = _loop("spmv", group=False).last_launch
-    assert len(third.sequence) == 6 and third.bin["base"] == int(np.argmax(np.bincount(np.digitize(lengths, [4, 32, 128], right=True), minlength=4)))
-    ok, worst = vo.within_budget(y2, ref, budget, TOL)
-    assert ok, worst
+    assert len(third.sequence) == 6 and third.bin["base"] == int(np.argmax(np.bincount(np.digitize(lengths, [4, 32, 256], right=True), minlength=4)))
+    assert np.array_equal(y1, y2)
 
 
 def test_spmv_columns_crowded_into_one_stripe(k):
@@ -212,7 +215,7 @@ def test_more_long_rows_than_the_streamed_arrays_account_for(k):
     indices = np.sort(rng.integers(0, n, nnz)).astype(np.int32)
     x = rng.standard_normal(n, dtype=np.float32)
 
-    @appy.jit
+    @appy.jit(hip_group=False)
     def windows(data, start, length, indices, x, y, m):
         #pragma parallel for
         for i in range(m):
@@ -226,7 +229,7 @@ def test_more_long_rows_than_the_streamed_arrays_account_for(k):
 
     y = np.empty(m, dtype=np.float32)
     windows(data, start, length, indices, x, y, m)
-    launch = _loop("windows").last_launch
+    launch = _loop("windows", group=False).last_launch
     assert len(launch.sequence) == 6
     assert launch.sequence is not None and launch.bin["cap"] < int((length > launch.bin["threshold"][2]).sum())
     terms = data.astype(np.float64) * x.astype(np.float64)[indices]

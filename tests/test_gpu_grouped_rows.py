@@ -1,7 +1,8 @@
 """Loops over short rows that sum terms gathered from an operand larger than an L2 (CSR SpMV with
-a few to a hundred elements per row): from their second launch on, the elements of every 256 rows
-are grouped by the stripe of the operand they read, the groups run with one stripe per XCD, and the
-sums of a row are added up afterwards.  Every result is compared with the float64 oracle to the bar
+a few to a hundred elements per row): the elements of every 256 rows are grouped by the stripe of the
+operand they read, the groups run with one stripe per XCD, and the sums of a row are added up
+afterwards.  The form of a launch follows from the sizes of its arrays; what the launch before it
+reported about the rows only leaves out kernels that would run empty, and never changes a bit of the result.  Every result is compared with the float64 oracle to the bar
 of the parity tests (``|out - oracle| <= 1e-5 * sum(|terms|)`` per output).
 
 Pattern: the CSR loop of the reference's examples/03-spmv.py:5-16 and
@@ -25,9 +26,17 @@ def k(gpu):
     return selfcheck.kernels()
 
 
-def _loop(name, index_type="int32"):
+FULL = ["clear", "bins", "group", "cells", "sums", "plan", "parts", "fold", "rowwise"]
+
+
+def _steps(launch):
+    return [step[0].src.name.rsplit("_", 1)[-1] if step[0] else "clear" for step in (launch.sequence or [])]
+
+
+def _loop(name, index_type="int32", reuse=True):
     hits = [v[0] for kk, v in cg.code_cache.items() if kk[-1] == name and v[0].options.get("hip_bins", True)
             and v[0].options.get("hip_group", True) and getattr(v[0], "last_launch", None) is not None
+            and bool(v[0].options.get("hip_reuse", True)) == reuse
             and (name != "spmv" or ("A_indptr" in v[0].analysis.arrays and v[0].analysis.arrays["A_indptr"].ty.name == index_type
                                    and v[0].analysis.arrays["x"].ty.name == "float32"))]
     return max(hits, key=lambda lp: lp.last_launch.serial if getattr(lp, "last_launch", None) is not None else -1)
@@ -69,7 +78,7 @@ def _matrix(lengths, n, seed):
     (33_000, 7 << 20, "8"),                  # sixteen stripes, two per XCD
     (36_000, 1 << 21, "1..127"),             # rows of the three classes that qualify
 ])
-def test_short_rows_are_grouped_from_the_second_launch_on(k, m, n, lengths):
+def test_short_rows_are_grouped_and_earlier_launches_change_no_bit(k, m, n, lengths):
     rng = np.random.default_rng(m)
     if lengths == "0,10,20":
         ln = rng.integers(0, 3, m) * 10
@@ -83,24 +92,24 @@ def test_short_rows_are_grouped_from_the_second_launch_on(k, m, n, lengths):
     _forget()
     y0 = k.spmv(data, indptr, indices, x, m, n)
     first = _loop("spmv").last_launch
-    assert first.spec.rows == "mixed"                       # nothing known about the rows yet: sorted by length
+    # nothing is believed about the rows yet: grouped, with the kernels for rows beyond the limit set up as well
+    assert _grouped(first) and _steps(first) == FULL and first.nsplit == (16 if n > (8 << 19) else 8)
     ok, worst = vo.within_budget(y0, ref, budget, TOL)
     assert ok, worst
     y1 = k.spmv(data, indptr, indices, x, m, n)
     second = _loop("spmv").last_launch
-    assert _grouped(second) and second.nsplit == (16 if n > (8 << 19) else 8)
-    assert [step[0].src.spec.aux if step[0] else "clear" for step in second.sequence] == ["clear", "group", "cells", "", ""]
-    ok, worst = vo.within_budget(y1, ref, budget, TOL)
-    assert ok, worst
+    # the first launch found no row beyond the limit: the kernels that would run empty are left out
+    assert _grouped(second) and _steps(second) == ["clear", "group", "cells", "sums", "rowwise"]
     assert np.all(y1[ln == 0] == 0.0)
-    # the same launch again gives the same bits: the order of the additions does not depend on timing
+    # the same bits from the first launch on: neither what earlier launches reported nor timing changes the order
+    # in which the terms of a row are added
+    assert np.array_equal(y0, y1)
     assert np.array_equal(y1, k.spmv(data, indptr, indices, x, m, n))
 
 
 def test_matrices_with_long_rows_group_their_short_rows_and_cut_the_long_ones(k):
-    """The form of a launch follows what the last launch reported.  Rows longer than it was told of are
-    still summed correctly (and reported); once the rows have been sorted again, the elements of the short
-    rows are grouped and the long rows run in parts cut at the stripes, in one launch."""
+    """What a launch reported is believed only by a launch over the same arrays.  Rows of up to 512 elements have
+    their elements grouped, longer rows run in parts cut at the stripes, in one launch, from the first launch on."""
     m, n = 40_000, 1 << 20
     short = _matrix(np.full(m, 12), n, seed=1)
     rng = np.random.default_rng(2)
@@ -112,31 +121,46 @@ def test_matrices_with_long_rows_group_their_short_rows_and_cut_the_long_ones(k)
     launch = _loop("spmv").last_launch
     assert _grouped(launch) and len(launch.sequence) == 5
     ref, budget = vo.spmv_csr(*long_, (m, n))
-    y = k.spmv(*long_, m, n)
-    launch = _loop("spmv").last_launch
-    assert _grouped(launch) and len(launch.sequence) == 5   # shaped by the report on the short rows
-    ok, worst = vo.within_budget(y, ref, budget, TOL)
-    assert ok, worst
-    y = k.spmv(*long_, m, n)
-    assert _loop("spmv").last_launch.spec.rows == "mixed"   # the grouping kernel has seen the long rows
-    ok, worst = vo.within_budget(y, ref, budget, TOL)
-    assert ok, worst
-    for _ in range(2):
+    results = []
+    for _ in range(3):
         y = k.spmv(*long_, m, n)
         launch = _loop("spmv").last_launch
-        assert _grouped(launch)
-        names = [step[0].src.name.rsplit("_", 1)[-1] if step[0] else "clear" for step in launch.sequence]
-        assert names == ["clear", "bins", "group", "cells", "sums", "plan", "parts", "fold", "rowwise"], names
+        assert _grouped(launch) and _steps(launch) == FULL       # other arrays: the report on the short rows is not theirs
         cut = launch.bin["rowmax"]
         assert cut == 512 and (ln > cut).sum() > 100 and (ln <= cut).sum() > 100
         ok, worst = vo.within_budget(y, ref, budget, TOL)
         assert ok, worst
-    # and back: a matrix of short rows after one with long rows (the lists of long rows are empty)
+        results.append(y)
+    assert np.array_equal(results[0], results[1]) and np.array_equal(results[1], results[2])
+    # and back: the matrix of short rows after the one with long rows
     ref, budget = vo.spmv_csr(*short, (m, n))
     y = k.spmv(*short, m, n)
     assert len(_loop("spmv").last_launch.sequence) == 9
     ok, worst = vo.within_budget(y, ref, budget, TOL)
     assert ok, worst
+    assert np.array_equal(y, k.spmv(*short, m, n)) and len(_loop("spmv").last_launch.sequence) == 5
+
+
+def test_longest_rows_just_below_and_above_the_limit_settle_on_one_form(k):
+    """One limit decides between grouped and cut rows in every form of the launch: a matrix whose longest rows
+    hold 257..512 elements (or 513..600) takes the same form, with the same bits, from its second launch on."""
+    m, n = 40_000, 1 << 20
+    for longest, steps in ((300, 5), (512, 5), (600, 9)):
+        rng = np.random.default_rng(longest)
+        ln = rng.integers(1, 20, m)
+        ln[::97] = longest
+        data, indptr, indices, x = _matrix(ln, n, seed=longest + 1)
+        ref, budget = vo.spmv_csr(data, indptr, indices, x, (m, n))
+        _forget()
+        seen, ys = [], []
+        for _ in range(5):
+            ys.append(k.spmv(data, indptr, indices, x, m, n))
+            seen.append(len(_loop("spmv").last_launch.sequence))
+            assert _grouped(_loop("spmv").last_launch)
+        assert seen == [9, steps, steps, steps, steps], (longest, seen)
+        assert all(np.array_equal(ys[0], y) for y in ys[1:]), longest
+        ok, worst = vo.within_budget(ys[-1], ref, budget, TOL)
+        assert ok, worst
 
 
 def test_rows_of_every_length_around_the_cut(k):
@@ -151,7 +175,7 @@ def test_rows_of_every_length_around_the_cut(k):
     data, indptr, indices, x = _matrix(ln, n, seed=15)
     ref, budget = vo.spmv_csr(data, indptr, indices, x, (m, n))
     _forget()
-    tags = []
+    tags, ys = [], []
     for _ in range(3):
         y = k.spmv(data, indptr, indices, x, m, n)
         launch = _loop("spmv").last_launch
@@ -159,7 +183,9 @@ def test_rows_of_every_length_around_the_cut(k):
         ok, worst = vo.within_budget(y, ref, budget, TOL)
         assert ok, worst
         assert np.all(y[ln == 0] == 0.0)
-    assert tags == [0, 9, 9]
+        ys.append(y)
+    assert tags == [9, 9, 9]
+    assert np.array_equal(ys[0], ys[1]) and np.array_equal(ys[1], ys[2])
 
 
 @pytest.mark.parametrize("with_long_rows", [False, True])
@@ -199,7 +225,7 @@ def test_blocks_whose_elements_end_on_step_boundaries(k, with_long_rows):
     data, indptr, indices, x = _matrix(ln, n, seed=32)
     ref, budget = vo.spmv_csr(data, indptr, indices, x, (m, n))
     _forget()
-    forms = []
+    forms, ys = [], []
     for _ in range(3):
         y = k.spmv(data, indptr, indices, x, m, n)
         launch = _loop("spmv").last_launch
@@ -207,7 +233,9 @@ def test_blocks_whose_elements_end_on_step_boundaries(k, with_long_rows):
         ok, worst = vo.within_budget(y, ref, budget, TOL)
         assert ok, (forms, worst)
         assert np.all(y[ln == 0] == 0.0)
-    assert forms == ([0, 9, 9] if with_long_rows else [0, 5, 5])
+        ys.append(y)
+    assert forms == ([9, 9, 9] if with_long_rows else [9, 5, 5])
+    assert np.array_equal(ys[0], ys[1]) and np.array_equal(ys[1], ys[2])
 
 
 def test_row_ranges_that_do_not_follow_one_another_run_row_by_row(gpu):
@@ -232,8 +260,8 @@ def test_row_ranges_that_do_not_follow_one_another_run_row_by_row(gpu):
 
     start, end = indptr[:-1].copy(), indptr[1:].copy()
     _forget("windows")
-    run(start, end, expect_grouped=False)       # first launch: rows sorted by length
-    run(start, end)                             # a CSR matrix in two arrays: grouped
+    run(start, end)                             # a CSR matrix in two arrays: grouped, from the first launch on
+    run(start, end)
     # two rows swapped: ranges out of order
     s2, e2 = start.copy(), end.copy()
     s2[[1000, 1001]] = s2[[1001, 1000]]
@@ -274,7 +302,7 @@ def test_refused_ranges_in_a_launch_that_also_cuts_long_rows(gpu):
         assert np.all(np.abs(y - ref) <= TOL * budget + 1e-9 * ca[-1]), np.max(np.abs(y - ref))
 
     _forget("windows")
-    run(start, end, 0)
+    run(start, end, 9)
     run(start, end, 9)
     long_row = int(np.flatnonzero(ln > 600)[5])
     s2, e2 = start.copy(), end.copy()
@@ -337,7 +365,7 @@ def test_terms_with_a_scalar_factor_integer_values_and_no_second_operand(gpu):
         for launch_no in range(2):
             y = np.zeros(m, dtype=dtype)
             call(y)
-            assert _grouped(_loop(name).last_launch) == (launch_no == 1), name
+            assert _grouped(_loop(name).last_launch), name
             if dtype is np.int32:
                 assert np.array_equal(y, ref.astype(np.int64)), name
             else:
@@ -394,11 +422,11 @@ def test_loops_that_do_not_qualify_keep_their_rows_sorted(k):
 
 
 def test_grouped_launches_on_gpu_tensors_follow_changes_of_the_matrix(gpu):
-    """Nothing about the matrix is kept between launches: the same tensors with other contents give the
-    other matrix's product."""
+    """With `hip_reuse=False` nothing about the matrix is kept between launches: the same tensors with other
+    contents give the other matrix's product."""
     import torch
 
-    k = selfcheck.kernels()
+    k = selfcheck.kernels(hip_reuse=False)
     m, n = 60_000, 1 << 20
     a = _matrix(np.full(m, 16), n, seed=11)
     b = _matrix(np.full(m, 16), n, seed=13)
@@ -406,13 +434,13 @@ def test_grouped_launches_on_gpu_tensors_follow_changes_of_the_matrix(gpu):
     _forget()
     for _ in range(2):
         y = k.spmv(*d, m, n)
-    assert _grouped(_loop("spmv").last_launch)
+    assert _grouped(_loop("spmv", reuse=False).last_launch)
     ref, budget = vo.spmv_csr(*a, (m, n))
     assert vo.within_budget(y.cpu().numpy(), ref, budget, TOL)[0]
     for t, v in zip(d, b):
         t.copy_(torch.from_numpy(v))
     y = k.spmv(*d, m, n)
-    assert _grouped(_loop("spmv").last_launch)
+    assert _grouped(_loop("spmv", reuse=False).last_launch)
     ref, budget = vo.spmv_csr(*b, (m, n))
     ok, worst = vo.within_budget(y.cpu().numpy(), ref, budget, TOL)
     assert ok, worst
@@ -442,8 +470,9 @@ def test_larger_blocks_of_rows(gpu, rows_per_block):
 
 
 def test_launches_recorded_into_a_graph_keep_their_rows_sorted(gpu):
-    """The grouped form clears a flag with a memory-set node; recorded launches use the kernels over sorted
-    rows instead, and every replay follows the contents of the tensors."""
+    """The grouped form clears a flag with a memory-set node, and a kept order of the elements would be that of
+    the values at the time of the recording; recorded launches use the kernels over sorted rows instead, and
+    every replay follows the contents of the tensors."""
     import torch
 
     k = selfcheck.kernels()
@@ -463,16 +492,17 @@ def test_launches_recorded_into_a_graph_keep_their_rows_sorted(gpu):
             y[i] = s
 
     _forget("spmv_into")
-    for _ in range(2):
-        spmv_into(*d, y, m)
+    spmv_into(*d, y, m)
     assert _grouped(_loop("spmv_into").last_launch)
+    spmv_into(*d, y, m)
+    assert _loop("spmv_into").last_launch.plan is not None      # GPU tensors seen twice: their order is kept
     with appy.graph() as g:
         spmv_into(*d, y, m)
     assert _loop("spmv_into").last_launch.spec.rows == "mixed"
     for replay in range(3):
         d[0].mul_(1.5)
         y.zero_()
-        spmv_into(*d, torch.empty_like(y), m)             # eager (grouped) launches between the replays
+        spmv_into(*d, torch.empty_like(y), m)             # eager launches between the replays
         g.launch()
         g.synchronize()
         ref, budget = vo.spmv_csr(d[0].cpu().numpy(), a[1], a[2], a[3], (m, n))
