@@ -493,6 +493,15 @@ class LoopAnalysis:
         if not any(isinstance(n, ast.Name) and (n.id in self.assigned or n.id == self.var)
                    for b in (lo, hi) for n in ast.walk(b)):
             return None
+        # the sorting kernel and the kernels that run the rows each evaluate the set-up and the bounds of a row;
+        # a body that stores to an array they read (`ln[i] = 0` after a loop over `range(ln[i])`) would have a
+        # row that has run already classified anew, and run again
+        body = self.outer.body
+        at = next(k for k, st in enumerate(body) if st is loop)
+        read_first = {n.id for st in body[:at] for n in ast.walk(st) if isinstance(n, ast.Name)}
+        read_first |= {n.id for b in (lo, hi) for n in ast.walk(b) if isinstance(n, ast.Name)}
+        if read_first & set(self.stored):
+            return None
         jv = loop.target.id
         pairs = set()
         for n in ast.walk(loop):

@@ -729,7 +729,7 @@ int appy_hip_launch_static_scratch(void* func,
     if (!func) return fail_arg("func is NULL");
     if (!args || args_bytes == 0) return fail_arg("args is NULL or empty");
     if (args_bytes > kMaxArgs) return fail_arg("argument block larger than 4096 bytes");
-    if (scratch_arg_offset % alignof(void*) || scratch_arg_offset + sizeof(void*) > args_bytes)
+    if (scratch_arg_offset % alignof(void*) || args_bytes < sizeof(void*) || scratch_arg_offset > args_bytes - sizeof(void*))
         return fail_arg("scratch_arg_offset does not name a pointer inside the argument block");
     if (scratch_bytes > APPY_HIP_STATIC_SCRATCH_BYTES)
         return fail_arg("scratch_bytes exceeds APPY_HIP_STATIC_SCRATCH_BYTES (the static scratch buffer holds 8 MiB)");

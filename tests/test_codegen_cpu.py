@@ -775,3 +775,49 @@ def test_simd_loops_of_a_wavefront_team_are_fenced_when_they_touch_stored_arrays
            "    t = 0.0\n    #pragma simd\n    for j in range(m):\n        t += B[i, j] * B[i, j]\n    y[i] = s * t\n")
     g, _ = compiled(src, B=A, y=np.zeros(23), n=23, m=61)
     assert "wave_fence();" not in body_of(g.kernel_for(Spec("team", block=256, vec=2, width=16)).src.text)
+
+
+def test_rows_whose_bounds_read_what_the_body_stores_are_not_sorted_by_length():
+    """`for j in range(ln[i]): ...; ln[i] = 0` is a legal loop, but the kernels over sorted rows evaluate the bounds
+    of a row more than once: such a nest keeps one team width for all rows."""
+    ln = np.zeros(8, np.int32)
+    v = np.zeros(64, np.float32)
+    y = np.zeros(8, np.float32)
+    src = ("#pragma parallel for\nfor i in range(m):\n    s = 0.0\n    #pragma simd\n    for j in range(ln[i]):\n"
+           "        s += v[i * 8 + j]\n    y[i] = s\n")
+    f, _ = compiled(src, ln=ln, v=v, y=y, m=8)
+    assert f.analysis.ragged is not None
+    g, _ = compiled(src + "    ln[i] = 0\n", ln=ln, v=v, y=y, m=8)
+    assert g.analysis.team_split is not None and g.analysis.ragged is None
+    assert g.choose_spec(1 << 20, {"m": 1 << 20}, {"v": v}).rows == ""
+
+
+def test_row_plans_kernel_that_writes_the_pairs_and_kernel_that_runs_a_plan():
+    """The two generated kernels of the kept order of elements: one (key, value) pair per element with the
+    checks that make an inspector refuse its input; tiles of products dropped into row-sorted slots in LDS and
+    added to per-row sums without atomics, every load issued from a scalar base plus a fixed lane offset."""
+    f, _ = selfcheck_loop("spmv")
+    keys = body_of(f.kernel_for(Spec("team", block=256, vec=1, width=64, aux="rkeys", block_rows=256)).src.text)
+    assert "__lp[__r + 1] == __hq[__r]" in keys and "__flag[0] = 1" in keys
+    assert "if (__cq < 0 || __cq >= __nx) { __inside = false; continue; }" in keys
+    assert "__keys[__j + __q] = ((__rel >> 15) << __lbits) | ((unsigned)__cq >> 5);" in keys
+    assert "x[" not in keys.split("{", 1)[1]                                  # the gathered operand is not read here
+    for unroll, tile in ((6, 6144), (4, 4096)):
+        run = body_of(f.kernel_for(Spec("team", block=1024, vec=1, width=1024, unroll=unroll, parts=8, aux="xcells")).src.text)
+        assert f"__shared__ float __sum[32768];" in run and f"__prod[{tile}];" in run
+        assert "atomicAdd" not in run and run.count("__syncthreads();") >= 4
+        assert "(__cv * __cx)" in run and "A_indptr[" not in run.split("{", 1)[1] and "A_indices[" not in run.split("{", 1)[1]
+        assert "__builtin_amdgcn_readfirstlane" in run
+    with pytest.raises(ValueError):
+        Spec("team", block=1024, vec=1, width=1024, unroll=8, parts=8, aux="xcells")
+    # the shape of a plan for the benchmark's matrices: 128 blocks of rows x 8 column ranges, 19 bits of column, tiles of 6144
+    arrays = {"A_data": np.broadcast_to(np.float32(0), (16 << 22,)), "A_indices": np.broadcast_to(np.int32(0), (16 << 22,)),
+              "A_indptr": np.broadcast_to(np.int32(0), ((1 << 22) + 1,)), "x": np.broadcast_to(np.float32(0), (1 << 22,))}
+    shape = f.plan_shape(1 << 22, {"M": 1 << 22}, arrays)
+    assert (shape.row_blocks, shape.groups, shape.group_width, shape.col_bits, shape.tile, shape.line_bits) == (128, 8, 1 << 19, 19, 6144, 17)
+    assert f.plan_arrays() == ["A_indptr", "A_indices", "A_data"]
+    arrays["x"] = np.broadcast_to(np.float32(0), (7 << 20,))
+    shape = f.plan_shape(1 << 22, {"M": 1 << 22}, arrays)
+    assert (shape.col_bits, shape.tile) == (20, 4096)
+    arrays["x"] = np.broadcast_to(np.float32(0), (1 << 19,))                  # an operand that every L2 holds anyway
+    assert f.plan_shape(1 << 22, {"M": 1 << 22}, arrays) is None

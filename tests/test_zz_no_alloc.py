@@ -111,3 +111,7 @@ def test_requests_beyond_the_static_buffer_are_refused(gpu):
                                               C.sizeof(launch.args), C.sizeof(launch.args), 64) != 0
     assert lib.appy_hip_launch_static_scratch(None, 1, 1, 1, 64, 1, 1, 0, None, C.byref(launch.args),
                                               C.sizeof(launch.args), off, 64) != 0
+    # offsets near the top of the address range, which wrap around when the size of a pointer is added to them
+    for wrap in (2 ** 64 - 8, 2 ** 64 - 16):
+        assert lib.appy_hip_launch_static_scratch(launch.function(), g[0], 1, 1, b[0], 1, 1, 0, None, C.byref(launch.args),
+                                                  C.sizeof(launch.args), C.c_size_t(wrap), 64) != 0
