@@ -323,6 +323,21 @@ class RowPlan:
                 _live_plans.remove(self)
 
 
+# Page-locked slots with device memory of their own for host arrays of a few bytes (`shared()` scalars):
+# (host address, device address) pairs, handed out per launch, per device.
+_SMALL_SLOT_BYTES = 64
+_small_free = {}
+_small_lock = threading.Lock()
+
+
+def _take_small_slot(device):
+    with _small_lock:
+        free = _small_free.get(device)
+        if free:
+            return free.pop()
+    return (rt.host_alloc(_SMALL_SLOT_BYTES), rt.malloc(256))
+
+
 _live_plans = []        # every valid plan of the process: launches that store into their arrays drop them
 _plans_lock = threading.Lock()
 
@@ -1088,6 +1103,7 @@ class Launch:
         self.sequence = None
         self.bin = None
         self.plan = None         # the row plan this launch runs, if any
+        self.small = []          # (slot, host ndarray, stored, name): arrays of a few bytes staged through page-locked slots
         try:
             self._stage(vals, arrays)
         except BaseException:
@@ -1095,6 +1111,7 @@ class Launch:
             for dptr, *_ in self.temps:
                 rt.free(dptr)
             self.temps = []
+            self._return_small_slots(wait=True)
             if self.oob:
                 rt.free(self.oob)
                 self.oob = 0
@@ -1177,6 +1194,8 @@ class Launch:
                 self._stage_host(name, host, v if tc is v else ("tensor", v, tc), arr.stored)
         for dptr, host, _orig, stored, name in self.temps:
             extents.append((name, dptr, host.nbytes, stored))
+        for slot, host, stored, name in self.small:
+            extents.append((name, slot[1], host.nbytes, stored))
         extents.extend(self.aliases)
         for _m, dptr, host, stored, name in self.mirrored:
             extents.append((name, dptr, host.nbytes, stored))
@@ -1688,6 +1707,24 @@ class Launch:
     def _stage_host(self, name, host, original, stored):
         nbytes = host.nbytes
         hit = residency.lookup(host.ctypes.data, nbytes) if (residency.active() and original is host) else None
+        if hit is None and 0 < nbytes <= _SMALL_SLOT_BYTES and self.capture is None and original is host:
+            # the one-element buffers of `shared()` scalars, and other arrays of a few bytes: through a page-locked
+            # slot that owns device memory - a small DMA each way, nothing allocated, nothing moved through the
+            # driver's path for pageable memory (which costs some 50 us per copy whatever its size)
+            for k, (slot, host0, stored0, name0) in enumerate(self.small):
+                if host0.ctypes.data == host.ctypes.data and host0.nbytes == nbytes:
+                    # the same array under a second name: one device copy serves both
+                    self.small[k] = (slot, host0, stored0 or stored, name0)
+                    self.aliases.append((name, slot[1], nbytes, stored))
+                    break
+            else:
+                slot = _take_small_slot(self.device)
+                C.memmove(slot[0], host.ctypes.data, nbytes)
+                rt.memcpy_h2d_async(slot[1], slot[0], nbytes, self.stream)
+                self.small.append((slot, host, stored, name))
+            self.ptr[name] = slot[1]
+            self.strides[name] = [s // host.itemsize for s in host.strides]
+            return
         if hit is not None:
             # the array (or the array this is a view of) has a standing mirror in HBM
             m, off = hit
@@ -1699,7 +1736,9 @@ class Launch:
                 if m.host_dirty:
                     m.upload(self.stream)
             elif nbytes and not (stored and self.loop.overwrites(name, self.lo, self.hi, self.env, host.shape)):
-                rt.memcpy_h2d(m.device_ptr() + off, host.ctypes.data, nbytes, self.stream)
+                # (from page-locked memory the upload is queued, not waited for: `finish` waits for the stream before
+                #  the caller can touch the host bytes again)
+                (rt.memcpy_h2d_async if m.pinned else rt.memcpy_h2d)(m.device_ptr() + off, host.ctypes.data, nbytes, self.stream)
             dptr = m.device_ptr() + off
             self.mirrored.append((m, dptr, host, stored, name))
             self.ptr[name] = dptr
@@ -1731,7 +1770,7 @@ class Launch:
 
     def replayable(self) -> bool:
         """True if nothing but the kernel launch happens when this call is repeated."""
-        return not (self.temps or self.mirrored or self.keepalive_copies or self.oob or self.capture is not None
+        return not (self.temps or self.mirrored or self.small or self.keepalive_copies or self.oob or self.capture is not None
                     or self.second is not None or self.sequence is not None)
 
     def _no_capture(self, name, why):
@@ -1812,6 +1851,14 @@ class Launch:
                     elif original is not host and is_numpy_array(original):
                         original[...] = host
             waited = bool(self.temps)
+            for slot, host, stored, _name in self.small:
+                if stored:
+                    rt.memcpy_d2h(slot[0], slot[1], host.nbytes, self.stream)       # one DMA; waits for the stream
+                    C.memmove(host.ctypes.data, slot[0], host.nbytes)
+                    waited = True
+            if self.small and not waited:
+                rt.sync(self.stream)        # the uploads must have left the slots before they are used again
+                waited = True
             for m, dptr, host, stored, _name in self.mirrored:
                 if m.resident:
                     m.stream, m.busy = self.stream, True
@@ -1836,6 +1883,19 @@ class Launch:
             self.temps = []
             self.mirrored = []
             self.keepalive = []
+            self._return_small_slots(wait=False)
+
+    def _return_small_slots(self, wait):
+        slots, self.small = [entry[0] for entry in self.small], []
+        if not slots:
+            return
+        if wait:
+            try:
+                rt.sync(self.stream)
+            except Exception:
+                pass
+        with _small_lock:
+            _small_free.setdefault(self.device, []).extend(slots)
 
     def run(self):
         try:
@@ -1844,6 +1904,7 @@ class Launch:
             for dptr, *_ in self.temps:
                 rt.free(dptr)
             self.temps = []
+            self._return_small_slots(wait=True)
             if self.oob:
                 rt.free(self.oob)
                 self.oob = 0

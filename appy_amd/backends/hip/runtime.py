@@ -85,6 +85,7 @@ SIGNATURES = {
     "appy_hip_pool_stats": (C.c_int, [C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
     "appy_hip_memcpy_h2d": (C.c_int, [_vp, _vp, C.c_size_t, _vp]),
     "appy_hip_memcpy_d2h": (C.c_int, [_vp, _vp, C.c_size_t, _vp]),
+    "appy_hip_memcpy_h2d_async": (C.c_int, [_vp, _vp, C.c_size_t, _vp]),
     "appy_hip_host_alloc": (C.c_int, [C.c_size_t, C.POINTER(_vp)]),
     "appy_hip_host_free": (C.c_int, [_vp]),
     "appy_hip_host_is_pinned": (C.c_int, [_vp, C.c_size_t]),
@@ -268,6 +269,11 @@ def free(dptr: int) -> None:
 
 def memcpy_h2d(dst: int, src_host_ptr: int, nbytes: int, stream: int = 0) -> None:
     check(lib().appy_hip_memcpy_h2d(_vp(dst), _vp(src_host_ptr), int(nbytes), _vp(stream)))
+
+
+def memcpy_h2d_async(dst: int, src_pinned_ptr: int, nbytes: int, stream: int = 0) -> None:
+    """Upload from page-locked memory that returns once it is queued on ``stream``."""
+    check(lib().appy_hip_memcpy_h2d_async(_vp(dst), _vp(src_pinned_ptr), int(nbytes), _vp(stream)))
 
 
 def memcpy_d2h(dst_host_ptr: int, src: int, nbytes: int, stream: int = 0) -> None:

@@ -627,6 +627,15 @@ int appy_hip_memcpy_h2d(void* dst_dev, const void* src_host, size_t nbytes, void
     return 0;
 }
 
+int appy_hip_memcpy_h2d_async(void* dst_dev, const void* src_pinned, size_t nbytes, void* stream) {
+    if (nbytes == 0) return 0;
+    if (!dst_dev || !src_pinned) return fail_arg("dst_dev/src_pinned is NULL");
+    if (!host_blocks().contains(src_pinned, nbytes))
+        return fail_arg("asynchronous uploads take memory from appy_hip_host_alloc only");
+    HIP_TRY(hipMemcpyAsync(dst_dev, src_pinned, nbytes, hipMemcpyHostToDevice, static_cast<hipStream_t>(stream)));
+    return 0;
+}
+
 int appy_hip_memcpy_d2h(void* dst_host, const void* src_dev, size_t nbytes, void* stream) {
     if (nbytes == 0) return 0;
     if (!dst_host || !src_dev) return fail_arg("dst_host/src_dev is NULL");

@@ -25,7 +25,7 @@ extern "C" {
 #endif
 
 /* 2: page-locked host memory, streams and graphs, appy_hip_rtc_version; 3: appy_hip_launch_static_scratch;
- * 4: row plans (appy_hip_rowplan_*), appy_hip_device_sync
+ * 4: row plans (appy_hip_rowplan_*), appy_hip_device_sync, appy_hip_memcpy_h2d_async
  * (additions only: every entry point of the earlier versions is unchanged). */
 #define APPY_HIP_ABI_VERSION 4
 
@@ -111,6 +111,10 @@ int appy_hip_pool_stats(uint64_t* bytes_in_use_out, uint64_t* bytes_cached_out);
  * finished (set APPY_HIP_NO_STAGING=1 to use the driver's pageable path). */
 int appy_hip_memcpy_h2d(void* dst_dev, const void* src_host, size_t nbytes, void* stream);
 int appy_hip_memcpy_d2h(void* dst_host, const void* src_dev, size_t nbytes, void* stream);
+/* Upload from page-locked memory (appy_hip_host_alloc; anything else is refused) that returns once the copy is
+ * queued on `stream`: the caller leaves the host bytes alone until it has waited for the stream.  Used for the
+ * one-element buffers of `shared()` scalars (appy/frontend/process_shared.py:27-53), which travel with every launch. */
+int appy_hip_memcpy_h2d_async(void* dst_dev, const void* src_pinned, size_t nbytes, void* stream);
 /* Page-locked host memory for arrays that travel often.  Replaces the device-
  * visible buffers behind the reference's shared NumPy arrays
  * (`device.buffer(n)` + `np.frombuffer`, appy/np_shared.py:11-17): on a
