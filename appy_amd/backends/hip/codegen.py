@@ -468,11 +468,14 @@ class CompiledLoop:
     def _indexed_arrays(self):
         """name -> element size of the arrays that are indexed by a variable (the
         candidates for wide loads); reduction targets like ``s[0]`` do not count."""
-        found = {}
-        for n in ast.walk(self.analysis.outer):
-            if (isinstance(n, ast.Subscript) and isinstance(n.value, ast.Name)
-                    and n.value.id in self.analysis.arrays and not isinstance(n.slice, ast.Constant)):
-                found[n.value.id] = self.analysis.arrays[n.value.id].ty.size
+        found = self.__dict__.get("_indexed_cache")
+        if found is None:       # (the loop does not change: walked once)
+            found = {}
+            for n in ast.walk(self.analysis.outer):
+                if (isinstance(n, ast.Subscript) and isinstance(n.value, ast.Name)
+                        and n.value.id in self.analysis.arrays and not isinstance(n.slice, ast.Constant)):
+                    found[n.value.id] = self.analysis.arrays[n.value.id].ty.size
+            self._indexed_cache = found
         return found
 
     def _elem_sizes(self):
@@ -996,7 +999,27 @@ class CompiledLoop:
                 # same tensors (address, shape, strides), same scalars, same stream: the staged
                 # launch of last time is still exact, so only the launch itself is repeated
                 _ensure_device(plan.device)
-                if self._value_only:
+                if plan.small_fixed:
+                    # host arrays of a few bytes (`shared()` scalars): through the slots the plan keeps for them
+                    with self._lock:        # the slots and the argument block are shared by all replays of this plan
+                        for slot, i, nbytes, _stored in plan.small_fixed:
+                            C.memmove(slot[0], args[i].ctypes.data, nbytes)
+                            rt.memcpy_h2d_async(slot[1], slot[0], nbytes, plan.stream)
+                        for i in self._value_only:
+                            fname = plan.scalar_fields.get(self.arg_names[i])
+                            if fname is not None:
+                                v = args[i]
+                                setattr(plan.args, fname, v.item() if isinstance(v, np.generic) else v)
+                        rt.launch(plan.function(), plan.grid, plan.block, plan.args, plan.stream)
+                        waited = False
+                        for slot, i, nbytes, stored in plan.small_fixed:
+                            if stored:
+                                rt.memcpy_d2h(slot[0], slot[1], nbytes, plan.stream)
+                                C.memmove(args[i].ctypes.data, slot[0], nbytes)
+                                waited = True
+                        if not waited:
+                            rt.sync(plan.stream)
+                elif self._value_only:
                     with self._lock:        # the argument block is shared by all replays of this plan
                         for i in self._value_only:
                             fname = plan.scalar_fields.get(self.arg_names[i])
@@ -1012,14 +1035,20 @@ class CompiledLoop:
         plan = self.prepare(vals)
         if plan is None:
             return
+        plan.keep_small = key is not None
         plan.run()
         if key is not None and plan.replayable():
+            plan.small_fixed = [(slot, self.arg_names.index(name), host.nbytes, stored) for slot, host, stored, name in plan.small_kept]
+            plan.small_kept = []
             with self._lock:        # launches may come from several interpreter threads
                 if len(self._replays) >= REPLAY_CACHE_ENTRIES:
                     # drop the older half (dicts keep insertion order)
                     for old in list(self._replays)[:REPLAY_CACHE_ENTRIES // 2]:
                         self._replays.pop(old, None)
                 self._replays[key] = plan
+        elif plan.small_kept:
+            plan.small, plan.small_kept = plan.small_kept, []
+            plan._return_small_slots(wait=False)
 
     def overwrites(self, name, lo, hi, env, shape) -> bool:
         """True if this launch stores every element of array ``name`` (so that its
@@ -1053,6 +1082,8 @@ class CompiledLoop:
                     return None
                 device = v.device.index or 0
                 key.append((v.data_ptr(), v.shape, v.stride()))
+            elif t is np.ndarray and 0 < v.nbytes <= _SMALL_SLOT_BYTES and v.flags["C_CONTIGUOUS"] and not residency.active():
+                key.append(("small", v.dtype.str, v.shape))      # travels through a slot of the plan at every call
             else:
                 return None
         if device < 0:
@@ -1104,6 +1135,9 @@ class Launch:
         self.bin = None
         self.plan = None         # the row plan this launch runs, if any
         self.small = []          # (slot, host ndarray, stored, name): arrays of a few bytes staged through page-locked slots
+        self.keep_small = False  # the slots stay with this launch when it is kept for repeats of the call
+        self.small_kept = []
+        self.small_fixed = []    # a launch kept for repeats: (slot, argument number, bytes, stored)
         try:
             self._stage(vals, arrays)
         except BaseException:
@@ -1770,7 +1804,7 @@ class Launch:
 
     def replayable(self) -> bool:
         """True if nothing but the kernel launch happens when this call is repeated."""
-        return not (self.temps or self.mirrored or self.small or self.keepalive_copies or self.oob or self.capture is not None
+        return not (self.temps or self.mirrored or self.aliases or self.keepalive_copies or self.oob or self.capture is not None
                     or self.second is not None or self.sequence is not None)
 
     def _no_capture(self, name, why):
@@ -1886,6 +1920,9 @@ class Launch:
             self._return_small_slots(wait=False)
 
     def _return_small_slots(self, wait):
+        if self.keep_small and not wait:
+            self.small_kept, self.small = self.small, []
+            return
         slots, self.small = [entry[0] for entry in self.small], []
         if not slots:
             return

@@ -234,3 +234,53 @@ def test_affine_subscripts_of_the_parallel_variable_are_checked_on_the_host(gpu)
         from_the_end(a, out, 100)
     with pytest.raises(IndexError, match="runs from 0 to 100"):
         reverse(a, np.zeros(101), 101)
+
+
+def test_shared_scalars_and_other_tiny_host_arrays_in_repeated_calls(gpu):
+    """Host arrays of a few bytes travel through page-locked slots, and a call that differs from an earlier one
+    only in their contents repeats that call's launch: every call must see its own values and get its own results."""
+    import torch
+
+    from appy_amd.backends.hip import codegen as cg
+
+    @appy.jit
+    def offset_sum(A, start):
+        s = start
+        #pragma parallel for simd shared(s)
+        for i in range(A.shape[0]):
+            s += A[i]
+        return s
+
+    @appy.jit
+    def two_names(A, acc, also, n):
+        #pragma parallel for simd
+        for i in range(n):
+            A[i] = A[i] + acc[0] + also[1]
+
+    @appy.jit
+    def bump(cell, by, n):
+        #pragma parallel for
+        for i in range(n):
+            cell[i] = cell[i] + by[i]
+
+    A = torch.arange(1000.0, device="cuda", dtype=torch.float64)
+    total = float(A.sum())
+    for start in (0.0, 2.5, -7.0, 1e6, 0.0):
+        assert offset_sum(A, start) == total + start
+    B = torch.arange(500.0, device="cuda", dtype=torch.float64)
+    assert offset_sum(B, 1.0) == float(B.sum()) + 1.0           # another tensor between two repeats
+    assert offset_sum(A, 3.0) == total + 3.0
+    loop = [v[0] for kk, v in cg.code_cache.items() if kk[-1] == "offset_sum"][-1]
+    assert loop._replays and all(plan.small_fixed for plan in loop._replays.values())
+    # the same small array under two names: one copy on the device serves both
+    X = torch.zeros(64, device="cuda", dtype=torch.float64)
+    for k in range(3):
+        pair = np.array([1.0 + k, 10.0])
+        two_names(X, pair, pair, 64)
+    assert torch.equal(X, torch.full((64,), 36.0, device="cuda", dtype=torch.float64))
+    # a stored small array, new contents at every call
+    for k in range(4):
+        cell = np.array([1.0, 2.0, 3.0]) * (k + 1)
+        by = torch.tensor([10.0, 20.0, 30.0], device="cuda", dtype=torch.float64)
+        bump(cell, by, 3)
+        assert np.array_equal(cell, np.array([11.0, 22.0, 33.0]) + np.array([1.0, 2.0, 3.0]) * k)
