@@ -64,10 +64,55 @@ class _ShapeView:
             raise TypeError("len() of a 0-d array")
         return self.shape[0]
 
-# Hardware facts used by the launch heuristics (MI355X: 256 CUs in 8 XCDs,
-# 256 MiB of memory-side cache in front of the HBM3E).
-DEFAULT_CUS = 256
-MALL_BYTES = 256 << 20
+@dataclasses.dataclass(frozen=True)
+class Hardware:
+    """What the launch heuristics know of a device.  The defaults are MI355X's: 256 CUs in 8 XCDs, an L2 of
+    4 MiB per XCD, 256 MiB of memory-side cache in front of the HBM3E (the one figure the runtime does not
+    report: `APPY_HIP_MALL_BYTES` overrides it)."""
+
+    cus: int = 256
+    xcds: int = 8
+    l2_bytes: int = 4 << 20
+    mall_bytes: int = 256 << 20
+
+    @property
+    def stripe_bytes(self) -> int:
+        """Most of a gathered operand that one XCD is given to keep in its L2 next to the streams: half the L2."""
+        return self.l2_bytes // 2
+
+    @property
+    def stripe_min_bytes(self) -> int:
+        """A gathered operand up to this size is left to every L2 as a whole."""
+        return 3 * self.l2_bytes // 4
+
+    @property
+    def pinned_stripes(self) -> bool:
+        """Stripes of a gathered operand are pinned to XCDs by workgroup number modulo 8 in the generated kernels."""
+        return self.xcds == 8
+
+
+MI355X = Hardware()
+_hardware = {}
+
+
+def hardware(device=None) -> Hardware:
+    """The facts of ``device`` as the runtime reports them; MI355X's when no device is named (kernels generated
+    and launch shapes chosen without a GPU)."""
+    if device is None:
+        return MI355X
+    hw = _hardware.get(device)
+    if hw is None:
+        t = rt.device_topology(device)
+        hw = Hardware(cus=int(t["compute_units"]) or MI355X.cus, xcds=int(t["xcds"]) or 1,
+                      l2_bytes=int(t["l2_bytes_per_xcd"]) or MI355X.l2_bytes,
+                      mall_bytes=int(os.environ.get("APPY_HIP_MALL_BYTES") or MI355X.mall_bytes))
+        _hardware[device] = hw
+    return hw
+
+
+# (the figures of MI355X under their old names: tests and tools that size their inputs by them)
+DEFAULT_CUS = MI355X.cus
+MALL_BYTES = MI355X.mall_bytes
 REDUCTION_WINDOW_BYTES = 6 << 20
 CACHED_REDUCTION_WINDOW_BYTES = 4 << 20
 TEAM_BYTES_IN_FLIGHT = 8.0e6
@@ -85,9 +130,8 @@ ROW_CACHE_STEPS = 16
 BIN_MIN_ROWS = 1 << 15
 # a gathered operand larger than this is walked one stripe at a time by long rows; eight stripes (one per
 # XCD and its 4 MiB L2) of at most STRIPE_BYTES each, or a multiple of eight
-STRIPE_MIN_BYTES = 3 << 20
-STRIPE_BYTES = 2 << 20
-GROUP_MAX_STRIPE_LOG = 19          # elements grouped by stripe: stripes of 2^19 elements of 4 bytes (half an L2) at most, 8 or 16 of them
+STRIPE_MIN_BYTES = MI355X.stripe_min_bytes
+STRIPE_BYTES = MI355X.stripe_bytes
 GROUP_MIN_TRIP = 4                 # ... for rows of this many elements on average, at least
 # row plans (the order of the elements of a CSR-like sum, worked out once and kept between launches)
 PLAN_ROW_BITS = 15                 # rows per block: what fits a workgroup's LDS as 4-byte sums
@@ -597,16 +641,18 @@ class CompiledLoop:
                 best = max(best, 64.0)
         return best, uniform
 
-    def choose_spec(self, n_outer, env, arrays, restrict=True, listable=True) -> Spec:
-        """``listable``: the iterations can be named by 32-bit numbers (rows sorted by length are)."""
-        spec = self._choose_spec(n_outer, env, arrays, restrict, listable)
+    def choose_spec(self, n_outer, env, arrays, restrict=True, listable=True, hw=None) -> Spec:
+        """``listable``: the iterations can be named by 32-bit numbers (rows sorted by length are); ``hw``: the
+        device the launch is for (MI355X's figures when none is named)."""
+        spec = self._choose_spec(n_outer, env, arrays, restrict, listable, hw or MI355X)
         if self.options.get("check_bounds"):
             # one element per access, every access through the checking path
             spec = dataclasses.replace(spec, vec=1, unroll=1, extent=0, lds_tile=0, stream_loads=False,
                                        stream_stores=False, checked=True)
         return spec
 
-    def _choose_spec(self, n_outer, env, arrays, restrict=True, listable=True) -> Spec:
+    def _choose_spec(self, n_outer, env, arrays, restrict=True, listable=True, hw=MI355X) -> Spec:
+        DEFAULT_CUS, MALL_BYTES = hw.cus, hw.mall_bytes      # (the names the rules below were written with)
         forced = self.options.get("hip_spec")
         d = self.default_spec
         if isinstance(forced, dict):
@@ -749,14 +795,14 @@ class CompiledLoop:
         return Spec("team", block=block, vec=v, width=w, restrict=restrict, stream_loads=stream, collapse=bool(nj),
                     row_steps=steps)
 
-    def team_parts(self, spec: Spec, n_outer: int, env, arrays) -> int:
+    def team_parts(self, spec: Spec, n_outer: int, env, arrays, hw=MI355X) -> int:
         """Workgroups per row of a two-phase team launch: two workgroups per CU in all, each
         part at least four vector steps per lane long."""
         trip, _uniform = self._estimate_trip(env, arrays, n_outer)
-        parts = min(2 * DEFAULT_CUS // max(1, n_outer), int(trip // (4 * spec.block * spec.vec)), 1024)
+        parts = min(2 * hw.cus // max(1, n_outer), int(trip // (4 * spec.block * spec.vec)), 1024)
         return max(1, parts)
 
-    def strip_parts(self, spec: Spec, n_outer: int, env) -> int:
+    def strip_parts(self, spec: Spec, n_outer: int, env, hw=MI355X) -> int:
         """Workgroups per strip of a two-phase strip launch: one workgroup of 1024 lanes per CU
         in all (2^20 x 64 floats: 79 us with 128 workgroups, 98 with 256, 156 with 512 - the
         finishing kernel walks the parts of a column one after the other), each part at least
@@ -767,10 +813,10 @@ class CompiledLoop:
         except Exception:
             trip = 0
         nw = spec.block // 64
-        parts = min(DEFAULT_CUS // max(1, strips), max(1, trip // (4 * nw)), 1024)
+        parts = min(hw.cus // max(1, strips), max(1, trip // (4 * nw)), 1024)
         return max(1, parts)
 
-    def grouped_shape(self, n_outer, env, arrays):
+    def grouped_shape(self, n_outer, env, arrays, hw=MI355X):
         """``(stripes, log2 of the elements per stripe, positions to group)`` for a launch that groups the
         elements of its rows by the stripe of the gathered operand they read, or None when the loop or
         these arrays do not qualify: the operand is larger than an L2 can keep next to the streams and
@@ -779,9 +825,10 @@ class CompiledLoop:
         if g is None or self._group_off or not self.options.get("hip_group", True):
             return None
         nx = int(arrays[g["x"]].shape[0])
-        if nx * 4 <= STRIPE_MIN_BYTES or nx > (16 << GROUP_MAX_STRIPE_LOG):
+        most = hw.stripe_bytes // 4         # elements per stripe: half an L2 at most, 8 or 16 stripes
+        if not hw.pinned_stripes or nx * 4 <= hw.stripe_min_bytes or nx > 16 * most:
             return None
-        parts = 8 if nx <= (8 << GROUP_MAX_STRIPE_LOG) else 16
+        parts = 8 if nx <= 8 * most else 16
         shift = max(1, (-(-nx // parts) - 1).bit_length())
         entries = min(int(arrays[nm].shape[0]) for nm in (g["idx"], g["carried"]) if nm)
         trip, _uniform = self._estimate_trip(env, arrays, n_outer)
@@ -896,11 +943,11 @@ class CompiledLoop:
                 names.append(nm)
         return names
 
-    def plan_shape(self, n_outer, env, arrays):
+    def plan_shape(self, n_outer, env, arrays, hw=MI355X):
         """The shape of a row plan for these arrays (runtime.RowPlanShape), or None when they do not
         qualify: the conditions of the grouped form (an operand too large for an L2, rows of a few
         elements), and keys and packed words of 32 bits."""
-        base = self.grouped_shape(n_outer, env, arrays)
+        base = self.grouped_shape(n_outer, env, arrays, hw)
         if base is None or self._plan_off:
             return None
         g = self.analysis.grouping
@@ -947,7 +994,7 @@ class CompiledLoop:
                 total += n * arr.ty.size
         return total
 
-    def grid_for(self, spec: Spec, n_outer: int, cus: int = DEFAULT_CUS, kernel=None, row_hint=(0.0, False)) -> int:
+    def grid_for(self, spec: Spec, n_outer: int, cus: int = MI355X.cus, kernel=None, row_hint=(0.0, False)) -> int:
         if spec.kind == "strip":
             return int(min(max(1, -(-n_outer // 64)), self.options.get("hip_max_blocks") or (1 << 22)))
         if spec.kind == "flat":
@@ -1238,7 +1285,8 @@ class Launch:
 
         # -- kernel variant, argument block, grid
         n_outer = hi - lo
-        spec = loop.choose_spec(n_outer, env, arrays, restrict=restrict, listable=hi < (1 << 31))
+        hw = self.hw = hardware(device)
+        spec = loop.choose_spec(n_outer, env, arrays, restrict=restrict, listable=hi < (1 << 31), hw=hw)
         if spec.kind == "flat" and spec.hoist_guarded and a.guarded_checks:
             # loads the program guards with a condition may only be issued early when
             # they cannot leave their array anywhere in the range
@@ -1252,11 +1300,11 @@ class Launch:
         self.nsplit = 1
         self.scratch_ptr = 0
         if spec.phase == 1 and spec.kind == "strip":
-            self.nsplit = loop.strip_parts(spec, n_outer, env)
+            self.nsplit = loop.strip_parts(spec, n_outer, env, hw)
             reds = len(a.strip[id(a.strip_split)])
             self.scratch_ptr = loop.scratch(device, self.stream, max(1, reds) * self.nsplit * n_outer * 8)
         elif spec.phase == 1:
-            self.nsplit = loop.team_parts(spec, n_outer, env, arrays)
+            self.nsplit = loop.team_parts(spec, n_outer, env, arrays, hw)
             reds = len(loop_ir.reductions_of(a.team_split))
             self.scratch_ptr = loop.scratch(device, self.stream, max(1, reds) * self.nsplit * n_outer * 8)
         if spec.phase == 1 and self.scratch_ptr is None:
@@ -1271,7 +1319,7 @@ class Launch:
                 loop.last_launch = self
                 return
             # not even the lists of rows fit what the loop may hold: one team width for all rows
-            spec = loop.choose_spec(n_outer, env, arrays, restrict=restrict, listable=False)
+            spec = loop.choose_spec(n_outer, env, arrays, restrict=restrict, listable=False, hw=hw)
             self.kernel, self.spec = loop.kernel_for(spec), spec
         self.args = self._argument_block(self.kernel, vals, arrays, lo, hi)
         if spec.phase == 1 and spec.kind == "strip":
@@ -1288,7 +1336,7 @@ class Launch:
         else:
             if spec.collapse:
                 n_outer *= max(1, loop.collapse_count(n_outer, env))
-            self.grid = (loop.grid_for(spec, n_outer, kernel=self.kernel,
+            self.grid = (loop.grid_for(spec, n_outer, cus=hw.cus, kernel=self.kernel,
                                        row_hint=loop.row_hint(n_outer, env, arrays)), 1, 1)
         self.block = (spec.block, 1, 1)
         loop.last_launch = self
@@ -1319,8 +1367,8 @@ class Launch:
         if gather is not None:
             x = arrays[gather[0]]
             x_bytes = int(x.shape[0]) * a.arrays[gather[0]].ty.size
-            if x_bytes > STRIPE_MIN_BYTES:
-                parts = min(64, 8 * -(-x_bytes // (8 * STRIPE_BYTES)))
+            if self.hw.pinned_stripes and x_bytes > self.hw.stripe_min_bytes:
+                parts = min(64, 8 * -(-x_bytes // (8 * self.hw.stripe_bytes)))
                 stripe = -(-int(x.shape[0]) // parts)
                 thresholds[2] = max(thresholds[2], 32 * parts)       # 32 elements per part at least
                 # rows longer than the threshold: no more of them than the streamed arrays have room for
@@ -1414,7 +1462,7 @@ class Launch:
         trusted = (loop.options.get("hip_hints", True) and loop._hint_key.get(self.device) == ident
                    and seen[0] == 1 and sum(seen[1:]) == n and min(seen[1:]) >= 0)
         long_rows = not trusted or seen[4] > 0
-        shape = loop.grouped_shape(n, env, arrays)
+        shape = loop.grouped_shape(n, env, arrays, self.hw)
         if shape is None:
             return False
         parts, shift, entries = shape
@@ -1430,7 +1478,7 @@ class Launch:
             group = loop.kernel_for(Spec("team", vec=1, width=64, parts=parts, aux="group", block_rows=R, skip_long=long_rows, **common))
             cells = loop.kernel_for(Spec("team", vec=1, width=64, parts=parts, aux="cells", block_rows=R, guard=1, **common))
             sums = loop.kernel_for(Spec("team", vec=V, width=1, phase=2, guard=1, skip_long=long_rows, **common))
-            plain = loop._choose_spec(n, env, arrays, restrict=spec.restrict, listable=False)
+            plain = loop._choose_spec(n, env, arrays, restrict=spec.restrict, listable=False, hw=self.hw)
             if plain.kind != "team" or plain.phase or plain.rows:
                 raise Unsupported("no plain team kernel to fall back to")
             rest = loop.kernel_for(dataclasses.replace(plain, guard=2))
@@ -1497,7 +1545,7 @@ class Launch:
         # (the kernel that runs the loop row by row when the input was refused: few workgroups that loop - it returns at
         #  once otherwise, and 65536 workgroups take 15 us to do that, 1024 take 3)
         seq.append((rest, self._argument_block(rest, vals, arrays, lo, hi),
-                    (min(1024, loop.grid_for(plain, n, kernel=rest, row_hint=loop.row_hint(n, env, arrays))), 1, 1), (plain.block, 1, 1)))
+                    (min(1024, loop.grid_for(plain, n, cus=self.hw.cus, kernel=rest, row_hint=loop.row_hint(n, env, arrays))), 1, 1), (plain.block, 1, 1)))
         self.sequence = seq
         self.kernel, self.spec = cells, cells.src.spec
         self.args, self.grid, self.block = args_of_cells[1], args_of_cells[2], args_of_cells[3]
@@ -1568,7 +1616,7 @@ class Launch:
         if plan is None:
             if key in loop._plan_refused:
                 return False
-            shape = loop.plan_shape(n, env, arrays)
+            shape = loop.plan_shape(n, env, arrays, self.hw)
             if shape is None:
                 return False
             with loop._lock:
@@ -1682,7 +1730,7 @@ class Launch:
         # few cells (a matrix of few blocks of rows): several workgroups share a cell, each with a run of its tiles,
         # until there are some four workgroups per compute unit or a workgroup is down to two tiles
         forced = loop.options.get("hip_plan_split")
-        plan.split = int(forced) if forced else max(1, min(-(-4 * DEFAULT_CUS // ncell), entries // (2 * plan.tile * ncell), 32))
+        plan.split = int(forced) if forced else max(1, min(-(-4 * self.hw.cus // ncell), entries // (2 * plan.tile * ncell), 32))
         plan.valid = True
         plan.owner = loop
         with loop._lock:

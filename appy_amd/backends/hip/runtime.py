@@ -31,6 +31,15 @@ class Props(C.Structure):
     ]
 
 
+class Topology(C.Structure):
+    _fields_ = [
+        ("xcds", C.c_int32),
+        ("compute_units", C.c_int32),
+        ("l2_bytes_per_xcd", C.c_int32),
+        ("lds_bytes_per_cu", C.c_int32),
+    ]
+
+
 class FuncInfo(C.Structure):
     _fields_ = [
         ("num_vgprs", C.c_int32),
@@ -68,6 +77,7 @@ SIGNATURES = {
     "appy_hip_device_count": (C.c_int, [C.POINTER(C.c_int)]),
     "appy_hip_init": (C.c_int, [C.c_int]),
     "appy_hip_device_props": (C.c_int, [C.c_int, C.POINTER(Props)]),
+    "appy_hip_device_topology": (C.c_int, [C.c_int, C.POINTER(Topology)]),
     "appy_hip_compile": (
         C.c_int,
         [C.c_char_p, C.c_char_p, C.c_char_p, C.POINTER(C.c_char_p), C.c_int, C.POINTER(_vp), C.POINTER(C.c_size_t)],
@@ -179,6 +189,12 @@ def device_props(device: int = 0) -> dict:
         v = getattr(p, f)
         out[f] = v.decode() if isinstance(v, bytes) else v
     return out
+
+
+def device_topology(device: int = 0) -> dict:
+    t = Topology()
+    check(lib().appy_hip_device_topology(int(device), C.byref(t)))
+    return {f: getattr(t, f) for f, _ in Topology._fields_}
 
 
 # Options every kernel is compiled with.  Contraction is off so that

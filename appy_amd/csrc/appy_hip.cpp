@@ -406,6 +406,24 @@ int appy_hip_device_props(int device, appy_hip_props* out) {
     return 0;
 }
 
+int appy_hip_device_topology(int device, appy_hip_topology* out) {
+    if (!out) return fail_arg("out is NULL");
+    std::memset(out, 0, sizeof(*out));
+    int xcds = 0, cus = 0, l2 = 0, lds = 0;
+    if (hipDeviceGetAttribute(&xcds, hipDeviceAttributeNumberOfXccs, device) != hipSuccess || xcds < 1) {
+        (void)hipGetLastError();
+        xcds = 1;
+    }
+    HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device));
+    HIP_TRY(hipDeviceGetAttribute(&l2, hipDeviceAttributeL2CacheSize, device));
+    HIP_TRY(hipDeviceGetAttribute(&lds, hipDeviceAttributeMaxSharedMemoryPerMultiprocessor, device));
+    out->xcds = xcds;
+    out->compute_units = cus;
+    out->l2_bytes_per_xcd = l2;
+    out->lds_bytes_per_cu = lds;
+    return 0;
+}
+
 // ---- run-time compilation ---------------------------------------------------
 
 int appy_hip_compile(const char* src, const char* name, const char* arch,

@@ -25,7 +25,7 @@ extern "C" {
 #endif
 
 /* 2: page-locked host memory, streams and graphs, appy_hip_rtc_version; 3: appy_hip_launch_static_scratch;
- * 4: row plans (appy_hip_rowplan_*), appy_hip_device_sync, appy_hip_memcpy_h2d_async
+ * 4: row plans (appy_hip_rowplan_*), appy_hip_device_sync, appy_hip_memcpy_h2d_async, appy_hip_device_topology
  * (additions only: every entry point of the earlier versions is unchanged). */
 #define APPY_HIP_ABI_VERSION 4
 
@@ -65,6 +65,16 @@ const char* appy_hip_last_error(void);
 int appy_hip_device_count(int* count_out);
 int appy_hip_init(int device);                 /* make `device` current for this thread */
 int appy_hip_device_props(int device, appy_hip_props* out);
+/* How the compute units are grouped (ABI 4; appy_hip_props keeps its layout).  On MI355X: 8 accelerator dies
+ * (XCDs) of 32 CUs, each with an L2 of its own (appy_hip_props.l2_bytes is that of one die) - the launch
+ * heuristics size grids by the CUs and pin stripes of gathered operands to dies, workgroup number modulo `xcds`. */
+typedef struct appy_hip_topology {
+    int32_t xcds;               /* accelerator dies with an L2 each; 1 where the device does not say */
+    int32_t compute_units;      /* all of them, as appy_hip_props.compute_units */
+    int32_t l2_bytes_per_xcd;
+    int32_t lds_bytes_per_cu;
+} appy_hip_topology;
+int appy_hip_device_topology(int device, appy_hip_topology* out);
 
 /* ---- run-time compilation ----------------------------------------------
  * Replaces @triton.jit on the generated `_kernel_loop_N`

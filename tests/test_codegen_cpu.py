@@ -821,3 +821,34 @@ def test_row_plans_kernel_that_writes_the_pairs_and_kernel_that_runs_a_plan():
     assert (shape.col_bits, shape.tile) == (20, 4096)
     arrays["x"] = np.broadcast_to(np.float32(0), (1 << 19,))                  # an operand that every L2 holds anyway
     assert f.plan_shape(1 << 22, {"M": 1 << 22}, arrays) is None
+
+
+def test_launch_shapes_follow_the_device_they_are_for():
+    """Grids and the forms that pin stripes of a gathered operand to XCDs are sized from what the runtime reports of
+    the device (compute units, XCDs, L2 per XCD), not from literals: another device, other shapes."""
+    small = cg.Hardware(cus=64, xcds=4, l2_bytes=2 << 20, mall_bytes=32 << 20)
+    assert cg.MI355X == cg.Hardware(cus=256, xcds=8, l2_bytes=4 << 20, mall_bytes=256 << 20)
+    assert (cg.MI355X.stripe_bytes, cg.MI355X.stripe_min_bytes, small.stripe_bytes) == (2 << 20, 3 << 20, 1 << 20)
+    # a streaming reduction: non-temporal loads from the size of the memory-side cache on
+    f, _ = compiled("#pragma parallel for simd shared(s)\nfor i in range(n):\n    s[0] += a[i]", s=np.zeros(1), a=np.zeros(8, np.float32), n=8)
+    arrays = {"s": np.zeros(1), "a": np.broadcast_to(np.float32(0), (1 << 24,))}
+    assert not f.choose_spec(1 << 24, {}, arrays).stream_loads and f.choose_spec(1 << 24, {}, arrays, hw=small).stream_loads
+    # few, very long rows: a workgroup per row up to as many rows as there are compute units
+    g, _ = selfcheck_loop("gemv")
+    rows = {"A": np.broadcast_to(np.float32(0), (128, 1 << 20)), "x": np.broadcast_to(np.float32(0), (1 << 20,)),
+            "y": np.broadcast_to(np.float32(0), (128,))}
+    env = {"A_shape_0": 128, "A_shape_1": 1 << 20}
+    big, little = g.choose_spec(128, env, rows), g.choose_spec(128, env, rows, hw=small)
+    assert (big.block, big.phase) == (1024, 1) and (little.block, little.phase) == (256, 0)
+    assert g.team_parts(big, 128, env, rows) == 4 and g.team_parts(big, 128, env, rows, hw=small) == 1
+    assert g.grid_for(f.default_spec, 1 << 30, cus=64) < g.grid_for(f.default_spec, 1 << 30)
+    # stripes per XCD: only where the kernels' mapping of workgroups to XCDs holds (eight of them)
+    sp, _ = selfcheck_loop("spmv")
+    csr = {"A_data": np.broadcast_to(np.float32(0), (16 << 20,)), "A_indices": np.broadcast_to(np.int32(0), (16 << 20,)),
+           "A_indptr": np.broadcast_to(np.int32(0), ((1 << 20) + 1,)), "x": np.broadcast_to(np.float32(0), (1 << 20,))}
+    assert sp.grouped_shape(1 << 20, {"M": 1 << 20}, csr)[0] == 8
+    assert sp.grouped_shape(1 << 20, {"M": 1 << 20}, csr, hw=small) is None and sp.plan_shape(1 << 20, {"M": 1 << 20}, csr, hw=small) is None
+    double = cg.Hardware(cus=256, xcds=8, l2_bytes=8 << 20)
+    assert sp.grouped_shape(1 << 20, {"M": 1 << 20}, csr, hw=double) is None       # 4 MiB stay in an 8 MiB L2 as a whole
+    csr["x"] = np.broadcast_to(np.float32(0), (4 << 20,))
+    assert sp.grouped_shape(1 << 20, {"M": 1 << 20}, csr, hw=double)[0] == 8
