@@ -109,6 +109,51 @@ def test_spmv_full_size_row_lengths_and_linearity(env, kind):
     assert bool(((y1.double() - ref).abs() <= TOL * budget).all())
 
 
+@pytest.mark.parametrize("kind", ["uniform", "powerlaw"])
+def test_spmv_full_size_with_the_order_of_the_elements_kept(env, kind):
+    """The same tensors launch after launch: the first launch reads the raw arrays, the second works out the
+    order of the elements and runs it, the third only runs it.  All three against a float64 sum built with
+    `index_add_`; exact cases (all ones) through the kept order as well; the same bits from launch to launch."""
+    import appy_amd as appy
+    from appy_amd.backends.hip import codegen as cg
+
+    torch, k = env
+    m = 1 << 22
+    if kind == "uniform":
+        lengths = np.full(m, 16, dtype=np.int64)
+    else:
+        lengths = np.clip(np.random.default_rng(104).zipf(1.5, m), 1, 4096).astype(np.int64)
+    data, indptr, indices = _csr(torch, lengths, m, seed=11)
+    x = torch.randn(m, device="cuda", generator=torch.Generator(device="cuda").manual_seed(12))
+    rows = torch.repeat_interleave(torch.arange(m, device="cuda"), torch.from_numpy(lengths).to("cuda"))
+    terms = data.double() * x[indices.long()].double()
+    ref = torch.zeros(m, dtype=torch.float64, device="cuda").index_add_(0, rows, terms)
+    budget = torch.zeros(m, dtype=torch.float64, device="cuda").index_add_(0, rows, terms.abs())
+    del terms, rows
+
+    def last_plan():
+        loops = [v[0] for kk, v in cg.code_cache.items() if kk[-1] == "spmv" and getattr(v[0], "last_launch", None) is not None
+                 and v[0].options.get("hip_reuse", True) is True]
+        return max(loops, key=lambda lp: lp.last_launch.serial).last_launch.plan
+
+    ys = []
+    for launch in range(3):
+        y = k.spmv(data, indptr, indices, x, m, m)
+        assert (last_plan() is not None) == (launch >= 1)
+        assert bool(((y.double() - ref).abs() <= TOL * budget).all())
+        ys.append(y)
+    assert torch.equal(ys[1], ys[2])
+    plan = last_plan()
+    assert plan.ncell == 8 * (m >> 15) and plan.split == 1 and plan.inspector_ms > 0
+    # all values 1 and x = 1: the row lengths, exactly - through a plan (the tensors are seen twice)
+    ones, ones_x = torch.ones_like(data), torch.ones(m, device="cuda")
+    for launch in range(2):
+        y = k.spmv(ones, indptr, indices, ones_x, m, m)
+        assert torch.equal(y, torch.from_numpy(lengths).to("cuda").float())
+    assert last_plan() is not None and last_plan() is not plan
+    appy.release()
+
+
 def test_spmm_full_size_against_spmv_columns(env):
     torch, k = env
     m = 1 << 20
