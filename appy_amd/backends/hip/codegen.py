@@ -1619,11 +1619,17 @@ class Launch:
             shape = loop.plan_shape(n, env, arrays, self.hw)
             if shape is None:
                 return False
+            import weakref
+
             with loop._lock:
-                seen = loop._plan_seen.get(key, 0) + 1
+                # sightings of these very tensor objects (an address is handed out again once a tensor is freed)
+                count, refs = loop._plan_seen.get(key, (0, ()))
+                if not (len(refs) == len(tensors) and all(r() is t for r, t in zip(refs, tensors))):
+                    count, refs = 0, tuple(weakref.ref(t) for t in tensors)
+                seen = count + 1
                 if len(loop._plan_seen) > 64:
                     loop._plan_seen.clear()
-                loop._plan_seen[key] = seen
+                loop._plan_seen[key] = (seen, refs)
             if seen < (1 if reuse == "now" else 2):
                 return False
             plan = self._build_plan(key, tensors, shape, vals, arrays, lo, hi, spec)
