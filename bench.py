@@ -634,6 +634,9 @@ def main():
         spec_tag, nbytes_prof = traffic.get(name, (None, None))
         r["traffic_profile_spec"] = spec_tag
         r["traffic_bytes_rocprof"] = nbytes_prof if spec_tag == r["spec"] else None
+        if "spec_reused" in r:
+            tag2, nbytes2 = traffic.get(name + "_reused", (None, None))
+            r["traffic_bytes_rocprof_reused"] = nbytes2 if tag2 == r["spec_reused"] else None
     # L2 requests per second of the launches whose request counts the committed counter runs hold (same kernel
     # shape), against one request per L2 channel and clock (16 channels in each of 8 XCDs)
     requests = load_profile_requests() if sc == 1.0 else {}
