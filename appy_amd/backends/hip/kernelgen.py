@@ -2680,11 +2680,6 @@ class KernelBuilder:
         w(f"int __cnt[{S}], __at[{S + 1}];")
         w("#pragma unroll")
         w(f"for (int __s = 0; __s < {S}; ++__s) __cnt[__s] = 0;")
-        if skip:
-            self._group_walk_kept(idx_c, car_c, U, find_row, count, starts, place_one, unrolled)
-            self.ind -= 1
-            w("}")
-            return
 
         def load_indices(k, j0, kk):
             w(f"{{ const int __j = {j0} + {kk} * 256 + __lid * 4;")
@@ -2716,6 +2711,11 @@ class KernelBuilder:
             self.ind -= 1
             w("}")
 
+        if skip:
+            # the sorting kernel, which ran before this one, has counted the rows beyond the limit: where there are none,
+            # every element is kept and the walk over the arrays as they lie does (the layout is the same either way)
+            w("if (__counts[3] == 0) {")
+            self.ind += 1
         # (indices of a whole block kept in registers between the two passes - 64 registers, half the wavefronts per
         #  SIMD - made this kernel slower: 455 us against 306 for 2^26 elements)
         w(f"for (int __j0 = __first; __j0 < __end; __j0 += {256 * U}) {{")
@@ -2733,6 +2733,13 @@ class KernelBuilder:
         unrolled(U, lambda: place("__k", "__k", "__j0", "__k"))
         self.ind -= 1
         w("}")
+        if skip:
+            self.ind -= 1
+            w("} else {")
+            self.ind += 1
+            self._group_walk_kept(idx_c, car_c, U, find_row, count, starts, place_one, unrolled)
+            self.ind -= 1
+            w("}")
         self.ind -= 1
         w("}")
 

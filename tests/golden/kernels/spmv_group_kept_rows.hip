@@ -84,36 +84,172 @@ _spmv_kernel_loop_1_group(
         int __cnt[8], __at[9];
         #pragma unroll
         for (int __s = 0; __s < 8; ++__s) __cnt[__s] = 0;
-        // where every row starts among the elements that are kept (rows beyond the limit hold none): lane l sums rows 4l .. 4l + 3
-        int* __kp = __hq;
-        int __kt[4], __mine = 0;
-        #pragma unroll
-        for (int __i = 0; __i < 4; ++__i) {
-            const int __r = 4 * __lid + __i;
-            const int __n = __r < __nr ? __hq[__r] - __lp[__r] : 0;
-            __kt[__i] = __n > __rowmax ? 0 : __n;
-            __mine += __kt[__i];
-        }
-        int __incl = __mine;
-        #pragma unroll
-        for (int __d = 1; __d < 64; __d <<= 1) {
-            const int __o = __shfl_up(__incl, __d, 64);
-            if (__lid >= __d) __incl += __o;
-        }
-        appy::wave_fence();       // the ends of the rows have been read: their table now holds the starts among the kept
-        {
-            int __run = __incl - __mine;
-        #pragma unroll
-            for (int __i = 0; __i < 4; ++__i) { __kp[4 * __lid + __i] = __run; __run += __kt[__i]; }
-        }
-        if (__lid == 63) __kp[256] = __incl;
-        appy::wave_fence();
-        const int __kept = __kp[256];
-        for (int __t0 = 0; __t0 < __kept; __t0 += 1024) {
-            appy::vec<int, 4>::type __c[4];
+        if (__counts[3] == 0) {
+            for (int __j0 = __first; __j0 < __end; __j0 += 1024) {
+                appy::vec<int, 4>::type __c[4];
+                #pragma unroll
+                for (int __k = 0; __k < 4; ++__k) {
+                    { const int __j = __j0 + __k * 256 + __lid * 4;
+                    if (__j + 4 <= __end) __c[__k] = appy::vload<int, 4>(A_indices + __j);
+                    else {
+                    #pragma unroll
+                        for (int __q = 0; __q < 4; ++__q) __c[__k][__q] = __j + __q < __end ? A_indices[__j + __q] : -1;
+                    } }
+                }
+                #pragma unroll
+                for (int __k = 0; __k < 4; ++__k) {
+                    #pragma unroll
+                    for (int __q = 0; __q < 4; ++__q)
+                    #pragma unroll
+                        for (int __s = 0; __s < 8; ++__s) __cnt[__s] += __popcll(__ballot((__c[__k][__q] >> __shiftc) == __s));
+                }
+            }
+            __at[0] = __first;
             #pragma unroll
-            for (int __k = 0; __k < 4; ++__k) {
-                {
+            for (int __s = 0; __s < 8; ++__s) __at[__s + 1] = __at[__s] + __cnt[__s];
+            #pragma unroll
+            for (int __s = 0; __s <= 8; ++__s) if (__lid == __s) __desc[__b * 9 + __s] = __at[__s];
+            for (int __j0 = __first; __j0 < __end; __j0 += 1024) {
+                appy::vec<int, 4>::type __c[4], __v[4];
+                #pragma unroll
+                for (int __k = 0; __k < 4; ++__k) {
+                    { const int __j = __j0 + __k * 256 + __lid * 4;
+                    if (__j + 4 <= __end) __c[__k] = appy::vload<int, 4>(A_indices + __j);
+                    else {
+                    #pragma unroll
+                        for (int __q = 0; __q < 4; ++__q) __c[__k][__q] = __j + __q < __end ? A_indices[__j + __q] : -1;
+                    } }
+                    { const int __j = __j0 + __k * 256 + __lid * 4;
+                    if (__j + 4 <= __end) __v[__k] = appy::vload<int, 4>(reinterpret_cast<const int*>(A_data) + __j);
+                    else {
+                    #pragma unroll
+                        for (int __q = 0; __q < 4; ++__q) __v[__k][__q] = __j + __q < __end ? reinterpret_cast<const int*>(A_data)[__j + __q] : 0;
+                    } }
+                }
+                #pragma unroll
+                for (int __k = 0; __k < 4; ++__k) {
+                    const int __j = __j0 + __k * 256 + __lid * 4;
+                    int __row = 0, __past = 256;       // the last row that starts at or before __j
+                    #pragma unroll
+                    for (int __it = 0; __it < 8; ++__it) {
+                        const int __mid = (__row + __past) >> 1;
+                        if (__lp[__mid] <= __j) __row = __mid; else __past = __mid;
+                    }
+                    #pragma unroll
+                    for (int __q = 0; __q < 4; ++__q) {
+                        if (__j + __q < __end) while (__lp[__row + 1] <= __j + __q) ++__row;
+                        const int __cq = __c[__k][__q];
+                        const int __sq = __cq >> __shiftc;          // negative past the end (and for negative indices: such elements are dropped)
+                        int __pos = 0;
+                        #pragma unroll
+                        for (int __s = 0; __s < 8; ++__s) {
+                            const unsigned long long __m = __ballot(__sq == __s);
+                            if (__sq == __s) __pos = __at[__s] + __popcll(__m & __below);
+                            __at[__s] += __popcll(__m);
+                        }
+                        if (__sq >= 0 && __sq < 8)
+                            __ent[__pos] = (long long)(((unsigned long long)(((unsigned)__row << 22) | (unsigned)(__cq & __cmask)) << 32) | (unsigned long long)(unsigned)__v[__k][__q]);
+                    }
+                }
+            }
+        } else {
+            // where every row starts among the elements that are kept (rows beyond the limit hold none): lane l sums rows 4l .. 4l + 3
+            int* __kp = __hq;
+            int __kt[4], __mine = 0;
+            #pragma unroll
+            for (int __i = 0; __i < 4; ++__i) {
+                const int __r = 4 * __lid + __i;
+                const int __n = __r < __nr ? __hq[__r] - __lp[__r] : 0;
+                __kt[__i] = __n > __rowmax ? 0 : __n;
+                __mine += __kt[__i];
+            }
+            int __incl = __mine;
+            #pragma unroll
+            for (int __d = 1; __d < 64; __d <<= 1) {
+                const int __o = __shfl_up(__incl, __d, 64);
+                if (__lid >= __d) __incl += __o;
+            }
+            appy::wave_fence();       // the ends of the rows have been read: their table now holds the starts among the kept
+            {
+                int __run = __incl - __mine;
+            #pragma unroll
+                for (int __i = 0; __i < 4; ++__i) { __kp[4 * __lid + __i] = __run; __run += __kt[__i]; }
+            }
+            if (__lid == 63) __kp[256] = __incl;
+            appy::wave_fence();
+            const int __kept = __kp[256];
+            for (int __t0 = 0; __t0 < __kept; __t0 += 1024) {
+                appy::vec<int, 4>::type __c[4];
+                #pragma unroll
+                for (int __k = 0; __k < 4; ++__k) {
+                    {
+                        const int __t = __t0 + __k * 256 + __lid * 4;
+                        int __row = 0, __past = 256;       // the last row that starts at or before __t
+                        #pragma unroll
+                        for (int __it = 0; __it < 8; ++__it) {
+                            const int __mid = (__row + __past) >> 1;
+                            if (__kp[__mid] <= __t) __row = __mid; else __past = __mid;
+                        }
+                        int __jq[4];
+                        #pragma unroll
+                        for (int __q = 0; __q < 4; ++__q) {
+                            if (__t + __q < __kept) while (__kp[__row + 1] <= __t + __q) ++__row;
+                            __jq[__q] = __lp[__row] + (__t + __q - __kp[__row]);
+                        }
+                        const bool __run = __t + 4 <= __kept && __jq[3] == __jq[0] + 3;       // four elements in a row of the arrays
+                        if (__run) __c[__k] = appy::vload<int, 4>(A_indices + __jq[0]);
+                        else {
+                        #pragma unroll
+                            for (int __q = 0; __q < 4; ++__q) __c[__k][__q] = __t + __q < __kept ? A_indices[__jq[__q]] : -1;
+                        }
+                    }
+                }
+                #pragma unroll
+                for (int __k = 0; __k < 4; ++__k) {
+                    #pragma unroll
+                    for (int __q = 0; __q < 4; ++__q)
+                    #pragma unroll
+                        for (int __s = 0; __s < 8; ++__s) __cnt[__s] += __popcll(__ballot((__c[__k][__q] >> __shiftc) == __s));
+                }
+            }
+            __at[0] = __first;
+            #pragma unroll
+            for (int __s = 0; __s < 8; ++__s) __at[__s + 1] = __at[__s] + __cnt[__s];
+            #pragma unroll
+            for (int __s = 0; __s <= 8; ++__s) if (__lid == __s) __desc[__b * 9 + __s] = __at[__s];
+            for (int __t0 = 0; __t0 < __kept; __t0 += 1024) {
+                appy::vec<int, 4>::type __c[4], __v[4];
+                #pragma unroll
+                for (int __k = 0; __k < 4; ++__k) {
+                    {
+                        const int __t = __t0 + __k * 256 + __lid * 4;
+                        int __row = 0, __past = 256;       // the last row that starts at or before __t
+                        #pragma unroll
+                        for (int __it = 0; __it < 8; ++__it) {
+                            const int __mid = (__row + __past) >> 1;
+                            if (__kp[__mid] <= __t) __row = __mid; else __past = __mid;
+                        }
+                        int __jq[4];
+                        #pragma unroll
+                        for (int __q = 0; __q < 4; ++__q) {
+                            if (__t + __q < __kept) while (__kp[__row + 1] <= __t + __q) ++__row;
+                            __jq[__q] = __lp[__row] + (__t + __q - __kp[__row]);
+                        }
+                        const bool __run = __t + 4 <= __kept && __jq[3] == __jq[0] + 3;       // four elements in a row of the arrays
+                        if (__run) __c[__k] = appy::vload<int, 4>(A_indices + __jq[0]);
+                        else {
+                        #pragma unroll
+                            for (int __q = 0; __q < 4; ++__q) __c[__k][__q] = __t + __q < __kept ? A_indices[__jq[__q]] : -1;
+                        }
+                        if (__run) __v[__k] = appy::vload<int, 4>(reinterpret_cast<const int*>(A_data) + __jq[0]);
+                        else {
+                        #pragma unroll
+                            for (int __q = 0; __q < 4; ++__q) __v[__k][__q] = __t + __q < __kept ? reinterpret_cast<const int*>(A_data)[__jq[__q]] : 0;
+                        }
+                    }
+                }
+                #pragma unroll
+                for (int __k = 0; __k < 4; ++__k) {
                     const int __t = __t0 + __k * 256 + __lid * 4;
                     int __row = 0, __past = 256;       // the last row that starts at or before __t
                     #pragma unroll
@@ -121,87 +257,21 @@ _spmv_kernel_loop_1_group(
                         const int __mid = (__row + __past) >> 1;
                         if (__kp[__mid] <= __t) __row = __mid; else __past = __mid;
                     }
-                    int __jq[4];
                     #pragma unroll
                     for (int __q = 0; __q < 4; ++__q) {
                         if (__t + __q < __kept) while (__kp[__row + 1] <= __t + __q) ++__row;
-                        __jq[__q] = __lp[__row] + (__t + __q - __kp[__row]);
+                        const int __cq = __c[__k][__q];
+                        const int __sq = __cq >> __shiftc;          // negative past the end (and for negative indices: such elements are dropped)
+                        int __pos = 0;
+                        #pragma unroll
+                        for (int __s = 0; __s < 8; ++__s) {
+                            const unsigned long long __m = __ballot(__sq == __s);
+                            if (__sq == __s) __pos = __at[__s] + __popcll(__m & __below);
+                            __at[__s] += __popcll(__m);
+                        }
+                        if (__sq >= 0 && __sq < 8)
+                            __ent[__pos] = (long long)(((unsigned long long)(((unsigned)__row << 22) | (unsigned)(__cq & __cmask)) << 32) | (unsigned long long)(unsigned)__v[__k][__q]);
                     }
-                    const bool __run = __t + 4 <= __kept && __jq[3] == __jq[0] + 3;       // four elements in a row of the arrays
-                    if (__run) __c[__k] = appy::vload<int, 4>(A_indices + __jq[0]);
-                    else {
-                    #pragma unroll
-                        for (int __q = 0; __q < 4; ++__q) __c[__k][__q] = __t + __q < __kept ? A_indices[__jq[__q]] : -1;
-                    }
-                }
-            }
-            #pragma unroll
-            for (int __k = 0; __k < 4; ++__k) {
-                #pragma unroll
-                for (int __q = 0; __q < 4; ++__q)
-                #pragma unroll
-                    for (int __s = 0; __s < 8; ++__s) __cnt[__s] += __popcll(__ballot((__c[__k][__q] >> __shiftc) == __s));
-            }
-        }
-        __at[0] = __first;
-        #pragma unroll
-        for (int __s = 0; __s < 8; ++__s) __at[__s + 1] = __at[__s] + __cnt[__s];
-        #pragma unroll
-        for (int __s = 0; __s <= 8; ++__s) if (__lid == __s) __desc[__b * 9 + __s] = __at[__s];
-        for (int __t0 = 0; __t0 < __kept; __t0 += 1024) {
-            appy::vec<int, 4>::type __c[4], __v[4];
-            #pragma unroll
-            for (int __k = 0; __k < 4; ++__k) {
-                {
-                    const int __t = __t0 + __k * 256 + __lid * 4;
-                    int __row = 0, __past = 256;       // the last row that starts at or before __t
-                    #pragma unroll
-                    for (int __it = 0; __it < 8; ++__it) {
-                        const int __mid = (__row + __past) >> 1;
-                        if (__kp[__mid] <= __t) __row = __mid; else __past = __mid;
-                    }
-                    int __jq[4];
-                    #pragma unroll
-                    for (int __q = 0; __q < 4; ++__q) {
-                        if (__t + __q < __kept) while (__kp[__row + 1] <= __t + __q) ++__row;
-                        __jq[__q] = __lp[__row] + (__t + __q - __kp[__row]);
-                    }
-                    const bool __run = __t + 4 <= __kept && __jq[3] == __jq[0] + 3;       // four elements in a row of the arrays
-                    if (__run) __c[__k] = appy::vload<int, 4>(A_indices + __jq[0]);
-                    else {
-                    #pragma unroll
-                        for (int __q = 0; __q < 4; ++__q) __c[__k][__q] = __t + __q < __kept ? A_indices[__jq[__q]] : -1;
-                    }
-                    if (__run) __v[__k] = appy::vload<int, 4>(reinterpret_cast<const int*>(A_data) + __jq[0]);
-                    else {
-                    #pragma unroll
-                        for (int __q = 0; __q < 4; ++__q) __v[__k][__q] = __t + __q < __kept ? reinterpret_cast<const int*>(A_data)[__jq[__q]] : 0;
-                    }
-                }
-            }
-            #pragma unroll
-            for (int __k = 0; __k < 4; ++__k) {
-                const int __t = __t0 + __k * 256 + __lid * 4;
-                int __row = 0, __past = 256;       // the last row that starts at or before __t
-                #pragma unroll
-                for (int __it = 0; __it < 8; ++__it) {
-                    const int __mid = (__row + __past) >> 1;
-                    if (__kp[__mid] <= __t) __row = __mid; else __past = __mid;
-                }
-                #pragma unroll
-                for (int __q = 0; __q < 4; ++__q) {
-                    if (__t + __q < __kept) while (__kp[__row + 1] <= __t + __q) ++__row;
-                    const int __cq = __c[__k][__q];
-                    const int __sq = __cq >> __shiftc;          // negative past the end (and for negative indices: such elements are dropped)
-                    int __pos = 0;
-                    #pragma unroll
-                    for (int __s = 0; __s < 8; ++__s) {
-                        const unsigned long long __m = __ballot(__sq == __s);
-                        if (__sq == __s) __pos = __at[__s] + __popcll(__m & __below);
-                        __at[__s] += __popcll(__m);
-                    }
-                    if (__sq >= 0 && __sq < 8)
-                        __ent[__pos] = (long long)(((unsigned long long)(((unsigned)__row << 22) | (unsigned)(__cq & __cmask)) << 32) | (unsigned long long)(unsigned)__v[__k][__q]);
                 }
             }
         }
