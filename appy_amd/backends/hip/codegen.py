@@ -1651,7 +1651,10 @@ class Launch:
             return False
         self.nsplit = PLAN_GROUPS * split
         self.plan = plan
-        seq = [(cells, self._argument_block(cells, vals, arrays, lo, hi), (plan.ncell * split, 1, 1), (1024, 1, 1)),
+        # one workgroup per CU (their LDS allows no more), a multiple of eight so that a workgroup stays with one column
+        # range; each walks the tiles of its runs as one sequence
+        grid = min(plan.ncell * split, int(loop.options.get("hip_plan_grid") or max(8, self.hw.cus // 8 * 8)))
+        seq = [(cells, self._argument_block(cells, vals, arrays, lo, hi), (max(8, grid // 8 * 8), 1, 1), (1024, 1, 1)),
                (sums, self._argument_block(sums, vals, arrays, lo, hi), (max(1, min(4096, -(-n // 256))), 1, 1), (256, 1, 1))]
         self.sequence = seq
         self.kernel, self.spec = cells, cells.src.spec
@@ -2027,7 +2030,7 @@ def codegen(loop_source, loop_name, val_map, options):
     key = (loop_source, loop_name, _signature(val_map), options.get("hip_spec") and repr(options.get("hip_spec")),
            options.get("hip_max_blocks"), bool(options.get("check_bounds")), bool(options.get("hip_bins", True)),
            bool(options.get("hip_group", True)), options.get("hip_group_rows"), bool(options.get("hip_hints", True)),
-           options.get("hip_reuse", True), options.get("hip_plan_split"), options.get("fn_name"))
+           options.get("hip_reuse", True), options.get("hip_plan_split"), options.get("hip_plan_grid"), options.get("fn_name"))
     # `clear_cache=True` regenerates the loop on every call instead of using the cached kernel
     # (reference: appy/backends/metal/codegen.py:23)
     fresh = bool(options.get("clear_cache"))

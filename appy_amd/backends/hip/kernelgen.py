@@ -3085,60 +3085,100 @@ class KernelBuilder:
         w("const unsigned __cmask = (1u << __colbits) - 1u;")
         w("const unsigned __xlast = (unsigned)(__nx - 1);")
         w("const char* __xb = reinterpret_cast<const char*>(" + xc + ");")
-        w("// a cell may be shared by __split workgroups, each with a run of its tiles and a slot of its own for the sums")
-        w("for (appy::i64 __vc = blockIdx.x; __vc < __ncell * __split; __vc += gridDim.x) {")
-        self.ind += 1
-        w("const int __g = (int)(__vc & 7);")
-        w("const appy::i64 __b = (__vc >> 3) / __split;")
-        w("const int __part = (int)((__vc >> 3) % __split);")
-        w("const appy::i64 __cell = __b * 8 + __g;")
-        w("const appy::i64 __ce = __cstart[__cell + 1];")
-        w("const int __nta = (int)(__tbase[__cell + 1] - __tbase[__cell]);")
-        w("const int __tlo = (int)((appy::i64)__part * __nta / __split), __nt = (int)((appy::i64)(__part + 1) * __nta / __split) - __tlo;")
-        w(f"const appy::i64 __cs = (appy::i64)__cstart[__cell] + (appy::i64)__tlo * {TILE};")
-        w("const unsigned __x0 = (unsigned)(__g * __gwidth);")
-        w("// tile t of this workgroup: elements at __eb + t * TILE, row stream at __sb + t * SEG")
-        w("const char* __eb = reinterpret_cast<const char*>(__ent + __cs);")
-        w("const char* __sb = reinterpret_cast<const char*>(__rstream + ((__cs >> 1) + 4 * ((appy::i64)__tbase[__cell] + __tlo)));")
+        w("// A cell may be shared by __split workgroups, each with a run of its tiles and a slot of its own for the sums: a")
+        w("// run is numbered (block * __split + part) * 8 + range.  The workgroup takes the runs blockIdx.x, blockIdx.x +")
+        w("// gridDim.x, ... (the grid is a multiple of eight workgroups: all of them read the same range) and walks their tiles")
+        w("// as one sequence, so that the loads of a run's first tiles travel while the run before it is finished.")
+        w("const unsigned __nrun = (unsigned)(__ncell * __split), __spl = (unsigned)__split;")
+        w("const unsigned __g = blockIdx.x & 7u;")
+        w("const unsigned __x0 = __g * (unsigned)__gwidth;")
         w("#pragma unroll")
         w(f"for (int __k = 0; __k < {ROWS // 1024}; ++__k) __sum[__k * 1024 + __tid] = 0;")
         w(f"unsigned long long __e0[{U}], __e1[{U}], __e2[{U}];")
         w(f"{x.elem_c} __xv[{U}], __x1[{U}];")
         w(f"unsigned __r0[{H}], __r1[{H}];")
         w("unsigned __da0, __db0, __da1, __db1;")
-        w("unsigned __h0, __h1, __h2;")
+        w("unsigned __h0, __h1, __hv2;        // headers of the tiles in flight (the newest as it was loaded, in a vector register)")
+        w("// the tile the next load fetches: run, tile within the run; of the run: its tiles, where its elements and its row")
+        w("// stream start, the elements from there to the end of the cell")
+        w("unsigned __vc = blockIdx.x, __tt = 0, __nt = 0;")
+        w("appy::i64 __eb = 0, __sb = 0;      // (in bytes from the start of the elements and of the row stream)")
+        w("const char* __entb = reinterpret_cast<const char*>(__ent);")
+        w("const char* __rsb = reinterpret_cast<const char*>(__rstream);")
+        w("appy::i64 __left = 0;")
+        w("// of the tiles in flight (0: the one that is added up, 1: the one whose gathers travel, 2: the one just requested):")
+        w("// whether it exists, its elements, whether it ends its run, the run, its part of the row stream")
+        w("bool __in0, __in1, __in2, __end0, __end1, __end2, __any0, __any1, __any2;")
+        w("unsigned __cnt0, __cnt1, __cnt2, __run0, __run1, __run2;")
+        w("appy::i64 __ps0, __ps1, __ps2;")
 
-        # (a tile beyond the end of the workgroup's run of tiles is read all the same - one position for every lane,
-        #  so that it costs one request per instruction - and never used)
-        def load_tile(dst, hdr, t):
-            w(f"{{ const bool __in = ({t}) < __nt;")
-            w(f"  const char* __p = __eb + (appy::i64)({t}) * {TILE * 8};")
+        def enter_run():
+            """Where the run __vc lies (when there is such a run)."""
+            w("if (__vc < __nrun) {")
+            w("    const unsigned __b = (__vc >> 3) / __spl, __part = (__vc >> 3) % __spl;")
+            w("    const appy::i64 __cell = (appy::i64)__b * 8 + __g;")
+            w("    const unsigned __nta = __tbase[__cell + 1] - __tbase[__cell];")
+            w("    const unsigned __tlo = __part * __nta / __spl;        // (at most 32 parts, and tiles of thousands of elements)")
+            w("    __nt = (__part + 1) * __nta / __spl - __tlo;")
+            w(f"    const appy::i64 __cs = (appy::i64)__cstart[__cell] + (appy::i64)__tlo * {TILE};")
+            w("    __left = (appy::i64)__cstart[__cell + 1] - __cs;")
+            w("    __eb = __cs * 8;")
+            w("    __sb = ((__cs >> 1) + 4 * ((appy::i64)__tbase[__cell] + __tlo)) * 4;")
+            w("} else {")
+            w("    __nt = 0;")
+            w("}")
+
+        # (a tile that does not exist - past the last run, or the one turn of a run without tiles - is read all the
+        #  same: one position for every lane, so that it costs one request per instruction, and never used)
+        def load_tile(dst):
+            """Requests the header and the elements of the next tile of the sequence into stage 2, and steps on.
+            (The header is asked for first and as a vector load, and turned into a scalar only when the tile moves on
+            to stage 1: a wait for it then covers no load younger than it, and none that misses.)"""
+            w("{")
+            w("  __any2 = __vc < __nrun; __in2 = __any2 && __tt < __nt; __end2 = __tt + 1 >= __nt; __run2 = __vc;")
+            w(f"  const char* __p = __entb + appy::uniform_i64(__in2 ? __eb + (appy::i64)__tt * {TILE * 8} : 0);")
+            w(f"  __ps2 = appy::uniform_i64(__in2 ? __sb + (appy::i64)__tt * {SEG * 4} : 0);")
+            w("  __hv2 = *reinterpret_cast<const unsigned*>(__rsb + __ps2 + appy::lane_offset(0u));")
+            w(f"  const appy::i64 __l = __left - (appy::i64)__tt * {TILE};")
+            w(f"  __cnt2 = __in2 ? (unsigned)(__l < {TILE} ? __l : {TILE}) : 0u;")
             w("#pragma unroll")
             w(f"  for (int __u = 0; __u < {U}; ++__u)")
-            w(f"      {dst}[__u] = __builtin_nontemporal_load(reinterpret_cast<const unsigned long long*>(__p + (__in ? (unsigned)((__u * 1024 + __tid) * 8) : 0u)));")
-            w(f"  {hdr} = __builtin_amdgcn_readfirstlane(*reinterpret_cast<const unsigned*>(__sb + (appy::i64)({t}) * {SEG * 4})); }}")
+            w(f"      {dst}[__u] = __builtin_nontemporal_load(reinterpret_cast<const unsigned long long*>(__p + appy::lane_offset(__in2 ? (unsigned)((__u * 1024 + __tid) * 8) : 0u)));")
+            w("  if (__any2) {")
+            w("      if (!__end2) ++__tt;")
+            w("      else {")
+            w("          __vc += gridDim.x; __tt = 0;")
+            self.ind += 3
+            enter_run()
+            self.ind -= 3
+            w("      }")
+            w("  }")
+            w("}")
 
-        def load_rows(dst, da, db, hdr, t):
+        def load_rows(dst, da, db, hdr, inn, ps):
             """Row numbers of the slots this lane adds up, and the first run of slots it may have to walk."""
-            w(f"{{ const bool __in = ({t}) < __nt;")
-            w(f"  const char* __p = __sb + (appy::i64)({t}) * {SEG * 4};")
+            w("{")
             w("#pragma unroll")
             w(f"  for (int __u = 0; __u < {H}; ++__u)")
-            w(f"      {dst}[__u] = __builtin_nontemporal_load(reinterpret_cast<const unsigned*>(__p + (__in ? (unsigned)((1 + __u * 1024 + __tid) * 4) : 0u)));")
+            w(f"      {dst}[__u] = __builtin_nontemporal_load(reinterpret_cast<const unsigned*>(__rsb + {ps} + appy::lane_offset({inn} ? (unsigned)((1 + __u * 1024 + __tid) * 4) : 0u)));")
             w(f"  const unsigned __runs = ({hdr} >> 16);")
-            w(f"  const char* __q = __p + (__in ? (appy::i64)(1 + ((({hdr} & 0xffffu) + 1) >> 1)) * 4 : 0);     // (a header beyond the run of tiles may hold anything)")
-            w("  const unsigned __at = __in && __tid < __runs ? __tid * 4 : 0u;        // (lanes without a run: one position)")
+            w(f"  const char* __q = __rsb + ({ps} + ({inn} ? (appy::i64)(1 + ((({hdr} & 0xffffu) + 1) >> 1)) * 4 : 0));     // (the header of a tile that does not exist may hold anything)")
+            w(f"  const unsigned __at = appy::lane_offset({inn} && __tid < __runs ? __tid * 4 : 0u);        // (lanes without a run: one position)")
             w(f"  {da} = *reinterpret_cast<const unsigned*>(__q + __at);")
             w(f"  {db} = *reinterpret_cast<const unsigned*>(__q + __at + 4); }}")
 
-        def gather(dst, src, t):
-            w(f"{{ const bool __in = ({t}) < __nt;")
+        def gather(dst, src, inn):
+            w("{")
             w("#pragma unroll")
             w(f"  for (int __u = 0; __u < {U}; ++__u) {{")
             w(f"    unsigned __c = __x0 + ((unsigned)({src}[__u] >> 32) & __cmask);")
             w("    __c = __c < __xlast ? __c : __xlast;        // (what was read beyond the cell may hold anything)")
-            w(f"    {dst}[__u] = *reinterpret_cast<const {x.elem_c}*>(__xb + (__in ? (unsigned)(__c << 2) : 0u));")
+            w(f"    {dst}[__u] = *reinterpret_cast<const {x.elem_c}*>(__xb + appy::lane_offset({inn} ? (unsigned)(__c << 2) : 0u));")
             w("  } }")
+
+        def shift(frm, to):
+            w(f"__in{to} = __in{frm}; __end{to} = __end{frm}; __any{to} = __any{frm}; __cnt{to} = __cnt{frm}; "
+              f"__run{to} = __run{frm}; __ps{to} = __ps{frm};")
 
         def add_run(d, d1):
             w(f"{{ const int __row = (int)({d} & {ROWS - 1}u), __from = (int)({d} >> {RB}), __to = (int)({d1} >> {RB});")
@@ -3153,17 +3193,20 @@ class KernelBuilder:
             w("  }")
             w("  __sum[__row] = __acc; }")
 
-        load_tile("__e0", "__h0", "0")
-        load_tile("__e1", "__h1", "1")
-        load_rows("__r0", "__da0", "__db0", "__h0", "0")
-        gather("__xv", "__e0", "0")
+        enter_run()
+        load_tile("__e0")
+        w("__h0 = __builtin_amdgcn_readfirstlane(__hv2);")
+        shift(2, 0)
+        load_tile("__e1")
+        w("__h1 = __builtin_amdgcn_readfirstlane(__hv2);")
+        shift(2, 1)
+        load_rows("__r0", "__da0", "__db0", "__h0", "__in0", "__ps0")
+        gather("__xv", "__e0", "__in0")
         w("__syncthreads();")
-        w("for (int __t = 0; __t < __nt; ++__t) {")
+        w("while (__any0) {")
         self.ind += 1
-        w(f"const appy::i64 __left = __ce - (__cs + (appy::i64)__t * {TILE});")
-        w(f"const unsigned __cnt = (unsigned)(__left < {TILE} ? __left : {TILE});")
-        w("const unsigned __ns = __h0 & 0xffffu, __nm = __h0 >> 16;")
-        w(f"if (__cnt == {TILE}u) {{")
+        w("const unsigned __ns = __in0 ? __h0 & 0xffffu : 0u, __nm = __in0 ? __h0 >> 16 : 0u;")
+        w(f"if (__cnt0 == {TILE}u) {{")
         w("#pragma unroll")
         w(f"    for (int __u = 0; __u < {U}; ++__u) {{")
         w(f"        {P} __val;")
@@ -3175,13 +3218,13 @@ class KernelBuilder:
         w(f"    for (int __u = 0; __u < {U}; ++__u) {{")
         w(f"        {P} __val;")
         w("        " + value("__e0[__u]", "__xv[__u]"))
-        w("        if (__u * 1024 + __tid < __cnt) __prod[(unsigned)(__e0[__u] >> 32) >> __colbits] = __val;")
+        w("        if (__u * 1024 + __tid < __cnt0) __prod[(unsigned)(__e0[__u] >> 32) >> __colbits] = __val;")
         w("    }")
         w("}")
         w("// the elements of the tile after the next, the row numbers and the gathers of the next one travel while this one is added up")
-        load_tile("__e2", "__h2", "__t + 2")
-        load_rows("__r1", "__da1", "__db1", "__h1", "__t + 1")
-        gather("__x1", "__e1", "__t + 1")
+        load_tile("__e2")
+        load_rows("__r1", "__da1", "__db1", "__h1", "__in1", "__ps1")
+        gather("__x1", "__e1", "__in1")
         w("__syncthreads();")
         w("{")
         w(f"    {P} __sa[{H}], __sb_[{H}];")
@@ -3206,7 +3249,7 @@ class KernelBuilder:
         self.ind -= 1
         w("}")
         w("if (__nm > 1024) {")
-        w(f"    const unsigned* __runs = reinterpret_cast<const unsigned*>(__sb + (appy::i64)__t * {SEG * 4}) + 1 + ((__ns + 1) >> 1);")
+        w("    const unsigned* __runs = reinterpret_cast<const unsigned*>(__rsb + __ps0) + 1 + ((__ns + 1) >> 1);")
         w("    for (unsigned __m = __tid + 1024; __m < __nm; __m += 1024) {")
         w("        const unsigned __d = __runs[__m], __d1 = __runs[__m + 1];")
         self.ind += 2
@@ -3217,22 +3260,30 @@ class KernelBuilder:
         self.ind -= 1
         w("}")
         w("__syncthreads();")
+        w("if (__end0) {")
+        self.ind += 1
+        w("// the run is through: its sums go out and start again at zero (every lane clears what it has read itself; the next")
+        w("// tile's terms are added after the barrier that follows their scatter)")
+        w("const unsigned __b = (__run0 >> 3) / __spl, __part = (__run0 >> 3) % __spl;")
+        w(f"{P}* __out = reinterpret_cast<{P}*>(__scratch) + ((appy::i64)__part * 8 + __g) * __n + (appy::i64)__b * {ROWS};")
+        w(f"if (((appy::i64)__b + 1) * {ROWS} <= __n) {{")
+        w("#pragma unroll")
+        w(f"    for (int __k = 0; __k < {ROWS // 1024}; ++__k) {{ __out[__k * 1024 + __tid] = __sum[__k * 1024 + __tid]; __sum[__k * 1024 + __tid] = 0; }}")
+        w("} else {")
+        w(f"    for (int __k = 0; __k < {ROWS // 1024}; ++__k) {{")
+        w(f"        if ((appy::i64)__b * {ROWS} + __k * 1024 + __tid < __n) __out[__k * 1024 + __tid] = __sum[__k * 1024 + __tid];")
+        w("        __sum[__k * 1024 + __tid] = 0;")
+        w("    }")
+        w("}")
+        self.ind -= 1
+        w("}")
         w("#pragma unroll")
         w(f"for (int __u = 0; __u < {U}; ++__u) {{ __e0[__u] = __e1[__u]; __e1[__u] = __e2[__u]; __xv[__u] = __x1[__u]; }}")
         w("#pragma unroll")
         w(f"for (int __u = 0; __u < {H}; ++__u) __r0[__u] = __r1[__u];")
-        w("__h0 = __h1; __h1 = __h2; __da0 = __da1; __db0 = __db1;")
-        self.ind -= 1
-        w("}")
-        w(f"{P}* __out = reinterpret_cast<{P}*>(__scratch) + ((appy::i64)__part * 8 + __g) * __n + __b * {ROWS};")
-        w(f"if ((__b + 1) * {ROWS} <= __n) {{")
-        w("#pragma unroll")
-        w(f"    for (int __k = 0; __k < {ROWS // 1024}; ++__k) __out[__k * 1024 + __tid] = __sum[__k * 1024 + __tid];")
-        w("} else {")
-        w(f"    for (int __k = 0; __k < {ROWS // 1024}; ++__k)")
-        w(f"        if (__b * {ROWS} + __k * 1024 + __tid < __n) __out[__k * 1024 + __tid] = __sum[__k * 1024 + __tid];")
-        w("}")
-        w("__syncthreads();")
+        w("__h0 = __h1; __h1 = __builtin_amdgcn_readfirstlane(__hv2); __da0 = __da1; __db0 = __db1;")
+        shift(1, 0)
+        shift(2, 1)
         self.ind -= 1
         w("}")
 
@@ -3412,10 +3463,12 @@ class KernelBuilder:
             params.append(Param("__lbits", "const int __lbits", C.c_int32, "lbits"))
             params.append(Param("__flag", "long long* __flag", C.c_void_p, "flag"))
         if sp.aux == "xcells":
-            params.append(Param("__ent", "const unsigned long long* __ent", C.c_void_p, "ent"))
-            params.append(Param("__cstart", "const unsigned* __cstart", C.c_void_p, "cstart"))
-            params.append(Param("__tbase", "const unsigned* __tbase", C.c_void_p, "tbase"))
-            params.append(Param("__rstream", "const unsigned* __rstream", C.c_void_p, "rstream"))
+            # (nothing the kernel stores to overlaps the plan: with `__restrict__` the starts of the cells, read once per run
+            #  of tiles, come through the scalar cache and no vector load in flight has to be waited for)
+            params.append(Param("__ent", "const unsigned long long* __restrict__ __ent", C.c_void_p, "ent"))
+            params.append(Param("__cstart", "const unsigned* __restrict__ __cstart", C.c_void_p, "cstart"))
+            params.append(Param("__tbase", "const unsigned* __restrict__ __tbase", C.c_void_p, "tbase"))
+            params.append(Param("__rstream", "const unsigned* __restrict__ __rstream", C.c_void_p, "rstream"))
             params.append(Param("__ncell", "const appy::i64 __ncell", C.c_int64, "ncell"))
             params.append(Param("__split", "const appy::i64 __split", C.c_int64, "split"))
             params.append(Param("__gwidth", "const appy::i64 __gwidth", C.c_int64, "gwidth"))

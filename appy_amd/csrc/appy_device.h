@@ -273,6 +273,23 @@ __device__ __forceinline__ i64 team_lane_below(i64 v, int lane) {
     return (i64)(((unsigned long long)hi << 32) | (unsigned long long)lo);
 }
 
+// A number that is the same in every lane, kept in scalar registers whatever it was computed from: with such an offset
+// from a kernel argument, loads at `base + offset + lane offset` take the scalar-base form of the memory instructions
+// (one 32-bit register per lane for the lane's offset instead of a 64-bit address worked out per lane).
+__device__ __forceinline__ unsigned lane_offset(unsigned v) {
+    // (the compiler may not look through this: a lane's offset stays one 32-bit register next to the scalar base, where it
+    //  would otherwise widen offsets chosen under a condition to 64 bits and add the base lane by lane)
+    asm("" : "+v"(v));
+    return v;
+}
+
+__device__ __forceinline__ i64 uniform_i64(i64 v) {
+    const unsigned long long u = (unsigned long long)v;
+    const unsigned lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(u & 0xffffffffull));
+    const unsigned hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(u >> 32));
+    return (i64)(((unsigned long long)hi << 32) | (unsigned long long)lo);
+}
+
 // Between two loops that the lanes of one wavefront share: what any lane stored in the first is
 // visible to every lane in the second, and nothing of the second is started before the first is
 // through.  The hardware runs the lanes in lockstep; this keeps the compiler from moving one
