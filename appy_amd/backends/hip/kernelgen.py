@@ -3206,6 +3206,7 @@ class KernelBuilder:
         w("while (__any0) {")
         self.ind += 1
         w("const unsigned __ns = __in0 ? __h0 & 0xffffu : 0u, __nm = __in0 ? __h0 >> 16 : 0u;")
+        load_tile("__e2")
         w(f"if (__cnt0 == {TILE}u) {{")
         w("#pragma unroll")
         w(f"    for (int __u = 0; __u < {U}; ++__u) {{")
@@ -3222,7 +3223,6 @@ class KernelBuilder:
         w("    }")
         w("}")
         w("// the elements of the tile after the next, the row numbers and the gathers of the next one travel while this one is added up")
-        load_tile("__e2")
         load_rows("__r1", "__da1", "__db1", "__h1", "__in1", "__ps1")
         gather("__x1", "__e1", "__in1")
         w("__syncthreads();")

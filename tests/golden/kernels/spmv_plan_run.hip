@@ -148,22 +148,6 @@ _spmv_kernel_loop_1_xcells(
     __syncthreads();
     while (__any0) {
         const unsigned __ns = __in0 ? __h0 & 0xffffu : 0u, __nm = __in0 ? __h0 >> 16 : 0u;
-        if (__cnt0 == 6144u) {
-        #pragma unroll
-            for (int __u = 0; __u < 6; ++__u) {
-                float __val;
-                { const float __cv = __int_as_float((int)(unsigned)(__e0[__u])); const float __cx = __xv[__u]; __val = (__cv * __cx); }
-                __prod[(unsigned)(__e0[__u] >> 32) >> __colbits] = __val;
-            }
-        } else {
-        #pragma unroll
-            for (int __u = 0; __u < 6; ++__u) {
-                float __val;
-                { const float __cv = __int_as_float((int)(unsigned)(__e0[__u])); const float __cx = __xv[__u]; __val = (__cv * __cx); }
-                if (__u * 1024 + __tid < __cnt0) __prod[(unsigned)(__e0[__u] >> 32) >> __colbits] = __val;
-            }
-        }
-        // the elements of the tile after the next, the row numbers and the gathers of the next one travel while this one is added up
         {
           __any2 = __vc < __nrun; __in2 = __any2 && __tt < __nt; __end2 = __tt + 1 >= __nt; __run2 = __vc;
           const char* __p = __entb + appy::uniform_i64(__in2 ? __eb + (appy::i64)__tt * 49152 : 0);
@@ -194,6 +178,22 @@ _spmv_kernel_loop_1_xcells(
               }
           }
         }
+        if (__cnt0 == 6144u) {
+        #pragma unroll
+            for (int __u = 0; __u < 6; ++__u) {
+                float __val;
+                { const float __cv = __int_as_float((int)(unsigned)(__e0[__u])); const float __cx = __xv[__u]; __val = (__cv * __cx); }
+                __prod[(unsigned)(__e0[__u] >> 32) >> __colbits] = __val;
+            }
+        } else {
+        #pragma unroll
+            for (int __u = 0; __u < 6; ++__u) {
+                float __val;
+                { const float __cv = __int_as_float((int)(unsigned)(__e0[__u])); const float __cx = __xv[__u]; __val = (__cv * __cx); }
+                if (__u * 1024 + __tid < __cnt0) __prod[(unsigned)(__e0[__u] >> 32) >> __colbits] = __val;
+            }
+        }
+        // the elements of the tile after the next, the row numbers and the gathers of the next one travel while this one is added up
         {
         #pragma unroll
           for (int __u = 0; __u < 3; ++__u)
