@@ -387,6 +387,43 @@ def test_a_part_of_the_rows_and_rows_with_many_elements_in_one_tile(env):
         assert _planned(_loop("part").last_launch)
 
 
+@pytest.mark.parametrize("grid,split", [(8, 3), (16, 1), (64, 5)])
+def test_few_workgroups_walk_many_cells_one_after_the_other(env, grid, split):
+    """The kernel that runs a plan gives every workgroup a sequence of runs of tiles (a cell, or a part of one)
+    and walks their tiles as one sequence: with few workgroups each walks many, among them cells without any
+    element (all columns of a block of rows in one range) and a last block of rows that is not full.  The result
+    must not depend on how the runs are dealt out."""
+    torch, _k = env
+    rng = np.random.default_rng(17)
+    m, n = 3 * 32768 + 1234, 1 << 21
+    ln = rng.integers(0, 40, m).astype(np.int64)
+    ln[32768:65536] = 12
+    indptr = np.zeros(m + 1, dtype=np.int64)
+    np.cumsum(ln, out=indptr[1:])
+    cols = rng.integers(0, n, int(indptr[-1]))
+    lo, hi = int(indptr[32768]), int(indptr[65536])
+    cols[lo:hi] = rng.integers(5 * (n // 8), 6 * (n // 8), hi - lo)          # the second block of rows: one range only
+    data = rng.standard_normal(len(cols), dtype=np.float32)
+    x = rng.standard_normal(n, dtype=np.float32)
+    indptr, cols = indptr.astype(np.int32), cols.astype(np.int32)
+    ref, budget = vo.spmv_csr(data, indptr, cols, x, (m, n))
+    td, tp, ti, tx = _gpu(torch, data, indptr, cols, x)
+    dealt = selfcheck.kernels(hip_reuse="now", hip_plan_grid=grid, hip_plan_split=split)
+    usual = selfcheck.kernels(hip_reuse="now", hip_plan_split=split)
+    ys = []
+    for k in (dealt, usual):
+        for it in range(2):
+            y = k.spmv(td, tp, ti, tx, m, n)
+            yh = y.cpu().numpy()
+            assert np.all(np.abs(yh - ref) <= TOL * budget)
+            ys.append(y)
+        launch = _loop(hip_plan_split=split).last_launch              # (the loop that ran last)
+        assert _planned(launch) and launch.plan.split == split and launch.plan.ncell == 32
+        assert launch.grid[0] == (grid if k is dealt else min(32 * split, launch.hw.cus // 8 * 8))
+    assert all(torch.equal(ys[0], y) for y in ys[1:])
+    appy.release()
+
+
 def test_plans_are_bounded_released_and_kept_out_of_the_way(env, monkeypatch):
     torch, k = env
     m, n = 40_000, 1 << 20
