@@ -1046,6 +1046,8 @@ class CompiledLoop:
                 # same tensors (address, shape, strides), same scalars, same stream: the staged
                 # launch of last time is still exact, so only the launch itself is repeated
                 _ensure_device(plan.device)
+                if _live_plans and plan.stored_extents:
+                    drop_plans_overlapping(plan.stored_extents)
                 if plan.small_fixed:
                     # host arrays of a few bytes (`shared()` scalars): through the slots the plan keeps for them
                     with self._lock:        # the slots and the argument block are shared by all replays of this plan
@@ -1281,6 +1283,9 @@ class Launch:
         for _m, dptr, host, stored, name in self.mirrored:
             extents.append((name, dptr, host.nbytes, stored))
         restrict = not _overlaps(extents)
+        # (what this launch stores into: a launch repeated without being staged again, and the replay of a graph it was
+        #  recorded into, must drop the row plans built from that memory just as this staging does)
+        self.stored_extents = [e for e in extents if e[3]]
         drop_plans_overlapping(extents)
 
         # -- kernel variant, argument block, grid
@@ -1893,6 +1898,7 @@ class Launch:
         if g is not None:
             g.launches += 1
             g.keepalive.extend(self.keepalive)
+            g.stored_extents.extend(self.stored_extents)
             for m, _dptr, _host, stored, _name in self.mirrored:
                 if m not in g.used_mirrors:
                     g.used_mirrors.append(m)

@@ -45,6 +45,7 @@ class graph:
         self.stored_mirrors = []   # resident host arrays the recorded kernels store to
         self.used_mirrors = []     # resident host arrays the recorded kernels touch at all
         self.keepalive = []        # tensors whose memory the graph refers to
+        self.stored_extents = []   # (name, address, bytes, True) of the memory the recorded kernels store into
 
     # ---- capture ----------------------------------------------------------------------
     def __enter__(self):
@@ -85,6 +86,11 @@ class graph:
         if not self.exec:
             raise RuntimeError("the graph has not been captured")
         s = self.stream if stream is None else int(stream)
+        if self.stored_extents:
+            # orders of CSR elements kept by other loops were built from the contents of their arrays: what this replay
+            # stores into is no longer what they were built from
+            from .backends.hip import codegen as _cg
+            _cg.drop_plans_overlapping(self.stored_extents)
         rt.graph_launch(self.exec, s)
         for m in self.used_mirrors:
             m.stream, m.busy = s, True
@@ -102,6 +108,7 @@ class graph:
             rt.stream_destroy(self.stream)
             self.stream = 0
         self.keepalive = []
+        self.stored_extents = []
         self.stored_mirrors = []
         self.used_mirrors = []
 

@@ -187,6 +187,45 @@ def test_arrays_stored_to_by_another_loop_drop_the_plan(env):
     _check(y, d2, indptr, indices, 2.0 * x, m, n)
 
 
+def test_stores_that_are_not_staged_again_drop_the_plan_too(env):
+    """A call with the same tensors and scalars as an earlier one repeats that call's launch without staging it
+    again, and a graph replays what was recorded: both must drop the plans built from what they store into."""
+    torch, k = env
+    m, n = 45_000, 1 << 20
+    data, indptr, indices, x = _matrix(np.full(m, 12), n, seed=4)
+    td, tp, ti, tx = _gpu(torch, data, indptr, indices, x)
+    scale_values(td, 2.0)
+    scale_values(td, 2.0)                           # from here on this call is a repeated launch
+    loop = [v[0] for kk, v in cg.code_cache.items() if kk[-1] == "scale_values"][-1]
+    assert loop._replays
+    for _ in range(3):
+        y = k.spmv(td, tp, ti, tx, m, n)
+    plan = _loop().last_launch.plan
+    assert plan is not None and plan.valid
+    _check(y, 4.0 * data, indptr, indices, x, m, n)
+    staged = cg.Launch.serial
+    scale_values(td, 2.0)
+    assert cg.Launch.serial == staged               # nothing was staged
+    assert not plan.valid
+    y = k.spmv(td, tp, ti, tx, m, n)
+    assert _loop().last_launch.plan is None
+    _check(y, 8.0 * data, indptr, indices, x, m, n)
+    # the same through a graph
+    with appy.graph() as g:
+        scale_values(td, 0.5)
+    torch.cuda.synchronize()
+    for _ in range(3):
+        y = k.spmv(td, tp, ti, tx, m, n)
+    plan = _loop().last_launch.plan
+    assert plan is not None and plan.valid
+    g.launch(torch.cuda.current_stream().cuda_stream)
+    assert not plan.valid
+    y = k.spmv(td, tp, ti, tx, m, n)
+    assert _loop().last_launch.plan is None
+    _check(y, 4.0 * data, indptr, indices, x, m, n)
+    g.close()
+
+
 def test_another_matrix_at_the_same_addresses(env):
     torch, k = env
     m, n = 45_000, 1 << 20
