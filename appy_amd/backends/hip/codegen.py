@@ -478,6 +478,7 @@ class CompiledLoop:
         self._hints = {}    # device -> (address, ctypes view) of page-locked words the binned kernels report to
         self._hint_key = {} # device -> which arrays the launch that reports next was about
         self._scratch_retired = []
+        self._scratch_gen = 0       # counts the times the scratch memory of this loop was (re)allocated or given back
         self._replays = {}  # call identity -> Launch that can simply be launched again
         self._plans = []    # row plans of this loop, most recently used last
         self._plan_seen = {}        # identity of the arrays of a launch that could use a plan -> launches seen with it
@@ -862,6 +863,7 @@ class CompiledLoop:
                     self._scratch_retired = [r for r in self._scratch_retired if r[2]]
             have = (rt.malloc(nbytes), nbytes)
             self._scratch[key] = have
+            self._scratch_gen += 1
         for ptr, st, _recorded in retired:
             rt.sync(st)
             rt.free(ptr)
@@ -894,6 +896,8 @@ class CompiledLoop:
         once the launches that use it have finished."""
         self.release_plans()
         with self._lock:
+            self._scratch_gen += 1
+            self._replays.clear()       # (staged launches name the memory that goes back)
             held, self._scratch, self._scratch_retired = (
                 [(k, p) for k, (p, _n) in self._scratch.items()] + [((None, st), p) for p, st, _rec in self._scratch_retired], {}, [])
         try:
@@ -1042,13 +1046,19 @@ class CompiledLoop:
         key = self._replay_key(args) if self._replayable else None
         if key is not None:
             plan = self._replays.get(key)
+            if plan is not None and plan.seq_replay is not None and not self._kept_order_still_true(plan, args):
+                with self._lock:
+                    self._replays.pop(key, None)
+                plan = None
             if plan is not None:
                 # same tensors (address, shape, strides), same scalars, same stream: the staged
                 # launch of last time is still exact, so only the launch itself is repeated
                 _ensure_device(plan.device)
                 if _live_plans and plan.stored_extents:
                     drop_plans_overlapping(plan.stored_extents)
-                if plan.small_fixed:
+                if plan.seq_replay is not None:
+                    plan.launch_only()      # the two kernels that run a kept order of the elements
+                elif plan.small_fixed:
                     # host arrays of a few bytes (`shared()` scalars): through the slots the plan keeps for them
                     with self._lock:        # the slots and the argument block are shared by all replays of this plan
                         for slot, i, nbytes, _stored in plan.small_fixed:
@@ -1098,6 +1108,20 @@ class CompiledLoop:
         elif plan.small_kept:
             plan.small, plan.small_kept = plan.small_kept, []
             plan._return_small_slots(wait=False)
+
+    def _kept_order_still_true(self, launch, args) -> bool:
+        """For a staged launch over a kept order of the elements (a row plan) that is about to be repeated
+        as it is: the plan still stands (no launch has stored into its arrays, it has not been given back),
+        the arrays are the very tensors it was built from with their version counters unmoved, and the
+        loop's scratch memory is the memory the launch names."""
+        plan, gen, tensors = launch.seq_replay
+        if not plan.valid or gen != self._scratch_gen:
+            return False
+        for i, ref, version in tensors:
+            t = args[i]
+            if ref() is not t or t._version != version:
+                return False
+        return True
 
     def overwrites(self, name, lo, hi, env, shape) -> bool:
         """True if this launch stores every element of array ``name`` (so that its
@@ -1318,6 +1342,7 @@ class Launch:
             self.kernel, self.spec, self.nsplit, self.scratch_ptr = loop.kernel_for(spec), spec, 1, 0
         self.scalar_fields = {}      # by-value scalar -> field of the argument block
         self.sequence = None         # binned rows: [(kernel, argument block, grid, block)] launched in this order
+        self.seq_replay = None       # for a sequence that may be repeated as it is: what must still hold then
         if spec.rows == "mixed":
             if (self._stage_planned(vals, arrays, lo, hi, spec) or self._stage_grouped(vals, arrays, lo, hi, spec)
                     or self._stage_binned(vals, arrays, lo, hi, spec)):
@@ -1664,6 +1689,13 @@ class Launch:
         self.sequence = seq
         self.kernel, self.spec = cells, cells.src.spec
         self.args, self.grid, self.block = seq[0][1], seq[0][2], seq[0][3]
+        if not loop._value_only and not self.small:
+            # a call with these same tensors may repeat the two launches without staging them again, as long as the plan
+            # stands (`CompiledLoop._kept_order_still_true`)
+            import weakref
+
+            self.seq_replay = (plan, loop._scratch_gen,
+                               [(loop.arg_names.index(nm), weakref.ref(t), t._version) for nm, t in zip(loop.plan_arrays(), tensors)])
         return True
 
     def _build_plan(self, key, tensors, shape, vals, arrays, lo, hi, spec):
@@ -1752,6 +1784,7 @@ class Launch:
             # what the launches before this one needed on this stream (8 bytes per element for the grouped form) is
             # not needed by the launches that run the plan; the stream has just been waited for
             stale = loop._scratch.pop((self.device, self.stream), None)
+            loop._scratch_gen += 1
         if stale is not None:
             rt.free(stale[0])
         with _plans_lock:
@@ -1867,7 +1900,7 @@ class Launch:
     def replayable(self) -> bool:
         """True if nothing but the kernel launch happens when this call is repeated."""
         return not (self.temps or self.mirrored or self.aliases or self.keepalive_copies or self.oob or self.capture is not None
-                    or self.second is not None or self.sequence is not None)
+                    or self.second is not None or (self.sequence is not None and self.seq_replay is None))
 
     def _no_capture(self, name, why):
         if self.capture is not None:

@@ -187,6 +187,73 @@ def test_arrays_stored_to_by_another_loop_drop_the_plan(env):
     _check(y, d2, indptr, indices, 2.0 * x, m, n)
 
 
+def test_a_launch_over_a_kept_order_is_repeated_without_staging_while_the_plan_stands(env):
+    """With the same tensors and scalars as the call before, the two kernels that run a plan are launched again as
+    they were staged; the repeat stops as soon as the plan may not be true any more: a value changed in place, a
+    store by another loop, other tensors at the same addresses, memory given back."""
+    torch, k = env
+    m, n = 45_000, 1 << 20
+    data, indptr, indices, x = _matrix(np.full(m, 12), n, seed=6)
+    td, tp, ti, tx = _gpu(torch, data, indptr, indices, x)
+    y = torch.empty(m, device="cuda")
+
+    @appy.jit
+    def into(data, indptr, indices, x, y, m):
+        #pragma parallel for
+        for i in range(m):
+            s = 0.0
+            #pragma simd
+            for j in range(indptr[i], indptr[i + 1]):
+                s += data[j] * x[indices[j]]
+            y[i] = s
+
+    def staged_by(call):
+        before = cg.Launch.serial
+        call()
+        return cg.Launch.serial - before
+
+    for _ in range(3):
+        into(td, tp, ti, tx, y, m)
+    assert _planned(_loop("into").last_launch)
+    _check(y, data, indptr, indices, x, m, n)
+    y.zero_()
+    assert staged_by(lambda: into(td, tp, ti, tx, y, m)) == 0          # repeated as it was
+    _check(y, data, indptr, indices, x, m, n)
+    tx.mul_(2.0)                                                         # the operand is not part of the plan
+    assert staged_by(lambda: into(td, tp, ti, tx, y, m)) == 0
+    _check(y, data, indptr, indices, 2.0 * x, m, n)
+    td.mul_(3.0)                                                         # a value changed in place: staged anew
+    assert staged_by(lambda: into(td, tp, ti, tx, y, m)) == 1
+    assert _loop("into").last_launch.plan is None
+    _check(y, 3.0 * data, indptr, indices, 2.0 * x, m, n)
+    for _ in range(2):
+        into(td, tp, ti, tx, y, m)
+    assert _planned(_loop("into").last_launch)
+    assert staged_by(lambda: into(td, tp, ti, tx, y, m)) == 0
+    scale_values(td, 0.5)                                                # a store by another loop
+    assert staged_by(lambda: into(td, tp, ti, tx, y, m)) == 1
+    _check(y, 1.5 * data, indptr, indices, 2.0 * x, m, n)
+    for _ in range(2):
+        into(td, tp, ti, tx, y, m)
+    assert staged_by(lambda: into(td, tp, ti, tx, y, m)) == 0
+    appy.release()                                                       # the memory the staged launch names is gone
+    assert staged_by(lambda: into(td, tp, ti, tx, y, m)) == 1
+    _check(y, 1.5 * data, indptr, indices, 2.0 * x, m, n)
+    # other tensors at the same addresses
+    for _ in range(2):
+        into(td, tp, ti, tx, y, m)
+    assert staged_by(lambda: into(td, tp, ti, tx, y, m)) == 0
+    ptr = td.data_ptr()
+    del td
+    gc.collect()
+    data2 = (data * -1.0).astype(np.float32)
+    td2 = torch.from_numpy(data2).cuda()
+    if td2.data_ptr() == ptr:
+        assert staged_by(lambda: into(td2, tp, ti, tx, y, m)) == 1
+        _check(y, data2, indptr, indices, 2.0 * x, m, n)
+    appy.release()
+
+
 def test_stores_that_are_not_staged_again_drop_the_plan_too(env):
     """A call with the same tensors and scalars as an earlier one repeats that call's launch without staging it
     again, and a graph replays what was recorded: both must drop the plans built from what they store into."""
