@@ -1046,7 +1046,7 @@ class CompiledLoop:
         key = self._replay_key(args) if self._replayable else None
         if key is not None:
             plan = self._replays.get(key)
-            if plan is not None and plan.seq_replay is not None and not self._kept_order_still_true(plan, args):
+            if plan is not None and plan.seq_replay is not None and not self._sequence_still_right(plan, args):
                 with self._lock:
                     self._replays.pop(key, None)
                 plan = None
@@ -1057,7 +1057,7 @@ class CompiledLoop:
                 if _live_plans and plan.stored_extents:
                     drop_plans_overlapping(plan.stored_extents)
                 if plan.seq_replay is not None:
-                    plan.launch_only()      # the two kernels that run a kept order of the elements
+                    plan.launch_only()      # the kernels of a CSR-like loop, as they were staged
                 elif plan.small_fixed:
                     # host arrays of a few bytes (`shared()` scalars): through the slots the plan keeps for them
                     with self._lock:        # the slots and the argument block are shared by all replays of this plan
@@ -1109,19 +1109,32 @@ class CompiledLoop:
             plan.small, plan.small_kept = plan.small_kept, []
             plan._return_small_slots(wait=False)
 
-    def _kept_order_still_true(self, launch, args) -> bool:
-        """For a staged launch over a kept order of the elements (a row plan) that is about to be repeated
-        as it is: the plan still stands (no launch has stored into its arrays, it has not been given back),
-        the arrays are the very tensors it was built from with their version counters unmoved, and the
-        loop's scratch memory is the memory the launch names."""
-        plan, gen, tensors = launch.seq_replay
-        if not plan.valid or gen != self._scratch_gen:
+    def _sequence_still_right(self, launch, args) -> bool:
+        """For a staged sequence of launches that is about to be repeated as it is: the loop's scratch memory
+        is the memory the launches name, and
+        - over a kept order of the elements (a row plan): the plan still stands (no launch has stored into its
+          arrays, it has not been given back) and the arrays are the very tensors it was built from with their
+          version counters unmoved;
+        - over the raw arrays, in a form chosen from what the last launch reported about the lengths of the
+          rows: the report is still about these arrays and still says the same (the results never depend on
+          it, the choice of the kernels does)."""
+        kind, gen = launch.seq_replay[0], launch.seq_replay[1]
+        if gen != self._scratch_gen:
             return False
-        for i, ref, version in tensors:
-            t = args[i]
-            if ref() is not t or t._version != version:
+        if kind == "plan":
+            plan, tensors = launch.seq_replay[2], launch.seq_replay[3]
+            if not plan.valid:
                 return False
-        return True
+            for i, ref, version in tensors:
+                t = args[i]
+                if ref() is not t or t._version != version:
+                    return False
+            return True
+        ident, seen = launch.seq_replay[2], launch.seq_replay[3]
+        if self._hint_key.get(launch.device) != ident:
+            return False
+        _addr, hint = self.hint(launch.device)
+        return all(int(hint[k]) == seen[k] for k in range(5))
 
     def overwrites(self, name, lo, hi, env, shape) -> bool:
         """True if this launch stores every element of array ``name`` (so that its
@@ -1343,6 +1356,7 @@ class Launch:
         self.scalar_fields = {}      # by-value scalar -> field of the argument block
         self.sequence = None         # binned rows: [(kernel, argument block, grid, block)] launched in this order
         self.seq_replay = None       # for a sequence that may be repeated as it is: what must still hold then
+        self.plan_pending = False    # a later launch over the same tensors would work out a row plan
         if spec.rows == "mixed":
             if (self._stage_planned(vals, arrays, lo, hi, spec) or self._stage_grouped(vals, arrays, lo, hi, spec)
                     or self._stage_binned(vals, arrays, lo, hi, spec)):
@@ -1462,6 +1476,8 @@ class Launch:
                         (max(1, min(1024, -(-cap // 256))), 1, 1), (256, 1, 1)))
         self.sequence = seq
         self.args, self.grid, self.block = seq[2][1], seq[2][2], seq[2][3]
+        if known and not self.plan_pending and not loop._value_only and not self.small:
+            self.seq_replay = ("hints", loop._scratch_gen, ident, tuple(seen))
         return True
 
     def _stage_grouped(self, vals, arrays, lo, hi, spec) -> bool:
@@ -1579,6 +1595,10 @@ class Launch:
         self.sequence = seq
         self.kernel, self.spec = cells, cells.src.spec
         self.args, self.grid, self.block = args_of_cells[1], args_of_cells[2], args_of_cells[3]
+        if trusted and not self.plan_pending and not loop._value_only and not self.small:
+            # (these kernels read the arrays themselves at every launch: a call with the same tensors may repeat them as they
+            #  are while the last launch reports the classes of rows that this form was chosen for)
+            self.seq_replay = ("hints", loop._scratch_gen, ident, tuple(seen))
         return True
 
     def _hint_identity(self, arrays, lo, hi):
@@ -1661,6 +1681,8 @@ class Launch:
                     loop._plan_seen.clear()
                 loop._plan_seen[key] = (seen, refs)
             if seen < (1 if reuse == "now" else 2):
+                # (the next launch over these tensors may build a plan: this one must not be repeated in its place)
+                self.plan_pending = True
                 return False
             plan = self._build_plan(key, tensors, shape, vals, arrays, lo, hi, spec)
             if plan is None:
@@ -1694,7 +1716,7 @@ class Launch:
             # stands (`CompiledLoop._kept_order_still_true`)
             import weakref
 
-            self.seq_replay = (plan, loop._scratch_gen,
+            self.seq_replay = ("plan", loop._scratch_gen, plan,
                                [(loop.arg_names.index(nm), weakref.ref(t), t._version) for nm, t in zip(loop.plan_arrays(), tensors)])
         return True
 

@@ -446,6 +446,69 @@ def test_grouped_launches_on_gpu_tensors_follow_changes_of_the_matrix(gpu):
     assert ok, worst
 
 
+def test_calls_with_the_same_tensors_repeat_the_staged_kernels_until_the_rows_change_class(gpu):
+    """A call whose tensors and scalars are those of an earlier call repeats that call's kernels without staging them
+    again, once the form has settled (it was chosen from what a launch over these arrays reported).  The kernels read
+    the arrays themselves: other contents give the other product; rows that change class are reported by the kernels,
+    and the next call is staged anew."""
+    import torch
+
+    k = selfcheck.kernels(hip_reuse=False)
+    m, n = 60_000, 1 << 20
+    a = _matrix(np.full(m, 16), n, seed=21)
+    data, indptr, indices, x = a
+    d = [torch.from_numpy(v).cuda() for v in a]
+    y = torch.empty(m, device="cuda")
+
+    @appy.jit(hip_reuse=False)
+    def into(data, indptr, indices, x, y, m):
+        #pragma parallel for
+        for i in range(m):
+            s = 0.0
+            #pragma simd
+            for j in range(indptr[i], indptr[i + 1]):
+                s += data[j] * x[indices[j]]
+            y[i] = s
+
+    def staged_by(call):
+        before = cg.Launch.serial
+        call()
+        return cg.Launch.serial - before
+
+    call = lambda: into(*d, y, m)
+    assert staged_by(call) == 1 and _steps(_loop("into", reuse=False).last_launch) == FULL      # nothing known yet
+    assert staged_by(call) == 1 and _steps(_loop("into", reuse=False).last_launch) == ["clear", "group", "cells", "sums", "rowwise"]
+    y.zero_()
+    assert staged_by(call) == 0                                                                 # repeated as staged
+    ref, budget = vo.spmv_csr(*a, (m, n))
+    assert vo.within_budget(y.cpu().numpy(), ref, budget, TOL)[0]
+    # other values and columns in the same tensors: the repeated kernels read them
+    b = _matrix(np.full(m, 16), n, seed=23)
+    for t, v in zip(d, b):
+        t.copy_(torch.from_numpy(v))
+    assert staged_by(call) == 0
+    ref, budget = vo.spmv_csr(*b, (m, n))
+    assert vo.within_budget(y.cpu().numpy(), ref, budget, TOL)[0]
+    # rows beyond the limit appear (same sizes of the arrays): the kernels report them, the call after is staged in full
+    ln = np.full(m, 16)
+    ln[:100] = 16 + 2000
+    ln[100:100 + 100 * 125] = 0
+    assert ln.sum() == 16 * m
+    c = _matrix(ln, n, seed=25)
+    for t, v in zip(d, c):
+        t.copy_(torch.from_numpy(v))
+    ref, budget = vo.spmv_csr(*c, (m, n))
+    assert staged_by(call) == 0                                                                 # still the short form: right, and reports
+    assert vo.within_budget(y.cpu().numpy(), ref, budget, TOL)[0]
+    torch.cuda.synchronize()
+    assert staged_by(call) == 1 and _steps(_loop("into", reuse=False).last_launch) == FULL
+    assert vo.within_budget(y.cpu().numpy(), ref, budget, TOL)[0]
+    assert staged_by(call) == 1 and _steps(_loop("into", reuse=False).last_launch) == FULL      # long rows: the form with kernels for them
+    assert staged_by(call) == 0
+    assert vo.within_budget(y.cpu().numpy(), ref, budget, TOL)[0]
+    appy.release()
+
+
 @pytest.mark.parametrize("rows_per_block", [512, 1024])
 def test_larger_blocks_of_rows(gpu, rows_per_block):
     """`hip_group_rows` sets the rows per block of the grouped form (256 unless told otherwise)."""
