@@ -3039,8 +3039,10 @@ class KernelBuilder:
         w("}")
 
     def _body_xcells(self):
-        """The kernel that runs a row plan: one workgroup of 1024 lanes per cell, the cells of column range
-        g on the workgroups g mod 8 (one XCD and its L2 per range).  Tile by tile: the lanes gather the
+        """The kernel that runs a row plan: workgroups of 1024 lanes (one per CU: their LDS allows no more), the
+        cells of column range g on the workgroups g mod 8 (one XCD and its L2 per range); a workgroup walks the
+        tiles of its cells as one sequence, so that the loads of a cell's first tiles travel while the cell before
+        it is finished, and puts out the sums of a cell when its last tile is through.  Tile by tile: the lanes gather the
         operand in the order of the plan (adjacent lanes read the same lines), put the value of each term into
         its slot in LDS, and after a barrier add the slots to the sums of the cell's rows, which are in LDS
         too - first the rows with one slot, a lane per row, then the rows with a run of slots, a lane per run,
@@ -3049,8 +3051,9 @@ class KernelBuilder:
 
         A wavefront instruction takes four cycles on a SIMD and only four wavefronts share one, so the loop is
         written for few instructions: every load is a per-tile base held in scalar registers plus a lane
-        offset that never changes, nothing is loaded under a branch (the plan's arrays end in spare room, and
-        what is read beyond a cell is masked where it would matter), and headers are scalars."""
+        offset that never changes, nothing is loaded under a branch (a tile that does not exist is read at one
+        position for every lane and never used), the starts of a cell come through the scalar cache, and the header
+        of a tile becomes a scalar one stage after it was asked for."""
         a, g = self.a, self.a.grouping
         U = self.spec.unroll
         TILE = 1024 * U
