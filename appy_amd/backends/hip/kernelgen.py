@@ -539,7 +539,9 @@ class LoopAnalysis:
                 and isinstance(st.targets[0], ast.Name) and st.targets[0].id == name):
             return None
         x, idx = self.arrays[x_name], self.arrays[idx_name]
-        if x.ty.size != 4 or x.ty.is_bool or idx.ty.name != "int32":
+        # (64-bit indices: the kernel that writes the pairs of a row plan narrows them; the kernels that group the elements
+        #  at every launch read 32-bit indices only, `CompiledLoop.grouped_shape`)
+        if x.ty.size != 4 or x.ty.is_bool or idx.ty.name not in ("int32", "int64"):
             return None
         jv = loop.target.id
         term = loop_ir.reduction_operand(st)
@@ -2999,8 +3001,10 @@ class KernelBuilder:
         self.ind += 1
         w("const int __j = __j0 + __k * 256 + __lid * 4;")
         w("if (__j >= __end) continue;")
-        w("appy::vec<int, 4>::type __c, __v;")
-        w(f"if (__j + 4 <= __end) __c = appy::vload<int, 4>({idx_c} + __j);")
+        ic = a.arrays[g["idx"]].elem_c           # int, or long long: narrowed once it is known to lie inside the operand
+        w(f"appy::vec<{ic}, 4>::type __c;")
+        w("appy::vec<int, 4>::type __v;")
+        w(f"if (__j + 4 <= __end) __c = appy::vload<{ic}, 4>({idx_c} + __j);")
         w("else {")
         w("#pragma unroll")
         w(f"    for (int __q = 0; __q < 4; ++__q) __c[__q] = __j + __q < __end ? {idx_c}[__j + __q] : 0;")
@@ -3023,7 +3027,7 @@ class KernelBuilder:
         w("for (int __q = 0; __q < 4; ++__q) {")
         w("    if (__j + __q >= __end) break;")
         w("    while (__lp[__row + 1] <= __j + __q) ++__row;")
-        w("    const int __cq = __c[__q];")
+        w(f"    const {ic} __cq = __c[__q];")
         w("    if (__cq < 0 || __cq >= __nx) { __inside = false; continue; }")
         w("    const unsigned __rel = __rel0 + (unsigned)__row;")
         w(f"    __keys[__j + __q] = ((__rel >> {RB}) << __lbits) | ((unsigned)__cq >> 5);")

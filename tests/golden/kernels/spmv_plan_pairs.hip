@@ -73,7 +73,8 @@ _spmv_kernel_loop_1_rkeys(
             for (int __k = 0; __k < 4; ++__k) {
                 const int __j = __j0 + __k * 256 + __lid * 4;
                 if (__j >= __end) continue;
-                appy::vec<int, 4>::type __c, __v;
+                appy::vec<int, 4>::type __c;
+                appy::vec<int, 4>::type __v;
                 if (__j + 4 <= __end) __c = appy::vload<int, 4>(A_indices + __j);
                 else {
                 #pragma unroll
