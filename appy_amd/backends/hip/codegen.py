@@ -817,7 +817,7 @@ class CompiledLoop:
         parts = min(hw.cus // max(1, strips), max(1, trip // (4 * nw)), 1024)
         return max(1, parts)
 
-    def grouped_shape(self, n_outer, env, arrays, hw=MI355X, wide_indices=False):
+    def grouped_shape(self, n_outer, env, arrays, hw=MI355X):
         """``(stripes, log2 of the elements per stripe, positions to group)`` for a launch that groups the
         elements of its rows by the stripe of the gathered operand they read, or None when the loop or
         these arrays do not qualify: the operand is larger than an L2 can keep next to the streams and
@@ -825,8 +825,6 @@ class CompiledLoop:
         g = self.analysis.grouping
         if g is None or self._group_off or not self.options.get("hip_group", True):
             return None
-        if self.analysis.arrays[g["idx"]].ty.size != 4 and not wide_indices:
-            return None                     # (the kernels of this form read 32-bit indices; a row plan narrows wider ones)
         nx = int(arrays[g["x"]].shape[0])
         most = hw.stripe_bytes // 4         # elements per stripe: half an L2 at most, 8 or 16 stripes
         if not hw.pinned_stripes or nx * 4 <= hw.stripe_min_bytes or nx > 16 * most:
@@ -953,7 +951,7 @@ class CompiledLoop:
         """The shape of a row plan for these arrays (runtime.RowPlanShape), or None when they do not
         qualify: the conditions of the grouped form (an operand too large for an L2, rows of a few
         elements), and keys and packed words of 32 bits."""
-        base = self.grouped_shape(n_outer, env, arrays, hw, wide_indices=True)
+        base = self.grouped_shape(n_outer, env, arrays, hw)
         if base is None or self._plan_off:
             return None
         g = self.analysis.grouping

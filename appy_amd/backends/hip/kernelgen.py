@@ -539,8 +539,8 @@ class LoopAnalysis:
                 and isinstance(st.targets[0], ast.Name) and st.targets[0].id == name):
             return None
         x, idx = self.arrays[x_name], self.arrays[idx_name]
-        # (64-bit indices: the kernel that writes the pairs of a row plan narrows them; the kernels that group the elements
-        #  at every launch read 32-bit indices only, `CompiledLoop.grouped_shape`)
+        # (64-bit indices are narrowed where they are loaded: by the kernels that group the elements and by the kernel that
+        #  writes the pairs of a row plan; the kernels that run the groups and the plan do not read them)
         if x.ty.size != 4 or x.ty.is_bool or idx.ty.name not in ("int32", "int64"):
             return None
         jv = loop.target.id
@@ -2560,6 +2560,7 @@ class KernelBuilder:
         self.mode = "lane"
         idx_c = cname(g["idx"])
         a.arrays[g["idx"]].loaded = True
+        self._group_wide = a.arrays[g["idx"]].ty.size == 8     # 64-bit indices are narrowed as they are loaded
         car_c = f"reinterpret_cast<const int*>({cname(g['carried'])})" if g["carried"] else None
         body = a.outer.body
         at = next(k for k, st in enumerate(body) if st is a.team_split)
@@ -2685,10 +2686,10 @@ class KernelBuilder:
 
         def load_indices(k, j0, kk):
             w(f"{{ const int __j = {j0} + {kk} * 256 + __lid * 4;")
-            w(f"if (__j + 4 <= __end) __c[{k}] = appy::vload<int, 4>({idx_c} + __j);")
+            w(f"if (__j + 4 <= __end) __c[{k}] = {self._group_index4(idx_c + ' + __j')};")
             w("else {")
             w("#pragma unroll")
-            w(f"    for (int __q = 0; __q < 4; ++__q) __c[{k}][__q] = __j + __q < __end ? {idx_c}[__j + __q] : -1;")
+            w(f"    for (int __q = 0; __q < 4; ++__q) __c[{k}][__q] = __j + __q < __end ? {self._group_index1(idx_c + '[__j + __q]')} : -1;")
             w("} }")
 
         def load_carried(k, j0, kk):
@@ -2745,6 +2746,16 @@ class KernelBuilder:
         self.ind -= 1
         w("}")
 
+    def _group_index4(self, pointer: str) -> str:
+        """Four indices of the grouping kernel from `pointer`, as 32-bit numbers (an index that does not fit
+        is negative afterwards, and dropped like every negative index)."""
+        if not self._group_wide:
+            return f"appy::vload<int, 4>({pointer})"
+        return f"appy::narrow_indices(appy::vload<long long, 4>({pointer}))"
+
+    def _group_index1(self, value: str) -> str:
+        return value if not self._group_wide else f"appy::narrow_index({value})"
+
     def _group_walk_kept(self, idx_c, car_c, U, find_row, count, starts, place_one, unrolled):
         """The two passes of the grouping kernel over the elements of the rows that are kept (rows
         beyond `__rowmax` elements run in planned parts): the lanes walk the kept elements of the block
@@ -2794,10 +2805,10 @@ class KernelBuilder:
             w("{")
             self.ind += 1
             positions(k)
-            w(f"if (__run) __c[{k}] = appy::vload<int, 4>({idx_c} + __jq[0]);")
+            w(f"if (__run) __c[{k}] = {self._group_index4(idx_c + ' + __jq[0]')};")
             w("else {")
             w("#pragma unroll")
-            w(f"    for (int __q = 0; __q < 4; ++__q) __c[{k}][__q] = __t + __q < __kept ? {idx_c}[__jq[__q]] : -1;")
+            w(f"    for (int __q = 0; __q < 4; ++__q) __c[{k}][__q] = __t + __q < __kept ? {self._group_index1(idx_c + '[__jq[__q]]')} : -1;")
             w("}")
             if both:
                 if car_c:

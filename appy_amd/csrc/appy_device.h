@@ -276,6 +276,17 @@ __device__ __forceinline__ i64 team_lane_below(i64 v, int lane) {
 // A number that is the same in every lane, kept in scalar registers whatever it was computed from: with such an offset
 // from a kernel argument, loads at `base + offset + lane offset` take the scalar-base form of the memory instructions
 // (one 32-bit register per lane for the lane's offset instead of a 64-bit address worked out per lane).
+// A 64-bit index as a 32-bit one; what does not fit becomes -1 (kernels that group elements drop negative indices).
+__device__ __forceinline__ int narrow_index(long long v) {
+    return v >= 0 && v <= 0x7fffffffll ? (int)v : -1;
+}
+__device__ __forceinline__ vec<int, 4>::type narrow_indices(vec<long long, 4>::type v) {
+    vec<int, 4>::type r;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) r[k] = narrow_index(v[k]);
+    return r;
+}
+
 __device__ __forceinline__ unsigned lane_offset(unsigned v) {
     // (the compiler may not look through this: a lane's offset stays one 32-bit register next to the scalar base, where it
     //  would otherwise widen offsets chosen under a condition to 64 bits and add the base lane by lane)

@@ -179,6 +179,15 @@ def test_sums_of_gathered_terms_can_be_grouped_by_the_stripe_they_read():
     wide = csr("v[j] * x[c[j]]", c=np.zeros(16, np.int64))
     assert wide.grouping is not None and wide.arrays["c"].ty.name == "int64"
     # the kernels
+    src = ("#pragma parallel for\nfor i in range(m):\n    s = 0.0\n    #pragma simd\n"
+           "    for j in range(p[i], p[i + 1]):\n        s += v[j] * x[c[j]]\n    y[i] = s")
+    fw, _ = compiled(src, p=i32, c=np.zeros(16, np.int64), v=f32, x=f32, y=np.zeros(8, np.float32), m=8)
+    for spec in (Spec("team", block=256, vec=1, width=64, parts=8, aux="group", block_rows=256),
+                 Spec("team", block=256, vec=1, width=64, parts=8, aux="group", block_rows=256, skip_long=True),
+                 Spec("team", block=256, vec=1, width=64, aux="rkeys", block_rows=256)):
+        kn = fw.kernel_for(spec)
+        assert ("appy::narrow_indices(appy::vload<long long, 4>(" in kn.src.text) == (spec.aux == "group")
+        assert kn.code                                                        # compiles for gfx950
     group = body_of(f.kernel_for(Spec("team", block=256, vec=1, width=64, parts=8, aux="group", block_rows=256)).src.text)
     assert "__lp[__r + 1] == __hq[__r]" in group and "__flag[0] = 1" in group and "__hint[0] = 2" in group
     assert "x[" not in group.split("{", 1)[1]                                 # the gathered operand is not read here

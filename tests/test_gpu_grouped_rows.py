@@ -446,6 +446,32 @@ def test_grouped_launches_on_gpu_tensors_follow_changes_of_the_matrix(gpu):
     assert ok, worst
 
 
+@pytest.mark.parametrize("lengths", ["16", "zipf"])
+def test_column_indices_of_64_bits_are_narrowed_by_the_grouping_kernels(gpu, lengths):
+    """Column indices (and row starts) of 64 bits: both walks of the grouping kernel - over the arrays as they lie and
+    over the kept rows of a matrix with long rows - load them as pairs of 16-byte vectors and narrow them."""
+    import torch
+
+    k = selfcheck.kernels(hip_reuse=False)
+    m, n = 60_000, 1 << 20
+    rng = np.random.default_rng(31)
+    ln = np.full(m, 16) if lengths == "16" else np.clip(rng.zipf(1.5, m), 1, 4096)
+    data, indptr, indices, x = _matrix(ln, n, seed=33)
+    d = [torch.from_numpy(v).cuda() for v in (data, indptr.astype(np.int64), indices.astype(np.int64), x)]
+    ref, budget = vo.spmv_csr(data, indptr, indices, x, (m, n))
+    _forget()
+    ys = []
+    for it in range(3):
+        y = k.spmv(*d, m, n)
+        launch = _loop("spmv", index_type="int64", reuse=False).last_launch
+        assert _grouped(launch)
+        assert (_steps(launch) == FULL) == (it == 0 or lengths == "zipf")
+        ok, worst = vo.within_budget(y.cpu().numpy(), ref, budget, TOL)
+        assert ok, worst
+        ys.append(y)
+    assert torch.equal(ys[0], ys[1]) and torch.equal(ys[1], ys[2])
+
+
 def test_calls_with_the_same_tensors_repeat_the_staged_kernels_until_the_rows_change_class(gpu):
     """A call whose tensors and scalars are those of an earlier call repeats that call's kernels without staging them
     again, once the form has settled (it was chosen from what a launch over these arrays reported).  The kernels read

@@ -110,8 +110,8 @@ def test_a_plan_is_built_on_the_second_launch_and_run_from_then_on(env, m, n, le
 @pytest.mark.parametrize("ptr_type,idx_type", [(np.int64, np.int64), (np.int32, np.int64), (np.int64, np.int32)])
 def test_index_arrays_of_64_bits(env, ptr_type, idx_type):
     """Row starts and column indices of 64 bits (what torch's CSR tensors hold): the kernel that writes the pairs
-    narrows them once it has checked that they lie inside the operand; the launches before the plan take the
-    forms that read such indices (rows sorted by length)."""
+    narrows them once it has checked that they lie inside the operand, and so do the kernels that group the
+    elements in the launch before the plan exists."""
     torch, k = env
     m, n = 50_000, 1 << 21
     data, indptr, indices, x = _matrix(np.full(m, 12), n, seed=9)
@@ -123,6 +123,7 @@ def test_index_arrays_of_64_bits(env, ptr_type, idx_type):
         launch = max((v[0] for kk, v in cg.code_cache.items() if kk[-1] == "spmv" and getattr(v[0], "last_launch", None) is not None),
                      key=lambda lp: lp.last_launch.serial).last_launch
         assert _planned(launch) == (it >= 1)
+        assert it >= 1 or launch.spec.aux == "cells"
 
 
 def test_values_and_indices_changed_in_place_give_the_new_result(env):
