@@ -342,6 +342,7 @@ class RowPlan:
         self.ncell = 0
         self.tile = 0
         self.split = 1              # workgroups per cell
+        self.entries = 0            # positions of the streamed arrays the plan was built from
         self.owner = None           # the loop the plan belongs to
         self.inspector_ms = None
 
@@ -404,6 +405,15 @@ def drop_plans_overlapping(extents):
         with _plans_lock:
             if plan in _live_plans:
                 _live_plans.remove(plan)
+
+
+def plan_kernel_spec(tile: int, entries: int, rows: int, restrict: bool = True) -> Spec:
+    """The kernel that runs a row plan of tiles of `tile` elements over `entries` elements of `rows` rows.  Where
+    rows are short (fewer than 48 elements on average) the row numbers are a larger share of what a tile loads:
+    they are asked for ahead of the scatter (uniform 16 per row: 0.257 -> 0.252 ms; a power-law matrix of 98 per
+    row loses 1.7 % that way and keeps them behind it)."""
+    return Spec("team", block=1024, vec=1, width=1024, unroll=tile // 1024, parts=PLAN_GROUPS, aux="xcells", restrict=restrict,
+                stream_loads=entries < 48 * rows)
 
 
 def release_all_plans():
@@ -1689,8 +1699,7 @@ class Launch:
                 return False
         V = spec.vec
         try:
-            cells = loop.kernel_for(Spec("team", block=1024, vec=1, width=1024, unroll=plan.tile // 1024, parts=PLAN_GROUPS,
-                                         aux="xcells", restrict=spec.restrict))
+            cells = loop.kernel_for(plan_kernel_spec(plan.tile, plan.entries, n, spec.restrict))
             sums = loop.kernel_for(Spec("team", block=256, vec=V, width=1, phase=2, guard=1, restrict=spec.restrict))
         except Unsupported:
             loop._plan_off = True
@@ -1799,6 +1808,7 @@ class Launch:
         # until there are some four workgroups per compute unit or a workgroup is down to two tiles
         forced = loop.options.get("hip_plan_split")
         plan.split = int(forced) if forced else max(1, min(-(-4 * self.hw.cus // ncell), entries // (2 * plan.tile * ncell), 32))
+        plan.entries = entries
         plan.valid = True
         plan.owner = loop
         with loop._lock:
