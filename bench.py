@@ -511,6 +511,9 @@ def main():
             if "kernel_ms" not in rec:
                 rec.update(r)           # a run of the reused form only: its figures stand for the workload
             rec.update(reused)
+            if rec.get("ms_no_reuse", 0) > reused["ms_reused"]:
+                # launches after which working the order out has paid for itself
+                rec["inspector_break_even_launches"] = reused["inspector_ms"] / (rec["ms_no_reuse"] - reused["ms_reused"])
             loop.release()
         rec["forms"] = ("kernel_ms, frac, ms_no_reuse, first_launch_ms: every launch reads the raw arrays (hip_reuse=False); "
                         "inspector_ms once, then ms_reused, frac_reused per launch: the kept order of the elements "
