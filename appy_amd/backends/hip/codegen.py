@@ -1731,8 +1731,9 @@ class Launch:
 
     def _build_plan(self, key, tensors, shape, vals, arrays, lo, hi, spec):
         """Runs the inspector for these arrays: the generated kernel writes one (key, value) pair per element, the
-        library sorts the pairs and lays out cells, tiles and slots.  Waits for the device once, to learn whether
-        the arrays were accepted (row ranges that follow one another, indices inside the operand)."""
+        library sorts the pairs and lays out cells, tiles and slots.  Waits for the device after that kernel, to learn
+        whether the arrays were accepted (row ranges that follow one another, indices inside the operand) and whether
+        every position holds an element, and once more at the end."""
         loop = self.loop
         n = hi - lo
         try:
@@ -1783,11 +1784,17 @@ class Launch:
             args = self._argument_block(rkeys, vals, arrays, lo, hi)
             nblk = -(-n // 256)
             rt.launch(rkeys_fn, (max(1, min(1 << 20, -(-nblk // 4))), 1, 1), (256, 1, 1), args, self.stream)
-            rt.check(lib.appy_hip_rowplan_build(C.byref(shape), keys, pairs, keys_sorted, elements, temp, temp_bytes.value,
-                                                cstart, tbase, rstream, self.stream))
+            # what the kernel found: whether the arrays are accepted, and how many positions the rows cover - all of them
+            # (the usual case: a loop over all rows of a CSR matrix) means that the sort needs one pass less
+            words = (C.c_int64 * 2)(0, 0)
+            rt.memcpy_d2h(C.addressof(words), flag, 16, self.stream)      # waits for the stream
+            word = C.c_int64(words[0])
+            if not word.value:
+                shape.full = 1 if words[1] == entries else 0
+                rt.check(lib.appy_hip_rowplan_build(C.byref(shape), keys, pairs, keys_sorted, elements, temp, temp_bytes.value,
+                                                    cstart, tbase, rstream, self.stream))
             t1.record(self.stream)
-            word = C.c_int64(0)
-            rt.memcpy_d2h(C.addressof(word), flag, 8, self.stream)      # waits for the stream
+            rt.sync(self.stream)          # (the temporary arrays go back below)
             plan.inspector_ms = t0.elapsed_ms(t1)
         except BaseException:
             plan.release()

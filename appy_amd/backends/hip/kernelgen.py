@@ -3004,6 +3004,8 @@ class KernelBuilder:
         w("    if (__lid == 0) __flag[0] = 1;")
         w("    continue;")
         w("}")
+        w("// (how many positions the rows of all blocks cover: when it is every position, no key stays unset and the sort needs a bit less)")
+        w("if (__lid == 0) atomicAdd(reinterpret_cast<unsigned long long*>(__flag) + 1, (unsigned long long)(__end - __first));")
         w(f"const unsigned __rel0 = (unsigned)(__b * {R});       // first row of the block, counted from the start of the range")
         w("bool __inside = true;")
         w(f"for (int __j0 = __first; __j0 < __end; __j0 += {256 * U}) {{")

@@ -12,7 +12,7 @@ import threading
 _LIB_NAME = "libappy_hip.so"
 _PKG_ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 
 class Props(C.Structure):
@@ -58,6 +58,7 @@ class RowPlanShape(C.Structure):
         ("col_bits", C.c_uint32),
         ("tile", C.c_uint32),
         ("line_bits", C.c_uint32),
+        ("full", C.c_uint32),
     ]
 
 

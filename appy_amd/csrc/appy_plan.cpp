@@ -207,7 +207,7 @@ bool shape_ok(const appy_hip_rowplan_shape* s) {
 uint32_t key_bits(const appy_hip_rowplan_shape* s) {
     uint32_t bits = s->line_bits;
     while ((1ull << bits) < ((uint64_t)s->row_blocks << s->line_bits)) ++bits;
-    return bits + 1;        // and the bit that only positions without an element have set
+    return bits + (s->full ? 0 : 1);        // and the bit that only positions without an element have set
 }
 
 }  // namespace

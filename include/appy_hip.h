@@ -27,7 +27,7 @@ extern "C" {
 /* 2: page-locked host memory, streams and graphs, appy_hip_rtc_version; 3: appy_hip_launch_static_scratch;
  * 4: row plans (appy_hip_rowplan_*), appy_hip_device_sync, appy_hip_memcpy_h2d_async, appy_hip_device_topology
  * (additions only: every entry point of the earlier versions is unchanged). */
-#define APPY_HIP_ABI_VERSION 4
+#define APPY_HIP_ABI_VERSION 5
 
 typedef struct appy_hip_props {
     char     name[128];        /* marketing name */
@@ -203,6 +203,8 @@ typedef struct appy_hip_rowplan_shape {
     uint32_t col_bits;      /* bits of the column within its range in a packed word */
     uint32_t tile;          /* elements per tile: 4096 or 6144 */
     uint32_t line_bits;     /* bits of IDX[j] >> 5 in a key */
+    uint32_t full;          /* 1: every position holds an element (no key is 0xFFFFFFFF), so the sort may leave
+                               out the bit that only such keys have set - one pass less; 0: not known */
 } appy_hip_rowplan_shape;
 int appy_hip_rowplan_sizes(const appy_hip_rowplan_shape* shape, size_t* sort_temp_bytes_out, size_t* max_tiles_out,
                            size_t* stream_words_out);

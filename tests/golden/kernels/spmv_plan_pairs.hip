@@ -66,6 +66,8 @@ _spmv_kernel_loop_1_rkeys(
             if (__lid == 0) __flag[0] = 1;
             continue;
         }
+        // (how many positions the rows of all blocks cover: when it is every position, no key stays unset and the sort needs a bit less)
+        if (__lid == 0) atomicAdd(reinterpret_cast<unsigned long long*>(__flag) + 1, (unsigned long long)(__end - __first));
         const unsigned __rel0 = (unsigned)(__b * 256);       // first row of the block, counted from the start of the range
         bool __inside = true;
         for (int __j0 = __first; __j0 < __end; __j0 += 1024) {
