@@ -1643,7 +1643,7 @@ class Launch:
         """The launches of a loop whose elements have been ordered by an earlier launch with the same arrays
         (a row plan): the kernel that runs the plan, then the kernel that adds the sums of a row's eight
         column ranges and runs the rest of the body.  A plan is built the second time a set of arrays is
-        seen unchanged (`hip_reuse="now"`: the first time); the first time the launch takes the forms that
+        seen unchanged (`hip_reuse="now"`: the first time, `hip_reuse=k`: the k-th); before that the launch takes the forms that
         keep nothing.  False (nothing staged) when the launch does not qualify or has no plan yet."""
         loop, a, env = self.loop, self.loop.analysis, self.env
         reuse = loop.options.get("hip_reuse", True)
@@ -1690,7 +1690,11 @@ class Launch:
                 if len(loop._plan_seen) > 64:
                     loop._plan_seen.clear()
                 loop._plan_seen[key] = (seen, refs)
-            if seen < (1 if reuse == "now" else 2):
+            # the sighting at which the order is worked out: the second by default, the first with "now", the k-th with
+            # an integer k (working it out costs some eight launches over the raw arrays: a program that knows it will
+            # launch a few times only may ask for a later sighting, or switch the reuse off)
+            wanted = 1 if reuse == "now" else (max(1, reuse) if isinstance(reuse, int) and not isinstance(reuse, bool) else 2)
+            if seen < wanted:
                 # (the next launch over these tensors may build a plan: this one must not be repeated in its place)
                 self.plan_pending = True
                 return False

@@ -360,6 +360,11 @@ def test_reuse_can_be_switched_off_and_forced(env):
     y = now.spmv(td, tp, ti, tx, m, n)
     assert _planned(_loop(hip_reuse="now").last_launch)            # built by the first launch
     _check(y, data, indptr, indices, x, m, n)
+    later = selfcheck.kernels(hip_reuse=4)                        # built by the fourth launch over the same tensors
+    for it in range(5):
+        y = later.spmv(td, tp, ti, tx, m, n)
+        assert _planned(_loop(hip_reuse=4).last_launch) == (it >= 3)
+    _check(y, data, indptr, indices, x, m, n)
     # NumPy callers keep the forms that keep nothing (their arrays are copied per call)
     k = selfcheck.kernels()
     for _ in range(3):
