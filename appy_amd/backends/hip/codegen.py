@@ -1974,7 +1974,9 @@ class Launch:
         if g is not None:
             g.launches += 1
             g.keepalive.extend(self.keepalive)
-            g.stored_extents.extend(self.stored_extents)
+            for e in self.stored_extents:
+                if e not in g.stored_extents:       # (a loop recorded many times over the same arrays)
+                    g.stored_extents.append(e)
             for m, _dptr, _host, stored, _name in self.mirrored:
                 if m not in g.used_mirrors:
                     g.used_mirrors.append(m)
