@@ -554,6 +554,66 @@ def test_few_workgroups_walk_many_cells_one_after_the_other(env, grid, split):
     appy.release()
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_random_shapes_ranges_and_row_lengths(env, seed):
+    """Matrices of random sizes and row-length laws, a random range of their rows, random numbers of workgroups:
+    the launches over the kept order must give the oracle's product for the rows of the range and touch no other."""
+    torch, _k = env
+    rng = np.random.default_rng(1000 + seed)
+    m = int(rng.integers(40_000, 150_000))
+    n = int(rng.integers((1 << 20) + 1, 1 << 23))
+    law = ["0..3", "16", "1..40", "zipf", "0,10,20", "banded"][seed % 6]
+    if law == "banded":
+        ln = rng.integers(1, 24, m)
+    else:
+        ln = _lengths(law, m, rng)
+    indptr = np.zeros(m + 1, dtype=np.int64)
+    np.cumsum(ln, out=indptr[1:])
+    nnz = int(indptr[-1])
+    if law == "banded":
+        # columns near the diagonal: most cells of a block of rows hold nothing
+        rows = np.repeat(np.arange(m), ln)
+        cols = np.clip((rows * (n / max(m, 1))).astype(np.int64) + rng.integers(-3000, 3000, nnz), 0, n - 1)
+    else:
+        cols = rng.integers(0, n, nnz)
+    data = rng.standard_normal(nnz).astype(np.float32)
+    x = rng.standard_normal(n).astype(np.float32)
+    indptr32, cols32 = indptr.astype(np.int32), cols.astype(np.int32)
+    lo = int(rng.integers(0, m // 8))
+    hi = int(rng.integers(m - m // 8, m + 1)) if seed % 2 else m
+    if seed % 2 == 0:
+        lo = 0
+
+    opts = {"hip_reuse": "now"}
+    if seed % 3 == 0:
+        opts["hip_plan_grid"] = int(rng.choice([8, 24, 64]))
+
+    @appy.jit(**opts)
+    def part(data, indptr, indices, x, y, lo, hi):
+        #pragma parallel for
+        for i in range(lo, hi):
+            s = 0.0
+            #pragma simd
+            for j in range(indptr[i], indptr[i + 1]):
+                s += data[j] * x[indices[j]]
+            y[i] = s
+
+    td, tp, ti, tx = _gpu(torch, data, indptr32, cols32, x)
+    ref, budget = vo.spmv_csr(data, indptr32, cols32, x, (m, n))
+    planned = 0
+    for it in range(2):
+        y = torch.full((m,), 7.0, device="cuda")
+        part(td, tp, ti, tx, y, lo, hi)
+        yh = y.cpu().numpy()
+        assert np.all(yh[:lo] == 7.0) and np.all(yh[hi:] == 7.0)
+        assert np.all(np.abs(yh[lo:hi] - ref[lo:hi]) <= TOL * budget[lo:hi]), (law, m, n, lo, hi)
+        planned += _planned(_loop("part").last_launch)
+    # (small or very sparse inputs do not qualify for a plan: then the other forms have been checked)
+    assert planned in (0, 2)
+    print(f"random shapes: law {law} m {m} n {n} rows [{lo}, {hi}) nnz {nnz}: {'kept order' if planned else 'other forms'}")
+    appy.release()
+
+
 def test_plans_are_bounded_released_and_kept_out_of_the_way(env, monkeypatch):
     torch, k = env
     m, n = 40_000, 1 << 20
