@@ -342,6 +342,7 @@ class RowPlan:
         self.ncell = 0
         self.tile = 0
         self.split = 1              # workgroups per cell
+        self.grid = 8               # workgroups of the kernel that runs the plan
         self.entries = 0            # positions of the streamed arrays the plan was built from
         self.owner = None           # the loop the plan belongs to
         self.inspector_ms = None
@@ -414,6 +415,51 @@ def plan_kernel_spec(tile: int, entries: int, rows: int, restrict: bool = True) 
     row loses 1.7 % that way and keeps them behind it)."""
     return Spec("team", block=1024, vec=1, width=1024, unroll=tile // 1024, parts=PLAN_GROUPS, aux="xcells", restrict=restrict,
                 stream_loads=entries < 48 * rows)
+
+
+def plan_split(tiles, cus: int, tile: int, entries: int, forced=None) -> int:
+    """Workgroups that share a cell of a row plan (each takes a run of its tiles and has a slot of its own for the
+    sums).  `tiles`: tiles per cell.  Few cells (a matrix of few blocks of rows): until there are some four runs per
+    compute unit or a run is down to two tiles.  Cells of very different sizes (a banded matrix: one of the eight
+    cells of a block of rows holds everything): until the largest run is no more than about what a workgroup gets
+    on average.  Every doubling doubles the sums the second kernel reads, so it stops at 32."""
+    if forced:
+        return int(forced)
+    ncell = len(tiles)
+    split = max(1, min(-(-4 * cus // ncell), entries // (2 * tile * ncell), 32))
+    total, largest = int(tiles.sum()), int(tiles.max()) if ncell else 0
+    workgroups = max(8, cus // 8 * 8)
+    while split < 32 and largest > 4 * split and -(-largest // split) > 1.25 * total / workgroups:
+        split *= 2
+    return split
+
+
+def deal_runs(tiles, split: int, grid: int):
+    """The runs of tiles of a row plan dealt to `grid` workgroups (a multiple of eight; workgroup w reads column
+    range w mod 8 only): entry w + grid * i of the result is the i-th run of workgroup w, 0xFFFFFFFF for none.
+    Run (block * split + part) * 8 + range holds the tiles [part * t / split, (part + 1) * t / split) of its
+    cell of t tiles.  Per range the runs are sorted by size and dealt out back and forth, so that workgroups
+    end up with about the same number of tiles whatever the sizes of the cells; runs without tiles are dealt
+    too (their sums must be written)."""
+    tiles = np.asarray(tiles, dtype=np.int64)
+    ncell = len(tiles)
+    per_range = grid // PLAN_GROUPS
+    blocks = ncell // PLAN_GROUPS
+    parts = np.arange(split, dtype=np.int64)
+    t = tiles.reshape(blocks, PLAN_GROUPS)                                               # [block, range]
+    size = ((parts[None, None, :] + 1) * t[:, :, None]) // split - (parts[None, None, :] * t[:, :, None]) // split
+    run = (np.arange(blocks, dtype=np.int64)[:, None, None] * split + parts[None, None, :]) * PLAN_GROUPS \
+        + np.arange(PLAN_GROUPS, dtype=np.int64)[None, :, None]
+    rounds = -(-(blocks * split) // per_range)
+    order = np.full(rounds * grid, 0xFFFFFFFF, dtype=np.uint32)
+    for g in range(PLAN_GROUPS):
+        sz, rn = size[:, g, :].reshape(-1), run[:, g, :].reshape(-1)
+        by_size = np.lexsort((rn, -sz))                                                  # largest first, ties by number
+        rank = np.arange(len(by_size))
+        rnd, pos = rank // per_range, rank % per_range
+        member = np.where(rnd % 2 == 0, pos, per_range - 1 - pos)
+        order[(g + PLAN_GROUPS * member) + grid * rnd] = rn[by_size].astype(np.uint32)
+    return order
 
 
 def release_all_plans():
@@ -1716,10 +1762,7 @@ class Launch:
             return False
         self.nsplit = PLAN_GROUPS * split
         self.plan = plan
-        # one workgroup per CU (their LDS allows no more), a multiple of eight so that a workgroup stays with one column
-        # range; each walks the tiles of its runs as one sequence
-        grid = min(plan.ncell * split, int(loop.options.get("hip_plan_grid") or max(8, self.hw.cus // 8 * 8)))
-        seq = [(cells, self._argument_block(cells, vals, arrays, lo, hi), (max(8, grid // 8 * 8), 1, 1), (1024, 1, 1)),
+        seq = [(cells, self._argument_block(cells, vals, arrays, lo, hi), (plan.grid, 1, 1), (1024, 1, 1)),
                (sums, self._argument_block(sums, vals, arrays, lo, hi), (max(1, min(4096, -(-n // 256))), 1, 1), (256, 1, 1))]
         self.sequence = seq
         self.kernel, self.spec = cells, cells.src.spec
@@ -1817,8 +1860,23 @@ class Launch:
         plan.tile = int(shape.tile)
         # few cells (a matrix of few blocks of rows): several workgroups share a cell, each with a run of its tiles,
         # until there are some four workgroups per compute unit or a workgroup is down to two tiles
-        forced = loop.options.get("hip_plan_split")
-        plan.split = int(forced) if forced else max(1, min(-(-4 * self.hw.cus // ncell), entries // (2 * plan.tile * ncell), 32))
+        # how the tiles lie over the cells decides how many workgroups share a cell and which runs a workgroup gets
+        tb = np.empty(ncell + 1, dtype=np.uint32)
+        rt.memcpy_d2h(tb.ctypes.data, tbase, 4 * (ncell + 1), self.stream)
+        tiles = np.diff(tb.astype(np.int64))
+        plan.split = plan_split(tiles, self.hw.cus, plan.tile, entries, loop.options.get("hip_plan_split"))
+        # one workgroup per CU (their LDS allows no more), a multiple of eight so that a workgroup stays with one column
+        # range; each walks the tiles of its runs as one sequence
+        grid = min(ncell * plan.split, int(loop.options.get("hip_plan_grid") or max(8, self.hw.cus // 8 * 8)))
+        plan.grid = max(8, grid // 8 * 8)
+        order = deal_runs(tiles, plan.split, plan.grid)
+        try:
+            dealt = plan.alloc(4 * len(order))
+            rt.memcpy_h2d(dealt, order.ctypes.data, 4 * len(order), self.stream)
+        except BaseException:
+            plan.release()
+            raise
+        plan.bin["order"], plan.bin["norder"] = dealt, len(order)
         plan.entries = entries
         plan.valid = True
         plan.owner = loop
@@ -1867,7 +1925,7 @@ class Launch:
                 val = self.bin[p.role][p.dim]
             elif p.role in ("rows", "counts", "zero", "nrows", "bnd", "cap", "stripe", "m", "base", "skip", "tlo", "thi", "load", "hint", "rowstart",
                             "flag", "desc", "ent", "shiftc", "entries", "rowmax", "keys", "vals", "nx", "lbits", "cstart", "tbase",
-                            "rstream", "ncell", "gwidth", "colbits", "split"):
+                            "rstream", "ncell", "gwidth", "colbits", "split", "order", "norder"):
                 val = self.bin[p.role]
             elif p.role == "lo":
                 val = lo

@@ -3107,9 +3107,10 @@ class KernelBuilder:
         w("const unsigned __xlast = (unsigned)(__nx - 1);")
         w("const char* __xb = reinterpret_cast<const char*>(" + xc + ");")
         w("// A cell may be shared by __split workgroups, each with a run of its tiles and a slot of its own for the sums: a")
-        w("// run is numbered (block * __split + part) * 8 + range.  The workgroup takes the runs blockIdx.x, blockIdx.x +")
-        w("// gridDim.x, ... (the grid is a multiple of eight workgroups: all of them read the same range) and walks their tiles")
-        w("// as one sequence, so that the loads of a run's first tiles travel while the run before it is finished.")
+        w("// run is numbered (block * __split + part) * 8 + range.  The workgroup takes the runs that the entries blockIdx.x,")
+        w("// blockIdx.x + gridDim.x, ... of __order name (dealt out on the host by size; the grid is a multiple of eight")
+        w("// workgroups and all runs of a workgroup read the same range) and walks their tiles as one sequence, so that")
+        w("// the loads of a run's first tiles travel while the run before it is finished.")
         w("const unsigned __nrun = (unsigned)(__ncell * __split), __spl = (unsigned)__split;")
         w("const unsigned __g = blockIdx.x & 7u;")
         w("const unsigned __x0 = __g * (unsigned)__gwidth;")
@@ -3122,7 +3123,8 @@ class KernelBuilder:
         w("unsigned __h0, __h1, __hv2;        // headers of the tiles in flight (the newest as it was loaded, in a vector register)")
         w("// the tile the next load fetches: run, tile within the run; of the run: its tiles, where its elements and its row")
         w("// stream start, the elements from there to the end of the cell")
-        w("unsigned __vc = blockIdx.x, __tt = 0, __nt = 0;")
+        w("unsigned __vi = blockIdx.x, __tt = 0, __nt = 0;")
+        w("unsigned __vc = __vi < __norder ? __order[__vi] : 0xffffffffu;        // (no run: a number beyond them all)")
         w("appy::i64 __eb = 0, __sb = 0;      // (in bytes from the start of the elements and of the row stream)")
         w("const char* __entb = reinterpret_cast<const char*>(__ent);")
         w("const char* __rsb = reinterpret_cast<const char*>(__rstream);")
@@ -3168,7 +3170,7 @@ class KernelBuilder:
             w("  if (__any2) {")
             w("      if (!__end2) ++__tt;")
             w("      else {")
-            w("          __vc += gridDim.x; __tt = 0;")
+            w("          __vi += gridDim.x; __vc = __vi < __norder ? __order[__vi] : 0xffffffffu; __tt = 0;")
             self.ind += 3
             enter_run()
             self.ind -= 3
@@ -3497,6 +3499,8 @@ class KernelBuilder:
             params.append(Param("__rstream", "const unsigned* __restrict__ __rstream", C.c_void_p, "rstream"))
             params.append(Param("__ncell", "const appy::i64 __ncell", C.c_int64, "ncell"))
             params.append(Param("__split", "const appy::i64 __split", C.c_int64, "split"))
+            params.append(Param("__order", "const unsigned* __restrict__ __order", C.c_void_p, "order"))
+            params.append(Param("__norder", "const appy::i64 __norder", C.c_int64, "norder"))
             params.append(Param("__gwidth", "const appy::i64 __gwidth", C.c_int64, "gwidth"))
             params.append(Param("__colbits", "const int __colbits", C.c_int32, "colbits"))
             params.append(Param("__nx", "const appy::i64 __nx", C.c_int64, "nx"))

@@ -12,6 +12,8 @@ _spmv_kernel_loop_1_xcells(
     const unsigned* __restrict__ __rstream,
     const appy::i64 __ncell,
     const appy::i64 __split,
+    const unsigned* __restrict__ __order,
+    const appy::i64 __norder,
     const appy::i64 __gwidth,
     const int __colbits,
     const appy::i64 __nx,
@@ -27,9 +29,10 @@ _spmv_kernel_loop_1_xcells(
     const unsigned __xlast = (unsigned)(__nx - 1);
     const char* __xb = reinterpret_cast<const char*>(x);
     // A cell may be shared by __split workgroups, each with a run of its tiles and a slot of its own for the sums: a
-    // run is numbered (block * __split + part) * 8 + range.  The workgroup takes the runs blockIdx.x, blockIdx.x +
-    // gridDim.x, ... (the grid is a multiple of eight workgroups: all of them read the same range) and walks their tiles
-    // as one sequence, so that the loads of a run's first tiles travel while the run before it is finished.
+    // run is numbered (block * __split + part) * 8 + range.  The workgroup takes the runs that the entries blockIdx.x,
+    // blockIdx.x + gridDim.x, ... of __order name (dealt out on the host by size; the grid is a multiple of eight
+    // workgroups and all runs of a workgroup read the same range) and walks their tiles as one sequence, so that
+    // the loads of a run's first tiles travel while the run before it is finished.
     const unsigned __nrun = (unsigned)(__ncell * __split), __spl = (unsigned)__split;
     const unsigned __g = blockIdx.x & 7u;
     const unsigned __x0 = __g * (unsigned)__gwidth;
@@ -42,7 +45,8 @@ _spmv_kernel_loop_1_xcells(
     unsigned __h0, __h1, __hv2;        // headers of the tiles in flight (the newest as it was loaded, in a vector register)
     // the tile the next load fetches: run, tile within the run; of the run: its tiles, where its elements and its row
     // stream start, the elements from there to the end of the cell
-    unsigned __vc = blockIdx.x, __tt = 0, __nt = 0;
+    unsigned __vi = blockIdx.x, __tt = 0, __nt = 0;
+    unsigned __vc = __vi < __norder ? __order[__vi] : 0xffffffffu;        // (no run: a number beyond them all)
     appy::i64 __eb = 0, __sb = 0;      // (in bytes from the start of the elements and of the row stream)
     const char* __entb = reinterpret_cast<const char*>(__ent);
     const char* __rsb = reinterpret_cast<const char*>(__rstream);
@@ -78,7 +82,7 @@ _spmv_kernel_loop_1_xcells(
       if (__any2) {
           if (!__end2) ++__tt;
           else {
-              __vc += gridDim.x; __tt = 0;
+              __vi += gridDim.x; __vc = __vi < __norder ? __order[__vi] : 0xffffffffu; __tt = 0;
                 if (__vc < __nrun) {
                     const unsigned __b = (__vc >> 3) / __spl, __part = (__vc >> 3) % __spl;
                     const appy::i64 __cell = (appy::i64)__b * 8 + __g;
@@ -110,7 +114,7 @@ _spmv_kernel_loop_1_xcells(
       if (__any2) {
           if (!__end2) ++__tt;
           else {
-              __vc += gridDim.x; __tt = 0;
+              __vi += gridDim.x; __vc = __vi < __norder ? __order[__vi] : 0xffffffffu; __tt = 0;
                 if (__vc < __nrun) {
                     const unsigned __b = (__vc >> 3) / __spl, __part = (__vc >> 3) % __spl;
                     const appy::i64 __cell = (appy::i64)__b * 8 + __g;
@@ -161,7 +165,7 @@ _spmv_kernel_loop_1_xcells(
           if (__any2) {
               if (!__end2) ++__tt;
               else {
-                  __vc += gridDim.x; __tt = 0;
+                  __vi += gridDim.x; __vc = __vi < __norder ? __order[__vi] : 0xffffffffu; __tt = 0;
                     if (__vc < __nrun) {
                         const unsigned __b = (__vc >> 3) / __spl, __part = (__vc >> 3) % __spl;
                         const appy::i64 __cell = (appy::i64)__b * 8 + __g;

@@ -822,7 +822,8 @@ def test_row_plans_kernel_that_writes_the_pairs_and_kernel_that_runs_a_plan():
         assert "__builtin_amdgcn_readfirstlane" in run
         # one sequence of tiles over all the runs of a workgroup: the next run is entered where the loads are issued, and
         # the sums of a run that is through go out inside the loop over the tiles
-        assert "while (__any0) {" in run and "__vc += gridDim.x; __tt = 0;" in run and "if (__end0) {" in run
+        assert "while (__any0) {" in run and "__vi += gridDim.x; __vc = __vi < __norder ? __order[__vi] : 0xffffffffu; __tt = 0;" in run
+        assert "if (__end0) {" in run
         assert "const unsigned* __restrict__ __cstart" in run.split("{", 1)[0] or "__restrict__ __cstart" in f.kernel_for(
             Spec("team", block=1024, vec=1, width=1024, unroll=unroll, parts=8, aux="xcells")).src.text
     with pytest.raises(ValueError):
@@ -838,6 +839,52 @@ def test_row_plans_kernel_that_writes_the_pairs_and_kernel_that_runs_a_plan():
     assert (shape.col_bits, shape.tile) == (20, 4096)
     arrays["x"] = np.broadcast_to(np.float32(0), (1 << 19,))                  # an operand that every L2 holds anyway
     assert f.plan_shape(1 << 22, {"M": 1 << 22}, arrays) is None
+
+
+def test_runs_of_a_row_plan_are_dealt_by_size():
+    """How many workgroups share a cell follows from the sizes of the cells, and the runs are dealt to the workgroups
+    of their column range largest first, back and forth: every run exactly once, every workgroup its own range only,
+    about the same number of tiles each."""
+    rng = np.random.default_rng(0)
+    # the uniform matrix of the benchmark: 1024 cells of 11 tiles, four per workgroup as they come
+    tiles = np.full(1024, 11)
+    assert cg.plan_split(tiles, 256, 6144, 16 << 22) == 1
+    order = cg.deal_runs(tiles, 1, 256)
+    assert len(order) == 1024 and sorted(order.tolist()) == list(range(1024))
+    assert all((int(order[w + 256 * i]) & 7) == (w & 7) for w in range(256) for i in range(4))
+    # a banded matrix: one cell of each block of rows holds all of its 86 tiles - two workgroups share a cell
+    tiles = np.zeros(1024, dtype=np.int64)
+    blocks = np.arange(128)
+    tiles[blocks * 8 + blocks * 8 // 128] = 86
+    assert cg.plan_split(tiles, 256, 6144, 16 << 22) == 2
+    assert cg.plan_split(tiles, 256, 6144, 16 << 22, forced=4) == 4
+    order = cg.deal_runs(tiles, 2, 256)
+    runs = order[order != 0xFFFFFFFF]
+    assert sorted(runs.tolist()) == list(range(2048))                      # runs without tiles are dealt too
+    size = lambda vc: (lambda b, part, g: ((part + 1) * tiles[b * 8 + g]) // 2 - (part * tiles[b * 8 + g]) // 2)((vc >> 3) // 2, (vc >> 3) % 2, vc & 7)
+    load = np.zeros(256, dtype=np.int64)
+    for p, vc in enumerate(order.tolist()):
+        if vc != 0xFFFFFFFF:
+            assert (vc & 7) == (p % 256) & 7
+            load[p % 256] += size(vc)
+    assert load.sum() == tiles.sum() and load.max() == 43 and load.min() == 43
+    # cells of random sizes: no workgroup far above the mean, lists without holes
+    tiles = rng.integers(0, 200, 1024)
+    split = cg.plan_split(tiles, 256, 6144, int(tiles.sum()) * 6144)
+    order = cg.deal_runs(tiles, split, 256)
+    load = np.zeros(256, dtype=np.int64)
+    for p, vc in enumerate(order.tolist()):
+        if vc != 0xFFFFFFFF:
+            b, part, g = (vc >> 3) // split, (vc >> 3) % split, vc & 7
+            load[p % 256] += ((part + 1) * tiles[b * 8 + g]) // split - (part * tiles[b * 8 + g]) // split
+            assert p < 256 or order[p - 256] != 0xFFFFFFFF
+    assert load.sum() == tiles.sum() and load.max() <= 1.15 * load.mean()
+    # few cells: several workgroups per cell, a workgroup per run
+    tiles = np.full(16, 40)
+    split = cg.plan_split(tiles, 256, 6144, 16 * 40 * 6144)
+    assert split == 20                                                     # until a run is down to two tiles
+    order = cg.deal_runs(tiles, split, min(16 * split, 256) // 8 * 8)
+    assert sorted(order[order != 0xFFFFFFFF].tolist()) == list(range(16 * split))
 
 
 def test_launch_shapes_follow_the_device_they_are_for():
