@@ -154,6 +154,41 @@ def test_spmv_full_size_with_the_order_of_the_elements_kept(env, kind):
     appy.release()
 
 
+def test_spmv_full_size_banded_matrix_shares_its_cells(env):
+    """A banded matrix of 2^22 rows (16 per row within 3000 columns of the diagonal): of the eight cells of a block of
+    rows one holds everything, so two workgroups share every cell and the runs are dealt by size; the product against a
+    float64 sum built with `index_add_`, the same bits from launch to launch."""
+    import appy_amd as appy
+    from appy_amd.backends.hip import codegen as cg
+
+    torch, k = env
+    m = n = 1 << 22
+    g = torch.Generator(device="cuda").manual_seed(5)
+    rows = torch.arange(m, device="cuda").repeat_interleave(16)
+    cols = (rows + torch.randint(-3000, 3000, (rows.numel(),), device="cuda", generator=g)).clamp_(0, n - 1)
+    cols, _ = cols.view(m, 16).sort(dim=1)
+    indices = cols.reshape(-1).to(torch.int32)
+    indptr = (torch.arange(m + 1, device="cuda") * 16).to(torch.int32)
+    data = torch.randn(rows.numel(), device="cuda", generator=g)
+    x = torch.randn(n, device="cuda", generator=g)
+    terms = data.double() * x.double()[indices.long()]
+    ref = torch.zeros(m, device="cuda", dtype=torch.float64).index_add_(0, rows, terms)
+    budget = torch.zeros(m, device="cuda", dtype=torch.float64).index_add_(0, rows, terms.abs())
+    del rows, cols, terms
+    ys = []
+    for launch in range(3):
+        y = k.spmv(data, indptr, indices, x, m, n)
+        assert bool(((y.double() - ref).abs() <= TOL * budget).all())
+        ys.append(y)
+    assert torch.equal(ys[1], ys[2])
+    loops = [v[0] for kk, v in cg.code_cache.items() if kk[-1] == "spmv" and getattr(v[0], "last_launch", None) is not None
+             and v[0].options.get("hip_reuse", True) is True]
+    launch = max(loops, key=lambda lp: lp.last_launch.serial).last_launch
+    plan = launch.plan
+    assert plan is not None and plan.ncell == 8 * (m >> 15) and plan.split == 2 and launch.grid[0] == plan.grid
+    appy.release()
+
+
 def test_spmm_full_size_against_spmv_columns(env):
     torch, k = env
     m = 1 << 20
