@@ -1769,7 +1769,7 @@ class Launch:
         self.args, self.grid, self.block = seq[0][1], seq[0][2], seq[0][3]
         if not loop._value_only and not self.small:
             # a call with these same tensors may repeat the two launches without staging them again, as long as the plan
-            # stands (`CompiledLoop._kept_order_still_true`)
+            # stands (`CompiledLoop._sequence_still_right`)
             import weakref
 
             self.seq_replay = ("plan", loop._scratch_gen, plan,
