@@ -409,12 +409,9 @@ def drop_plans_overlapping(extents):
 
 
 def plan_kernel_spec(tile: int, entries: int, rows: int, restrict: bool = True) -> Spec:
-    """The kernel that runs a row plan of tiles of `tile` elements over `entries` elements of `rows` rows.  Where
-    rows are short (fewer than 48 elements on average) the row numbers are a larger share of what a tile loads:
-    they are asked for ahead of the scatter (uniform 16 per row: 0.257 -> 0.252 ms; a power-law matrix of 98 per
-    row loses 1.7 % that way and keeps them behind it)."""
-    return Spec("team", block=1024, vec=1, width=1024, unroll=tile // 1024, parts=PLAN_GROUPS, aux="xcells", restrict=restrict,
-                stream_loads=entries < 48 * rows)
+    """The kernel that runs a row plan of tiles of `tile` elements (over `entries` elements of `rows` rows: one
+    shape for all of them)."""
+    return Spec("team", block=1024, vec=1, width=1024, unroll=tile // 1024, parts=PLAN_GROUPS, aux="xcells", restrict=restrict)
 
 
 def plan_split(tiles, cus: int, tile: int, entries: int, forced=None) -> int:

@@ -92,8 +92,7 @@ class Spec:
                                  # than a limit given at the launch are passed over (they run in planned parts)
                                  # 'rkeys' = the kernel that turns the elements of `block_rows` rows per wavefront into the
                                  # (key, value) pairs a row plan is built from, 'xcells' = the kernel that runs a row plan
-                                 # (`parts` column ranges, `unroll` x 1024 elements per tile; `stream_loads`: the row
-                                 # numbers of the next tile are asked for ahead of the scatter of the current one)
+                                 # (`parts` column ranges, `unroll` x 1024 elements per tile)
     guard: int = 0               # 1 = the kernel returns at once when the grouping kernel of this launch has refused
                                  # its input (row ranges that do not follow one another: a flag in device memory),
                                  # 2 = when it has not
@@ -3190,10 +3189,10 @@ class KernelBuilder:
             w(f"  {da} = *reinterpret_cast<const unsigned*>(__q + __at);")
             w(f"  {db} = *reinterpret_cast<const unsigned*>(__q + __at + 4); }}")
 
-        def gather(dst, src, inn):
+        def gather(dst, src, inn, first, last):
             w("{")
             w("#pragma unroll")
-            w(f"  for (int __u = 0; __u < {U}; ++__u) {{")
+            w(f"  for (int __u = {first}; __u < {last}; ++__u) {{")
             w(f"    unsigned __c = __x0 + ((unsigned)({src}[__u] >> 32) & __cmask);")
             w("    __c = __c < __xlast ? __c : __xlast;        // (what was read beyond the cell may hold anything)")
             w(f"    {dst}[__u] = *reinterpret_cast<const {x.elem_c}*>(__xb + appy::lane_offset({inn} ? (unsigned)(__c << 2) : 0u));")
@@ -3224,16 +3223,18 @@ class KernelBuilder:
         w("__h1 = __builtin_amdgcn_readfirstlane(__hv2);")
         shift(2, 1)
         load_rows("__r0", "__da0", "__db0", "__h0", "__in0", "__ps0")
-        gather("__xv", "__e0", "__in0")
+        gather("__xv", "__e0", "__in0", 0, U)
         w("__syncthreads();")
         w("while (__any0) {")
         self.ind += 1
         w("const unsigned __ns = __in0 ? __h0 & 0xffffu : 0u, __nm = __in0 ? __h0 >> 16 : 0u;")
+        # Where the loads of the next tiles are asked for was settled with cycle counters at the boundaries of the phases: a
+        # wave that asks for a load waits until the texture addresser takes it, and with every load ahead of the first
+        # barrier all waves stood in that queue together (7000 of 11300 cycles per tile) while LDS was idle, and then
+        # added up together while the addresser was idle.  So the element stream of the tile after the next goes first (it
+        # comes from HBM), the row numbers follow the scatter, and the gathers are asked for in two halves between the
+        # phases that add up: waves that have been served go on adding while the others queue.
         load_tile("__e2")
-        if self.spec.stream_loads:
-            # (matrices of short rows: the row numbers of the next tile leave with the element stream, ahead of the scatter;
-            #  measured on one box: uniform 16 per row 0.257 -> 0.252 ms, power law of mean 98 1.086 -> 1.104 ms)
-            load_rows("__r1", "__da1", "__db1", "__h1", "__in1", "__ps1")
         w(f"if (__cnt0 == {TILE}u) {{")
         w("#pragma unroll")
         w(f"    for (int __u = 0; __u < {U}; ++__u) {{")
@@ -3249,10 +3250,7 @@ class KernelBuilder:
         w("        if (__u * 1024 + __tid < __cnt0) __prod[(unsigned)(__e0[__u] >> 32) >> __colbits] = __val;")
         w("    }")
         w("}")
-        w("// the elements of the tile after the next, the row numbers and the gathers of the next one travel while this one is added up")
-        if not self.spec.stream_loads:
-            load_rows("__r1", "__da1", "__db1", "__h1", "__in1", "__ps1")
-        gather("__x1", "__e1", "__in1")
+        load_rows("__r1", "__da1", "__db1", "__h1", "__in1", "__ps1")
         w("__syncthreads();")
         w("{")
         w(f"    {P} __sa[{H}], __sb_[{H}];")
@@ -3269,6 +3267,7 @@ class KernelBuilder:
         w("        if (__s + 1 < __ns) __sum[(__r0[__u] >> 16) & 0x7fffu] = __sb_[__u] + __pp[__u][1];")
         w("    }")
         w("}")
+        gather("__x1", "__e1", "__in1", 0, H)
         w("if (__nm > 0) {")
         self.ind += 1
         w("if (__tid < __nm) {")
@@ -3287,6 +3286,7 @@ class KernelBuilder:
         w("}")
         self.ind -= 1
         w("}")
+        gather("__x1", "__e1", "__in1", H, U)
         w("__syncthreads();")
         w("if (__end0) {")
         self.ind += 1

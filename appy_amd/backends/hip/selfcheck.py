@@ -195,7 +195,6 @@ def compile_all_patterns() -> int:
                          # sort, the kernel that runs the plan
                          Spec("team", block=256, vec=1, width=64, aux="rkeys", block_rows=256),
                          Spec("team", block=1024, vec=1, width=1024, unroll=6, parts=8, aux="xcells"),
-                         Spec("team", block=1024, vec=1, width=1024, unroll=6, parts=8, aux="xcells", stream_loads=True),
                          Spec("team", block=1024, vec=1, width=1024, unroll=4, parts=8, aux="xcells")]
         for spec in more:
             loop.kernel_for(spec).code

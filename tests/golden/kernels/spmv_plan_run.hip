@@ -1,4 +1,4 @@
-// kernel for spmv_kernel_loop_1_xcells: team_b1024_v1_u6_w1024_r_nt_s8_xcells
+// kernel for spmv_kernel_loop_1_xcells: team_b1024_v1_u6_w1024_r_s8_xcells
 extern "C" __global__ void __launch_bounds__(1024)
 _spmv_kernel_loop_1_xcells(
     const int* __restrict__ A_indptr,
@@ -182,15 +182,6 @@ _spmv_kernel_loop_1_xcells(
               }
           }
         }
-        {
-        #pragma unroll
-          for (int __u = 0; __u < 3; ++__u)
-              __r1[__u] = __builtin_nontemporal_load(reinterpret_cast<const unsigned*>(__rsb + __ps1 + appy::lane_offset(__in1 ? (unsigned)((1 + __u * 1024 + __tid) * 4) : 0u)));
-          const unsigned __runs = (__h1 >> 16);
-          const char* __q = __rsb + (__ps1 + (__in1 ? (appy::i64)(1 + (((__h1 & 0xffffu) + 1) >> 1)) * 4 : 0));     // (the header of a tile that does not exist may hold anything)
-          const unsigned __at = appy::lane_offset(__in1 && __tid < __runs ? __tid * 4 : 0u);        // (lanes without a run: one position)
-          __da1 = *reinterpret_cast<const unsigned*>(__q + __at);
-          __db1 = *reinterpret_cast<const unsigned*>(__q + __at + 4); }
         if (__cnt0 == 6144u) {
         #pragma unroll
             for (int __u = 0; __u < 6; ++__u) {
@@ -206,14 +197,15 @@ _spmv_kernel_loop_1_xcells(
                 if (__u * 1024 + __tid < __cnt0) __prod[(unsigned)(__e0[__u] >> 32) >> __colbits] = __val;
             }
         }
-        // the elements of the tile after the next, the row numbers and the gathers of the next one travel while this one is added up
         {
         #pragma unroll
-          for (int __u = 0; __u < 6; ++__u) {
-            unsigned __c = __x0 + ((unsigned)(__e1[__u] >> 32) & __cmask);
-            __c = __c < __xlast ? __c : __xlast;        // (what was read beyond the cell may hold anything)
-            __x1[__u] = *reinterpret_cast<const float*>(__xb + appy::lane_offset(__in1 ? (unsigned)(__c << 2) : 0u));
-          } }
+          for (int __u = 0; __u < 3; ++__u)
+              __r1[__u] = __builtin_nontemporal_load(reinterpret_cast<const unsigned*>(__rsb + __ps1 + appy::lane_offset(__in1 ? (unsigned)((1 + __u * 1024 + __tid) * 4) : 0u)));
+          const unsigned __runs = (__h1 >> 16);
+          const char* __q = __rsb + (__ps1 + (__in1 ? (appy::i64)(1 + (((__h1 & 0xffffu) + 1) >> 1)) * 4 : 0));     // (the header of a tile that does not exist may hold anything)
+          const unsigned __at = appy::lane_offset(__in1 && __tid < __runs ? __tid * 4 : 0u);        // (lanes without a run: one position)
+          __da1 = *reinterpret_cast<const unsigned*>(__q + __at);
+          __db1 = *reinterpret_cast<const unsigned*>(__q + __at + 4); }
         __syncthreads();
         {
             float __sa[3], __sb_[3];
@@ -230,6 +222,13 @@ _spmv_kernel_loop_1_xcells(
                 if (__s + 1 < __ns) __sum[(__r0[__u] >> 16) & 0x7fffu] = __sb_[__u] + __pp[__u][1];
             }
         }
+        {
+        #pragma unroll
+          for (int __u = 0; __u < 3; ++__u) {
+            unsigned __c = __x0 + ((unsigned)(__e1[__u] >> 32) & __cmask);
+            __c = __c < __xlast ? __c : __xlast;        // (what was read beyond the cell may hold anything)
+            __x1[__u] = *reinterpret_cast<const float*>(__xb + appy::lane_offset(__in1 ? (unsigned)(__c << 2) : 0u));
+          } }
         if (__nm > 0) {
             if (__tid < __nm) {
                 { const int __row = (int)(__da0 & 32767u), __from = (int)(__da0 >> 15), __to = (int)(__db0 >> 15);
@@ -260,6 +259,13 @@ _spmv_kernel_loop_1_xcells(
                 }
             }
         }
+        {
+        #pragma unroll
+          for (int __u = 3; __u < 6; ++__u) {
+            unsigned __c = __x0 + ((unsigned)(__e1[__u] >> 32) & __cmask);
+            __c = __c < __xlast ? __c : __xlast;        // (what was read beyond the cell may hold anything)
+            __x1[__u] = *reinterpret_cast<const float*>(__xb + appy::lane_offset(__in1 ? (unsigned)(__c << 2) : 0u));
+          } }
         __syncthreads();
         if (__end0) {
             // the run is through: its sums go out and start again at zero (every lane clears what it has read itself; the next

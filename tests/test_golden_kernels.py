@@ -38,7 +38,7 @@ CASES = {
     "spmv_sums_of_cells": ("spmv", Spec("team", block=256, vec=4, width=1, phase=2, guard=1)),
     # the kept order of the elements (row plans): the kernel that writes the pairs the inspector sorts, the kernel that runs a plan
     "spmv_plan_pairs": ("spmv", Spec("team", block=256, vec=1, width=64, aux="rkeys", block_rows=256)),
-    "spmv_plan_run": ("spmv", Spec("team", block=1024, vec=1, width=1024, unroll=6, parts=8, aux="xcells", stream_loads=True)),
+    "spmv_plan_run": ("spmv", Spec("team", block=1024, vec=1, width=1024, unroll=6, parts=8, aux="xcells")),
     "spmm": ("spmm", Spec("team", block=256, vec=4, width=32, extent=128)),
 }
 
