@@ -203,3 +203,24 @@ def identity_literal(op: str, t: Ty) -> str:
         return "((long long)(-9223372036854775807LL - 1))"
     suffix = "ULL" if t.kind == "u" else "LL"
     return f"(({t.c}){val}{suffix})"
+
+
+def partial_type(ty: Ty) -> Ty:
+    """Type of the per-lane partial results of a reduction: registers and cross-lane
+    steps are 32 or 64 bits wide, so 16-bit floats accumulate in float32 (rounded once,
+    when the team combines) and 8/16-bit integers and flags in 32-bit integers (sums wrap
+    to the narrow type at the end exactly as they would have step by step)."""
+    if ty.size >= 4:
+        return ty
+    if ty.is_float:
+        return F32
+    return Ty("uint32") if ty.kind == "u" else I32
+
+
+def partial_identity(op: str, ty: Ty, pty: Ty) -> str:
+    """Neutral element of ``op`` over ``ty``, written in the partial type ``pty``."""
+    if pty == ty or ty.is_float:
+        return identity_literal(op, pty)
+    if ty.is_bool:
+        return "0" if op in ("max", "+") else "1"
+    return f"(({pty.c}){identity_literal(op, ty)})"
