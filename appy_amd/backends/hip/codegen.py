@@ -19,9 +19,7 @@ from __future__ import annotations
 import ast
 import ctypes as C
 import dataclasses
-import hashlib
 import math
-import os
 import threading
 import types as _types
 
@@ -33,10 +31,12 @@ from . import dtypes as T
 from . import runtime as rt
 from ... import graphs, residency
 from .exprs import ArrayParam, ScalarParam
-from .kernelgen import KernelBuilder, KernelSource, LoopAnalysis, Spec, Unsupported  # noqa: F401 - Unsupported is part of this module's interface
-
-ARCH = "gfx950"
-_HEADER_PATH = os.path.join(os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__)))), "csrc", "appy_device.h")
+from .csr_staging import CsrStaging
+from .device import (ARCH, Hardware, Kernel, MI355X, compile_source, device_header, hardware, scratch_limit,  # noqa: F401 - part of this module's interface
+                     _current_raw_stream, _ensure_device)
+from .kernelgen import KernelBuilder, KernelSource, LoopAnalysis, Spec, Unsupported  # noqa: F401 - part of this module's interface
+from .row_plans import (PLAN_GROUPS, PLAN_ROW_BITS, PLANS_PER_LOOP, RowPlan, _live_plans, deal_runs,  # noqa: F401 - part of this module's interface
+                        drop_plans_overlapping, plan_kernel_spec, plan_split)
 
 code_cache = {}
 _cache_lock = threading.Lock()
@@ -45,7 +45,6 @@ _cache_lock = threading.Lock()
 # only these builtins (a bound like ``range(min(n, m))`` is ordinary Python).
 _HOST_EVAL_GLOBALS = {"__builtins__": {"min": min, "max": max, "abs": abs, "int": int, "len": len, "float": float,
                                        "round": round, "bool": bool}}
-_device_header = None
 
 
 class _ShapeView:
@@ -63,51 +62,6 @@ class _ShapeView:
         if not self.shape:
             raise TypeError("len() of a 0-d array")
         return self.shape[0]
-
-@dataclasses.dataclass(frozen=True)
-class Hardware:
-    """What the launch heuristics know of a device.  The defaults are MI355X's: 256 CUs in 8 XCDs, an L2 of
-    4 MiB per XCD, 256 MiB of memory-side cache in front of the HBM3E (the one figure the runtime does not
-    report: `APPY_HIP_MALL_BYTES` overrides it)."""
-
-    cus: int = 256
-    xcds: int = 8
-    l2_bytes: int = 4 << 20
-    mall_bytes: int = 256 << 20
-
-    @property
-    def stripe_bytes(self) -> int:
-        """Most of a gathered operand that one XCD is given to keep in its L2 next to the streams: half the L2."""
-        return self.l2_bytes // 2
-
-    @property
-    def stripe_min_bytes(self) -> int:
-        """A gathered operand up to this size is left to every L2 as a whole."""
-        return 3 * self.l2_bytes // 4
-
-    @property
-    def pinned_stripes(self) -> bool:
-        """Stripes of a gathered operand are pinned to XCDs by workgroup number modulo 8 in the generated kernels."""
-        return self.xcds == 8
-
-
-MI355X = Hardware()
-_hardware = {}
-
-
-def hardware(device=None) -> Hardware:
-    """The facts of ``device`` as the runtime reports them; MI355X's when no device is named (kernels generated
-    and launch shapes chosen without a GPU)."""
-    if device is None:
-        return MI355X
-    hw = _hardware.get(device)
-    if hw is None:
-        t = rt.device_topology(device)
-        hw = Hardware(cus=int(t["compute_units"]) or MI355X.cus, xcds=int(t["xcds"]) or 1,
-                      l2_bytes=int(t["l2_bytes_per_xcd"]) or MI355X.l2_bytes,
-                      mall_bytes=int(os.environ.get("APPY_HIP_MALL_BYTES") or MI355X.mall_bytes))
-        _hardware[device] = hw
-    return hw
 
 
 # (the figures of MI355X under their old names: tests and tools that size their inputs by them)
@@ -133,32 +87,6 @@ BIN_MIN_ROWS = 1 << 15
 STRIPE_MIN_BYTES = MI355X.stripe_min_bytes
 STRIPE_BYTES = MI355X.stripe_bytes
 GROUP_MIN_TRIP = 4                 # ... for rows of this many elements on average, at least
-# row plans (the order of the elements of a CSR-like sum, worked out once and kept between launches)
-PLAN_ROW_BITS = 15                 # rows per block: what fits a workgroup's LDS as 4-byte sums
-PLAN_GROUPS = 8                    # column ranges of the gathered operand, one per XCD
-PLANS_PER_LOOP = 2                 # plans a loop keeps (least recently used goes first)
-
-
-def scratch_limit(device: int) -> int:
-    """Most bytes of device memory one loop may hold for its own purposes (scratch buffers of launches made of
-    several kernels, row plans): `APPY_HIP_SCRATCH_MAX_BYTES`, or a quarter of the device's memory."""
-    env = os.environ.get("APPY_HIP_SCRATCH_MAX_BYTES")
-    if env:
-        return int(env)
-    if device not in _hbm_bytes:
-        _hbm_bytes[device] = int(rt.device_props(device)["hbm_bytes"])
-    return _hbm_bytes[device] // 4
-
-
-_hbm_bytes = {}
-
-
-def device_header() -> str:
-    global _device_header
-    if _device_header is None:
-        with open(_HEADER_PATH) as f:
-            _device_header = f.read()
-    return _device_header
 
 
 # ---------------------------------------------------------------------------
@@ -213,160 +141,12 @@ def _signature(val_map):
     return tuple(sig)
 
 
-# ---------------------------------------------------------------------------
-# compiled kernels
-# ---------------------------------------------------------------------------
-def _disk_cache_dir():
-    if os.environ.get("APPY_HIP_NO_DISK_CACHE") == "1":
-        return None
-    d = os.environ.get("APPY_HIP_CACHE_DIR") or os.path.join(os.path.expanduser("~"), ".cache", "appy_hip")
-    try:
-        os.makedirs(d, exist_ok=True)
-    except OSError:
-        return None
-    return d
-
-
-def compile_source(text: str, name: str) -> bytes:
-    """HIP C++ -> gfx950 code object, through hiprtc, with an on-disk cache
-    keyed on the source text, the compiler options and the compiler version."""
-    d = _disk_cache_dir()
-    path = None
-    if d:
-        h = hashlib.sha256()
-        h.update(text.encode())
-        h.update(repr(rt.BASE_COMPILE_OPTIONS + rt.extra_compile_options()).encode())
-        h.update(ARCH.encode())
-        h.update(str(rt.rtc_version()).encode())
-        path = os.path.join(d, h.hexdigest() + ".co")
-        if os.path.exists(path):
-            with open(path, "rb") as f:
-                code = f.read()
-            if code[:4] == b"\x7fELF":
-                return code
-    code = rt.compile_to_code_object(text, name + ".hip", ARCH)
-    if path:
-        tmp = path + f".{os.getpid()}.tmp"
-        try:
-            with open(tmp, "wb") as f:
-                f.write(code)
-            os.replace(tmp, path)
-        except OSError:
-            pass
-    return code
-
-
-class Kernel:
-    """One compiled variant of a loop."""
-
-    def __init__(self, src: KernelSource):
-        self.src = src
-        self._code = None
-        self._compile_lock = threading.Lock()
-        self._funcs = {}   # device -> function handle
-        fields = [(f"f{i}", p.ctype) for i, p in enumerate(src.params)]
-        self.ArgStruct = type("Args" + src.name, (C.Structure,), {"_fields_": fields})
-        self._field_names = [f for f, _ in fields]
-
-    @property
-    def code(self) -> bytes:
-        """The code object, compiled when first asked for: a loop is generated in its default
-        shape when it is first seen, but the launch may pick another shape, and hiprtc takes a
-        few hundred milliseconds per variant."""
-        if self._code is None:
-            with self._compile_lock:
-                if self._code is None:
-                    self._code = compile_source(self.src.text, self.src.name)
-        return self._code
-
-    def function(self, device: int):
-        f = self._funcs.get(device)
-        if f is None:
-            mod = rt.Module(self.code)
-            f = (mod, mod.function(self.src.name))
-            self._funcs[device] = f
-        return f[1]
-
-
-# ---------------------------------------------------------------------------
-# the launcher
-# ---------------------------------------------------------------------------
-_tls = threading.local()
-
-
-def _ensure_device(dev: int):
-    """HIP's current device is a per-thread setting."""
-    if getattr(_tls, "device", None) != dev:
-        rt.init(dev)
-        _tls.device = dev
-
-
-_raw_stream_getter = None
-
-
-def _current_raw_stream(device: int) -> int:
-    """PyTorch's current stream on ``device`` as a raw handle."""
-    global _raw_stream_getter
-    if _raw_stream_getter is None:
-        import torch
-
-        _raw_stream_getter = getattr(torch._C, "_cuda_getCurrentRawStream", None) or (
-            lambda dev: torch.cuda.current_stream(dev).cuda_stream)
-    return _raw_stream_getter(device)
-
-
 def _pow2ceil(x: float) -> int:
     n = 1
     while n < x:
         n <<= 1
     return n
 
-
-
-class RowPlan:
-    """The elements of one set of arrays in the order `xcells` kernels walk them, in device memory
-    that this object owns.  It describes the arrays as they were when it was built: it is used only
-    while every array it read is still the same object with the same version counter (tensors count
-    the in-place operations PyTorch performs on them), and it is dropped when a launch of this
-    package stores into memory one of those arrays occupies."""
-
-    def __init__(self, device, key, refs, ranges):
-        self.device = device
-        self.key = key
-        self.refs = refs            # weak references to the tensors the plan was built from
-        self.ranges = ranges        # (address, bytes) of those tensors
-        self.buffers = []           # device allocations of the plan
-        self.nbytes = 0
-        self.valid = False
-        self.bin = {}               # arguments of the kernels that run the plan
-        self.ncell = 0
-        self.tile = 0
-        self.split = 1              # workgroups per cell
-        self.grid = 8               # workgroups of the kernel that runs the plan
-        self.entries = 0            # positions of the streamed arrays the plan was built from
-        self.owner = None           # the loop the plan belongs to
-        self.inspector_ms = None
-
-    def alloc(self, nbytes):
-        ptr = rt.malloc(max(256, nbytes))
-        self.buffers.append(ptr)
-        self.nbytes += nbytes
-        return ptr
-
-    def alive(self, tensors) -> bool:
-        return self.valid and all(r() is t for r, t in zip(self.refs, tensors))
-
-    def release(self):
-        self.valid = False
-        bufs, self.buffers = self.buffers, []
-        for ptr in bufs:
-            try:
-                rt.free(ptr)
-            except Exception:       # the runtime may be shutting down
-                pass
-        with _plans_lock:
-            if self in _live_plans:
-                _live_plans.remove(self)
 
 
 # Page-locked slots with device memory of their own for host arrays of a few bytes (`shared()` scalars):
@@ -382,81 +162,6 @@ def _take_small_slot(device):
         if free:
             return free.pop()
     return (rt.host_alloc(_SMALL_SLOT_BYTES), rt.malloc(256))
-
-
-_live_plans = []        # every valid plan of the process: launches that store into their arrays drop them
-_plans_lock = threading.Lock()
-
-
-def drop_plans_overlapping(extents):
-    """``extents``: (name, address, bytes, stored) of a launch's arrays.  Plans built from memory that
-    the launch stores into are no longer true."""
-    if not _live_plans:
-        return
-    stored = [(p, n) for _name, p, n, st in extents if st]
-    if not stored:
-        return
-    with _plans_lock:
-        hit = [plan for plan in _live_plans
-               if any(p < q + m and q < p + n for p, n in stored for q, m in plan.ranges)]
-    for plan in hit:
-        plan.valid = False      # its memory goes back once the launches that use it have drained (CompiledLoop.release / next build)
-        if plan.owner is not None:
-            plan.owner._plan_seen.clear()       # the arrays have changed: they count as new
-        with _plans_lock:
-            if plan in _live_plans:
-                _live_plans.remove(plan)
-
-
-def plan_kernel_spec(tile: int, entries: int, rows: int, restrict: bool = True) -> Spec:
-    """The kernel that runs a row plan of tiles of `tile` elements (over `entries` elements of `rows` rows: one
-    shape for all of them)."""
-    return Spec("team", block=1024, vec=1, width=1024, unroll=tile // 1024, parts=PLAN_GROUPS, aux="xcells", restrict=restrict)
-
-
-def plan_split(tiles, cus: int, tile: int, entries: int, forced=None) -> int:
-    """Workgroups that share a cell of a row plan (each takes a run of its tiles and has a slot of its own for the
-    sums).  `tiles`: tiles per cell.  Few cells (a matrix of few blocks of rows): until there are some four runs per
-    compute unit or a run is down to two tiles.  Cells of very different sizes (a banded matrix: one of the eight
-    cells of a block of rows holds everything): until the largest run is no more than about what a workgroup gets
-    on average.  Every doubling doubles the sums the second kernel reads, so it stops at 32."""
-    if forced:
-        return int(forced)
-    ncell = len(tiles)
-    split = max(1, min(-(-4 * cus // ncell), entries // (2 * tile * ncell), 32))
-    total, largest = int(tiles.sum()), int(tiles.max()) if ncell else 0
-    workgroups = max(8, cus // 8 * 8)
-    while split < 32 and largest > 4 * split and -(-largest // split) > 1.25 * total / workgroups:
-        split *= 2
-    return split
-
-
-def deal_runs(tiles, split: int, grid: int):
-    """The runs of tiles of a row plan dealt to `grid` workgroups (a multiple of eight; workgroup w reads column
-    range w mod 8 only): entry w + grid * i of the result is the i-th run of workgroup w, 0xFFFFFFFF for none.
-    Run (block * split + part) * 8 + range holds the tiles [part * t / split, (part + 1) * t / split) of its
-    cell of t tiles.  Per range the runs are sorted by size and dealt out back and forth, so that workgroups
-    end up with about the same number of tiles whatever the sizes of the cells; runs without tiles are dealt
-    too (their sums must be written)."""
-    tiles = np.asarray(tiles, dtype=np.int64)
-    ncell = len(tiles)
-    per_range = grid // PLAN_GROUPS
-    blocks = ncell // PLAN_GROUPS
-    parts = np.arange(split, dtype=np.int64)
-    t = tiles.reshape(blocks, PLAN_GROUPS)                                               # [block, range]
-    size = ((parts[None, None, :] + 1) * t[:, :, None]) // split - (parts[None, None, :] * t[:, :, None]) // split
-    run = (np.arange(blocks, dtype=np.int64)[:, None, None] * split + parts[None, None, :]) * PLAN_GROUPS \
-        + np.arange(PLAN_GROUPS, dtype=np.int64)[None, :, None]
-    rounds = -(-(blocks * split) // per_range)
-    order = np.full(rounds * grid, 0xFFFFFFFF, dtype=np.uint32)
-    for g in range(PLAN_GROUPS):
-        sz, rn = size[:, g, :].reshape(-1), run[:, g, :].reshape(-1)
-        by_size = np.lexsort((rn, -sz))                                                  # largest first, ties by number
-        rank = np.arange(len(by_size))
-        rnd, pos = rank // per_range, rank % per_range
-        member = np.where(rnd % 2 == 0, pos, per_range - 1 - pos)
-        order[(g + PLAN_GROUPS * member) + grid * rnd] = rn[by_size].astype(np.uint32)
-    return order
 
 
 def release_all_plans():
@@ -1251,7 +956,7 @@ class CompiledLoop:
         return Launch(self, vals, arrays, env, lo, hi)
 
 
-class Launch:
+class Launch(CsrStaging):
     """One staged launch: device pointers, argument block, grid."""
 
     serial = 0      # launches staged so far in this process (a diagnostic: which of two loops ran last)
@@ -1437,458 +1142,6 @@ class Launch:
                                        row_hint=loop.row_hint(n_outer, env, arrays)), 1, 1)
         self.block = (spec.block, 1, 1)
         loop.last_launch = self
-
-    def _stage_binned(self, vals, arrays, lo, hi, spec):
-        """The launches of a loop whose rows are sorted by the trip count of their simd loop first:
-        clear the counters, sort (`bins`), the rows of all classes (`mixed`), and for long rows that
-        gather from a large operand: cut them at the stripes of that operand (`plan`), run the parts
-        (phase 1), fold the partial results and run the rest of the body (phase 2)."""
-        loop, a, env = self.loop, self.loop.analysis, self.env
-        n = hi - lo
-        V = spec.vec
-        thresholds = [V, 8 * V, 32 * V]
-        widthlog = [0, 2, 4, 6]
-        trip, _uniform = loop._estimate_trip(env, arrays, n)
-        base = sum(1 for t in thresholds if trip > t)
-        # what the last launch of this loop found in its classes, if it was about the same arrays (a hint: their
-        # contents may have changed).  The class with most rows is the one to take in natural order; without
-        # long rows last time, this launch sets nothing up for parts (long rows, if there are some after
-        # all, then run whole).  Neither changes the order in which the terms of a row are added.
-        hint_addr, hint = loop.hint(self.device)
-        seen = [int(hint[k]) for k in range(5)] if self.loop.options.get("hip_hints", True) else [0] * 5
-        ident = self._hint_identity(arrays, lo, hi) if a.grouping is not None else (lo, hi)
-        known = loop._hint_key.get(self.device) == ident and seen[0] == 1 and sum(seen[1:]) == n and min(seen[1:]) >= 0
-        loop._hint_key[self.device] = ident
-        parts, stripe, cap = 0, 0, 0
-        gather = a.ragged[1]
-        if gather is not None:
-            x = arrays[gather[0]]
-            x_bytes = int(x.shape[0]) * a.arrays[gather[0]].ty.size
-            if self.hw.pinned_stripes and x_bytes > self.hw.stripe_min_bytes:
-                parts = min(64, 8 * -(-x_bytes // (8 * self.hw.stripe_bytes)))
-                stripe = -(-int(x.shape[0]) // parts)
-                thresholds[2] = max(thresholds[2], 32 * parts)       # 32 elements per part at least
-                # rows longer than the threshold: no more of them than the streamed arrays have room for
-                bound = max([int(arrays[nm].shape[0]) for _code, streamed in loop._simd_loops for nm in streamed
-                             if arrays[nm].ndim == 1] or [0])
-                cap = min(n, bound // thresholds[2] + 1) if bound else n
-        if known:
-            # (the thresholds follow from element sizes and the size of the gathered operand, so the classes
-            #  of the hint are the classes of this launch whenever the hint is about these arrays)
-            base = max(range(4), key=lambda c: seen[c + 1])
-            if seen[4] == 0:
-                parts, stripe, cap = 0, 0, 0
-        reds = max(1, len(loop_ir.reductions_of(a.team_split)))
-        # one buffer: counters | row lists of the four classes | part boundaries | row starts | partial results
-        # header: 8 counters, 64 part loads (8 bytes each), and a second such block that the binning kernel
-        # clears instead when it is not run to clear the first
-        off_rows = 2048
-        off_bnd = off_rows + 4 * 4 * n
-        off_start = (off_bnd + 4 * (parts + 1) * cap + 255) // 256 * 256        # where each listed row starts (8 bytes)
-        off_part = (off_start + 8 * cap + 255) // 256 * 256
-        total = off_part + 8 * reds * parts * cap
-        buf = loop.scratch(self.device, self.stream, total)
-        if buf is None:
-            return False
-        self.bin = {
-            "counts": buf, "load": buf + 32, "zero": buf + 1024, "rows": buf + off_rows, "m": n, "base": base, "threshold": thresholds,
-            "widthlog": widthlog, "skip": cap if parts else 0, "bnd": buf + off_bnd, "rowstart": buf + off_start, "cap": cap, "stripe": stripe,
-            "nrows": buf + 4 * 3, "hint": hint_addr, "tlo": thresholds[base - 1] if base > 0 else -(1 << 62),
-            "thi": thresholds[base] if base < 3 else (1 << 62),
-        }
-        self.scratch_ptr = buf + off_part
-        self.nsplit = parts
-        common = dict(block=256, vec=V, restrict=spec.restrict, stream_loads=spec.stream_loads)
-        bins = loop.kernel_for(Spec("team", block=1024, vec=1, width=1, restrict=spec.restrict, aux="bins"))
-        seq = []
-        # the counters are cleared by the binning kernel itself, run over an empty range
-        self.bin["zero"] = buf
-        seq.append((bins, self._argument_block(bins, vals, arrays, 0, 0), (1, 1, 1), (1024, 1, 1)))
-        self.bin["zero"] = buf + 1024
-        seq.append((bins, self._argument_block(bins, vals, arrays, lo, hi),
-                    (max(1, min(512, -(-n // 4096))), 1, 1), (1024, 1, 1)))
-        # a wavefront for every slot of the base class: the other classes follow in further passes of the grid
-        # (uniform rows of 16: 0.927 ms, as without binning, against 0.936 ms with 16384 workgroups that loop)
-        waves = -(-(n << widthlog[base]) // 64)
-        seq.append((self.kernel, self._argument_block(self.kernel, vals, arrays, lo, hi),
-                    (max(256, min(loop.options.get("hip_max_blocks") or (1 << 20), -(-waves // 4))), 1, 1), (256, 1, 1)))
-        if parts:
-            ts = 8
-            while ts < parts:
-                ts *= 2
-            self.bin["rows"] = buf + off_rows + 4 * 3 * n         # the list of class 3
-            plan = loop.kernel_for(Spec("team", width=ts, rows="list", parts=parts, aux="plan",
-                                        **{**common, "vec": 1, "stream_loads": False}))
-            first = loop.kernel_for(Spec("team", width=16, phase=1, rows="list", parts=parts, **common))
-            last = loop.kernel_for(Spec("team", width=1, phase=2, rows="list", parts=parts, **common))
-            seq.append((plan, self._argument_block(plan, vals, arrays, lo, hi),
-                        (max(1, min(2048, -(-cap * ts // 256))), 1, 1), (256, 1, 1)))
-            seq.append((first, self._argument_block(first, vals, arrays, lo, hi),
-                        (max(8, min(2048, 8 * -(-cap * 16 // 256))), 1, 1), (256, 1, 1)))
-            seq.append((last, self._argument_block(last, vals, arrays, lo, hi),
-                        (max(1, min(1024, -(-cap // 256))), 1, 1), (256, 1, 1)))
-        self.sequence = seq
-        self.args, self.grid, self.block = seq[2][1], seq[2][2], seq[2][3]
-        if known and not self.plan_pending and not loop._value_only and not self.small:
-            self.seq_replay = ("hints", loop._scratch_gen, ident, tuple(seen))
-        return True
-
-    def _stage_grouped(self, vals, arrays, lo, hi, spec) -> bool:
-        """The launches of a loop of short rows whose simd loop sums terms that gather from an operand
-        larger than an L2: group the elements of every 256 rows by the stripe of the operand they read
-        (`group`), run the groups, stripe s on XCD s mod 8, sums per row and stripe to the scratch buffer
-        (`cells`), add the sums of a row and run the rest of the body (phase 2).  The grouping kernel
-        checks that the rows' ranges follow one another (as those of a CSR matrix do); where they do
-        not, it raises a flag, the kernels after it return at once, and the loop runs row by row.
-        When the last launch has reported rows in the class of the longest, the same launch lists those
-        rows (`bins`), leaves them out of the groups and runs them in parts cut at the stripes (`plan`,
-        `parts`, `fold`).  False (nothing staged) when the launch does not qualify."""
-        loop, a, env = self.loop, self.loop.analysis, self.env
-        n = hi - lo
-        g = a.grouping
-        if g is None or self.capture is not None:
-            # (a launch recorded into a graph keeps its rows sorted by length: this form clears its flag with a
-            #  memory-set node, and those are kept out of graphs)
-            return False
-        V = spec.vec
-        # The form of the launch follows from what the host knows of these arrays (their sizes).  What the last
-        # launch of the loop reported about the lengths of the rows only prunes it: when that launch was about
-        # these same arrays and found no row beyond the limit, the kernels for such rows - which would run
-        # empty - are left out.  Both forms add the terms of a row in the same order.
-        _addr, hint = loop.hint(self.device)
-        seen = [int(hint[k]) for k in range(5)]
-        ident = self._hint_identity(arrays, lo, hi)
-        trusted = (loop.options.get("hip_hints", True) and loop._hint_key.get(self.device) == ident
-                   and seen[0] == 1 and sum(seen[1:]) == n and min(seen[1:]) >= 0)
-        long_rows = not trusted or seen[4] > 0
-        shape = loop.grouped_shape(n, env, arrays, self.hw)
-        if shape is None:
-            return False
-        parts, shift, entries = shape
-        # rows per block (blocks of 512 rows where the kept rows hold 7 elements on average - the power-law matrix with
-        # mean 16 - were measured slower: 0.780 ms against 0.745; there are half as many wavefronts to group them)
-        R = int(loop.options.get("hip_group_rows") or 256)
-        nblk = -(-n // R)
-        common = dict(block=256, restrict=spec.restrict)
-        # rows beyond this many elements are cut at the stripes of the gathered operand, the others have their elements
-        # grouped (power-law matrix: 3.14 ms with 128, 3.05 with 256, 3.02 with 512, 3.09 with 1024)
-        cut = max(32 * V, 64 * parts)
-        try:
-            group = loop.kernel_for(Spec("team", vec=1, width=64, parts=parts, aux="group", block_rows=R, skip_long=long_rows, **common))
-            cells = loop.kernel_for(Spec("team", vec=1, width=64, parts=parts, aux="cells", block_rows=R, guard=1, **common))
-            sums = loop.kernel_for(Spec("team", vec=V, width=1, phase=2, guard=1, skip_long=long_rows, **common))
-            plain = loop._choose_spec(n, env, arrays, restrict=spec.restrict, listable=False, hw=self.hw)
-            if plain.kind != "team" or plain.phase or plain.rows:
-                raise Unsupported("no plain team kernel to fall back to")
-            rest = loop.kernel_for(dataclasses.replace(plain, guard=2))
-            if long_rows:
-                ts = 8
-                while ts < parts:
-                    ts *= 2
-                listed = dict(common, rows="list", parts=parts, guard=1)
-                bins = loop.kernel_for(Spec("team", block=1024, vec=1, width=1, restrict=spec.restrict, aux="bins"))
-                plan = loop.kernel_for(Spec("team", vec=1, width=ts, aux="plan", **listed))
-                first = loop.kernel_for(Spec("team", vec=V, width=16, phase=1, stream_loads=spec.stream_loads, **listed))
-                last = loop.kernel_for(Spec("team", vec=V, width=1, phase=2, stream_loads=spec.stream_loads, **listed))
-        except Unsupported:
-            loop._group_off = True
-            return False
-        reds = max(1, len(loop_ir.reductions_of(a.team_split)))
-        cap = 0
-        if long_rows:
-            bound = max([int(arrays[nm].shape[0]) for _code, streamed in loop._simd_loops for nm in streamed
-                         if arrays[nm].ndim == 1] or [0])
-            cap = min(n, bound // cut + 1) if bound else n
-        # one buffer: header (counters of the sorting kernel, the flag) | lists of rows by class | cuts of the long rows |
-        # their starts | their partial results | where the cells start | the grouped elements | sums per row and stripe
-        off_rows = 2048
-        off_bnd = off_rows + (4 * 4 * n if long_rows else 0)
-        off_start = (off_bnd + 4 * (parts + 1) * cap + 255) // 256 * 256
-        off_long = (off_start + 8 * cap + 255) // 256 * 256
-        off_desc = (off_long + 8 * reds * parts * cap + 255) // 256 * 256
-        off_ent = (off_desc + 4 * (parts + 1) * nblk + 255) // 256 * 256
-        off_part = (off_ent + 8 * entries + 255) // 256 * 256
-        buf = loop.scratch(self.device, self.stream, off_part + 4 * parts * n)
-        if buf is None:
-            return False
-        hint_addr, _ = loop.hint(self.device)
-        if trusted:
-            base = max(range(3), key=lambda c: seen[c + 1])
-        else:
-            trip, _uniform = loop._estimate_trip(env, arrays, n)
-            base = sum(1 for t in (V, 8 * V) if trip > t)
-        loop._hint_key[self.device] = ident
-        self.bin = {"flag": buf + 1984, "desc": buf + off_desc, "ent": buf + off_ent, "shiftc": shift, "entries": entries,
-                    # (one limit in every form: rows beyond it are cut at the stripes when the launch has kernels for
-                    #  them, and reported by the grouping kernel when it has not)
-                    "rowmax": cut, "hint": hint_addr,
-                    "counts": buf, "load": buf + 32, "zero": buf + 1024, "rows": buf + off_rows, "m": n, "base": base,
-                    "threshold": [V, 8 * V, cut], "bnd": buf + off_bnd, "rowstart": buf + off_start, "cap": cap,
-                    "stripe": -(-int(arrays[g["x"]].shape[0]) // parts), "nrows": buf + 4 * 3}
-        self.scratch_ptr = buf + off_part
-        self.nsplit = parts
-        # the flag starts at zero, and with it the counters of the sorting kernel
-        seq = [(None, ((buf, 2048) if long_rows else (buf + 1984, 8)), None, None)]
-        if long_rows:
-            seq.append((bins, self._argument_block(bins, vals, arrays, lo, hi), (max(1, min(512, -(-n // 4096))), 1, 1), (1024, 1, 1)))
-        seq.append((group, self._argument_block(group, vals, arrays, lo, hi), (max(1, min(1 << 20, -(-nblk // 4))), 1, 1), (256, 1, 1)))
-        seq.append((cells, self._argument_block(cells, vals, arrays, lo, hi), (8 * max(1, min(8192, -(-nblk // 4))), 1, 1), (256, 1, 1)))
-        args_of_cells = seq[-1]
-        seq.append((sums, self._argument_block(sums, vals, arrays, lo, hi), (max(1, min(4096, -(-n // 256))), 1, 1), (256, 1, 1)))
-        if long_rows:
-            self.bin["rows"] = buf + off_rows + 4 * 3 * n         # the list of the longest class
-            self.scratch_ptr = buf + off_long
-            seq.append((plan, self._argument_block(plan, vals, arrays, lo, hi), (max(1, min(2048, -(-cap * ts // 256))), 1, 1), (256, 1, 1)))
-            seq.append((first, self._argument_block(first, vals, arrays, lo, hi), (max(8, min(2048, 8 * -(-cap * 16 // 256))), 1, 1), (256, 1, 1)))
-            seq.append((last, self._argument_block(last, vals, arrays, lo, hi), (max(1, min(1024, -(-cap // 256))), 1, 1), (256, 1, 1)))
-        # (the kernel that runs the loop row by row when the input was refused: few workgroups that loop - it returns at
-        #  once otherwise, and 65536 workgroups take 15 us to do that, 1024 take 3)
-        seq.append((rest, self._argument_block(rest, vals, arrays, lo, hi),
-                    (min(1024, loop.grid_for(plain, n, cus=self.hw.cus, kernel=rest, row_hint=loop.row_hint(n, env, arrays))), 1, 1), (plain.block, 1, 1)))
-        self.sequence = seq
-        self.kernel, self.spec = cells, cells.src.spec
-        self.args, self.grid, self.block = args_of_cells[1], args_of_cells[2], args_of_cells[3]
-        if trusted and not self.plan_pending and not loop._value_only and not self.small:
-            # (these kernels read the arrays themselves at every launch: a call with the same tensors may repeat them as they
-            #  are while the last launch reports the classes of rows that this form was chosen for)
-            self.seq_replay = ("hints", loop._scratch_gen, ident, tuple(seen))
-        return True
-
-    def _hint_identity(self, arrays, lo, hi):
-        """Names the arrays the lengths of the rows come from (address and shape, not contents): what a launch
-        reports about the rows is only believed by a launch over the same arrays."""
-        out = [lo, hi]
-        for nm in self.loop.plan_arrays():
-            v = arrays[nm]
-            out.append((nm, v.ctypes.data if isinstance(v, np.ndarray) else v.data_ptr(), tuple(v.shape)))
-        return tuple(out)
-
-    def _plan_identity(self, arrays, lo, hi, vals):
-        """``(key, tensors)`` naming the contents a row plan of this launch would describe, or None when
-        they cannot be named: every array the plan reads must be a tensor on the GPU (its version counter
-        tells of in-place changes)."""
-        loop = self.loop
-        names = loop.plan_arrays()
-        tensors, key = [], [self.device, lo, hi, int(arrays[loop.analysis.grouping["x"]].shape[0])]
-        for nm in names:
-            t = arrays[nm]
-            if isinstance(t, np.ndarray) or not getattr(t, "is_cuda", False) or not hasattr(t, "_version"):
-                return None
-            tensors.append(t)
-            key.append((nm, t.data_ptr(), tuple(t.shape), tuple(t.stride()), t._version))
-        for nm in loop.arg_names:
-            if nm in loop.analysis.scalars:
-                v = vals[nm]
-                key.append((nm, v.item() if isinstance(v, np.generic) else v))
-        return tuple(key), tensors
-
-    def _stage_planned(self, vals, arrays, lo, hi, spec) -> bool:
-        """The launches of a loop whose elements have been ordered by an earlier launch with the same arrays
-        (a row plan): the kernel that runs the plan, then the kernel that adds the sums of a row's eight
-        column ranges and runs the rest of the body.  A plan is built the second time a set of arrays is
-        seen unchanged (`hip_reuse="now"`: the first time, `hip_reuse=k`: the k-th); before that the launch takes the forms that
-        keep nothing.  False (nothing staged) when the launch does not qualify or has no plan yet."""
-        loop, a, env = self.loop, self.loop.analysis, self.env
-        reuse = loop.options.get("hip_reuse", True)
-        if a.grouping is None or not reuse or loop._plan_off or self.capture is not None:
-            # (a launch recorded into a graph is replayed without being staged again: it must read the arrays
-            #  themselves every time, not an order worked out from what they held when it was recorded)
-            return False
-        n = hi - lo
-        ident = self._plan_identity(arrays, lo, hi, vals)
-        if ident is None:
-            return False
-        key, tensors = ident
-        plan = None
-        if any(not pl.valid for pl in loop._plans):
-            # plans that a store into their arrays has made untrue: their memory goes back once the launches
-            # that were queued with them have finished
-            with loop._lock:
-                dead = [pl for pl in loop._plans if not pl.valid]
-                loop._plans = [pl for pl in loop._plans if pl.valid]
-            rt.device_sync()
-            for pl in dead:
-                pl.release()
-        with loop._lock:
-            for cand in loop._plans:
-                if cand.key == key and cand.alive(tensors):
-                    plan = cand
-                    loop._plans.remove(cand)
-                    loop._plans.append(cand)
-                    break
-        if plan is None:
-            if key in loop._plan_refused:
-                return False
-            shape = loop.plan_shape(n, env, arrays, self.hw)
-            if shape is None:
-                return False
-            import weakref
-
-            with loop._lock:
-                # sightings of these very tensor objects (an address is handed out again once a tensor is freed)
-                count, refs = loop._plan_seen.get(key, (0, ()))
-                if not (len(refs) == len(tensors) and all(r() is t for r, t in zip(refs, tensors))):
-                    count, refs = 0, tuple(weakref.ref(t) for t in tensors)
-                seen = count + 1
-                if len(loop._plan_seen) > 64:
-                    loop._plan_seen.clear()
-                loop._plan_seen[key] = (seen, refs)
-            # the sighting at which the order is worked out: the second by default, the first with "now", the k-th with
-            # an integer k (working it out costs some eight launches over the raw arrays: a program that knows it will
-            # launch a few times only may ask for a later sighting, or switch the reuse off)
-            wanted = 1 if reuse == "now" else (max(1, reuse) if isinstance(reuse, int) and not isinstance(reuse, bool) else 2)
-            if seen < wanted:
-                # (the next launch over these tensors may build a plan: this one must not be repeated in its place)
-                self.plan_pending = True
-                return False
-            plan = self._build_plan(key, tensors, shape, vals, arrays, lo, hi, spec)
-            if plan is None:
-                return False
-        V = spec.vec
-        try:
-            cells = loop.kernel_for(plan_kernel_spec(plan.tile, plan.entries, n, spec.restrict))
-            sums = loop.kernel_for(Spec("team", block=256, vec=V, width=1, phase=2, guard=1, restrict=spec.restrict))
-        except Unsupported:
-            loop._plan_off = True
-            return False
-        self.bin = dict(plan.bin)
-        split = plan.split
-        self.bin["split"] = split
-        self.scratch_ptr = loop.scratch(self.device, self.stream, 4 * PLAN_GROUPS * split * n)
-        if self.scratch_ptr is None:
-            return False
-        self.nsplit = PLAN_GROUPS * split
-        self.plan = plan
-        seq = [(cells, self._argument_block(cells, vals, arrays, lo, hi), (plan.grid, 1, 1), (1024, 1, 1)),
-               (sums, self._argument_block(sums, vals, arrays, lo, hi), (max(1, min(4096, -(-n // 256))), 1, 1), (256, 1, 1))]
-        self.sequence = seq
-        self.kernel, self.spec = cells, cells.src.spec
-        self.args, self.grid, self.block = seq[0][1], seq[0][2], seq[0][3]
-        if not loop._value_only and not self.small:
-            # a call with these same tensors may repeat the two launches without staging them again, as long as the plan
-            # stands (`CompiledLoop._sequence_still_right`)
-            import weakref
-
-            self.seq_replay = ("plan", loop._scratch_gen, plan,
-                               [(loop.arg_names.index(nm), weakref.ref(t), t._version) for nm, t in zip(loop.plan_arrays(), tensors)])
-        return True
-
-    def _build_plan(self, key, tensors, shape, vals, arrays, lo, hi, spec):
-        """Runs the inspector for these arrays: the generated kernel writes one (key, value) pair per element, the
-        library sorts the pairs and lays out cells, tiles and slots.  Waits for the device after that kernel, to learn
-        whether the arrays were accepted (row ranges that follow one another, indices inside the operand) and whether
-        every position holds an element, and once more at the end."""
-        loop = self.loop
-        n = hi - lo
-        try:
-            rkeys = loop.kernel_for(Spec("team", block=256, vec=1, width=64, aux="rkeys", block_rows=256, restrict=spec.restrict))
-        except Unsupported:
-            loop._plan_off = True
-            return None
-        lib = rt.lib()
-        temp_bytes, max_tiles, words = C.c_size_t(0), C.c_size_t(0), C.c_size_t(0)
-        rt.check(lib.appy_hip_rowplan_sizes(C.byref(shape), C.byref(temp_bytes), C.byref(max_tiles), C.byref(words)))
-        entries = int(shape.entries)
-        ncell = int(shape.row_blocks) * int(shape.groups)
-        limit = scratch_limit(self.device)
-        slack = 4 * int(shape.tile)      # the kernel that runs the plan reads whole tiles, a few beyond the end of a cell
-        kept = 8 * (entries + slack) + 4 * (words.value + slack) + 8 * (ncell + 1) + 256
-        if kept + 16 * entries + temp_bytes.value > limit:
-            return None
-        # older plans of this loop make room first (their launches have been queued before this one on their streams)
-        with loop._lock:
-            old = [pl for pl in loop._plans if not pl.valid] + [pl for pl in loop._plans if pl.valid][:-(PLANS_PER_LOOP - 1) or None]
-            loop._plans = [pl for pl in loop._plans if pl not in old]
-        if old:
-            rt.device_sync()
-            for pl in old:
-                pl.release()
-        import weakref
-
-        plan = RowPlan(self.device, key, [weakref.ref(t) for t in tensors],
-                       [(t.data_ptr(), t.numel() * t.element_size()) for t in tensors])
-        temps = []
-        t0 = t1 = None
-        try:
-            elements = plan.alloc(8 * (entries + slack))
-            cstart = plan.alloc(4 * (ncell + 1))
-            tbase = plan.alloc(4 * (ncell + 1))
-            rstream = plan.alloc(4 * (words.value + slack))
-            flag = plan.alloc(256)
-            for nb in (4 * entries, 8 * entries, 4 * entries, temp_bytes.value):
-                temps.append(rt.malloc(max(256, nb)))
-            keys, pairs, keys_sorted, temp = temps
-            rkeys_fn = rkeys.function(self.device)      # (loads the code object: not part of the inspector's time)
-            t0, t1 = rt.Event(), rt.Event()
-            t0.record(self.stream)
-            rt.memset_async(keys, 0xFF, 4 * entries, self.stream)
-            rt.memset_async(flag, 0, 256, self.stream)
-            self.bin = {"keys": keys, "vals": pairs, "entries": entries, "nx": int(arrays[loop.analysis.grouping["x"]].shape[0]),
-                        "lbits": int(shape.line_bits), "flag": flag}
-            args = self._argument_block(rkeys, vals, arrays, lo, hi)
-            nblk = -(-n // 256)
-            rt.launch(rkeys_fn, (max(1, min(1 << 20, -(-nblk // 4))), 1, 1), (256, 1, 1), args, self.stream)
-            # what the kernel found: whether the arrays are accepted, and how many positions the rows cover - all of them
-            # (the usual case: a loop over all rows of a CSR matrix) means that the sort needs one pass less
-            words = (C.c_int64 * 2)(0, 0)
-            rt.memcpy_d2h(C.addressof(words), flag, 16, self.stream)      # waits for the stream
-            word = C.c_int64(words[0])
-            if not word.value:
-                shape.full = 1 if words[1] == entries else 0
-                rt.check(lib.appy_hip_rowplan_build(C.byref(shape), keys, pairs, keys_sorted, elements, temp, temp_bytes.value,
-                                                    cstart, tbase, rstream, self.stream))
-            t1.record(self.stream)
-            rt.sync(self.stream)          # (the temporary arrays go back below)
-            plan.inspector_ms = t0.elapsed_ms(t1)
-        except BaseException:
-            plan.release()
-            raise
-        finally:
-            for ptr in temps:
-                rt.free(ptr)
-        if word.value:
-            plan.release()
-            loop._plan_refused.add(key)
-            return None
-        plan.bin = {"ent": elements, "cstart": cstart, "tbase": tbase, "rstream": rstream, "ncell": ncell,
-                    "gwidth": int(shape.group_width), "colbits": int(shape.col_bits), "flag": flag,
-                    "nx": int(arrays[loop.analysis.grouping["x"]].shape[0])}
-        plan.ncell = ncell
-        plan.tile = int(shape.tile)
-        # few cells (a matrix of few blocks of rows): several workgroups share a cell, each with a run of its tiles,
-        # until there are some four workgroups per compute unit or a workgroup is down to two tiles
-        # how the tiles lie over the cells decides how many workgroups share a cell and which runs a workgroup gets
-        tb = np.empty(ncell + 1, dtype=np.uint32)
-        rt.memcpy_d2h(tb.ctypes.data, tbase, 4 * (ncell + 1), self.stream)
-        tiles = np.diff(tb.astype(np.int64))
-        plan.split = plan_split(tiles, self.hw.cus, plan.tile, entries, loop.options.get("hip_plan_split"))
-        # one workgroup per CU (their LDS allows no more), a multiple of eight so that a workgroup stays with one column
-        # range; each walks the tiles of its runs as one sequence
-        grid = min(ncell * plan.split, int(loop.options.get("hip_plan_grid") or max(8, self.hw.cus // 8 * 8)))
-        plan.grid = max(8, grid // 8 * 8)
-        order = deal_runs(tiles, plan.split, plan.grid)
-        try:
-            dealt = plan.alloc(4 * len(order))
-            rt.memcpy_h2d(dealt, order.ctypes.data, 4 * len(order), self.stream)
-        except BaseException:
-            plan.release()
-            raise
-        plan.bin["order"], plan.bin["norder"] = dealt, len(order)
-        plan.entries = entries
-        plan.valid = True
-        plan.owner = loop
-        with loop._lock:
-            loop._plans.append(plan)
-            # what the launches before this one needed on this stream (8 bytes per element for the grouped form) is
-            # not needed by the launches that run the plan; the stream has just been waited for
-            stale = loop._scratch.pop((self.device, self.stream), None)
-            loop._scratch_gen += 1
-        if stale is not None:
-            rt.free(stale[0])
-        with _plans_lock:
-            _live_plans.append(plan)
-        loop.last_plan = plan
-        return plan
 
     def _argument_block(self, kernel, vals, arrays, lo, hi):
         loop = self.loop
