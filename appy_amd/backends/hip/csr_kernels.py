@@ -329,7 +329,6 @@ class CsrKernels:
             w("}")
         w(f"const appy::i64 __nblk = (__hi - __lo + {R - 1}) / {R};")
         w("const int __cmask = (1 << __shiftc) - 1;")
-        w("const unsigned long long __below = (1ull << __lid) - 1ull;")
         w("for (appy::i64 __b = (appy::i64)blockIdx.x * 4 + __wvl; __b < __nblk; __b += (appy::i64)gridDim.x * 4) {")
         self.ind += 1
         w(f"const appy::i64 __r0 = __lo + __b * {R};")
@@ -402,18 +401,31 @@ class CsrKernels:
             w(f"for (int __s = 0; __s < {S}; ++__s) __at[__s + 1] = __at[__s] + __cnt[__s];")
             w("#pragma unroll")
             w(f"for (int __s = 0; __s <= {S}; ++__s) if (__lid == __s) __desc[__b * {S + 1} + __s] = __at[__s];")
+            w("int __atv = 0;       // lane s: where the next element of stripe s goes")
+            w("#pragma unroll")
+            w(f"for (int __s = 0; __s < {S}; ++__s) __atv = __lid == __s ? __at[__s] : __atv;")
 
         def place_one(kc, kv):
             w(f"const int __cq = __c[{kc}][__q];")
             w("const int __sq = __cq >> __shiftc;          // negative past the end (and for negative indices: such elements are dropped)")
-            w("int __pos = 0;")
+            # the lanes whose element goes to the same stripe, from one ballot per bit of the stripe number (a lane whose
+            # bit is set keeps the lanes of the ballot, the others keep the rest); lane s holds where stripe s stands
+            w(f"const bool __ok = __sq >= 0 && __sq < {S};")
+            w("const unsigned long long __okm = __ballot(__ok);")
+            w("unsigned __olo = (unsigned)__okm, __ohi = (unsigned)(__okm >> 32);")
             w("#pragma unroll")
-            w(f"for (int __s = 0; __s < {S}; ++__s) {{")
-            w("    const unsigned long long __m = __ballot(__sq == __s);")
-            w("    if (__sq == __s) __pos = __at[__s] + __popcll(__m & __below);")
-            w("    __at[__s] += __popcll(__m);")
+            w(f"for (int __bit = 0; __bit < {(S - 1).bit_length()}; ++__bit) {{")
+            w("    const unsigned __e = (unsigned)((__sq << (31 - __bit)) >> 31);       // all ones where the bit is set")
+            w("    const unsigned long long __bm = __ballot(__e != 0u);")
+            w("    __olo &= ~((unsigned)__bm ^ __e);")
+            w("    __ohi &= ~((unsigned)(__bm >> 32) ^ __e);")
             w("}")
-            w(f"if (__sq >= 0 && __sq < {S})")
+            w("const int __pos = __builtin_amdgcn_ds_bpermute(__sq << 2, __atv) "
+              "+ (int)__builtin_amdgcn_mbcnt_hi(__ohi, __builtin_amdgcn_mbcnt_lo(__olo, 0u));")
+            w("// every lane tells the lane of its stripe how many elements the stripe takes in this step (all of them the same")
+            w("// number; a lane that no one tells receives zero; a lane without an element tells what holds for the number it has)")
+            w("__atv += __builtin_amdgcn_ds_permute(__sq << 2, __popc(__olo) + __popc(__ohi));")
+            w("if (__ok)")
             w("    __ent[__pos] = (long long)(((unsigned long long)(((unsigned)__row << 22) | (unsigned)(__cq & __cmask)) << 32) "
               f"| (unsigned long long)(unsigned)__v[{kv}][__q]);")
 

@@ -24,7 +24,6 @@ _spmv_kernel_loop_1_group(
     int* __hq = __hq_all[__wvl];
     const appy::i64 __nblk = (__hi - __lo + 255) / 256;
     const int __cmask = (1 << __shiftc) - 1;
-    const unsigned long long __below = (1ull << __lid) - 1ull;
     for (appy::i64 __b = (appy::i64)blockIdx.x * 4 + __wvl; __b < __nblk; __b += (appy::i64)gridDim.x * 4) {
         const appy::i64 __r0 = __lo + __b * 256;
         const int __nr = (int)((__hi - __r0) < 256 ? (__hi - __r0) : 256);
@@ -99,6 +98,9 @@ _spmv_kernel_loop_1_group(
         for (int __s = 0; __s < 8; ++__s) __at[__s + 1] = __at[__s] + __cnt[__s];
         #pragma unroll
         for (int __s = 0; __s <= 8; ++__s) if (__lid == __s) __desc[__b * 9 + __s] = __at[__s];
+        int __atv = 0;       // lane s: where the next element of stripe s goes
+        #pragma unroll
+        for (int __s = 0; __s < 8; ++__s) __atv = __lid == __s ? __at[__s] : __atv;
         for (int __j0 = __first; __j0 < __end; __j0 += 1024) {
             appy::vec<int, 4>::type __c[4], __v[4];
             #pragma unroll
@@ -130,14 +132,21 @@ _spmv_kernel_loop_1_group(
                     if (__j + __q < __end) while (__lp[__row + 1] <= __j + __q) ++__row;
                     const int __cq = __c[__k][__q];
                     const int __sq = __cq >> __shiftc;          // negative past the end (and for negative indices: such elements are dropped)
-                    int __pos = 0;
+                    const bool __ok = __sq >= 0 && __sq < 8;
+                    const unsigned long long __okm = __ballot(__ok);
+                    unsigned __olo = (unsigned)__okm, __ohi = (unsigned)(__okm >> 32);
                     #pragma unroll
-                    for (int __s = 0; __s < 8; ++__s) {
-                        const unsigned long long __m = __ballot(__sq == __s);
-                        if (__sq == __s) __pos = __at[__s] + __popcll(__m & __below);
-                        __at[__s] += __popcll(__m);
+                    for (int __bit = 0; __bit < 3; ++__bit) {
+                        const unsigned __e = (unsigned)((__sq << (31 - __bit)) >> 31);       // all ones where the bit is set
+                        const unsigned long long __bm = __ballot(__e != 0u);
+                        __olo &= ~((unsigned)__bm ^ __e);
+                        __ohi &= ~((unsigned)(__bm >> 32) ^ __e);
                     }
-                    if (__sq >= 0 && __sq < 8)
+                    const int __pos = __builtin_amdgcn_ds_bpermute(__sq << 2, __atv) + (int)__builtin_amdgcn_mbcnt_hi(__ohi, __builtin_amdgcn_mbcnt_lo(__olo, 0u));
+                    // every lane tells the lane of its stripe how many elements the stripe takes in this step (all of them the same
+                    // number; a lane that no one tells receives zero; a lane without an element tells what holds for the number it has)
+                    __atv += __builtin_amdgcn_ds_permute(__sq << 2, __popc(__olo) + __popc(__ohi));
+                    if (__ok)
                         __ent[__pos] = (long long)(((unsigned long long)(((unsigned)__row << 22) | (unsigned)(__cq & __cmask)) << 32) | (unsigned long long)(unsigned)__v[__k][__q]);
                 }
             }
