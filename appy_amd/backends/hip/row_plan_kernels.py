@@ -119,16 +119,32 @@ class RowPlanKernels:
         w("    const int __mid = (__row + __past) >> 1;")
         w("    if (__lp[__mid] <= __j) __row = __mid; else __past = __mid;")
         w("}")
+        # (four keys and four values leave as vectors where the lane holds four elements inside the operand: one store
+        #  of 16 bytes and two instead of eight single ones)
+        w("appy::vec<unsigned, 4>::type __kq;")
+        w("appy::vec<unsigned long long, 4>::type __vq;")
+        w("bool __all = __j + 4 <= __end;")
         w("#pragma unroll")
         w("for (int __q = 0; __q < 4; ++__q) {")
-        w("    if (__j + __q >= __end) break;")
-        w("    while (__lp[__row + 1] <= __j + __q) ++__row;")
+        w("    if (__j + __q < __end) while (__lp[__row + 1] <= __j + __q) ++__row;")
         w(f"    const {ic} __cq = __c[__q];")
-        w("    if (__cq < 0 || __cq >= __nx) { __inside = false; continue; }")
+        w("    const bool __in = __cq >= 0 && __cq < __nx;")
+        w("    if (__j + __q < __end && !__in) __inside = false;")
+        w("    __all = __all && __in;")
         w("    const unsigned __rel = __rel0 + (unsigned)__row;")
-        w(f"    __keys[__j + __q] = ((__rel >> {RB}) << __lbits) | ((unsigned)__cq >> 5);")
-        w(f"    __vals[__j + __q] = (unsigned long long)(unsigned)__v[__q] | ((unsigned long long)((__rel & {(1 << RB) - 1}u) "
+        w(f"    __kq[__q] = ((__rel >> {RB}) << __lbits) | ((unsigned)__cq >> 5);")
+        w(f"    __vq[__q] = (unsigned long long)(unsigned)__v[__q] | ((unsigned long long)((__rel & {(1 << RB) - 1}u) "
           f"| (((unsigned)__cq & 31u) << {RB})) << 32);")
+        w("}")
+        w("if (__all) {")
+        w("    appy::vstore<unsigned, 4>(__keys + __j, __kq);")
+        w("    appy::vstore<unsigned long long, 4>(__vals + __j, __vq);")
+        w("} else {")
+        w("#pragma unroll")
+        w("    for (int __q = 0; __q < 4; ++__q) {")
+        w(f"        const {ic} __cq = __c[__q];")
+        w("        if (__j + __q < __end && __cq >= 0 && __cq < __nx) { __keys[__j + __q] = __kq[__q]; __vals[__j + __q] = __vq[__q]; }")
+        w("    }")
         w("}")
         self.ind -= 1
         w("}")

@@ -93,15 +93,29 @@ _spmv_kernel_loop_1_rkeys(
                     const int __mid = (__row + __past) >> 1;
                     if (__lp[__mid] <= __j) __row = __mid; else __past = __mid;
                 }
+                appy::vec<unsigned, 4>::type __kq;
+                appy::vec<unsigned long long, 4>::type __vq;
+                bool __all = __j + 4 <= __end;
                 #pragma unroll
                 for (int __q = 0; __q < 4; ++__q) {
-                    if (__j + __q >= __end) break;
-                    while (__lp[__row + 1] <= __j + __q) ++__row;
+                    if (__j + __q < __end) while (__lp[__row + 1] <= __j + __q) ++__row;
                     const int __cq = __c[__q];
-                    if (__cq < 0 || __cq >= __nx) { __inside = false; continue; }
+                    const bool __in = __cq >= 0 && __cq < __nx;
+                    if (__j + __q < __end && !__in) __inside = false;
+                    __all = __all && __in;
                     const unsigned __rel = __rel0 + (unsigned)__row;
-                    __keys[__j + __q] = ((__rel >> 15) << __lbits) | ((unsigned)__cq >> 5);
-                    __vals[__j + __q] = (unsigned long long)(unsigned)__v[__q] | ((unsigned long long)((__rel & 32767u) | (((unsigned)__cq & 31u) << 15)) << 32);
+                    __kq[__q] = ((__rel >> 15) << __lbits) | ((unsigned)__cq >> 5);
+                    __vq[__q] = (unsigned long long)(unsigned)__v[__q] | ((unsigned long long)((__rel & 32767u) | (((unsigned)__cq & 31u) << 15)) << 32);
+                }
+                if (__all) {
+                    appy::vstore<unsigned, 4>(__keys + __j, __kq);
+                    appy::vstore<unsigned long long, 4>(__vals + __j, __vq);
+                } else {
+                #pragma unroll
+                    for (int __q = 0; __q < 4; ++__q) {
+                        const int __cq = __c[__q];
+                        if (__j + __q < __end && __cq >= 0 && __cq < __nx) { __keys[__j + __q] = __kq[__q]; __vals[__j + __q] = __vq[__q]; }
+                    }
                 }
             }
         }

@@ -811,8 +811,9 @@ def test_row_plans_kernel_that_writes_the_pairs_and_kernel_that_runs_a_plan():
     f, _ = selfcheck_loop("spmv")
     keys = body_of(f.kernel_for(Spec("team", block=256, vec=1, width=64, aux="rkeys", block_rows=256)).src.text)
     assert "__lp[__r + 1] == __hq[__r]" in keys and "__flag[0] = 1" in keys
-    assert "if (__cq < 0 || __cq >= __nx) { __inside = false; continue; }" in keys
-    assert "__keys[__j + __q] = ((__rel >> 15) << __lbits) | ((unsigned)__cq >> 5);" in keys
+    assert "const bool __in = __cq >= 0 && __cq < __nx;" in keys and "if (__j + __q < __end && !__in) __inside = false;" in keys
+    assert "appy::vstore<unsigned, 4>(__keys + __j, __kq);" in keys         # four pairs of a lane leave as vectors
+    assert "__kq[__q] = ((__rel >> 15) << __lbits) | ((unsigned)__cq >> 5);" in keys
     assert "x[" not in keys.split("{", 1)[1]                                  # the gathered operand is not read here
     for unroll, tile in ((6, 6144), (4, 4096)):
         run = body_of(f.kernel_for(Spec("team", block=1024, vec=1, width=1024, unroll=unroll, parts=8, aux="xcells")).src.text)
